@@ -1,0 +1,120 @@
+"""The batch of one step: ragged segments of (request, its next tokens).
+
+All integer metadata of a step is laid out in one host array and reaches the
+device in one copy: token ids, positions, the segment of each token, per
+segment the offset of its first token, its length, the context length after
+the step and its state slot, the rows whose logits are wanted, and per page
+group the block tables [segments, max_blocks] and the page slot of every
+token.  The reference builds the same flat layout (src/llaisys/models/qwen2.cpp:942-957)
+but uploads the tables again for every layer (:993-1007).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, Hashable, List, Sequence
+
+import numpy as np
+import torch
+
+
+@dataclass
+class StepEntry:
+    rid: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()          # places among `tokens` whose logits are asked for
+
+
+@dataclass
+class AttentionMeta:
+    """Device arrays the attention kernels index, and the host numbers their
+    launches are sized by."""
+    block_table: torch.Tensor        # [segments, max_blocks] int32, -1 = given back
+    max_blocks: int
+    seg_of_token: torch.Tensor       # [T]
+    q_start: torch.Tensor            # [segments]
+    q_len: torch.Tensor              # [segments]
+    ctx_len: torch.Tensor            # [segments]  cached length after this step
+    num_segments: int
+    num_tokens: int
+    max_q_len: int
+    max_ctx_len: int
+    host_q_start: np.ndarray
+    host_q_len: np.ndarray
+    host_ctx_len: np.ndarray
+    extra: Dict[Any, Any] = field(default_factory=dict)    # what kernels derive and keep for the step
+
+
+class StepContext:
+    """What parts may read during a step."""
+
+    def __init__(self, ws, num_tokens: int, num_segments: int):
+        self.ws = ws
+        self.num_tokens = num_tokens
+        self.num_segments = num_segments
+        self.ids: torch.Tensor = None
+        self.positions: torch.Tensor = None
+        self.state_slots: torch.Tensor = None        # [segments] int32, device
+        self.host_state_slots: np.ndarray = None
+        self.host_q_start: np.ndarray = None
+        self.host_q_len: np.ndarray = None
+        self.host_ctx_len: np.ndarray = None
+        self.want_rows: torch.Tensor = None
+        self.num_want = 0
+        self._slot_maps: List[torch.Tensor] = []
+        self._attn: List[AttentionMeta] = []
+        self._shared: Dict[Any, Any] = {}
+
+    def slot_map(self, group: int) -> torch.Tensor:
+        return self._slot_maps[group]
+
+    def attention_meta(self, group: int) -> AttentionMeta:
+        return self._attn[group]
+
+    def shared(self, key, make: Callable[[], Any]):
+        """Per-step value shared by every part that asks with the same key."""
+        if key not in self._shared:
+            self._shared[key] = make()
+        return self._shared[key]
+
+
+class BatchUploader:
+    """Packs the step's integers into pinned host memory and copies them to
+    the device once.  Two host buffers alternate, each guarded by an event, so
+    a buffer is not rewritten while its copy may still be in flight."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        self._host = [None, None]
+        self._events = [None, None]
+        self._dev = None
+        self._turn = 0
+
+    def upload(self, parts: List[np.ndarray]) -> List[torch.Tensor]:
+        offs, total = [], 0
+        for p in parts:
+            offs.append(total)
+            total += (p.size + 3) // 4 * 4            # 16-byte alignment of every array
+        total = max(total, 4)
+        i = self._turn
+        self._turn ^= 1
+        cuda = self.device.type == "cuda"
+        if self._host[i] is None or self._host[i].numel() < total:
+            cap = total * 2
+            self._host[i] = torch.empty(cap, dtype=torch.int32, pin_memory=cuda)
+        elif self._events[i] is not None:
+            self._events[i].synchronize()
+        if self._dev is None or self._dev.numel() < total:
+            self._dev = torch.empty(total * 2, dtype=torch.int32, device=self.device)
+        h = self._host[i].numpy()
+        for p, o in zip(parts, offs):
+            h[o:o + p.size] = p.reshape(-1)
+        if cuda:
+            # a fresh device buffer per step would be simpler; one buffer is enough because the
+            # copy is ordered on the stream after the kernels of the step before
+            self._dev[:total].copy_(self._host[i][:total], non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            self._events[i] = ev
+        else:
+            self._dev[:total].copy_(self._host[i][:total])
+        return [self._dev[o:o + p.size].view(p.shape) for p, o in zip(parts, offs)]

@@ -1,0 +1,232 @@
+"""The engine: a model, its cache and ONE step function.
+
+`step(entries)` takes a batch of (request, its next tokens): portions of
+prompts beside single decoded tokens, cut anywhere.  It runs only the tokens
+it is given, as one batch, against the cache that earlier steps left, and
+returns float32 logits at the wanted places.  Generation (the scheduler) and
+trace replay are two callers of this one function.
+
+The reference's step builds its batch itself from its request list and admits
+only whole prompts and single tokens (src/llaisys/models/qwen2.cpp:922-957);
+its attention already derives each query's horizon as ctx - qlen + i
+(src/ops/paged_attention/op.cpp:204), which is what makes portions sound.
+"""
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Any, Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheFull, CacheManager
+from ..config import load_config, lookup, architecture_name
+from ..config.spec import ModelSpec
+from ..parts.base import Runtime
+from ..weights import load_into, random_tensor
+from .batch import AttentionMeta, BatchUploader, StepContext, StepEntry
+from .model import Model
+from .workspace import Workspace
+
+DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+          "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"engine dtype must be bfloat16 or float32, found {dtype}")
+        return dtype
+    if str(dtype) not in DTYPES:
+        raise ValueError(f"engine dtype must be one of {sorted(DTYPES)}, found {dtype!r}")
+    return DTYPES[str(dtype)]
+
+
+class StepError(ValueError):
+    """The batch is not valid; nothing was changed."""
+
+
+class Engine:
+    def __init__(self, spec: ModelSpec, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
+                 num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
+                 max_seqs: int = 64, page_order_seed: Optional[int] = None,
+                 config: Any = None):
+        self.spec = spec
+        self.config = config
+        self.rt = Runtime(torch.device(device), parse_dtype(dtype))
+        if self.rt.device.type == "cuda":
+            from ..kernels import ops
+            ops.require_gpu(self.rt.device)
+        self.model = Model(spec, self.rt)
+        self.page_size = int(page_size)
+        self.max_seqs = int(max_seqs)
+        self._num_pages = num_pages
+        self._max_tokens = max_tokens
+        self._page_order_seed = page_order_seed
+        self.cache: Optional[CacheManager] = None
+        self.ws = Workspace(self.rt.device)
+        self._uploader = BatchUploader(self.rt.device)
+        self.steps_run = 0
+
+    # ---- construction -----------------------------------------------------
+    @classmethod
+    def from_dir(cls, model_dir, **kw) -> "Engine":
+        """Model class, sizes and constants come from config.json; weights from
+        the folder's safetensors files."""
+        arch, cfg, spec = load_config(model_dir)
+        eng = cls(spec, config=cfg, **kw)
+        load_into(eng.model, model_dir)
+        eng._make_cache()
+        return eng
+
+    @classmethod
+    def from_random(cls, config: Dict[str, Any], seed: int, **kw) -> "Engine":
+        """Random weights drawn straight on the device (no files): for
+        measurements at sizes where writing a checkpoint first would only cost time."""
+        arch = lookup(architecture_name(config))
+        cfg = arch.config_from_dict(config)
+        spec = arch.model_spec(cfg)
+        eng = cls(spec, config=cfg, **kw)
+        expected = eng.model.expected_params()
+        stored = torch.float32 if eng.rt.dtype is torch.float32 else torch.bfloat16
+
+        def get(name):
+            return random_tensor(seed, name, expected[name], stored, device=eng.rt.device)
+
+        eng.model.load_params(get)
+        eng._make_cache()
+        return eng
+
+    def _bytes_per_page(self) -> int:
+        needs, sources = self.model.cache_needs()
+        from ..parts.base import PagedKVNeed
+        es = 4 if self.rt.dtype is torch.float32 else 2
+        return sum(2 * n.num_kv_heads * n.head_dim * self.page_size * es
+                   for n, s in zip(needs, sources) if s is None and isinstance(n, PagedKVNeed))
+
+    def _make_cache(self) -> None:
+        needs, sources = self.model.cache_needs()
+        pages = self._num_pages
+        if pages is None and self._max_tokens is not None:
+            pages = -(-int(self._max_tokens) // self.page_size)
+        if pages is None:
+            per_seq = -(-self.spec.max_positions // self.page_size)
+            pages = per_seq * self.max_seqs
+            if self.rt.device.type == "cuda":
+                free, _ = torch.cuda.mem_get_info(self.rt.device)
+                bpp = max(1, self._bytes_per_page())
+                pages = max(1, min(pages, int(free * 0.85) // bpp))
+        self.cache = CacheManager(needs, sources, page_size=self.page_size, num_pages=int(pages),
+                                  max_seqs=self.max_seqs, dtype=self.rt.dtype, device=self.rt.device,
+                                  page_order_seed=self._page_order_seed)
+
+    # ---- the step ---------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("step: empty batch")
+        seen = set()
+        vocab = self.spec.vocab_size
+        for e in entries:
+            if e.rid in seen:
+                raise StepError(f"step: request {e.rid!r} appears twice in one batch")
+            seen.add(e.rid)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"step: request {e.rid!r} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise StepError(f"step: token id {t} of request {e.rid!r} is outside the "
+                                    f"vocabulary of {vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"step: request {e.rid!r} wants logits at place {w} of {n} tokens")
+            have = self.cache.cached_len(e.rid) if self.cache.has(e.rid) else 0
+            if have + n > self.spec.max_positions:
+                raise StepError(f"step: request {e.rid!r} would reach {have + n} positions, the "
+                                f"model max sequence length is {self.spec.max_positions}")
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Run one batch.  Returns float32 logits [wanted, vocab] in the order of
+        the entries and of their `want` lists, or None when nothing is wanted.
+        Raises StepError for a bad batch and CacheFull when pages or slots do
+        not suffice; in both cases the cache is as before."""
+        self._validate(entries)
+        cache = self.cache
+        admitted, reserved = [], []
+        try:
+            for e in entries:
+                if not cache.has(e.rid):
+                    cache.admit(e.rid)
+                    admitted.append(e.rid)
+            # all-or-nothing over the batch: check the sum first
+            total = [0] * len(cache.groups)
+            for e in entries:
+                for gi, n in enumerate(cache.pages_needed(e.rid, len(e.tokens))):
+                    total[gi] += n
+            for gi, g in enumerate(cache.groups):
+                if total[gi] > g.pool.free:
+                    raise CacheFull(f"step: the batch needs {total[gi]} more pages, "
+                                    f"{g.pool.free} of {g.pool.capacity} are free")
+            for e in entries:
+                cache.reserve(e.rid, len(e.tokens))
+        except CacheFull:
+            for rid in admitted:
+                cache.release(rid)
+            raise
+        ctx = self._build_context(entries)
+        logits = self.model.forward(ctx, cache)
+        for e in entries:
+            cache.commit(e.rid, len(e.tokens))
+        self.steps_run += 1
+        return logits
+
+    def finish(self, rid: Hashable) -> None:
+        """The request is over: what it holds is given back."""
+        if self.cache.has(rid):
+            self.cache.release(rid)
+
+    def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        cache, P = self.cache, self.page_size
+        nseg = len(entries)
+        q_len = np.array([len(e.tokens) for e in entries], dtype=np.int32)
+        q_start = np.zeros(nseg + 1, dtype=np.int32)
+        np.cumsum(q_len, out=q_start[1:])
+        T = int(q_start[-1])
+        cached = np.array([cache.cached_len(e.rid) for e in entries], dtype=np.int32)
+        ctx_len = cached + q_len
+        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+        seg_of_token = np.repeat(np.arange(nseg, dtype=np.int32), q_len)
+        pos = (np.arange(T, dtype=np.int32) - q_start[seg_of_token] + cached[seg_of_token]).astype(np.int32)
+        slots = np.array([cache.slot(e.rid) for e in entries], dtype=np.int32)
+        want = [int(q_start[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
+        want_rows = np.asarray(want, dtype=np.int32)
+        parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows]
+        tables, max_blocks = [], []
+        for gi in range(len(cache.groups)):
+            tabs = [cache.block_table(e.rid, gi) for e in entries]
+            mb = max(1, max(len(t) for t in tabs))
+            tab = np.full((nseg, mb), -1, dtype=np.int32)
+            for i, t in enumerate(tabs):
+                tab[i, :len(t)] = t
+            page = tab[seg_of_token, pos // P]
+            if (page < 0).any():
+                raise AssertionError("step: a token of the batch has no page")
+            slot_map = (page.astype(np.int64) * P + pos % P).astype(np.int32)
+            tables.append(tab)
+            max_blocks.append(mb)
+            parts += [tab, slot_map]
+        dev = self._uploader.upload(parts)
+        ctx = StepContext(self.ws, T, nseg)
+        (ctx.ids, ctx.positions, d_seg, d_qs, d_ql, d_cl, ctx.state_slots, ctx.want_rows) = dev[:8]
+        ctx.num_want = len(want)
+        ctx.host_state_slots = slots
+        ctx.host_q_start, ctx.host_q_len, ctx.host_ctx_len = q_start[:-1], q_len, ctx_len
+        for gi in range(len(cache.groups)):
+            d_tab, d_slot = dev[8 + 2 * gi], dev[9 + 2 * gi]
+            ctx._slot_maps.append(d_slot)
+            ctx._attn.append(AttentionMeta(
+                block_table=d_tab, max_blocks=max_blocks[gi], seg_of_token=d_seg, q_start=d_qs,
+                q_len=d_ql, ctx_len=d_cl, num_segments=nseg, num_tokens=T,
+                max_q_len=int(q_len.max()), max_ctx_len=int(ctx_len.max()),
+                host_q_start=q_start[:-1], host_q_len=q_len, host_ctx_len=ctx_len))
+        return ctx

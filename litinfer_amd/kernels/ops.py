@@ -1,0 +1,319 @@
+"""Python side of the HIP kernels: argument checks and the ctypes calls.
+
+Every function checks on the host that devices, dtypes, shapes and strides are
+what its kernel and launch assume, because a kernel that reads out of bounds
+can take the GPU down.  There is no fallback: on a tensor that is not on the
+GPU, or without the built library, a call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+from typing import Optional
+
+import torch
+
+from . import build
+
+float32 = torch.float32
+bfloat16 = torch.bfloat16
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+MAX_HEAD_DIM = 256
+
+P, I, F, L = c_void_p, c_int, c_float, c_long
+_SIGNATURES = {
+    "elementwise": {
+        "li_embedding": [P, P, I, P, I, I, I],
+        "li_rmsnorm": [P, I, P, F, P, I, I, I],
+        "li_gather_rows": [P, P, P, I, I],
+        "li_cast": [P, I, P, I, L],
+        "li_swiglu": [P, P, I, I, I],
+        "li_rope_table": [P, F, I, P, P, I],
+        "li_rope_apply": [P, I, I, I, I, I, P, P, I],
+        "li_kv_store": [P, I, I, I, I, I, P, P, P, I, I, I],
+        "li_rope_kv_store": [P, I, I, I, I, I, I, P, P, P, P, P, I, I, I],
+    },
+    "gemm": {
+        "li_linear": [P, P, P, P, I, I, I, I, I, I],
+    },
+    "attention": {
+        "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
+    },
+    "sampling": {
+        "li_argmax_rows": [P, P, I, I],
+        "li_sample_rows": [P, P, P, P, P, P, P, P, I, I],
+    },
+}
+_fn_cache = {}
+
+
+def _fn(module: str, name: str):
+    key = (module, name)
+    f = _fn_cache.get(key)
+    if f is None:
+        lib = build.load(module)
+        f = getattr(lib, name)
+        f.argtypes = _SIGNATURES[module][name] + [c_void_p]      # + stream
+        f.restype = c_int
+        _fn_cache[key] = f
+    return f
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _run(module: str, name: str, *args) -> None:
+    rc = _fn(module, name)(*args, _stream())
+    if rc != 0:
+        raise RuntimeError(f"{name}: the kernel library refused the call (code {rc}): "
+                           f"{_ERRORS.get(rc, 'unknown')}")
+
+
+_ERRORS = {1: "unsupported dtype combination", 2: "unsupported size", 3: "launch failed"}
+
+
+def require_gpu(device) -> None:
+    if not torch.cuda.is_available():
+        raise RuntimeError("litinfer_amd runs on an AMD GPU through its HIP kernels; "
+                           "no GPU is visible and there is no CPU path")
+
+
+def _gpu(*ts) -> None:
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("kernel call on a tensor that is not on the GPU "
+                               "(there is no CPU path)")
+
+
+def _chk(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _rows_ok(t: torch.Tensor) -> bool:
+    return t.dim() == 2 and t.stride(1) == 1 and t.stride(0) >= t.shape[1]
+
+
+def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> None:
+    """Sizes the attention and position kernels take; anything else is refused
+    here, when the model is built."""
+    _chk(num_heads > 0 and num_kv_heads > 0 and num_heads % num_kv_heads == 0,
+         f"attention: {num_heads} heads and {num_kv_heads} kv heads: the first must be a "
+         f"multiple of the second")
+    _chk(head_dim % 2 == 0 and 2 <= head_dim <= MAX_HEAD_DIM,
+         f"attention: head size {head_dim} is not supported (even, at most {MAX_HEAD_DIM})")
+
+
+# ---------------------------------------------------------------- elementwise
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, :] = table[ids[t], :] as float32.  Ids must already be inside the
+    table (the step checks them on the host)."""
+    _gpu(ids, table, out)
+    t, h = out.shape
+    _chk(ids.dtype is torch.int32 and ids.numel() == t and ids.is_contiguous(), "embedding: ids")
+    _chk(table.dim() == 2 and table.shape[1] == h and table.is_contiguous() and table.dtype in _DT,
+         "embedding: table")
+    _chk(out.dtype is torch.float32 and out.is_contiguous(), "embedding: out must be float32")
+    if t:
+        _run("elementwise", "li_embedding", ids.data_ptr(), table.data_ptr(), _DT[table.dtype],
+             out.data_ptr(), t, h, table.shape[0])
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    _gpu(x, weight, out)
+    _chk(x.dim() == 2 and x.shape == out.shape and x.is_contiguous() and out.is_contiguous(),
+         "rmsnorm: x and out must be contiguous [T, H] of one shape")
+    _chk(x.dtype in _DT and out.dtype in _DT, "rmsnorm: dtype")
+    _chk(weight.dtype is torch.float32 and weight.numel() == x.shape[1] and weight.is_contiguous(),
+         "rmsnorm: weight must be float32 [H]")
+    if x.shape[0]:
+        _run("elementwise", "li_rmsnorm", x.data_ptr(), _DT[x.dtype], weight.data_ptr(), float(eps),
+             out.data_ptr(), _DT[out.dtype], x.shape[0], x.shape[1])
+
+
+def gather_rows(x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:
+    """out[i, :] = x[rows[i], :]; rows must be valid row numbers of x."""
+    _gpu(x, rows, out)
+    _chk(x.dtype is torch.float32 and out.dtype is torch.float32 and x.is_contiguous()
+         and out.is_contiguous() and x.dim() == 2 and out.dim() == 2 and x.shape[1] == out.shape[1],
+         "gather_rows: x, out")
+    _chk(rows.dtype is torch.int32 and rows.numel() == out.shape[0] and rows.is_contiguous(),
+         "gather_rows: rows")
+    if out.shape[0]:
+        _run("elementwise", "li_gather_rows", x.data_ptr(), rows.data_ptr(), out.data_ptr(),
+             out.shape[0], x.shape[1])
+
+
+def cast(src: torch.Tensor, dst: torch.Tensor) -> None:
+    _gpu(src, dst)
+    _chk(src.numel() == dst.numel() and src.is_contiguous() and dst.is_contiguous()
+         and src.dtype in _DT and dst.dtype in _DT, "cast: src, dst")
+    if src.numel():
+        _run("elementwise", "li_cast", src.data_ptr(), _DT[src.dtype], dst.data_ptr(), _DT[dst.dtype],
+             src.numel())
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, i] = up * gate / (1 + exp(-gate)) with gate = gate_up[t, i],
+    up = gate_up[t, I + i]."""
+    _gpu(gate_up, out)
+    t, inter = out.shape
+    _chk(gate_up.shape == (t, 2 * inter) and gate_up.is_contiguous() and out.is_contiguous()
+         and gate_up.dtype is out.dtype and out.dtype in _DT, "swiglu: gate_up [T, 2I], out [T, I]")
+    if t:
+        _run("elementwise", "li_swiglu", gate_up.data_ptr(), out.data_ptr(), _DT[out.dtype], t, inter)
+
+
+def rope_table(positions: torch.Tensor, theta: float, rotary_dim: int, cos: torch.Tensor,
+               sin: torch.Tensor) -> None:
+    """cos/sin [T, rotary_dim/2] of angle = float(pos) / theta^(2j/rotary_dim), in float32."""
+    _gpu(positions, cos, sin)
+    t = positions.numel()
+    _chk(positions.dtype is torch.int32 and positions.is_contiguous(), "rope_table: positions")
+    _chk(cos.shape == (t, rotary_dim // 2) and sin.shape == cos.shape and cos.is_contiguous()
+         and sin.is_contiguous() and cos.dtype is torch.float32 and sin.dtype is torch.float32,
+         "rope_table: cos, sin")
+    if t:
+        _run("elementwise", "li_rope_table", positions.data_ptr(), float(theta), rotary_dim,
+             cos.data_ptr(), sin.data_ptr(), t)
+
+
+def _check_qkv(qkv, heads_total, head_dim):
+    _chk(_rows_ok(qkv) and qkv.dtype in _DT and qkv.shape[1] >= heads_total * head_dim,
+         "qkv: needs rows of at least heads*head_dim elements")
+
+
+def rope_apply(qkv: torch.Tensor, n_heads: int, head_dim: int, rotary_dim: int, cos: torch.Tensor,
+               sin: torch.Tensor) -> None:
+    """Rotate heads 0..n_heads-1 of every row of qkv in place (half-split pairs)."""
+    _gpu(qkv, cos, sin)
+    _check_qkv(qkv, n_heads, head_dim)
+    t = qkv.shape[0]
+    _chk(cos.shape == (t, rotary_dim // 2) and sin.shape == cos.shape and rotary_dim <= head_dim,
+         "rope_apply: tables")
+    if t:
+        _run("elementwise", "li_rope_apply", qkv.data_ptr(), _DT[qkv.dtype], qkv.stride(0), n_heads,
+             head_dim, rotary_dim, cos.data_ptr(), sin.data_ptr(), t)
+
+
+def _check_cache(k, v, nkv, dh, page_size, dtype):
+    _chk(k.shape == v.shape and k.dim() == 4 and k.shape[1:] == (nkv, page_size, dh)
+         and k.is_contiguous() and v.is_contiguous() and k.dtype is dtype and v.dtype is dtype,
+         "kv cache: expected contiguous [pages, kv_heads, page_size, head_dim] of the activation dtype")
+
+
+def kv_store(qkv: torch.Tensor, nh: int, nkv: int, dh: int, slot_map: torch.Tensor, k: torch.Tensor,
+             v: torch.Tensor, page_size: int) -> None:
+    """Write the key and value heads of every row of qkv (columns nh*dh.. and
+    (nh+nkv)*dh..) to the page slot slot_map[t] = page*page_size + offset."""
+    _gpu(qkv, slot_map, k, v)
+    _check_qkv(qkv, nh + 2 * nkv, dh)
+    _check_cache(k, v, nkv, dh, page_size, qkv.dtype)
+    t = qkv.shape[0]
+    _chk(slot_map.dtype is torch.int32 and slot_map.numel() == t and slot_map.is_contiguous(),
+         "kv_store: slot_map")
+    if t:
+        _run("elementwise", "li_kv_store", qkv.data_ptr(), _DT[qkv.dtype], qkv.stride(0), nh, nkv, dh,
+             slot_map.data_ptr(), k.data_ptr(), v.data_ptr(), page_size, k.shape[0], t)
+
+
+def rope_kv_store(qkv: torch.Tensor, nh: int, nkv: int, dh: int, rotary_dim: int, cos: torch.Tensor,
+                  sin: torch.Tensor, slot_map: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                  page_size: int) -> None:
+    """Fused: rotate the query heads in place, rotate the key heads and write
+    them, and copy the value heads, to the pages."""
+    _gpu(qkv, cos, sin, slot_map, k, v)
+    _check_qkv(qkv, nh + 2 * nkv, dh)
+    _check_cache(k, v, nkv, dh, page_size, qkv.dtype)
+    t = qkv.shape[0]
+    _chk(cos.shape == (t, rotary_dim // 2) and sin.shape == cos.shape and rotary_dim <= dh
+         and cos.dtype is torch.float32, "rope_kv_store: tables")
+    _chk(slot_map.dtype is torch.int32 and slot_map.numel() == t and slot_map.is_contiguous(),
+         "rope_kv_store: slot_map")
+    if t:
+        _run("elementwise", "li_rope_kv_store", qkv.data_ptr(), _DT[qkv.dtype], qkv.stride(0), nh, nkv,
+             dh, rotary_dim, cos.data_ptr(), sin.data_ptr(), slot_map.data_ptr(), k.data_ptr(),
+             v.data_ptr(), page_size, k.shape[0], t)
+
+
+# ---------------------------------------------------------------------- gemm
+def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+           accumulate: bool = False) -> None:
+    """out = x w^T + bias, or out += x w^T + bias when `accumulate`.
+    x [M, K] and w [N, K] of one dtype (float32 or bfloat16); out [M, N] of that
+    dtype or float32; accumulation of the product is float32."""
+    _gpu(x, w, bias, out)
+    _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear: needs matrices")
+    m, k = x.shape
+    n = w.shape[0]
+    _chk(w.shape[1] == k and out.shape == (m, n), f"linear: shapes x {tuple(x.shape)}, "
+         f"w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+    _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear: contiguous operands")
+    _chk(x.dtype is w.dtype and x.dtype in _DT, f"linear: x is {x.dtype}, w is {w.dtype}")
+    _chk(out.dtype is x.dtype or out.dtype is torch.float32, "linear: out dtype")
+    _chk(not accumulate or out.dtype is torch.float32, "linear: accumulation needs a float32 out")
+    _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
+         "linear: bias must be float32 [N]")
+    if m:
+        _run("gemm", "li_linear", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
+             out.data_ptr(), m, n, k, _DT[x.dtype], _DT[out.dtype], int(bool(accumulate)))
+
+
+# ----------------------------------------------------------------- attention
+def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: torch.Tensor, meta,
+                    nh: int, nkv: int, dh: int, page_size: int, window: int, scale: float) -> None:
+    """Causal grouped-query attention of the batch's queries (heads 0..nh-1 of
+    qkv's rows) over the paged keys and values; out [T, nh*dh].  Query i of a
+    segment stands at position ctx_len - q_len + i and sees the keys at
+    positions <= its own and, with window > 0, closer than `window`."""
+    _gpu(qkv, out, k, v, meta.block_table)
+    check_attention_sizes(nh, nkv, dh)
+    _check_qkv(qkv, nh, dh)
+    _check_cache(k, v, nkv, dh, page_size, qkv.dtype)
+    t = qkv.shape[0]
+    _chk(out.shape == (t, nh * dh) and out.is_contiguous() and out.dtype is qkv.dtype, "attention: out")
+    _chk(t == meta.num_tokens, "attention: batch metadata is of another batch")
+    bt = meta.block_table
+    _chk(bt.dtype is torch.int32 and bt.shape == (meta.num_segments, meta.max_blocks)
+         and bt.is_contiguous(), "attention: block table")
+    _chk(meta.max_blocks * page_size >= meta.max_ctx_len, "attention: block table too short")
+    if t:
+        _run("attention", "li_paged_attention", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
+             k.data_ptr(), v.data_ptr(), _DT[qkv.dtype], bt.data_ptr(), meta.max_blocks,
+             meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(),
+             meta.ctx_len.data_ptr(), meta.num_segments, t, meta.max_q_len, meta.max_ctx_len,
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale))
+
+
+# ------------------------------------------------------------------ sampling
+def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """out[i] = index of the maximum of row i, the lowest index on ties."""
+    _gpu(logits, out)
+    _chk(logits.dim() == 2 and logits.dtype is torch.float32 and logits.is_contiguous(), "argmax: logits")
+    _chk(out.dtype is torch.int32 and out.numel() == logits.shape[0] and out.is_contiguous(), "argmax: out")
+    if logits.shape[0]:
+        _run("sampling", "li_argmax_rows", logits.data_ptr(), out.data_ptr(), logits.shape[0],
+             logits.shape[1])
+
+
+def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+                top_p: torch.Tensor, uniform: torch.Tensor, scratch: torch.Tensor,
+                out: torch.Tensor) -> None:
+    """One token per row: temperature <= 0 takes the argmax; else the softmax
+    of logits/temperature, restricted to the top_k largest (0 < top_k < V) and
+    then to the shortest prefix, in descending order, whose mass reaches top_p
+    (0 < top_p < 1), is sampled by inverse CDF over ascending ids with the
+    row's uniform number u in [0, 1).  scratch: float32 [rows, V]."""
+    _gpu(logits, temperature, top_k, top_p, uniform, scratch, out)
+    n, vocab = logits.shape
+    _chk(logits.dtype is torch.float32 and logits.is_contiguous(), "sample: logits")
+    for t_, dt in ((temperature, torch.float32), (top_k, torch.int32), (top_p, torch.float32),
+                   (uniform, torch.float32), (out, torch.int32)):
+        _chk(t_.dtype is dt and t_.numel() == n and t_.is_contiguous(), "sample: per-row arrays")
+    _chk(scratch.dtype is torch.float32 and scratch.numel() >= n * vocab and scratch.is_contiguous(),
+         "sample: scratch")
+    if n:
+        _run("sampling", "li_sample_rows", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(),
+             top_p.data_ptr(), uniform.data_ptr(), scratch.data_ptr(), out.data_ptr(), 0, n, vocab)

@@ -1,0 +1,13 @@
+from .base import (Block, FeedForward, Mixer, Norm, PagedKVNeed, Part, Runtime, StateNeed,
+                   build_part, register_part)
+from .position import Position, RopeNeox
+from .linear import Linear
+from .norm import RMSNorm
+from .attention import GQAttention
+from .mlp import SwiGLUMLP
+from .block import PreNormBlock
+from .embedding import LinearHead, TokenEmbedding
+
+__all__ = ["Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "Part", "Runtime", "StateNeed",
+           "build_part", "register_part", "Position", "RopeNeox", "Linear", "RMSNorm",
+           "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding"]

@@ -1,0 +1,134 @@
+"""Interfaces of the parts a layer is put together from, and their registry.
+
+A part is built from a `PartSpec` (its sizes and constants, and the prefix of
+its tensors) and a `Runtime` (device and activation dtype).  It says which
+tensors it expects, takes them, and then runs on the step's batch.  No part
+knows which model it is in; the model and the block only use what is written
+here.
+
+Interfaces (T = tokens of the step, H = hidden size):
+
+* Norm.forward(x [T, H] float32) -> [T, H] in the activation dtype.
+* Mixer.cache_need() -> PagedKVNeed | StateNeed | None;
+  Mixer.forward(xn [T, H], residual [T, H] float32, ctx, cache): ADDS its
+  output to `residual` in 32-bit.  `cache` is the CacheView of the entry of the
+  execution order that is running; `cache.owned` is False when the entry reads
+  another entry's cache and must write nothing.
+* FeedForward.forward(xn, residual): adds its output to `residual`.
+* Position: prepares per-step tables and rotates (or otherwise encodes) the
+  mixer's queries and keys; see `parts/position.py`.
+* Block.forward(x [T, H] float32 residual stream, ctx, cache).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Callable, Dict, Optional, Tuple
+
+import torch
+
+from ..config.spec import PartSpec
+from ..weights.loader import ParamSpec
+
+
+@dataclass(frozen=True)
+class Runtime:
+    """Where and in which precision a model runs.  `dtype` is the activation and
+    matrix dtype: torch.bfloat16 (serving) or torch.float32 (everything in true
+    32-bit)."""
+    device: torch.device
+    dtype: torch.dtype
+
+    def matrix(self, t: torch.Tensor) -> torch.Tensor:
+        """A stored matrix as this runtime multiplies with it.  In 32-bit mode
+        everything is widened (exactly); in bfloat16 mode a bfloat16 matrix stays
+        and a matrix stored in 32-bit stays 32-bit (its product then runs in
+        32-bit)."""
+        if self.dtype is torch.float32:
+            t = t.to(torch.float32)
+        return t.to(self.device).contiguous()
+
+    def vector(self, t: torch.Tensor) -> torch.Tensor:
+        """Norm weights and biases are held in float32 in both modes."""
+        return t.to(torch.float32).to(self.device).contiguous()
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """Keys and values of every token in pages; `window` > 0 keeps only the
+    last `window` positions visible (older pages are given back)."""
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Per-request state of fixed size, zero when a request is admitted."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class Part:
+    category = "part"
+
+    def __init__(self, spec: PartSpec, rt: Runtime):
+        self.spec = spec
+        self.rt = rt
+        self.prefix = spec.prefix
+
+    def expected_params(self) -> Dict[str, ParamSpec]:
+        """Full tensor name -> ParamSpec."""
+        return {}
+
+    def load_params(self, get: Callable[[str], Optional[torch.Tensor]]) -> None:
+        """`get(name)` returns the stored tensor on the CPU, or None when an
+        optional tensor is absent."""
+
+
+class Norm(Part):
+    category = "norm"
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    category = "mixer"
+
+    def cache_need(self):
+        return None
+
+    def forward(self, xn, residual, ctx, cache) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    category = "feed_forward"
+
+    def forward(self, xn, residual, ctx) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    category = "block"
+
+    def cache_need(self):
+        return None
+
+    def forward(self, x, ctx, cache) -> None:
+        raise NotImplementedError
+
+
+_PARTS: Dict[Tuple[str, str], type] = {}
+
+
+def register_part(category: str, kind: str, cls: type) -> None:
+    _PARTS[(category, kind)] = cls
+
+
+def build_part(category: str, spec: PartSpec, rt: Runtime, **extra) -> Any:
+    key = (category, spec.kind)
+    if key not in _PARTS:
+        known = sorted(k for c, k in _PARTS if c == category)
+        raise KeyError(f"no {category} part named '{spec.kind}'; registered: {', '.join(known)}")
+    return _PARTS[key](spec, rt, **extra)

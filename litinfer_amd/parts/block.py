@@ -1,0 +1,39 @@
+"""The pre-norm arrangement of a layer's parts
+(src/llaisys/models/qwen2.cpp:272-317): x += mixer(norm1(x)); x += ffn(norm2(x)).
+The residual stream x is float32; mixer and feed-forward add into it."""
+from __future__ import annotations
+
+from .base import Block, build_part, register_part
+
+
+class PreNormBlock(Block):
+    def __init__(self, spec, rt, parts):
+        super().__init__(spec, rt)
+        self.norm1 = build_part("norm", parts["norm1"], rt)
+        self.mixer = build_part("mixer", parts["mixer"], rt)
+        self.norm2 = build_part("norm", parts["norm2"], rt)
+        self.ffn = build_part("feed_forward", parts["feed_forward"], rt)
+        self._all = (self.norm1, self.mixer, self.norm2, self.ffn)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def expected_params(self):
+        e = {}
+        for p in self._all:
+            e.update(p.expected_params())
+        return e
+
+    def load_params(self, get):
+        for p in self._all:
+            p.load_params(get)
+
+    def forward(self, x, ctx, cache):
+        xn = ctx.ws.buffer("block.xn", x.shape, self.rt.dtype)
+        self.norm1.forward(x, xn)
+        self.mixer.forward(xn, x, ctx, cache)
+        self.norm2.forward(x, xn)
+        self.ffn.forward(xn, x, ctx)
+
+
+register_part("block", "prenorm", PreNormBlock)

@@ -1,0 +1,35 @@
+"""A weight matrix [out, in] with an optional bias: y = x W^T + b
+(src/ops/linear/cpu/linear_cpu.cpp:32-37).  Not a part of its own in a layer;
+mixers, feed-forwards and the head hold these."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+
+
+class Linear:
+    def __init__(self, rt, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
+        self.rt = rt
+        self.weight = rt.matrix(weight)      # the same buffer when it already is as needed
+        self.bias = None if bias is None else rt.vector(bias)
+        self.out_features, self.in_features = self.weight.shape
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ws=None):
+        """out = x W^T + b, or out += ... when `accumulate` (out is float32 then).
+        A matrix that is stored in 32-bit is multiplied in 32-bit also when the
+        activations are bfloat16: they are widened for it, exactly."""
+        if self.weight.dtype is torch.float32 and x.dtype is not torch.float32:
+            x32 = ws.buffer("linear.x32", x.shape, torch.float32)
+            ops.cast(x, x32)
+            if out.dtype is torch.float32:
+                ops.linear(x32, self.weight, self.bias, out, accumulate)
+            else:
+                y32 = ws.buffer("linear.y32", out.shape, torch.float32)
+                ops.linear(x32, self.weight, self.bias, y32, False)
+                ops.cast(y32, out)
+        else:
+            ops.linear(x, self.weight, self.bias, out, accumulate)
+        return out

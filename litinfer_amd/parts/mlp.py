@@ -1,0 +1,45 @@
+"""Dense SwiGLU feed-forward: y = (up * gate / (1 + exp(-gate))) Wd^T with
+gate = xn Wg^T, up = xn Wu^T, no biases (src/llaisys/models/qwen2.cpp:744-759,
+src/ops/swiglu/op.cpp:19-22).  Gate and up are one product with the packed
+matrix [Wg; Wu]; the result is added to the residual stream."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import ParamSpec
+from .base import FeedForward, register_part
+from .linear import Linear
+
+
+class SwiGLUMLP(FeedForward):
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.hidden = int(spec.args["hidden_size"])
+        self.inter = int(spec.args["intermediate_size"])
+        self.gate_up = None
+        self.down = None
+
+    def expected_params(self):
+        p = self.prefix
+        return {p + "gate_proj.weight": ParamSpec((self.inter, self.hidden)),
+                p + "up_proj.weight": ParamSpec((self.inter, self.hidden)),
+                p + "down_proj.weight": ParamSpec((self.hidden, self.inter))}
+
+    def load_params(self, get):
+        p = self.prefix
+        g, u = get(p + "gate_proj.weight"), get(p + "up_proj.weight")
+        dt = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
+        self.gate_up = Linear(self.rt, torch.cat([g.to(dt), u.to(dt)], dim=0))
+        self.down = Linear(self.rt, get(p + "down_proj.weight"))
+
+    def forward(self, xn, residual, ctx):
+        t = xn.shape[0]
+        gu = ctx.ws.buffer("mlp.gate_up", (t, 2 * self.inter), self.rt.dtype)
+        self.gate_up(xn, gu, ws=ctx.ws)
+        h = ctx.ws.buffer("mlp.h", (t, self.inter), self.rt.dtype)
+        ops.swiglu(gu, h)
+        self.down(h, residual, accumulate=True, ws=ctx.ws)
+
+
+register_part("feed_forward", "swiglu_mlp", SwiGLUMLP)

@@ -1,0 +1,118 @@
+"""A stand-in for the HIP kernels, written with torch on the CPU, for tests
+that check the engine's bookkeeping (batches, pages, block tables, schedules)
+where there is no GPU.  It is a test double: the package has no CPU path, and
+the tests patch these functions over `litinfer_amd.kernels.ops` themselves.
+Each function follows the documented contract of the kernel it stands for,
+with the cache addressed through the block table exactly as on the device."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def require_gpu(device):
+    return None
+
+
+def embedding(ids, table, out):
+    out.copy_(table[ids.long()].float())
+
+
+def rmsnorm(x, weight, eps, out):
+    xf = x.float()
+    inv = torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+    out.copy_((weight * xf * inv).to(out.dtype))
+
+
+def gather_rows(x, rows, out):
+    out.copy_(x[rows.long()])
+
+
+def cast(src, dst):
+    dst.copy_(src.view(dst.shape).to(dst.dtype))
+
+
+def swiglu(gate_up, out):
+    inter = out.shape[1]
+    g, u = gate_up[:, :inter].float(), gate_up[:, inter:].float()
+    out.copy_((u * (g / (1 + torch.exp(-g)))).to(out.dtype))
+
+
+def rope_table(positions, theta, rotary_dim, cos, sin):
+    j = torch.arange(rotary_dim // 2, dtype=torch.float32)
+    ang = positions.float()[:, None] / torch.pow(torch.tensor(theta, dtype=torch.float32),
+                                                  2 * j / rotary_dim)
+    cos.copy_(torch.cos(ang))
+    sin.copy_(torch.sin(ang))
+
+
+def rope_apply(qkv, n_heads, head_dim, rotary_dim, cos, sin):
+    t = qkv.shape[0]
+    x = qkv[:, :n_heads * head_dim].reshape(t, n_heads, head_dim).float()
+    half = rotary_dim // 2
+    a, b = x[..., :half].clone(), x[..., half:rotary_dim].clone()
+    c, s = cos[:, None, :], sin[:, None, :]
+    x[..., :half] = a * c - b * s
+    x[..., half:rotary_dim] = b * c + a * s
+    qkv[:, :n_heads * head_dim] = x.reshape(t, -1).to(qkv.dtype)
+
+
+def kv_store(qkv, nh, nkv, dh, slot_map, k, v, page_size):
+    t = qkv.shape[0]
+    kk = qkv[:, nh * dh:(nh + nkv) * dh].reshape(t, nkv, dh)
+    vv = qkv[:, (nh + nkv) * dh:(nh + 2 * nkv) * dh].reshape(t, nkv, dh)
+    page = (slot_map // page_size).long()
+    off = (slot_map % page_size).long()
+    k[page, :, off, :] = kk
+    v[page, :, off, :] = vv
+
+
+def rope_kv_store(qkv, nh, nkv, dh, rotary_dim, cos, sin, slot_map, k, v, page_size):
+    rope_apply(qkv, nh + nkv, dh, rotary_dim, cos, sin)
+    kv_store(qkv, nh, nkv, dh, slot_map, k, v, page_size)
+
+
+def linear(x, w, bias, out, accumulate=False):
+    y = x.float() @ w.float().T
+    if bias is not None:
+        y = y + bias
+    if accumulate:
+        out += y
+    else:
+        out.copy_(y.to(out.dtype))
+
+
+def check_attention_sizes(num_heads, num_kv_heads, head_dim):
+    assert num_heads % num_kv_heads == 0 and head_dim % 2 == 0
+
+
+def paged_attention(qkv, out, k, v, meta, nh, nkv, dh, page_size, window, scale):
+    g = nh // nkv
+    for s in range(meta.num_segments):
+        q0, ql, cl = int(meta.host_q_start[s]), int(meta.host_q_len[s]), int(meta.host_ctx_len[s])
+        table = meta.block_table[s].long()
+        for i in range(ql):
+            p = cl - ql + i
+            lo = max(0, p - window + 1) if window > 0 else 0
+            pos = torch.arange(lo, p + 1)
+            pages = table[pos // page_size]
+            assert (pages >= 0).all(), "attention addressed a page that was given back"
+            off = pos % page_size
+            for h in range(nh):
+                kh = h // g
+                qv = qkv[q0 + i, h * dh:(h + 1) * dh].float()
+                kk = k[pages, kh, off, :].float()
+                vv = v[pages, kh, off, :].float()
+                sc = (kk @ qv) * scale
+                w = torch.softmax(sc, dim=0)
+                out[q0 + i, h * dh:(h + 1) * dh] = (w @ vv).to(out.dtype)
+
+
+def argmax_rows(logits, out):
+    out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
+
+
+ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
+       "rope_apply", "kv_store", "rope_kv_store", "linear", "check_attention_sizes",
+       "paged_attention", "argmax_rows"]
