@@ -1,0 +1,199 @@
+// out[M, N] = x[M, K] w[N, K]^T (+ bias[N]) (+ out), float32 accumulation.
+//
+// float32 operands: an LDS-tiled FMA kernel (true 32-bit, no reduced-precision
+// matrix mode).  bfloat16 operands: MFMA tiles for 64-wide waves.  For each
+// output element the sum over K runs in an order that depends on K alone, not
+// on M or on the element's place, so a row's result does not depend on which
+// other rows are in the batch.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+template <typename TO>
+__device__ __forceinline__ void epilogue_store(TO* out, size_t idx, float acc, const float* bias,
+                                               int col, bool accumulate) {
+    if (bias) acc += bias[col];
+    if (accumulate) acc += load_as_float(out + idx);
+    store_from_float(out + idx, acc);
+}
+
+// ------------------------------------------------------------ float32 tiles
+// 64 x 64 tile per block of 256 threads, 4 x 4 outputs per thread, K in steps of 16.
+#define F32_BM 64
+#define F32_BN 64
+#define F32_BK 16
+
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ x,
+                                                        const float* __restrict__ w,
+                                                        const float* __restrict__ bias,
+                                                        float* __restrict__ out, int M, int N, int K,
+                                                        int accumulate) {
+    __shared__ float As[F32_BK][F32_BM + 4];
+    __shared__ float Bs[F32_BK][F32_BN + 4];
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.y * F32_BM, n0 = blockIdx.x * F32_BN;
+    const int ty = tid / 16, tx = tid % 16;
+    const int lrow = tid / 4, lk = (tid % 4) * 4;            // this thread's 4 consecutive k of one row
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += F32_BK) {
+        float a[4], b[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = k0 + lk + i;
+            a[i] = (m0 + lrow < M && k < K) ? x[(size_t)(m0 + lrow) * K + k] : 0.f;
+            b[i] = (n0 + lrow < N && k < K) ? w[(size_t)(n0 + lrow) * K + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { As[lk + i][lrow] = a[i]; Bs[lk + i][lrow] = b[i]; }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < F32_BK; ++k) {
+            float av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { av[i] = As[k][ty * 4 + i]; bv[i] = Bs[k][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = m0 + ty * 4 + i;
+        if (row >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int col = n0 + tx * 4 + j;
+            if (col < N) epilogue_store(out, (size_t)row * N + col, acc[i][j], bias, col, accumulate);
+        }
+    }
+}
+
+// ----------------------------------------------------------- bfloat16 MFMA
+// Block tile 128 x 128, K in steps of 32, 4 waves in a 2 x 2 grid, each wave a
+// 64 x 64 tile made of 2 x 2 MFMA 32x32x16 tiles.  Operand layout of
+// v_mfma_f32_32x32x16_bf16: lane l holds 8 consecutive k of row (l % 32),
+// starting at k = 8 * (l / 32), for A and for B alike; the result's register r
+// of lane l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
+#define BF_BM 128
+#define BF_BN 128
+#define BF_BK 32
+#define BF_LDS_STRIDE (BF_BK + 8)           // in elements; the pad spreads rows over banks
+
+struct __attribute__((aligned(16))) chunk16 { uint32_t w[4]; };
+
+template <bool ALIGNED>
+__device__ __forceinline__ chunk16 load_chunk(const bf16_t* __restrict__ base, int row, int rows,
+                                              int k, int K) {
+    chunk16 c = {{0u, 0u, 0u, 0u}};
+    if (row >= rows || k >= K) return c;
+    const bf16_t* p = base + (size_t)row * K + k;
+    if (ALIGNED) {                                   // K % 8 == 0: the chunk is whole and 16-byte aligned
+        c = *reinterpret_cast<const chunk16*>(p);
+    } else {
+        uint16_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e[i] = (k + i < K) ? p[i].bits : (uint16_t)0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c.w[i] = (uint32_t)e[2 * i] | ((uint32_t)e[2 * i + 1] << 16);
+    }
+    return c;
+}
+
+template <typename TO, bool ALIGNED>
+__global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict__ x,
+                                                         const bf16_t* __restrict__ w,
+                                                         const float* __restrict__ bias,
+                                                         TO* __restrict__ out, int M, int N, int K,
+                                                         int accumulate) {
+    __shared__ __attribute__((aligned(16))) uint16_t As[BF_BM * BF_LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t Bs[BF_BN * BF_LDS_STRIDE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int m0 = blockIdx.y * BF_BM, n0 = blockIdx.x * BF_BN;
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // each thread moves two 16-byte chunks of A and two of B per K step
+    const int crow0 = tid >> 2, ck = (tid & 3) * 8;
+    chunk16 ra[2], rb[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        ra[i] = load_chunk<ALIGNED>(x, m0 + crow0 + 64 * i, M, ck, K);
+        rb[i] = load_chunk<ALIGNED>(w, n0 + crow0 + 64 * i, N, ck, K);
+    }
+    const int frow = lane & 31, fk = (lane >> 5) * 8;
+    for (int k0 = 0; k0 < K; k0 += BF_BK) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            *reinterpret_cast<chunk16*>(&As[(crow0 + 64 * i) * BF_LDS_STRIDE + ck]) = ra[i];
+            *reinterpret_cast<chunk16*>(&Bs[(crow0 + 64 * i) * BF_LDS_STRIDE + ck]) = rb[i];
+        }
+        __syncthreads();
+        if (k0 + BF_BK < K) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                ra[i] = load_chunk<ALIGNED>(x, m0 + crow0 + 64 * i, M, k0 + BF_BK + ck, K);
+                rb[i] = load_chunk<ALIGNED>(w, n0 + crow0 + 64 * i, N, k0 + BF_BK + ck, K);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < BF_BK; ks += 16) {
+            bf16x8 af[2], bfr[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                af[i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + frow) * BF_LDS_STRIDE + ks + fk]);
+                bfr[i] = *reinterpret_cast<const bf16x8*>(&Bs[(wn + 32 * i + frow) * BF_LDS_STRIDE + ks + fk]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    const int ccol = lane & 31, crow = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wn + 32 * j + ccol;
+            if (col >= N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm + 32 * i + 8 * (r >> 2) + crow + (r & 3);
+                if (row < M) epilogue_store(out, (size_t)row * N + col, acc[i][j][r], bias, col, accumulate);
+            }
+        }
+}
+
+extern "C" int li_linear(const void* x, const void* w, const float* bias, void* out, int M, int N,
+                         int K, int in_dtype, int out_dtype, int accumulate, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0) return LI_ERR_SIZE;
+    if (accumulate && out_dtype != LI_F32) return LI_ERR_DTYPE;
+    if (in_dtype == LI_F32) {
+        if (out_dtype != LI_F32) return LI_ERR_DTYPE;
+        dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
+        if (grid.y > 65535) return LI_ERR_SIZE;
+        gemm_f32_kernel<<<grid, 256, 0, stream>>>((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate);
+    } else if (in_dtype == LI_BF16) {
+        dim3 grid((N + BF_BN - 1) / BF_BN, (M + BF_BM - 1) / BF_BM);
+        if (grid.y > 65535) return LI_ERR_SIZE;
+        const bool aligned = (K % 8) == 0;
+#define LI_GEMM(TO, AL) gemm_bf16_kernel<TO, AL><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, accumulate)
+        if (out_dtype == LI_F32) { if (aligned) LI_GEMM(float, true); else LI_GEMM(float, false); }
+        else if (out_dtype == LI_BF16) { if (aligned) LI_GEMM(bf16_t, true); else LI_GEMM(bf16_t, false); }
+        else return LI_ERR_DTYPE;
+#undef LI_GEMM
+    } else return LI_ERR_DTYPE;
+    return li_launch_status();
+}

@@ -66,16 +66,25 @@ def _lib_dirs() -> List[Path]:
     return dirs
 
 
+_dir_lock = threading.Lock()
+_chosen_dir: Optional[Path] = None
+
+
 def _writable_dir() -> Path:
-    for d in _lib_dirs():
-        try:
-            d.mkdir(parents=True, exist_ok=True)
-            probe = d / f".probe-{os.getpid()}"
-            probe.write_bytes(b"")
-            probe.unlink()
-            return d
-        except OSError:
-            continue
+    global _chosen_dir
+    with _dir_lock:
+        if _chosen_dir is not None:
+            return _chosen_dir
+        for d in _lib_dirs():
+            try:
+                d.mkdir(parents=True, exist_ok=True)
+                probe = d / f".probe-{os.getpid()}-{threading.get_ident()}"
+                probe.write_bytes(b"")
+                probe.unlink()
+                _chosen_dir = d
+                return d
+            except OSError:
+                continue
     raise KernelBuildError("no writable folder for the built libraries: tried "
                            + ", ".join(str(d) for d in _lib_dirs()))
 

@@ -42,7 +42,6 @@ _SIGNATURES = {
     },
     "sampling": {
         "li_argmax_rows": [P, P, I, I],
-        "li_sample_rows": [P, P, P, P, P, P, P, P, I, I],
     },
 }
 _fn_cache = {}
@@ -296,24 +295,3 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
     if logits.shape[0]:
         _run("sampling", "li_argmax_rows", logits.data_ptr(), out.data_ptr(), logits.shape[0],
              logits.shape[1])
-
-
-def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
-                top_p: torch.Tensor, uniform: torch.Tensor, scratch: torch.Tensor,
-                out: torch.Tensor) -> None:
-    """One token per row: temperature <= 0 takes the argmax; else the softmax
-    of logits/temperature, restricted to the top_k largest (0 < top_k < V) and
-    then to the shortest prefix, in descending order, whose mass reaches top_p
-    (0 < top_p < 1), is sampled by inverse CDF over ascending ids with the
-    row's uniform number u in [0, 1).  scratch: float32 [rows, V]."""
-    _gpu(logits, temperature, top_k, top_p, uniform, scratch, out)
-    n, vocab = logits.shape
-    _chk(logits.dtype is torch.float32 and logits.is_contiguous(), "sample: logits")
-    for t_, dt in ((temperature, torch.float32), (top_k, torch.int32), (top_p, torch.float32),
-                   (uniform, torch.float32), (out, torch.int32)):
-        _chk(t_.dtype is dt and t_.numel() == n and t_.is_contiguous(), "sample: per-row arrays")
-    _chk(scratch.dtype is torch.float32 and scratch.numel() >= n * vocab and scratch.is_contiguous(),
-         "sample: scratch")
-    if n:
-        _run("sampling", "li_sample_rows", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(),
-             top_p.data_ptr(), uniform.data_ptr(), scratch.data_ptr(), out.data_ptr(), 0, n, vocab)

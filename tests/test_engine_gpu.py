@@ -1,0 +1,69 @@
+"""The engine on the GPU against the plain implementation: whole requests,
+tails decoded one by one, portions of changing size, mixed batches with pages
+used again; in 32-bit and in bfloat16."""
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import schedules
+from tiny_configs import TINY_A, TINY_A_PAGE, TINY_B, TINY_B_PAGE, TINY_C, TINY_C_PAGE
+
+pytestmark = pytest.mark.gpu
+
+CASES = {"A": (TINY_A, TINY_A_PAGE, 0), "B": (TINY_B, TINY_B_PAGE, 1), "C": (TINY_C, TINY_C_PAGE, 2)}
+LENGTHS = [5, 17, 33, 70, 100, 41, 64, 2, 1]
+# float32: rounding of a different summation order only.  bfloat16: weights are
+# bfloat16 on both sides (the plain side computes in float64 from the stored
+# values); what differs is the rounding of activations to bfloat16 between kernels.
+TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, (cfg, page, seed) in CASES.items():
+        for dt in ("float32", "bfloat16"):
+            stored = torch.float32 if dt == "float32" else torch.bfloat16
+            d = helpers.make_model(tmp_path_factory.mktemp(f"m{name}{dt}"), cfg, seed, stored)
+            reqs = helpers.random_requests(cfg["vocab_size"], LENGTHS, seed + 10)
+            out[(name, dt)] = (d, reqs, helpers.plain_logits(d, reqs))
+    return out
+
+
+def _engine(d, dt, page, max_tokens, **kw):
+    from litinfer_amd.engine import Engine
+    return Engine.from_dir(d, dtype=dt, device="cuda:0", page_size=page, max_tokens=max_tokens,
+                           max_seqs=4, page_order_seed=11, **kw)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CASES))
+@pytest.mark.parametrize("kind", ["whole", "tail", "chunks", "mixed"])
+def test_schedules_match_the_plain_implementation(models, name, dt, kind):
+    cfg, page, _ = CASES[name]
+    d, reqs, ref = models[(name, dt)]
+    steps = getattr(schedules, kind)(reqs)
+    # the mixed schedule gets exactly the pages its fullest moment needs, so that the pages of a
+    # finished request are taken by the next one
+    eng = _engine(d, dt, page, schedules.max_live_tokens(reqs, steps, page if kind == "mixed" else 64))
+    out = schedules.run(eng, reqs, steps)
+    eng.cache.check_invariants()
+    assert all(f == g.pool.capacity for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
+    if kind == "mixed":
+        assert all(g.pool.total_allocations > g.pool.capacity for g in eng.cache.groups), "no page was used again"
+    worst = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
+    assert worst < TOL[dt], f"{name} {dt} {kind}: {worst}"
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_float32_schedules_agree_with_each_other_closely(models, name):
+    cfg, page, _ = CASES[name]
+    d, reqs, _ = models[(name, "float32")]
+    outs = {}
+    for kind in ("whole", "tail", "chunks", "mixed"):
+        steps = getattr(schedules, kind)(reqs)
+        outs[kind] = schedules.run(_engine(d, "float32", page, schedules.max_live_tokens(reqs, steps)), reqs, steps)
+    for kind in ("tail", "chunks", "mixed"):
+        for r in reqs:
+            assert schedules.rel_err(outs[kind][r], outs["whole"][r].astype(np.float64)) < 5e-6

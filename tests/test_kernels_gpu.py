@@ -1,0 +1,277 @@
+"""Each HIP kernel alone against a plain float32 reference of the same
+operation, at sizes other than the engine's (odd widths, tails of tiles)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_impl
+from litinfer_amd.engine.batch import AttentionMeta
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, f32=1e-5, bf16=2e-2):
+    return f32 if dtype is torch.float32 else bf16
+
+
+def rel(got, ref):
+    got = got.double().cpu().numpy() if isinstance(got, torch.Tensor) else got
+    return float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from litinfer_amd.kernels import ops
+    ops.require_gpu(DEV)
+    return ops
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(1, 2, 3), (50, 301, 120), (7, 1000, 4096)])
+def test_embedding(ops, dtype, shape):
+    t, v, h = shape
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(v, h, generator=g).to(dtype)
+    ids = torch.randint(0, v, (t,), generator=g, dtype=torch.int32)
+    out = torch.empty(t, h, device=DEV)
+    ops.embedding(ids.to(DEV), table.to(DEV), out)
+    ref = plain_impl.embedding(ids.numpy(), table.double().numpy())
+    assert np.array_equal(out.double().cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,eps", [((1, 4), 1e-5), ((33, 120), 1e-6), ((512, 4096), 1e-5), ((3, 3584), 1e-6)])
+def test_rmsnorm(ops, dtype, shape, eps):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(*shape, generator=g) * 3
+    w = 1 + 0.1 * torch.randn(shape[1], generator=g)
+    out = torch.empty(*shape, dtype=dtype, device=DEV)
+    ops.rmsnorm(x.to(DEV), w.to(DEV), eps, out)
+    ref = plain_impl.rms_norm(x.double().numpy(), w.double().numpy(), eps)
+    assert rel(out, ref) < tol(dtype, 2e-6, 8e-3)
+
+
+def test_rmsnorm_zero_row_is_zero_not_nan(ops):
+    x = torch.zeros(2, 64, device=DEV)
+    out = torch.empty(2, 64, device=DEV)
+    ops.rmsnorm(x, torch.ones(64, device=DEV), 1e-6, out)
+    assert torch.equal(out, torch.zeros_like(out))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mnk,bias,acc", [
+    ((2, 3, 4), True, False), ((1, 8, 16), False, False), ((5, 301, 120), True, False),
+    ((70, 200, 96), False, True), ((130, 129, 264), True, True), ((512, 512, 1024), True, False),
+    ((64, 3584, 3584), False, False), ((3, 37, 90), True, False), ((257, 64, 36), False, False)])
+def test_linear(ops, dtype, mnk, bias, acc):
+    m, n, k = mnk
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(m, k, generator=g).to(dtype)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(dtype)
+    b = torch.randn(n, generator=g) if bias else None
+    ref = plain_impl.linear(x.double().numpy(), w.double().numpy(), None if b is None else b.double().numpy())
+    if acc:
+        base = torch.randn(m, n, generator=g)
+        out = base.to(DEV)
+        ref = ref + base.double().numpy()
+    else:
+        out = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops.linear(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, accumulate=acc)
+    # operands are exact in both dtypes; what differs is the float32 accumulation over K terms
+    # (a random-walk error of about sqrt(K) half-ulps) and, for a bfloat16 out, its rounding
+    assert rel(out, ref) < (4 * math.sqrt(k) * 2.0 ** -24 if out.dtype is torch.float32 else 5e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_rows_do_not_depend_on_the_batch(ops, dtype):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(200, 264, generator=g).to(dtype).to(DEV)
+    w = torch.randn(150, 264, generator=g).to(dtype).to(DEV)
+    full = torch.empty(200, 150, dtype=torch.float32, device=DEV)
+    ops.linear(x, w, None, full)
+    for rows in (slice(0, 1), slice(17, 19), slice(100, 200)):
+        part = torch.empty(rows.stop - rows.start, 150, dtype=torch.float32, device=DEV)
+        ops.linear(x[rows].contiguous(), w, None, part)
+        assert rel(part, full[rows].double().cpu().numpy()) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(2, 3), (33, 200), (512, 4096)])
+def test_swiglu(ops, dtype, shape):
+    t, i = shape
+    g = torch.Generator().manual_seed(4)
+    gu = (torch.randn(t, 2 * i, generator=g) * 3).to(dtype)
+    out = torch.empty(t, i, dtype=dtype, device=DEV)
+    ops.swiglu(gu.to(DEV), out)
+    gd = gu.double().numpy()
+    ref = plain_impl.swiglu(gd[:, :i], gd[:, i:])
+    assert rel(out, ref) < tol(dtype, 1e-6, 8e-3)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("t,heads,dh,theta,start", [(3, 1, 4, 1e4, 0), (40, 5, 48, 5e4, 7), (64, 4, 128, 1e6, 500)])
+def test_rope(ops, dtype, t, heads, dh, theta, start):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(t, heads * dh, generator=g).to(dtype)
+    pos = torch.arange(start, start + t, dtype=torch.int32)
+    cos = torch.empty(t, dh // 2, device=DEV)
+    sin = torch.empty(t, dh // 2, device=DEV)
+    ops.rope_table(pos.to(DEV), theta, dh, cos, sin)
+    xd = x.to(DEV).clone()
+    ops.rope_apply(xd, heads, dh, dh, cos, sin)
+    ref = plain_impl.rope_neox(x.double().numpy().reshape(t, heads, dh), pos.numpy(), theta).reshape(t, -1)
+    # float32 angles: an angle near `start + t` carries an absolute error of about its ulp
+    assert rel(xd, ref) < tol(dtype, 2e-4 if start else 2e-6, 8e-3)
+
+
+def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_one=None):
+    """seg_specs: list of (ctx_len, q_len).  Builds random K/V for every
+    segment, scatters them into shuffled pages, and compares the kernel with
+    the plain attention on the logical sequences."""
+    g = torch.Generator().manual_seed(seed)
+    nseg = len(seg_specs)
+    blocks = [-(-c // page) for c, _ in seg_specs]
+    num_pages = sum(blocks) + 3
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    kc = torch.randn(num_pages, nkv, page, dh, generator=g).to(dtype)      # garbage everywhere first
+    vc = torch.randn(num_pages, nkv, page, dh, generator=g).to(dtype)
+    tab = np.full((nseg, max(blocks)), -1, dtype=np.int32)
+    T = sum(q for _, q in seg_specs)
+    q = (torch.randn(T, nh * dh, generator=g)).to(dtype)
+    ks, vs = [], []
+    o = 0
+    for s, (c, ql) in enumerate(seg_specs):
+        k = torch.randn(c, nkv, dh, generator=g).to(dtype)
+        v = torch.randn(c, nkv, dh, generator=g).to(dtype)
+        if scale_one is not None:             # make one far key stand out for the last query
+            far = scale_one
+            k[far] = 0
+            k[far, :, 0] = 6.0
+            q[o + ql - 1].view(nh, dh)[:, :] = 0
+            q[o + ql - 1].view(nh, dh)[:, 0] = 6.0
+        for b in range(blocks[s]):
+            tab[s, b] = perm.pop()
+            n = min(page, c - b * page)
+            kc[tab[s, b], :, :n] = k[b * page:b * page + n].transpose(0, 1)
+            vc[tab[s, b], :, :n] = v[b * page:b * page + n].transpose(0, 1)
+        ks.append(k)
+        vs.append(v)
+        o += ql
+    q_len = np.array([ql for _, ql in seg_specs], dtype=np.int32)
+    ctx_len = np.array([c for c, _ in seg_specs], dtype=np.int32)
+    q_start = np.concatenate([[0], np.cumsum(q_len)[:-1]]).astype(np.int32)
+    seg_of = np.repeat(np.arange(nseg, dtype=np.int32), q_len)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    meta = AttentionMeta(block_table=dev(tab), max_blocks=tab.shape[1], seg_of_token=dev(seg_of),
+                         q_start=dev(q_start), q_len=dev(q_len), ctx_len=dev(ctx_len), num_segments=nseg,
+                         num_tokens=T, max_q_len=int(q_len.max()), max_ctx_len=int(ctx_len.max()),
+                         host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len)
+    out = torch.empty(T, nh * dh, dtype=dtype, device=DEV)
+    scale = 1.0 / math.sqrt(dh)
+    ops.paged_attention(q.to(DEV), out, kc.to(DEV), vc.to(DEV), meta, nh, nkv, dh, page, window, scale)
+    refs = []
+    o = 0
+    for s, (c, ql) in enumerate(seg_specs):
+        qq = q[o:o + ql].double().numpy().reshape(ql, nh, dh)
+        refs.append(plain_impl.attention(qq, ks[s].double().numpy(), vs[s].double().numpy(),
+                                         np.arange(c - ql, c), np.arange(c), scale, window).reshape(ql, -1))
+        o += ql
+    return out, np.concatenate(refs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("segs,nh,nkv,dh,page,window", [
+    ([(2, 2)], 1, 1, 4, 16, 0),                       # the reference's smallest case
+    ([(11, 5)], 4, 2, 8, 16, 0),                      # a 5-token portion after 6 cached tokens
+    ([(20, 20), (20, 1)], 4, 2, 8, 16, 0),            # shuffled table, last page partly filled
+    ([(20, 1), (28, 1)], 4, 2, 8, 16, 0),             # two decoding requests with interleaved pages
+    ([(100, 37), (1, 1), (300, 1), (64, 64)], 6, 2, 48, 8, 0),
+    ([(100, 37), (33, 2), (300, 1), (70, 70)], 5, 5, 32, 16, 20),    # window crosses pages
+    ([(130, 130), (257, 3)], 28, 4, 128, 16, 0),      # the 7B layer's head layout
+    ([(200, 8)], 3, 1, 112, 16, 64),
+])
+def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
+    out, ref = _paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=6)
+    assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_finds_one_far_key(ops, dtype):
+    # one key among hundreds carries almost all the weight: a kernel that skips
+    # or misplaces a page gives a visibly different output
+    for far in (0, 15, 16, 333, 511):
+        out, ref = _paged_case(ops, dtype, [(512, 1)], 4, 2, 64, 16, 0, seed=7, scale_one=far)
+        assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_window_edge(ops, dtype):
+    # the key just outside the window must not count, the one just inside must
+    for window, far, visible in ((32, 512 - 32, True), (32, 512 - 33, False)):
+        out, ref = _paged_case(ops, dtype, [(512, 1)], 2, 1, 32, 8, window, seed=8, scale_one=far)
+        assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rope_kv_store_and_plain_store(ops, dtype):
+    g = torch.Generator().manual_seed(9)
+    t, nh, nkv, dh, page, pages = 37, 3, 2, 48, 8, 11
+    qkv = torch.randn(t, (nh + 2 * nkv) * dh + 5, generator=g).to(dtype)[:, :(nh + 2 * nkv) * dh]
+    pos = torch.randint(0, 200, (t,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(pages * page, generator=g)[:t].to(torch.int32)
+    cos = torch.empty(t, dh // 2, device=DEV)
+    sin = torch.empty(t, dh // 2, device=DEV)
+    ops.rope_table(pos.to(DEV), 1e4, dh, cos, sin)
+    outs = []
+    for fused in (True, False):
+        d = qkv.to(DEV)
+        d = d.clone() if d.is_contiguous() else d      # keep the row stride with its pad
+        kc = torch.zeros(pages, nkv, page, dh, dtype=dtype, device=DEV)
+        vc = torch.zeros_like(kc)
+        if fused:
+            ops.rope_kv_store(d, nh, nkv, dh, dh, cos, sin, slots.to(DEV), kc, vc, page)
+        else:
+            ops.rope_apply(d, nh + nkv, dh, dh, cos, sin)
+            ops.kv_store(d, nh, nkv, dh, slots.to(DEV), kc, vc, page)
+        outs.append((d[:, :nh * dh].clone(), kc, vc))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    x = qkv.double().numpy()
+    kref = plain_impl.rope_neox(x[:, nh * dh:(nh + nkv) * dh].reshape(t, nkv, dh), pos.numpy(), 1e4)
+    got = outs[0][1].double().cpu().numpy()
+    for i in range(t):
+        s = int(slots[i])
+        assert np.abs(got[s // page, :, s % page] - kref[i]).max() < tol(dtype, 1e-4, 3e-2)
+        assert torch.equal(outs[0][2][s // page, :, s % page].cpu(),
+                           qkv[i, (nh + nkv) * dh:].reshape(nkv, dh))
+
+
+@pytest.mark.parametrize("shape", [(1, 4), (3, 4096), (5, 152064), (2, 301)])
+def test_argmax_rows_lowest_index_wins(ops, shape):
+    g = torch.Generator().manual_seed(10)
+    x = torch.randn(*shape, generator=g)
+    x[0, shape[1] // 2] = 50.0
+    x[0, shape[1] - 1] = 50.0          # an equal maximum later in the row
+    out = torch.empty(shape[0], dtype=torch.int32, device=DEV)
+    ops.argmax_rows(x.to(DEV), out)
+    assert out.cpu().tolist() == [plain_impl.argmax_first(r) for r in x.numpy()]
+    assert out[0].item() == shape[1] // 2
+
+
+def test_gather_and_cast(ops):
+    x = torch.randn(10, 37)
+    rows = torch.tensor([9, 0, 0, 4], dtype=torch.int32)
+    out = torch.empty(4, 37, device=DEV)
+    ops.gather_rows(x.to(DEV), rows.to(DEV), out)
+    assert torch.equal(out.cpu(), x[rows.long()])
+    b = torch.empty(10, 37, dtype=torch.bfloat16, device=DEV)
+    ops.cast(x.to(DEV), b)
+    assert torch.equal(b.cpu(), x.to(torch.bfloat16))       # round to nearest even, as torch does
+    f = torch.empty(10, 37, device=DEV)
+    ops.cast(b, f)
+    assert torch.equal(f.cpu(), x.to(torch.bfloat16).float())

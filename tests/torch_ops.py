@@ -49,7 +49,7 @@ def rope_table(positions, theta, rotary_dim, cos, sin):
 
 def rope_apply(qkv, n_heads, head_dim, rotary_dim, cos, sin):
     t = qkv.shape[0]
-    x = qkv[:, :n_heads * head_dim].reshape(t, n_heads, head_dim).float()
+    x = qkv[:, :n_heads * head_dim].reshape(t, n_heads, head_dim).float().clone()
     half = rotary_dim // 2
     a, b = x[..., :half].clone(), x[..., half:rotary_dim].clone()
     c, s = cos[:, None, :], sin[:, None, :]
