@@ -46,3 +46,203 @@ extern "C" int li_argmax_rows(const float* logits, int* out, int n, int V, hipSt
     argmax_rows_kernel<<<n, SMP_NT, 0, stream>>>(logits, out, V);
     return li_launch_status();
 }
+
+// ---------------------------------------------------------------- sampling
+// One block per row.  The candidates are ordered by (value descending, index
+// ascending); top-k keeps the first k, top-p then the shortest prefix whose
+// softmax mass (among the top-k survivors) reaches p; the survivors' softmax is
+// sampled by inverse CDF over ASCENDING ids with the given uniform number.
+// Thresholds are found by a bitwise search over the order-preserving integer
+// image of the floats, every count and mass being a block reduction in a fixed
+// order, so the same inputs always give the same token.
+__device__ __forceinline__ uint32_t sort_key(float z) {
+    const uint32_t b = __float_as_uint(z);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+__device__ __forceinline__ int block_sum_int(int v, int* smem) {
+#pragma unroll
+    for (int o = LI_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, LI_WAVE);
+    const int lane = threadIdx.x & (LI_WAVE - 1), w = threadIdx.x / LI_WAVE;
+    __syncthreads();
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    int t = 0;
+#pragma unroll
+    for (int i = 0; i < SMP_NT / LI_WAVE; ++i) t += smem[i];
+    return t;
+}
+
+__device__ __forceinline__ float block_max_f(float v, float* smem) {
+    v = wave_max(v);
+    const int lane = threadIdx.x & (LI_WAVE - 1), w = threadIdx.x / LI_WAVE;
+    __syncthreads();
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    float t = smem[0];
+#pragma unroll
+    for (int i = 1; i < SMP_NT / LI_WAVE; ++i) t = fmaxf(t, smem[i]);
+    return t;
+}
+
+__global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
+    const float* __restrict__ logits, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p,
+    const float* __restrict__ uniform, int* __restrict__ out, int V) {
+    __shared__ float sf[SMP_NT / LI_WAVE];
+    __shared__ int si[SMP_NT / LI_WAVE];
+    __shared__ float part_f[SMP_NT];
+    __shared__ int part_i[SMP_NT];
+    __shared__ int chosen_thread;
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* row = logits + (size_t)r * V;
+    const float T = temperature[r];
+    if (!(T > 0.f)) {                                          // greedy
+        float v = -INFINITY;
+        int i = 0x7fffffff;
+        for (int j = tid; j < V; j += SMP_NT) {
+            const float x = row[j];
+            if (x > v || i == 0x7fffffff) { v = x; i = j; }
+        }
+        block_argmax(v, i, sf, si);
+        if (tid == 0) out[r] = i;
+        return;
+    }
+    // contiguous chunk of ids per thread, so that block scans run in id order
+    const int chunk = (V + SMP_NT - 1) / SMP_NT;
+    const int c0 = min(tid * chunk, V), c1 = min(c0 + chunk, V);
+
+    float m = -INFINITY;
+    for (int j = c0; j < c1; ++j) m = fmaxf(m, row[j] / T);
+    m = block_max_f(m, sf);
+
+    // ---- top-k: tau_k = k-th largest key, need_k = how many of its ties count
+    uint32_t tau = 0u;
+    int need = 0x7fffffff;
+    const int k = top_k[r];
+    if (k > 0 && k < V) {
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = tau | (1u << bit);
+            int c = 0;
+            for (int j = c0; j < c1; ++j) c += sort_key(row[j] / T) >= cand;
+            if (block_sum_int(c, si) >= k) tau = cand;
+        }
+        int c = 0;
+        for (int j = c0; j < c1; ++j) c += sort_key(row[j] / T) > tau;
+        need = k - block_sum_int(c, si);
+    }
+    // ---- top-p among the top-k survivors
+    const float p = top_p[r];
+    if (p > 0.f && p < 1.f) {
+        // Z_k: mass of the top-k survivors (ties at tau in id order, `need` of them)
+        int eq = 0;
+        for (int j = c0; j < c1; ++j) eq += sort_key(row[j] / T) == tau;
+        part_i[tid] = eq;
+        __syncthreads();
+        int before = 0;
+        for (int t = 0; t < tid; ++t) before += part_i[t];
+        float zk = 0.f;
+        {
+            int rank = before;
+            for (int j = c0; j < c1; ++j) {
+                const float z = row[j] / T;
+                const uint32_t key = sort_key(z);
+                if (key > tau || (key == tau && rank++ < need)) zk += expf(z - m);
+            }
+        }
+        zk = block_sum<SMP_NT>(zk, sf);
+        const float target = p * zk;
+        // tp = the largest c with f(c) >= target, where f(c) = Z_k for c <= tau (the top-k
+        // survivors as a whole) and the mass of the keys >= c above it; f does not increase
+        uint32_t tp = 0u;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = tp | (1u << bit);
+            if (cand <= tau) { tp = cand; continue; }
+            float s = 0.f;
+            for (int j = c0; j < c1; ++j) {
+                const float z = row[j] / T;
+                if (sort_key(z) >= cand) s += expf(z - m);
+            }
+            if (block_sum<SMP_NT>(s, sf) >= target) tp = cand;
+        }
+        float s = 0.f;
+        for (int j = c0; j < c1; ++j) {
+            const float z = row[j] / T;
+            if (sort_key(z) > tp) s += expf(z - m);
+        }
+        const float mass_gt = block_sum<SMP_NT>(s, sf);
+        const float e_tau = expf(key_value(tp) - m);
+        int need_p = 0x7fffffff;                               // ties without mass: all of them
+        if (e_tau > 0.f) {
+            const float q = ceilf((target - mass_gt) / e_tau);
+            need_p = q < 1.f ? 1 : (q > 2.0e9f ? 0x7fffffff : (int)q);
+        }
+        need = (tp == tau) ? min(need, need_p) : need_p;
+        tau = tp;
+    }
+    // ---- inverse CDF over ascending ids among the survivors
+    int eq = 0;
+    for (int j = c0; j < c1; ++j) eq += sort_key(row[j] / T) == tau;
+    __syncthreads();
+    part_i[tid] = eq;
+    __syncthreads();
+    int before = 0;
+    for (int t = 0; t < tid; ++t) before += part_i[t];
+    __syncthreads();                 // part_i is written again below
+    float mine = 0.f;
+    int last_in = -1;
+    {
+        int rank = before;
+        for (int j = c0; j < c1; ++j) {
+            const float z = row[j] / T;
+            const uint32_t key = sort_key(z);
+            if (key > tau || (key == tau && rank++ < need)) { mine += expf(z - m); last_in = j; }
+        }
+    }
+    part_f[tid] = mine;
+    part_i[tid] = last_in;           // (the tie counts are no longer needed: `before` is in a register)
+    if (tid == 0) chosen_thread = -1;
+    __syncthreads();
+    if (tid == 0) {                  // sequential scan in id order: 1024 additions, fixed order
+        float total = 0.f;
+        for (int t = 0; t < SMP_NT; ++t) total += part_f[t];
+        const float target = uniform[r] * total;
+        float run = 0.f;
+        int pick = -1, last_nonempty = -1;
+        for (int t = 0; t < SMP_NT; ++t) {
+            if (part_i[t] >= 0) last_nonempty = t;
+            if (pick < 0 && part_i[t] >= 0 && run + part_f[t] >= target) pick = t;
+            if (pick < 0) run += part_f[t];
+        }
+        if (pick < 0) pick = last_nonempty;               // rounding left the target just above the total
+        chosen_thread = pick;
+        sf[0] = run;                                       // mass before the chosen thread's chunk
+        sf[1] = target;
+    }
+    __syncthreads();
+    if (tid == chosen_thread) {
+        float run = sf[0];
+        const float target = sf[1];
+        int rank = before, pick = last_in;
+        for (int j = c0; j < c1; ++j) {
+            const float z = row[j] / T;
+            const uint32_t key = sort_key(z);
+            if (key > tau || (key == tau && rank++ < need)) {
+                run += expf(z - m);
+                if (run >= target) { pick = j; break; }
+            }
+        }
+        out[r] = pick;
+    }
+}
+
+extern "C" int li_sample_rows(const float* logits, const float* temperature, const int* top_k,
+                              const float* top_p, const float* uniform, int* out, int n, int V,
+                              hipStream_t stream) {
+    if (n <= 0 || V <= 0) return LI_ERR_SIZE;
+    sample_rows_kernel<<<n, SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V);
+    return li_launch_status();
+}

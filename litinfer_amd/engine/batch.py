@@ -118,3 +118,53 @@ class BatchUploader:
         else:
             self._dev[:total].copy_(self._host[i][:total])
         return [self._dev[o:o + p.size].view(p.shape) for p, o in zip(parts, offs)]
+
+
+def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploader") -> StepContext:
+    """Lay out the step's integers (see the module text) for the given entries
+    against the cache's current tables, upload them, and return the context.
+    Pages for the entries' tokens must have been reserved."""
+    P = cache.page_size
+    nseg = len(entries)
+    q_len = np.array([len(e.tokens) for e in entries], dtype=np.int32)
+    q_start = np.zeros(nseg + 1, dtype=np.int32)
+    np.cumsum(q_len, out=q_start[1:])
+    T = int(q_start[-1])
+    cached = np.array([cache.cached_len(e.rid) for e in entries], dtype=np.int32)
+    ctx_len = cached + q_len
+    ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+    seg_of_token = np.repeat(np.arange(nseg, dtype=np.int32), q_len)
+    pos = (np.arange(T, dtype=np.int32) - q_start[seg_of_token] + cached[seg_of_token]).astype(np.int32)
+    slots = np.array([cache.slot(e.rid) for e in entries], dtype=np.int32)
+    want = [int(q_start[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
+    want_rows = np.asarray(want, dtype=np.int32)
+    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows]
+    tables, max_blocks = [], []
+    for gi in range(len(cache.groups)):
+        tabs = [cache.block_table(e.rid, gi) for e in entries]
+        mb = max(1, max(len(t) for t in tabs))
+        tab = np.full((nseg, mb), -1, dtype=np.int32)
+        for i, t in enumerate(tabs):
+            tab[i, :len(t)] = t
+        page = tab[seg_of_token, pos // P]
+        if (page < 0).any():
+            raise AssertionError("step: a token of the batch has no page")
+        slot_map = (page.astype(np.int64) * P + pos % P).astype(np.int32)
+        tables.append(tab)
+        max_blocks.append(mb)
+        parts += [tab, slot_map]
+    dev = uploader.upload(parts)
+    ctx = StepContext(ws, T, nseg)
+    (ctx.ids, ctx.positions, d_seg, d_qs, d_ql, d_cl, ctx.state_slots, ctx.want_rows) = dev[:8]
+    ctx.num_want = len(want)
+    ctx.host_state_slots = slots
+    ctx.host_q_start, ctx.host_q_len, ctx.host_ctx_len = q_start[:-1], q_len, ctx_len
+    for gi in range(len(cache.groups)):
+        d_tab, d_slot = dev[8 + 2 * gi], dev[9 + 2 * gi]
+        ctx._slot_maps.append(d_slot)
+        ctx._attn.append(AttentionMeta(
+            block_table=d_tab, max_blocks=max_blocks[gi], seg_of_token=d_seg, q_start=d_qs,
+            q_len=d_ql, ctx_len=d_cl, num_segments=nseg, num_tokens=T,
+            max_q_len=int(q_len.max()), max_ctx_len=int(ctx_len.max()),
+            host_q_start=q_start[:-1], host_q_len=q_len, host_ctx_len=ctx_len))
+    return ctx

@@ -1,0 +1,282 @@
+"""The scheduler above the step function: it admits requests, cuts prompts into
+portions under a token budget, decodes, finishes and frees.
+
+Every step it plans one batch:
+ 1. one token for every running request that is decoding;
+ 2. the rest of the token budget to running requests still in their prompt,
+    oldest first, each at most `chunk_size` tokens and no more than the free
+    pages allow; a portion that does not reach the prompt's end asks for no
+    logits;
+ 3. requests from the waiting queue, first come first served, while budget and
+    a state slot remain and the free pages cover all of the request's prompt.
+When the pages do not even cover the decoding requests, the most recently
+admitted running request is PREEMPTED: all it holds is given back, it goes to
+the head of the waiting queue, and when it is admitted again its prompt plus
+what it had generated is computed anew (its random stream goes on where it
+was, so its tokens are the same as without preemption).  A request that could
+never fit the pool alone is refused when it is submitted.
+
+The reference admits every request into the very next step whole, without a
+budget or a look at the free pages, and when its pool is full the step throws
+and the caller spins (src/llaisys/models/qwen2.cpp:789-800, 832-845, 925-944;
+serving/engine_runtime.py:42-62).  Its finishing rules are kept: an end token
+is dropped and ends the request, the token that reaches max_new_tokens is kept
+(:1058-1073).
+"""
+from __future__ import annotations
+
+import itertools
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
+
+from ..cache import CacheFull
+from ..sampling import Sampler, SamplingParams
+from .batch import StepEntry
+
+WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+
+
+@dataclass
+class Request:
+    rid: Hashable
+    prompt: List[int]
+    max_new_tokens: int
+    params: Optional[SamplingParams]
+    first_token_greedy: bool = False
+    state: str = WAITING
+    generated: List[int] = field(default_factory=list)
+    computed: int = 0                # tokens of prompt + generated that are in the cache
+    samples_drawn: int = 0           # position in the request's random stream
+    finish_reason: Optional[str] = None
+    preemptions: int = 0
+    arrival: int = 0
+
+    @property
+    def tokens(self) -> List[int]:
+        return self.prompt + self.generated
+
+    @property
+    def remaining(self) -> int:
+        return len(self.prompt) + len(self.generated) - self.computed
+
+
+@dataclass
+class Planned:
+    request: Request
+    start: int
+    n: int
+    wants_logits: bool
+
+
+class Scheduler:
+    def __init__(self, engine, *, max_batch_tokens: int = 2048, chunk_size: int = 512,
+                 max_running: Optional[int] = None, eos_token_ids: Optional[Sequence[int]] = None,
+                 sampler=None):
+        if max_batch_tokens <= 0 or chunk_size <= 0:
+            raise ValueError("scheduler: max_batch_tokens and chunk_size must be positive")
+        self.engine = engine
+        self.cache = engine.cache
+        self.max_batch_tokens = int(max_batch_tokens)
+        self.chunk_size = int(chunk_size)
+        self.max_running = int(max_running) if max_running else self.cache.max_seqs
+        self.eos = tuple(engine.spec.eos_token_ids if eos_token_ids is None else eos_token_ids)
+        self.sampler = sampler if sampler is not None else Sampler(engine.rt.device)
+        self.waiting: Deque[Request] = deque()
+        self.running: List[Request] = []          # in order of admission
+        self.requests: Dict[Hashable, Request] = {}
+        self._ids = itertools.count()
+        self._arrivals = itertools.count()
+        self.steps = 0
+        self.preemptions = 0
+        self.last_batch_tokens = 0
+
+    # ---- submitting -----------------------------------------------------
+    def add_request(self, prompt: Sequence[int], max_new_tokens: int = 128,
+                    params: Optional[SamplingParams] = None, rid: Hashable = None,
+                    first_token_greedy: bool = False) -> Hashable:
+        prompt = [int(t) for t in prompt]
+        if not prompt:
+            raise ValueError("add_request: inputs must not be empty")
+        if max_new_tokens <= 0:
+            max_new_tokens = 512                       # src/llaisys/models/qwen2.cpp:793
+        vocab = self.engine.spec.vocab_size
+        if min(prompt) < 0 or max(prompt) >= vocab:
+            raise ValueError(f"add_request: a token id is outside the vocabulary of {vocab}")
+        limit = self.engine.spec.max_positions
+        if len(prompt) + max_new_tokens - 1 > limit:
+            raise ValueError("add_request: requested prompt and output exceed model max sequence "
+                             f"length ({limit})")
+        need = self.cache.pages_needed(None, len(prompt) + max_new_tokens - 1, cached=0)
+        for g, n in zip(self.cache.groups, need):
+            if g.need.window <= 0 and n > g.pool.capacity:
+                raise ValueError(f"add_request: the request needs {n} cache pages, the pool has "
+                                 f"{g.pool.capacity}: it could never run")
+        if rid is None:
+            rid = next(self._ids)
+            while rid in self.requests:
+                rid = next(self._ids)
+        elif rid in self.requests and self.requests[rid].state != FINISHED:
+            raise ValueError(f"add_request: request id {rid!r} is in use")
+        req = Request(rid, prompt, int(max_new_tokens), params, first_token_greedy,
+                      arrival=next(self._arrivals))
+        self.requests[rid] = req
+        self.waiting.append(req)
+        return rid
+
+    # ---- queries -----------------------------------------------------------
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def num_requests(self) -> int:
+        return len(self.requests)
+
+    def is_finished(self, rid) -> bool:
+        return self.requests[rid].state == FINISHED
+
+    def output(self, rid) -> List[int]:
+        return list(self.requests[rid].generated)
+
+    def abort(self, rid) -> None:
+        req = self.requests[rid]
+        if req.state == FINISHED:
+            return
+        if req.state == RUNNING:
+            self.running.remove(req)
+            self.engine.finish(rid)
+        else:
+            self.waiting.remove(req)
+        req.state, req.finish_reason = FINISHED, "aborted"
+
+    # ---- planning ------------------------------------------------------------
+    def _preempt(self, req: Request) -> None:
+        self.running.remove(req)
+        self.engine.finish(req.rid)
+        req.state, req.computed = WAITING, 0
+        req.preemptions += 1
+        self.preemptions += 1
+        self.waiting.appendleft(req)
+
+    def _fits(self, free: List[int], rid, n: int, cached: Optional[int] = None) -> Optional[List[int]]:
+        need = self.cache.pages_needed(rid, n, cached)
+        return need if all(a <= b for a, b in zip(need, free)) else None
+
+    def _largest_fitting(self, free: List[int], rid, n: int, cached: Optional[int]) -> int:
+        """The largest portion <= n whose pages are free (0 if not even one token fits)."""
+        while n > 0:
+            if self._fits(free, rid, n, cached) is not None:
+                return n
+            have = (self.cache.cached_len(rid) if cached is None else cached) + n
+            n -= ((have - 1) % self.cache.page_size) + 1        # drop the last, partly used page
+        return 0
+
+    def plan(self) -> List[Planned]:
+        """Decide the next batch.  Preempts if it must; changes nothing else."""
+        while True:
+            free = self.cache.free_pages()
+            plan: List[Planned] = []
+            budget = self.max_batch_tokens
+            decoding = [r for r in self.running if r.remaining == 1]
+            short = False
+            for r in decoding:
+                need = self._fits(free, r.rid, 1)
+                if need is None or budget <= 0:
+                    short = need is None
+                    break
+                free = [a - b for a, b in zip(free, need)]
+                budget -= 1
+                plan.append(Planned(r, r.computed, 1, True))
+            if short and len(self.running) > 1:
+                self._preempt(self.running[-1])
+                continue
+            if short:                                   # a lone request that outgrew the pool
+                r = self.running[0]
+                self.running.remove(r)
+                self.engine.finish(r.rid)
+                r.state, r.finish_reason = FINISHED, "error: kv capacity"
+                continue
+            break
+        for r in self.running:
+            if r.remaining <= 1 or budget <= 0:
+                continue
+            n = self._largest_fitting(free, r.rid, min(r.remaining, self.chunk_size, budget), None)
+            if n <= 0:
+                continue
+            free = [a - b for a, b in zip(free, self.cache.pages_needed(r.rid, n))]
+            budget -= n
+            plan.append(Planned(r, r.computed, n, n == r.remaining))
+        slots = self.cache.free_slots()
+        while self.waiting and budget > 0 and slots > 0 and len(self.running) < self.max_running:
+            r = self.waiting[0]
+            # admitted only when everything it has to compute fits the free pages now: a
+            # request let in on its first portion alone would soon be preempted again
+            if self._fits(free, None, r.remaining, 0) is None:
+                break                                   # first come first served: nobody overtakes
+            n = min(r.remaining, self.chunk_size, budget)
+            self.waiting.popleft()
+            r.state = RUNNING
+            self.running.append(r)
+            free = [a - b for a, b in zip(free, self.cache.pages_needed(None, n, cached=0))]
+            budget -= n
+            slots -= 1
+            plan.append(Planned(r, 0, n, n == r.remaining))
+        return plan
+
+    # ---- one step ------------------------------------------------------------
+    def step(self, default_params: Optional[SamplingParams] = None) -> List[Tuple[Hashable, int]]:
+        """Plan a batch, run it, sample, finish.  Returns (request id, token)
+        for every token appended in this step."""
+        plan = self.plan()
+        if not plan:
+            if self.has_unfinished() and not self.running:
+                # nothing runs and the head of the queue still does not fit: it never will
+                r = self.waiting.popleft()
+                r.state, r.finish_reason = FINISHED, "error: kv capacity"
+            return []
+        entries = [StepEntry(p.request.rid, p.request.tokens[p.start:p.start + p.n],
+                             [p.n - 1] if p.wants_logits else []) for p in plan]
+        self.last_batch_tokens = sum(p.n for p in plan)
+        logits = self.engine.step(entries)
+        self.steps += 1
+        for p in plan:
+            p.request.computed += p.n
+        sampled = [p.request for p in plan if p.wants_logits]
+        produced: List[Tuple[Hashable, int]] = []
+        if sampled:
+            params, counters = [], []
+            for r in sampled:
+                sp = r.params or default_params or SamplingParams()
+                if r.first_token_greedy and not r.generated:
+                    sp = SamplingParams()
+                params.append(sp)
+                counters.append(r.samples_drawn)
+            tokens = self.sampler.sample(logits, params, counters)
+            for r, sp, tok in zip(sampled, params, tokens):
+                if not sp.greedy:
+                    r.samples_drawn += 1
+                if self._append(r, int(tok)):
+                    produced.append((r.rid, int(tok)))
+        return produced
+
+    def _append(self, r: Request, tok: int) -> bool:
+        """Apply the finishing rules; True if the token was kept."""
+        if tok in self.eos:
+            self._finish(r, "eos")
+            return False
+        r.generated.append(tok)
+        if len(r.generated) >= r.max_new_tokens:
+            self._finish(r, "length")
+        elif len(r.prompt) + len(r.generated) >= self.engine.spec.max_positions:
+            self._finish(r, "max_pos")
+        return True
+
+    def _finish(self, r: Request, reason: str) -> None:
+        r.state, r.finish_reason = FINISHED, reason
+        if r in self.running:
+            self.running.remove(r)
+        self.engine.finish(r.rid)
+
+    def run_to_completion(self, default_params: Optional[SamplingParams] = None, max_steps: int = 10 ** 9):
+        while self.has_unfinished() and max_steps > 0:
+            self.step(default_params)
+            max_steps -= 1

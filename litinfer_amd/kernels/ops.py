@@ -42,6 +42,7 @@ _SIGNATURES = {
     },
     "sampling": {
         "li_argmax_rows": [P, P, I, I],
+        "li_sample_rows": [P, P, P, P, P, P, I, I],
     },
 }
 _fn_cache = {}
@@ -295,3 +296,22 @@ def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
     if logits.shape[0]:
         _run("sampling", "li_argmax_rows", logits.data_ptr(), out.data_ptr(), logits.shape[0],
              logits.shape[1])
+
+
+def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+                top_p: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:
+    """One token per row.  temperature <= 0: the argmax (lowest index on ties).
+    Otherwise the candidates, ordered by (logit descending, index ascending),
+    are cut to the first top_k (when 0 < top_k < V) and then to the shortest
+    prefix whose softmax mass among them reaches top_p (when 0 < top_p < 1);
+    the softmax of logits/temperature over the survivors is sampled by inverse
+    CDF over ascending ids with the row's uniform number in [0, 1)."""
+    _gpu(logits, temperature, top_k, top_p, uniform, out)
+    _chk(logits.dim() == 2 and logits.dtype is torch.float32 and logits.is_contiguous(), "sample: logits")
+    n = logits.shape[0]
+    for t_, dt in ((temperature, torch.float32), (top_k, torch.int32), (top_p, torch.float32),
+                   (uniform, torch.float32), (out, torch.int32)):
+        _chk(t_.dtype is dt and t_.numel() == n and t_.is_contiguous(), "sample: per-row arrays")
+    if n:
+        _run("sampling", "li_sample_rows", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(),
+             top_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), n, logits.shape[1])

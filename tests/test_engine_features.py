@@ -1,0 +1,382 @@
+"""The engine's parts and paths, each on its own: on the CPU with the torch
+stand-ins of tests/torch_ops.py (bookkeeping), and on the GPU with the HIP
+kernels (`-m gpu`).  Compared with the plain implementation."""
+import math
+from dataclasses import dataclass, replace
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_impl as P
+import schedules
+from litinfer_amd.cache import CacheFull, CacheManager
+from litinfer_amd.config import ExecEntry, LayerSpec, ModelSpec, PartSpec, Qwen2Config, qwen2_model_spec, register_architecture
+from litinfer_amd.engine import Engine, StepEntry, StepError
+from litinfer_amd.engine.batch import BatchUploader, build_context
+from litinfer_amd.engine.workspace import Workspace
+from litinfer_amd.parts import Mixer, Runtime, StateNeed, build_part, register_part
+from litinfer_amd.weights import ParamSpec
+from tiny_configs import TINY_A, TINY_B, TINY_C
+
+
+@pytest.fixture(params=[pytest.param("cpu"), pytest.param("gpu", marks=pytest.mark.gpu)])
+def device(request):
+    if request.param == "cpu":
+        request.getfixturevalue("cpu_ops")
+        return "cpu"
+    return "cuda:0"
+
+
+F32_TOL, BF16_TOL = 2e-5, 4e-2
+
+
+def engine_for(d, device, dtype="float32", page=16, max_tokens=512, **kw):
+    return Engine.from_dir(d, dtype=dtype, device=device, page_size=page, max_tokens=max_tokens, max_seqs=4, **kw)
+
+
+# ------------------------------------------------------------- whole paths
+def test_long_decoding_rolls_the_window_and_matches(tmp_path, device):
+    d = helpers.make_model(tmp_path, TINY_B, 1)
+    toks = helpers.random_requests(320, [250], 5)["r0"]
+    ref = helpers.plain_logits(d, {"r0": toks})["r0"]
+    eng = engine_for(d, device, page=8, max_tokens=256)
+    rows = [eng.step([StepEntry("r0", toks[:3], [0, 1, 2])]).cpu().numpy()]
+    for t in toks[3:]:
+        rows.append(eng.step([StepEntry("r0", [t], [0])]).cpu().numpy())
+    assert schedules.rel_err(np.concatenate(rows), ref) < F32_TOL
+    assert eng.cache.groups[1].pool.used <= 32 // 8 + 1          # the windowed layers keep a few pages only
+    assert eng.cache.groups[0].pool.used == -(-250 // 8)
+
+
+def test_first_tokens_of_a_sequence(tmp_path, device):
+    d = helpers.make_model(tmp_path, TINY_C, 2)
+    for n in (1, 2, 3):
+        toks = helpers.random_requests(301, [n], n)["r0"]
+        ref = helpers.plain_logits(d, {"r0": toks})["r0"]
+        eng = engine_for(d, device)
+        assert schedules.rel_err(eng.step([StepEntry("x", toks, list(range(n)))]).cpu().numpy(), ref) < F32_TOL
+
+
+def test_greedy_generation_through_the_entry_point(tmp_path, device):
+    from litinfer_amd.models import Qwen2, load
+    for cfg, seed in ((TINY_A, 0), (TINY_B, 1)):
+        d = helpers.make_model(tmp_path / str(seed), cfg, seed)
+        pcfg, w = P.load_folder(d)
+        model = load(d, device=device, dtype="float32", max_tokens=512, max_seqs=4, chunk_size=24)
+        assert isinstance(model, Qwen2)
+        for n in (5, 17, 33):
+            prompt = helpers.random_requests(cfg["vocab_size"], [n], n)["r0"]
+            got = model.generate(prompt, max_new_tokens=16)
+            assert got == P.greedy_generate(pcfg, w, prompt, 16, eos=cfg.get("eos_token_id", []) or [])
+        assert model.generate(prompt) == got[:1]                       # max_new_tokens=None means one token
+        assert model.generate(prompt, max_new_tokens=0) == []
+        with pytest.raises(ValueError, match="max sequence length"):
+            model.generate([1] * (cfg["max_position_embeddings"] + 1))   # test/test_kv_cache.py:87-93
+        with pytest.raises(ValueError, match="must not be empty"):
+            model.generate([])
+        assert model.generate(prompt, max_new_tokens=16) == got          # the cache was given back in between
+        assert model.engine.cache.free_slots() == 4
+
+
+def test_continuous_batching_calls_give_each_request_its_own_greedy_tokens(tmp_path, device):
+    from litinfer_amd.models import Qwen2
+    d = helpers.make_model(tmp_path, TINY_A, 0)
+    pcfg, w = P.load_folder(d)
+    model = Qwen2(d, device=device, dtype="float32", max_tokens=256, max_seqs=4, chunk_size=8, max_batch_tokens=16)
+    prompts = list(helpers.random_requests(256, [5, 17, 33], 9).values())
+    model.engine_start()
+    ids = [model.engine_add_request(p, max_new_tokens=6) for p in prompts]
+    finished = 0
+    while model.engine_has_unfinished():
+        finished += model.engine_step()
+    assert finished == 3 and model.engine_num_seqs() == 3
+    for i, p in zip(ids, prompts):
+        assert model.engine_is_finished(i) and model.engine_get_output(i) == P.greedy_generate(pcfg, w, p, 6)
+    model.engine_stop()
+
+
+def test_seeded_sampling_does_not_depend_on_the_batch(tmp_path, device):
+    from litinfer_amd.engine import Scheduler
+    from litinfer_amd.sampling import SamplingParams
+    d = helpers.make_model(tmp_path, TINY_B, 1)
+    prompts = list(helpers.random_requests(320, [1, 16, 40, 100], 3).values())
+    params = [SamplingParams(temperature=0.8, seed=s) for s in range(4)]
+
+    def run(which, **kw):
+        eng = engine_for(d, device, page=8, max_tokens=1024)
+        s = Scheduler(eng, eos_token_ids=(), **kw)
+        ids = [s.add_request(prompts[i], 24, params[i]) for i in which]
+        s.run_to_completion()
+        return [s.output(i) for i in ids]
+    together = run(range(4), chunk_size=24, max_batch_tokens=48)
+    alone = [run([i])[0] for i in range(4)]
+    assert together == alone and all(len(t) == 24 for t in together)
+    assert len({tuple(t) for t in together}) == 4
+
+
+def test_step_refuses_bad_batches_and_leaves_the_cache_alone(tmp_path, device):
+    d = helpers.make_model(tmp_path, TINY_A, 0)
+    eng = engine_for(d, device, max_tokens=64)
+    eng.step([StepEntry("a", [1, 2, 3], [])])
+    before = (eng.cache.free_pages(), eng.cache.cached_len("a"))
+    for bad in ([], [StepEntry("a", [], [])], [StepEntry("a", [256], [0])], [StepEntry("a", [-1], [0])],
+                [StepEntry("a", [1], [1])], [StepEntry("a", [1], []), StepEntry("a", [2], [])],
+                [StepEntry("b", [1] * 129, [])]):
+        with pytest.raises(StepError):
+            eng.step(bad)
+    with pytest.raises(CacheFull):
+        eng.step([StepEntry("a", [1], []), StepEntry("c", [1] * 60, [])])
+    assert (eng.cache.free_pages(), eng.cache.cached_len("a")) == before and not eng.cache.has("c")
+    assert eng.step([StepEntry("a", [4], [])]) is None                 # nothing wanted: nothing returned
+    eng.finish("a")
+    eng.finish("a")                                                    # ending twice is harmless
+    assert eng.cache.free_pages() == [4]
+
+
+def test_matrices_stored_in_32_bit_stay_32_bit_in_the_bfloat16_engine(tmp_path, device):
+    d = helpers.make_model(tmp_path, TINY_A, 0, torch.float32)
+    toks = helpers.random_requests(256, [40], 1)["r0"]
+    ref = helpers.plain_logits(d, {"r0": toks})["r0"]
+    eng = engine_for(d, device, dtype="bfloat16")
+    assert eng.model.layers[0].mixer.qkv.weight.dtype is torch.float32
+    assert eng.model.layers[0].norm1.weight.dtype is torch.float32
+    out = eng.step([StepEntry("a", toks, list(range(40)))]).cpu().numpy()
+    assert schedules.rel_err(out, ref) < BF16_TOL
+
+
+# ------------------------------------------------------ each part on its own
+def _rt(device, dtype=torch.float32):
+    return Runtime(torch.device(device), dtype)
+
+
+def _load(part, tensors):
+    part.load_params(lambda name: tensors.get(name))
+    return part
+
+
+def test_norm_part_alone(device):
+    g = torch.Generator().manual_seed(0)
+    x, w = torch.randn(9, 120, generator=g), 1 + 0.1 * torch.randn(120, generator=g)
+    part = _load(build_part("norm", PartSpec("rmsnorm", "n.", {"size": 120, "eps": 1e-4}), _rt(device)), {"n.weight": w})
+    assert part.expected_params() == {"n.weight": ParamSpec((120,))}
+    out = torch.empty(9, 120, device=device)
+    part.forward(x.to(device), out)
+    assert schedules.rel_err(out.cpu().numpy(), P.rms_norm(x.double().numpy(), w.double().numpy(), 1e-4)) < 2e-6
+
+
+def test_feed_forward_part_alone(device):
+    g = torch.Generator().manual_seed(1)
+    h, i, t = 72, 200, 11
+    ws = {f"f.{n}_proj.weight": torch.randn(*s, generator=g) * 0.1 for n, s in
+          (("gate", (i, h)), ("up", (i, h)), ("down", (h, i)))}
+    part = _load(build_part("feed_forward", PartSpec("swiglu_mlp", "f.", {"hidden_size": h, "intermediate_size": i}),
+                            _rt(device)), ws)
+    x = torch.randn(t, h, generator=g)
+    res = torch.randn(t, h, generator=g)
+    out = res.clone().to(device)
+    ctx = type("Ctx", (), {"ws": Workspace(device)})()
+    part.forward(x.to(device), out, ctx)
+    xd = x.double().numpy()
+    d = {k: v.double().numpy() for k, v in ws.items()}
+    ref = res.double().numpy() + P.swiglu(xd @ d["f.gate_proj.weight"].T, xd @ d["f.up_proj.weight"].T) @ d["f.down_proj.weight"].T
+    assert schedules.rel_err(out.cpu().numpy(), ref) < 2e-6
+
+
+def _mixer_case(device, window, cache_steps):
+    """Run the attention mixer alone over two requests in several steps and
+    return (its additions to a zero residual, the plain result)."""
+    g = torch.Generator().manual_seed(2)
+    h, nh, nkv, dh, page = 40, 6, 2, 16, 4
+    args = {"hidden_size": h, "num_heads": nh, "num_kv_heads": nkv, "head_dim": dh, "qkv_bias": True,
+            "window": window, "scale": None,
+            "position": PartSpec("rope_neox", "", {"head_dim": dh, "rotary_dim": dh, "theta": 1e4})}
+    ws = {f"a.{n}_proj.weight": torch.randn(o, h, generator=g) * 0.2 for n, o in (("q", nh * dh), ("k", nkv * dh), ("v", nkv * dh))}
+    ws.update({f"a.{n}_proj.bias": torch.randn(o, generator=g) * 0.2 for n, o in (("q", nh * dh), ("k", nkv * dh), ("v", nkv * dh))})
+    ws["a.o_proj.weight"] = torch.randn(h, nh * dh, generator=g) * 0.2
+    mixer = _load(build_part("mixer", PartSpec("gqa_attention", "a.", args), _rt(device)), ws)
+    cache = CacheManager([mixer.cache_need()], [None], page_size=page, num_pages=16, max_seqs=2,
+                         dtype=torch.float32, device=device, page_order_seed=3)
+    xs = {"p": torch.randn(19, h, generator=g), "q": torch.randn(7, h, generator=g)}
+    wsp, up = Workspace(device), BatchUploader(device)
+    got = {k: [] for k in xs}
+    done = {k: 0 for k in xs}
+    for step in cache_steps:
+        entries = [StepEntry(r, [0] * n, []) for r, n in step]
+        for e in entries:
+            if not cache.has(e.rid):
+                cache.admit(e.rid)
+            cache.reserve(e.rid, len(e.tokens))
+        ctx = build_context(cache, entries, wsp, up)
+        x = torch.cat([xs[r][done[r]:done[r] + n] for r, n in step]).to(device)
+        res = torch.zeros(x.shape[0], h, device=device)
+        mixer.forward(x, res, ctx, cache.view(0))
+        o = 0
+        for r, n in step:
+            got[r].append(res[o:o + n].cpu().numpy())
+            cache.commit(r, n)
+            done[r] += n
+            o += n
+    d = {k: v.double().numpy() for k, v in ws.items()}
+    ref = {}
+    for r, x in xs.items():
+        xd, t = x.double().numpy(), x.shape[0]
+        q = P.rope_neox((xd @ d["a.q_proj.weight"].T + d["a.q_proj.bias"]).reshape(t, nh, dh), np.arange(t), 1e4)
+        k = P.rope_neox((xd @ d["a.k_proj.weight"].T + d["a.k_proj.bias"]).reshape(t, nkv, dh), np.arange(t), 1e4)
+        v = (xd @ d["a.v_proj.weight"].T + d["a.v_proj.bias"]).reshape(t, nkv, dh)
+        a = P.attention(q, k, v, np.arange(t), np.arange(t), 1 / math.sqrt(dh), window)
+        ref[r] = a.reshape(t, -1) @ d["a.o_proj.weight"].T
+    return {r: np.concatenate(v) for r, v in got.items()}, ref
+
+
+@pytest.mark.parametrize("window", [0, 5])
+def test_attention_mixer_alone_over_a_cut_up_batch(device, window):
+    steps = [[("p", 6)], [("p", 2), ("q", 3)], [("p", 1), ("q", 1)], [("q", 3), ("p", 10)]]
+    got, ref = _mixer_case(device, window, steps)
+    for r in ref:
+        assert schedules.rel_err(got[r], ref[r]) < 3e-6
+
+
+def test_position_part_alone(device):
+    g = torch.Generator().manual_seed(4)
+    part = build_part("position", PartSpec("rope_neox", "", {"head_dim": 24, "rotary_dim": 24, "theta": 5e4}), _rt(device))
+    x = torch.randn(5, 3 * 24, generator=g)
+    pos = np.array([0, 1, 7, 8, 100], dtype=np.int32)
+    ctx = type("Ctx", (), {})()
+    ctx.ws, ctx.num_tokens, ctx.positions, ctx._s = Workspace(device), 5, torch.from_numpy(pos).to(device), {}
+    ctx.shared = lambda key, make: ctx._s.setdefault(key, make())
+    xd = x.clone().to(device)
+    part.apply(xd, 3, 24, ctx)
+    ref = P.rope_neox(x.double().numpy().reshape(5, 3, 24), pos, 5e4).reshape(5, -1)
+    assert schedules.rel_err(xd.cpu().numpy(), ref) < 1e-5
+    with pytest.raises(ValueError):
+        build_part("position", PartSpec("rope_neox", "", {"head_dim": 24, "rotary_dim": 26, "theta": 1.0}), _rt(device))
+    with pytest.raises(KeyError, match="registered: .*rope_neox"):
+        build_part("position", PartSpec("nope"), _rt(device))
+
+
+def test_embedding_and_head_alone(device):
+    g = torch.Generator().manual_seed(5)
+    table = torch.randn(301, 56, generator=g)
+    emb = _load(build_part("embedding", PartSpec("token_embedding", "e.", {"vocab_size": 301, "hidden_size": 56}),
+                           _rt(device)), {"e.weight": table})
+    ids = torch.tensor([300, 0, 7, 7], dtype=torch.int32)
+    out = torch.empty(4, 56, device=device)
+    emb.forward(ids.to(device), out)
+    assert torch.equal(out.cpu(), table[ids.long()])
+    head = build_part("head", PartSpec("linear_head", "h.", {"vocab_size": 301, "hidden_size": 56, "tied_to": "e.weight"}),
+                      _rt(device))
+    head.load_params(lambda n: None, tied_table=emb.table)
+    assert head.expected_params() == {}
+    logits = torch.empty(4, 301, device=device)
+    head.forward(out, logits, Workspace(device))
+    assert schedules.rel_err(logits.cpu().numpy(), (table[ids.long()] @ table.T).double().numpy()) < 2e-6
+
+
+# ------------------------------------- the order of layers is data: twice, shared cache
+def _looped_spec(c: Qwen2Config) -> ModelSpec:
+    base = qwen2_model_spec(c)
+    return replace(base, architecture="LoopedQwen2Test",
+                   order=(ExecEntry(0), ExecEntry(1), ExecEntry(0), ExecEntry(1, cache_from=1)))
+
+
+register_architecture("LoopedQwen2Test", Qwen2Config.from_dict, _looped_spec)
+
+
+def test_a_layer_named_twice_and_a_layer_reading_anothers_cache(tmp_path, device):
+    cfg = dict(TINY_A, architectures=["LoopedQwen2Test"])
+    d = helpers.make_model(tmp_path, cfg, 3)
+    pcfg, w = P.load_folder(d)
+    reqs = helpers.random_requests(256, [37, 9], 4)
+    order = [(0, None), (1, None), (0, None), (1, 1)]
+    ref = {r: P.forward(pcfg, w, t, order=order) for r, t in reqs.items()}
+    eng = engine_for(d, device)
+    assert len(eng.cache.groups) == 1 and eng.cache.groups[0].entries == [0, 1, 2]   # three caches, four entries
+    for kind in ("whole", "chunks", "mixed"):
+        out = schedules.run(eng, reqs, getattr(schedules, kind)(reqs))
+        assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind
+
+
+# ------------------------------ a toy mixer with state of its own, defined here
+class ToyStateMixer(Mixer):
+    """s_t = decay * s_{t-1} + xn_t, y_t = s_t W^T: a recurrent mixer whose state
+    lives in the request's state slot.  Written with torch: it is a toy."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.h = spec.args["hidden_size"]
+        self.decay = spec.args["decay"]
+        self.w = None
+
+    def cache_need(self):
+        return StateNeed((self.h,), torch.float32)
+
+    def expected_params(self):
+        return {self.prefix + "w": ParamSpec((self.h, self.h))}
+
+    def load_params(self, get):
+        self.w = get(self.prefix + "w").to(torch.float32).to(self.rt.device)
+
+    def forward(self, xn, residual, ctx, cache):
+        for s in range(ctx.num_segments):
+            q0, n, slot = int(ctx.host_q_start[s]), int(ctx.host_q_len[s]), int(ctx.host_state_slots[s])
+            state = cache.state[slot]
+            for t in range(q0, q0 + n):
+                state.mul_(self.decay).add_(xn[t].float())
+                residual[t] += state @ self.w.T
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    hidden_size: int
+    vocab_size: int
+    decay: float
+    inner: Qwen2Config
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(raw["hidden_size"], raw["vocab_size"], raw["toy_decay"], Qwen2Config.from_dict(raw))
+
+
+def _toy_spec(c: ToyConfig) -> ModelSpec:
+    base = qwen2_model_spec(c.inner)
+    l0 = base.layers[0]
+    toy = LayerSpec("prenorm", dict(l0.parts, mixer=PartSpec("toy_state", "model.layers.0.toy.",
+                                                             {"hidden_size": c.hidden_size, "decay": c.decay})))
+    return replace(base, architecture="ToyStateLM", layers=(toy,) + base.layers[1:])
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, device):
+    register_part("mixer", "toy_state", ToyStateMixer)
+    register_architecture("ToyStateLM", ToyConfig.from_dict, _toy_spec)
+    cfg = dict(TINY_A, architectures=["ToyStateLM"], toy_decay=0.9)
+    d = helpers.make_model(tmp_path, cfg, 6)
+    pcfg, w = P.load_folder(d)
+    assert "model.layers.0.toy.w" in w and "model.layers.0.self_attn.q_proj.weight" not in w
+
+    def plain(ids):
+        pos = np.arange(len(ids))
+        x = P.embedding(ids, w["model.embed_tokens.weight"])
+        xn = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], 1e-6)
+        s = np.zeros(64)
+        y = np.zeros_like(x)
+        for t in range(len(ids)):
+            s = 0.9 * s + xn[t]
+            y[t] = s @ w["model.layers.0.toy.w"].T
+        x = x + y
+        xn = P.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], 1e-6)
+        p = "model.layers.0.mlp."
+        x = x + P.swiglu(xn @ w[p + "gate_proj.weight"].T, xn @ w[p + "up_proj.weight"].T) @ w[p + "down_proj.weight"].T
+        x, _ = P.decoder_layer(x, pos, w, "model.layers.1.", pcfg, 0)
+        return P.rms_norm(x, w["model.norm.weight"], 1e-6) @ w["model.embed_tokens.weight"].T
+
+    reqs = helpers.random_requests(256, [21, 40, 3, 30, 12], 7)
+    ref = {r: plain(np.asarray(t)) for r, t in reqs.items()}
+    eng = engine_for(d, device)
+    assert len(eng.cache.groups) == 1 and eng.cache.groups[0].entries == [1]
+    assert eng.cache.view(0).state.shape == (4, 64)
+    for kind in ("whole", "tail", "chunks", "mixed"):
+        out = schedules.run(eng, reqs, getattr(schedules, kind)(reqs))
+        assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind   # slots reused, state zeroed
+    eng.cache.check_invariants()

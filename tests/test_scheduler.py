@@ -1,0 +1,173 @@
+"""The scheduler's decisions, on the CPU with a stand-in engine whose logits
+are canned: budget, portions, first come first served, finishing rules,
+preemption when pages run out."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from litinfer_amd.cache import CacheManager
+from litinfer_amd.engine import Scheduler
+from litinfer_amd.parts import PagedKVNeed
+from litinfer_amd.sampling import SamplingParams, uniform
+
+VOCAB = 50
+
+
+class FakeEngine:
+    """Owns a real cache manager; `step` does the bookkeeping of the real one
+    and returns logits whose argmax is (last token + 1) % VOCAB."""
+
+    def __init__(self, num_pages=8, page=4, max_seqs=4, max_positions=64, eos=()):
+        self.cache = CacheManager([PagedKVNeed(1, 4, 0)], [None], page_size=page, num_pages=num_pages,
+                                  max_seqs=max_seqs, dtype=torch.float32, device="cpu")
+        self.spec = SimpleNamespace(vocab_size=VOCAB, max_positions=max_positions, eos_token_ids=tuple(eos))
+        self.rt = SimpleNamespace(device=torch.device("cpu"))
+        self.batches = []
+
+    def step(self, entries):
+        for e in entries:
+            if not self.cache.has(e.rid):
+                self.cache.admit(e.rid)
+        for e in entries:
+            self.cache.reserve(e.rid, len(e.tokens))
+        rows = []
+        for e in entries:
+            self.cache.commit(e.rid, len(e.tokens))
+            for w in e.want:
+                row = torch.zeros(VOCAB)
+                row[(e.tokens[w] + 1) % VOCAB] = 5.0
+                rows.append(row)
+        self.batches.append([(e.rid, len(e.tokens), list(e.want)) for e in entries])
+        self.cache.check_invariants()
+        return torch.stack(rows) if rows else None
+
+    def finish(self, rid):
+        if self.cache.has(rid):
+            self.cache.release(rid)
+
+
+class HostSampler:
+    def sample(self, logits, params, counters):
+        import torch_ops
+        n = logits.shape[0]
+        out = torch.empty(n, dtype=torch.int32)
+        torch_ops.sample_rows(logits, torch.tensor([p.temperature for p in params]),
+                              torch.tensor([p.top_k for p in params]), torch.tensor([p.top_p for p in params]),
+                              torch.tensor([uniform(p.seed, c) for p, c in zip(params, counters)]), out)
+        return out.tolist()
+
+
+def sched(engine, **kw):
+    return Scheduler(engine, sampler=HostSampler(), **kw)
+
+
+def test_budget_portions_and_logits_only_at_the_prompts_end():
+    e = FakeEngine(num_pages=32)
+    s = sched(e, max_batch_tokens=10, chunk_size=6)
+    a = s.add_request(list(range(14)), max_new_tokens=3)
+    b = s.add_request(list(range(20, 25)), max_new_tokens=2)
+    s.run_to_completion()
+    assert e.batches[0] == [(a, 6, []), (b, 4, [])]               # budget 10 = 6 + 4, no logits yet
+    assert e.batches[1] == [(b, 1, [0]), (a, 6, [])]              # b's prompt ends: one row of logits
+    assert e.batches[2] == [(b, 1, [0]), (a, 2, [1])]             # single tokens first, then a's last portion
+    assert all(sum(n for _, n, _ in batch) <= 10 for batch in e.batches)
+    assert s.output(a) == [14, 15, 16] and s.output(b) == [25, 26]
+    assert s.requests[a].finish_reason == "length" and e.cache.free_pages() == [32]
+
+
+def test_first_come_first_served_and_short_requests_finish_first():
+    # the reference's scheduler test: requests of length 2, 5, 10 all finish, in length order
+    # (scripts/test_engine_runtime.py:56-83)
+    e = FakeEngine(num_pages=32)
+    s = sched(e)
+    ids = [s.add_request([1, 2, 3], max_new_tokens=n) for n in (10, 2, 5)]
+    done = []
+    while s.has_unfinished():
+        s.step()
+        done += [i for i in ids if s.is_finished(i) and i not in done]
+    assert done == [ids[1], ids[2], ids[0]]
+    assert [r for r, _, _ in e.batches[0]] == ids                  # admitted in arrival order
+
+
+def test_end_token_is_dropped_and_length_token_is_kept():
+    e = FakeEngine(eos=(7,))
+    s = sched(e)
+    a = s.add_request([4], max_new_tokens=10)                      # 5, 6, then 7 = end: dropped
+    b = s.add_request([6], max_new_tokens=10)                      # the very first token is the end token
+    c = s.add_request([10], max_new_tokens=2)
+    s.run_to_completion()
+    assert s.output(a) == [5, 6] and s.requests[a].finish_reason == "eos"
+    assert s.output(b) == [] and s.requests[b].finish_reason == "eos"
+    assert s.output(c) == [11, 12] and s.requests[c].finish_reason == "length"
+
+
+def test_submission_checks():
+    e = FakeEngine(num_pages=4, page=4, max_positions=32)
+    s = sched(e)
+    with pytest.raises(ValueError, match="must not be empty"):
+        s.add_request([], 4)
+    with pytest.raises(ValueError, match="max sequence length"):
+        s.add_request(list(range(30)), 4)                          # 30 + 4 - 1 > 32
+    with pytest.raises(ValueError, match="could never run"):
+        s.add_request(list(range(10)), 10)                         # 19 tokens need 5 pages of 4
+    with pytest.raises(ValueError, match="vocabulary"):
+        s.add_request([VOCAB], 1)
+    s.add_request(list(range(10)), 7)                              # 16 tokens: exactly the pool
+
+
+def test_out_of_pages_preempts_the_latest_and_tokens_stay_the_same():
+    def run(num_pages):
+        e = FakeEngine(num_pages=num_pages, page=4, max_seqs=3)
+        s = sched(e, max_batch_tokens=64, chunk_size=64)
+        ids = [s.add_request([i * 10 + j for j in range(6)], max_new_tokens=9,
+                             params=SamplingParams(temperature=0.9, seed=i)) for i in range(3)]
+        s.run_to_completion(max_steps=500)
+        assert not s.has_unfinished() and e.cache.free_pages() == [num_pages]
+        return [s.output(i) for i in ids], s
+    plenty, s0 = run(32)
+    scarce, s1 = run(8)                     # 3 requests x 15 tokens need 12 pages: they cannot all stay
+    assert s0.preemptions == 0 and s1.preemptions > 0
+    assert scarce == plenty
+    victim = max(s1.requests.values(), key=lambda r: r.preemptions)
+    assert victim.rid == 2                  # the most recently admitted one is the one that yields
+
+
+def test_waiting_request_is_admitted_when_pages_come_back():
+    e = FakeEngine(num_pages=4, page=4, max_seqs=4)
+    s = sched(e)
+    a = s.add_request(list(range(12)), max_new_tokens=4)           # 15 tokens: 4 pages, the whole pool
+    b = s.add_request(list(range(5)), max_new_tokens=2)
+    s.step()
+    assert [r for r, _, _ in e.batches[0]] == [a] and s.requests[b].state == "waiting"
+    s.run_to_completion()
+    assert s.output(b) == [5, 6] and s.requests[a].preemptions == 0
+
+
+def test_a_lone_request_that_outgrows_the_pool_ends_with_an_error():
+    e = FakeEngine(num_pages=2, page=4)
+    s = sched(e)
+    a = s.add_request([1, 2, 3], max_new_tokens=6)
+    e.cache.admit("other")                                         # someone else holds a page for good
+    e.cache.reserve("other", 4)
+    s.run_to_completion(max_steps=50)
+    assert s.is_finished(a) and s.requests[a].finish_reason == "error: kv capacity"
+    assert len(s.output(a)) == 2                                   # it got as far as its one page allowed
+
+
+def test_abort_gives_everything_back():
+    e = FakeEngine()
+    s = sched(e)
+    a = s.add_request(list(range(9)), 5)
+    s.step()
+    s.abort(a)
+    assert s.is_finished(a) and e.cache.free_pages() == [8] and not s.has_unfinished()
+    assert s.requests[a].finish_reason == "aborted"
+
+
+def test_sampling_stream_is_per_request():
+    # the k-th draw of a request depends on (seed, k) only
+    assert uniform(3, 0) == uniform(3, 0) and uniform(3, 0) != uniform(3, 1) != uniform(4, 1)
+    assert all(0.0 <= uniform(s, c) < 1.0 for s in range(20) for c in range(50))
+    mean = sum(uniform(1, c) for c in range(4000)) / 4000
+    assert abs(mean - 0.5) < 0.03

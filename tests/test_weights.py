@@ -1,0 +1,127 @@
+"""The safetensors reader and writer, the loader's one error, random weights."""
+import json
+import struct
+
+import numpy as np
+import pytest
+import torch
+
+import plain_impl
+from litinfer_amd.config import Qwen2Config, qwen2_model_spec
+from litinfer_amd.engine import expected_params_of_spec
+from litinfer_amd.weights import (CheckpointFolder, ParamSpec, SafetensorsFile, WeightError, check_entries,
+                                  stored_precision, write_random_model, write_safetensors)
+from tiny_configs import TINY_A, TINY_B
+
+
+def test_safetensors_round_trip_and_own_reader_agrees(tmp_path):
+    g = torch.Generator().manual_seed(0)
+    tensors = [("a", torch.randn(3, 5, generator=g)), ("b.c", torch.randn(7, generator=g).to(torch.bfloat16)),
+               ("t", torch.arange(6, dtype=torch.int64).reshape(2, 3))]
+    write_safetensors(tmp_path / "x.safetensors", tensors, metadata={"k": "v"})
+    f = SafetensorsFile(tmp_path / "x.safetensors")
+    assert f.entries == {"a": ("F32", (3, 5)), "b.c": ("BF16", (7,)), "t": ("I64", (2, 3))}
+    for n, t in tensors:
+        assert torch.equal(f.tensor(n), t)
+    other = plain_impl.read_safetensors(tmp_path / "x.safetensors", np.float64)     # the tests' own reader
+    assert np.array_equal(other["b.c"], tensors[1][1].double().numpy())
+    from safetensors import safe_open                                               # and the format's library
+    with safe_open(str(tmp_path / "x.safetensors"), "pt") as sf:
+        assert torch.equal(sf.get_tensor("b.c"), tensors[1][1])
+
+
+def test_offsets_are_checked(tmp_path):
+    header = json.dumps({"w": {"dtype": "F32", "shape": [4], "data_offsets": [0, 12]}}).encode()
+    (tmp_path / "bad.safetensors").write_bytes(struct.pack("<Q", len(header)) + header + b"\0" * 16)
+    with pytest.raises(ValueError, match="data_offsets"):
+        SafetensorsFile(tmp_path / "bad.safetensors")
+
+
+def test_stored_precision():
+    assert stored_precision(torch.zeros(2, dtype=torch.bfloat16), False).dtype is torch.bfloat16
+    assert stored_precision(torch.zeros(2, dtype=torch.float32), False).dtype is torch.float32
+    assert stored_precision(torch.zeros(2, dtype=torch.float16), False).dtype is torch.float32
+    assert stored_precision(torch.zeros(2, dtype=torch.int64), True).dtype is torch.int32
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes():
+    expected = {"a": ParamSpec((2, 3)), "b": ParamSpec((4,)), "bias": ParamSpec((4,), required=False),
+                "c": ParamSpec((5,))}
+    found = {"a": ("F32", (3, 2)), "zzz": ("F32", (1,)), "c": ("I32", (5,)),
+             "x.rotary_emb.inv_freq": ("F32", (8,))}
+    with pytest.raises(WeightError) as e:
+        check_entries(expected, found, lambda n: n.endswith("rotary_emb.inv_freq"))
+    err = e.value
+    assert err.missing == ["b"] and err.unexpected == ["zzz"]
+    assert err.wrong_shape == [("a", (2, 3), (3, 2))] and err.wrong_dtype[0][0] == "c"
+    msg = str(err)
+    for word in ("missing tensors (1)", "- b", "unexpected tensors (1)", "- zzz", "wrong shapes (1)",
+                 "a: expected [2, 3], found [3, 2]"):
+        assert word in msg
+
+
+def test_expected_tensor_names_are_the_checkpoints():
+    names = expected_params_of_spec(qwen2_model_spec(Qwen2Config.from_dict(TINY_B)))
+    assert names["model.embed_tokens.weight"].shape == (320, 96)
+    assert names["lm_head.weight"].shape == (320, 96) and names["model.norm.weight"].shape == (96,)
+    p = "model.layers.2."
+    assert names[p + "self_attn.q_proj.weight"].shape == (96, 96)
+    assert names[p + "self_attn.k_proj.weight"].shape == (32, 96)
+    assert names[p + "self_attn.v_proj.bias"].shape == (32,) and not names[p + "self_attn.v_proj.bias"].required
+    assert names[p + "self_attn.o_proj.weight"].shape == (96, 96)
+    assert names[p + "mlp.gate_proj.weight"].shape == (224, 96)
+    assert names[p + "mlp.down_proj.weight"].shape == (96, 224)
+    assert names[p + "post_attention_layernorm.weight"].shape == (96,)
+    assert len(names) == 3 + 3 * 12
+    tied = expected_params_of_spec(qwen2_model_spec(Qwen2Config.from_dict(TINY_A)))
+    assert "lm_head.weight" not in tied
+
+
+def test_random_model_folder_is_seeded_and_distributed_as_said(tmp_path):
+    a = write_random_model(tmp_path / "a", TINY_B, seed=3, dtype=torch.float32)
+    b = write_random_model(tmp_path / "b", TINY_B, seed=3, dtype=torch.float32)
+    c = write_random_model(tmp_path / "c", TINY_B, seed=4, dtype=torch.float32)
+    fa, fb, fc = (CheckpointFolder(x) for x in (a, b, c))
+    name = "model.layers.1.mlp.up_proj.weight"
+    assert torch.equal(fa.tensor(name), fb.tensor(name)) and not torch.equal(fa.tensor(name), fc.tensor(name))
+    w = fa.tensor(name)
+    assert abs(float(w.mean())) < 2e-3 and abs(float(w.std()) - 0.02) < 2e-3
+    n = fa.tensor("model.layers.0.input_layernorm.weight")
+    assert abs(float(n.mean()) - 1.0) < 1e-2 and float(n.std()) < 0.04
+    assert abs(float(fa.tensor("model.layers.0.self_attn.q_proj.bias").mean())) < 2e-2
+    assert json.loads((a / "config.json").read_text())["num_hidden_layers"] == 3
+    assert SafetensorsFile(write_random_model(tmp_path / "d", TINY_B, 3, torch.bfloat16) /
+                           "model.safetensors").entries[name][0] == "BF16"
+
+
+def _load(folder, cpu_ops):
+    from litinfer_amd.engine import Engine
+    return Engine.from_dir(folder, dtype="float32", device="cpu", max_tokens=64, max_seqs=2)
+
+
+def test_loader_raises_one_error_for_a_broken_folder(tmp_path, cpu_ops):
+    d = write_random_model(tmp_path / "m", TINY_A, seed=0, dtype=torch.float32)
+    f = SafetensorsFile(d / "model.safetensors")
+    tensors = {n: f.tensor(n).clone() for n in f.entries}
+    f.close()
+    del tensors["model.layers.1.mlp.down_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(16, 64)
+    tensors["model.layers.9.mlp.up_proj.weight"] = torch.zeros(2, 2)
+    write_safetensors(d / "model.safetensors", tensors.items())
+    with pytest.raises(WeightError) as e:
+        _load(d, cpu_ops)
+    assert e.value.missing == ["model.layers.1.mlp.down_proj.weight", "model.norm.weight"]
+    assert e.value.unexpected == ["model.layers.9.mlp.up_proj.weight"]
+    assert e.value.wrong_shape == [("model.layers.0.self_attn.k_proj.weight", (32, 64), (16, 64))]
+
+
+def test_biases_are_optional_and_tied_head_shares_the_table(tmp_path, cpu_ops):
+    d = write_random_model(tmp_path / "m", TINY_A, seed=0, dtype=torch.float32)
+    f = SafetensorsFile(d / "model.safetensors")
+    tensors = {n: f.tensor(n).clone() for n in f.entries if not n.endswith("bias")}
+    f.close()
+    write_safetensors(d / "model.safetensors", tensors.items())
+    eng = _load(d, cpu_ops)
+    assert eng.model.layers[0].mixer.qkv.bias is None
+    assert eng.model.head.proj.weight.data_ptr() == eng.model.embedding.table.data_ptr()

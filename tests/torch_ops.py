@@ -116,3 +116,30 @@ def argmax_rows(logits, out):
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
        "rope_apply", "kv_store", "rope_kv_store", "linear", "check_attention_sizes",
        "paged_attention", "argmax_rows"]
+
+
+def sample_rows(logits, temperature, top_k, top_p, uniform, out):
+    import numpy as np
+    lg = logits.double().numpy()
+    for r in range(lg.shape[0]):
+        t = float(temperature[r])
+        if not t > 0:
+            out[r] = int(np.argmax(lg[r]))
+            continue
+        z = lg[r] / t
+        order = np.lexsort((np.arange(z.size), -z))
+        k, p = int(top_k[r]), float(top_p[r])
+        if 0 < k < z.size:
+            order = order[:k]
+        if 0 < p < 1:
+            e = np.exp(z[order] - z[order[0]])
+            cum = np.cumsum(e / e.sum())
+            order = order[:int(np.argmax(cum >= p)) + 1] if (cum >= p).any() else order
+        keep = np.sort(order)
+        e = np.exp(z[keep] - z[keep].max())
+        cum = np.cumsum(e)
+        i = int(np.searchsorted(cum, float(uniform[r]) * cum[-1], side="left"))
+        out[r] = int(keep[min(i, keep.size - 1)])
+
+
+ALL.append("sample_rows")
