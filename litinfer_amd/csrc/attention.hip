@@ -18,13 +18,13 @@ template <typename T>
 __global__ __launch_bounds__(64) void paged_attention_wave_kernel(
     const T* __restrict__ q, int q_row_stride, T* __restrict__ out, const T* __restrict__ kc,
     const T* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
-    const int* __restrict__ seg_of_token, const int* __restrict__ q_start,
-    const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int dh,
-    int page_size, int num_pages, int window, float scale) {
+    const int* __restrict__ token_list, const int* __restrict__ seg_of_token,
+    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+    int nh, int nkv, int dh, int page_size, int num_pages, int window, float scale) {
     __shared__ float qs[ATT_MAX_DH];
     __shared__ float ps[LI_WAVE];
     __shared__ int rowoff[LI_WAVE];          // element offset / dh of each key's row, -1 = not there
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int t = token_list ? token_list[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int s = seg_of_token[t];
     const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
@@ -81,10 +81,279 @@ __global__ __launch_bounds__(64) void paged_attention_wave_kernel(
     }
 }
 
+// ------------------------------------------------------ single-query tokens
+// Decode: one query per sequence, so the work is reading the keys and values
+// once.  A block of 4 waves takes one (token, kv head, split of the keys) and
+// all the query heads of that kv head, so a page is read once for the whole
+// group.  A key's row is spread over LPK lanes (16 bytes each); a wave handles
+// 64 / LPK keys a round and U rounds are in flight.  Every lane group keeps an
+// online softmax (m, l, acc) per head over its keys; the groups of a wave are
+// merged by a butterfly, the waves through LDS in wave order, the splits by
+// `attention_merge_kernel` in split order: all fixed orders.
+template <typename T> struct raw16;
+template <> struct raw16<bf16_t> { static constexpr int E = 8; };
+template <> struct raw16<float> { static constexpr int E = 4; };
+
+struct __attribute__((aligned(16))) u32x4 { uint32_t w[4]; };
+
+template <typename T, int E>
+__device__ __forceinline__ void unpack16(const u32x4& r, float* f) {
+    if constexpr (E == 8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(r.w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(r.w[i] & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(r.w[i]);
+    }
+}
+
+__device__ __forceinline__ void softmax_merge(float& m, float& l, float* acc, int n, float mo, float lo,
+                                              const float* acco) {
+    const float mx = fmaxf(m, mo);
+    if (mx == -INFINITY) return;                       // both sides empty
+    const float a = expf(m - mx), b = expf(mo - mx);   // exp(-inf) = 0 for an empty side
+    l = l * a + lo * b;
+    for (int j = 0; j < n; ++j) acc[j] = acc[j] * a + acco[j] * b;
+    m = mx;
+}
+
+template <typename T, int LPK, int GB>
+__global__ __launch_bounds__(256) void paged_attention_decode_kernel(
+    const T* __restrict__ q, int q_row_stride, T* __restrict__ out, const T* __restrict__ kc,
+    const T* __restrict__ vc, const int* __restrict__ block_table, int max_blocks,
+    const int* __restrict__ token_list, const int* __restrict__ seg_of_token,
+    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv, int dh, int page_size,
+    int num_pages, int window, float scale, int nsplit) {
+    constexpr int E = raw16<T>::E;
+    constexpr int KPW = 64 / LPK;
+    constexpr int U = 4;
+    __shared__ float sm_acc[4][GB][ATT_MAX_DH];
+    __shared__ float sm_ml[4][GB][2];
+    const int ti = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+    const int t = token_list ? token_list[ti] : ti;
+    const int G = nh / nkv;
+    const int s = seg_of_token[t];
+    const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int nkeys = p - lo + 1;
+    const int per = (((nkeys + nsplit - 1) / nsplit) + 63) & ~63;
+    const int k_begin = lo + split * per;
+    const int k_end = (k_begin + per < p + 1) ? k_begin + per : p + 1;
+    const int* table = block_table + (size_t)s * max_blocks;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int grp = lane / LPK, sub = lane % LPK;
+    const int d0 = sub * E;
+
+    for (int h0 = 0; h0 < G; h0 += GB) {
+        const int gcount = (G - h0 < GB) ? G - h0 : GB;
+        float qr[GB][E], acc[GB][E], m[GB], l[GB];
+#pragma unroll
+        for (int h = 0; h < GB; ++h) {
+            m[h] = -INFINITY;
+            l[h] = 0.f;
+#pragma unroll
+            for (int j = 0; j < E; ++j) { acc[h][j] = 0.f; qr[h][j] = 0.f; }
+            if (h < gcount) {
+                const T* qp = q + (size_t)t * q_row_stride + (size_t)(kvh * G + h0 + h) * dh + d0;
+                u32x4 r = *reinterpret_cast<const u32x4*>(qp);
+                unpack16<T, E>(r, qr[h]);
+            }
+        }
+        for (int r0 = 0;; r0 += U) {
+            const int wbase = k_begin + (r0 * 4 + wave) * KPW;
+            if (wbase >= k_end) break;
+            u32x4 kraw[U], vraw[U];
+            bool ok[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int key = wbase + u * 4 * KPW + grp;
+                ok[u] = key < k_end;
+                kraw[u] = u32x4{{0u, 0u, 0u, 0u}};
+                vraw[u] = kraw[u];
+                if (ok[u]) {
+                    const int page = table[key / page_size];
+                    ok[u] = page >= 0 && page < num_pages;
+                    if (ok[u]) {
+                        const size_t off = (((size_t)page * nkv + kvh) * page_size + key % page_size) * dh + d0;
+                        kraw[u] = *reinterpret_cast<const u32x4*>(kc + off);
+                        vraw[u] = *reinterpret_cast<const u32x4*>(vc + off);
+                    }
+                }
+            }
+            float sc[U][GB];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float kf[E];
+                unpack16<T, E>(kraw[u], kf);
+#pragma unroll
+                for (int h = 0; h < GB; ++h) {
+                    float dot = 0.f;
+#pragma unroll
+                    for (int j = 0; j < E; ++j) dot = fmaf(qr[h][j], kf[j], dot);
+#pragma unroll
+                    for (int o = 1; o < LPK; o <<= 1) dot += __shfl_xor(dot, o, LI_WAVE);
+                    sc[u][h] = ok[u] ? dot * scale : -INFINITY;
+                }
+            }
+            float vf[U][E];
+#pragma unroll
+            for (int u = 0; u < U; ++u) unpack16<T, E>(vraw[u], vf[u]);
+#pragma unroll
+            for (int h = 0; h < GB; ++h) {
+                float mx = m[h];
+#pragma unroll
+                for (int u = 0; u < U; ++u) mx = fmaxf(mx, sc[u][h]);
+                if (mx == -INFINITY) continue;
+                const float alpha = expf(m[h] - mx);
+                float pu[U], ps = 0.f;
+#pragma unroll
+                for (int u = 0; u < U; ++u) { pu[u] = expf(sc[u][h] - mx); ps += pu[u]; }
+                l[h] = l[h] * alpha + ps;
+#pragma unroll
+                for (int j = 0; j < E; ++j) {
+                    float a = acc[h][j] * alpha;
+#pragma unroll
+                    for (int u = 0; u < U; ++u) a = fmaf(pu[u], vf[u][j], a);
+                    acc[h][j] = a;
+                }
+                m[h] = mx;
+            }
+        }
+        // the lane groups of the wave
+#pragma unroll
+        for (int o = LPK; o < 64; o <<= 1) {
+#pragma unroll
+            for (int h = 0; h < GB; ++h) {
+                const float mo = __shfl_xor(m[h], o, LI_WAVE), lo2 = __shfl_xor(l[h], o, LI_WAVE);
+                float ao[E];
+#pragma unroll
+                for (int j = 0; j < E; ++j) ao[j] = __shfl_xor(acc[h][j], o, LI_WAVE);
+                softmax_merge(m[h], l[h], acc[h], E, mo, lo2, ao);
+            }
+        }
+        __syncthreads();                               // the last pass's readers are done
+        if (grp == 0) {
+#pragma unroll
+            for (int h = 0; h < GB; ++h) {
+#pragma unroll
+                for (int j = 0; j < E; ++j) sm_acc[wave][h][d0 + j] = acc[h][j];
+                if (sub == 0) { sm_ml[wave][h][0] = m[h]; sm_ml[wave][h][1] = l[h]; }
+            }
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < gcount * dh; idx += 256) {
+            const int h = idx / dh, d = idx - h * dh;
+            float mx = sm_ml[0][h][0];
+#pragma unroll
+            for (int w = 1; w < 4; ++w) mx = fmaxf(mx, sm_ml[w][h][0]);
+            float lt = 0.f, at = 0.f;
+            if (mx != -INFINITY) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const float f = expf(sm_ml[w][h][0] - mx);
+                    lt += sm_ml[w][h][1] * f;
+                    at += sm_acc[w][h][d] * f;
+                }
+            }
+            const int head = kvh * G + h0 + h;
+            if (nsplit == 1) {
+                store_from_float(out + (size_t)t * nh * dh + (size_t)head * dh + d, lt != 0.f ? at / lt : 0.f);
+            } else {
+                const size_t pi = ((size_t)ti * nh + head) * nsplit + split;
+                part_acc[pi * dh + d] = at;
+                if (d == 0) { part_ml[pi * 2] = mx; part_ml[pi * 2 + 1] = lt; }
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ void attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                       const int* __restrict__ token_list, T* __restrict__ out, int nh,
+                                       int dh, int nsplit) {
+    const int ti = blockIdx.x, head = blockIdx.y;
+    const int t = token_list ? token_list[ti] : ti;
+    const size_t base = ((size_t)ti * nh + head) * nsplit;
+    float mx = -INFINITY;
+    for (int sp = 0; sp < nsplit; ++sp) mx = fmaxf(mx, part_ml[(base + sp) * 2]);
+    for (int d = threadIdx.x; d < dh; d += blockDim.x) {
+        float lt = 0.f, at = 0.f;
+        if (mx != -INFINITY) {
+            for (int sp = 0; sp < nsplit; ++sp) {
+                const float f = expf(part_ml[(base + sp) * 2] - mx);
+                lt += part_ml[(base + sp) * 2 + 1] * f;
+                at += part_acc[(base + sp) * dh + d] * f;
+            }
+        }
+        store_from_float(out + (size_t)t * nh * dh + (size_t)head * dh + d, lt != 0.f ? at / lt : 0.f);
+    }
+}
+
+template <typename T>
+static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, const T* vc,
+                         const int* block_table, int max_blocks, const int* token_list, int n_tokens,
+                         const int* seg_of_token, const int* q_start, const int* q_len, const int* ctx_len,
+                         float* part_acc, float* part_ml, int nh, int nkv, int dh, int page_size,
+                         int num_pages, int window, float scale, int nsplit, hipStream_t stream) {
+    constexpr int E = raw16<T>::E;
+    if (dh % E) return LI_ERR_SIZE;
+    const int lpk = dh / E;
+    if (n_tokens > 0x7fffffff / 1 || nkv > 65535 || nsplit > 65535 || nsplit < 1) return LI_ERR_SIZE;
+    dim3 grid(n_tokens, nkv, nsplit);
+#define LI_DEC(LPK) paged_attention_decode_kernel<T, LPK, 8><<<grid, 256, 0, stream>>>( \
+        q, q_row_stride, out, kc, vc, block_table, max_blocks, token_list, seg_of_token, q_start, q_len, \
+        ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages, window, scale, nsplit)
+    switch (lpk) {
+        case 1: LI_DEC(1); break;
+        case 2: LI_DEC(2); break;
+        case 4: LI_DEC(4); break;
+        case 8: LI_DEC(8); break;
+        case 16: LI_DEC(16); break;
+        case 32: LI_DEC(32); break;
+        case 64: LI_DEC(64); break;
+        default: return LI_ERR_SIZE;
+    }
+#undef LI_DEC
+    if (nsplit > 1) {
+        dim3 g2(n_tokens, nh);
+        attention_merge_kernel<T><<<g2, 64, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit);
+    }
+    return li_launch_status();
+}
+
+// Single-query tokens of the batch (token_list, or all tokens when it is null).
+// part_acc: float [n_tokens, nh, nsplit, dh]; part_ml: float [n_tokens, nh, nsplit, 2] (unused when nsplit is 1).
+extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* out, const void* kc,
+                                         const void* vc, int dtype, const int* block_table, int max_blocks,
+                                         const int* token_list, int n_tokens, const int* seg_of_token,
+                                         const int* q_start, const int* q_len, const int* ctx_len,
+                                         float* part_acc, float* part_ml, int nh, int nkv, int dh,
+                                         int page_size, int num_pages, int window, float scale, int nsplit,
+                                         hipStream_t stream) {
+    if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dh <= 0 || dh > ATT_MAX_DH || page_size <= 0 ||
+        max_blocks <= 0)
+        return LI_ERR_SIZE;
+    if (dtype == LI_F32)
+        return launch_decode<float>((const float*)q, q_row_stride, (float*)out, (const float*)kc, (const float*)vc,
+                                    block_table, max_blocks, token_list, n_tokens, seg_of_token, q_start, q_len,
+                                    ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages, window, scale,
+                                    nsplit, stream);
+    if (dtype == LI_BF16)
+        return launch_decode<bf16_t>((const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc,
+                                     (const bf16_t*)vc, block_table, max_blocks, token_list, n_tokens,
+                                     seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, dh,
+                                     page_size, num_pages, window, scale, nsplit, stream);
+    return LI_ERR_DTYPE;
+}
+
 extern "C" int li_paged_attention(const void* q, int q_row_stride, void* out, const void* kc,
                                   const void* vc, int dtype, const int* block_table, int max_blocks,
-                                  const int* seg_of_token, const int* q_start, const int* q_len,
-                                  const int* ctx_len, int num_segments, int T, int max_q_len,
+                                  const int* token_list, const int* seg_of_token, const int* q_start,
+                                  const int* q_len, const int* ctx_len, int num_segments, int T, int max_q_len,
                                   int max_ctx_len, int nh, int nkv, int dh, int page_size,
                                   int num_pages, int window, float scale, hipStream_t stream) {
     if (T <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dh <= 0 || dh > ATT_MAX_DH || nh > 65535 ||
@@ -94,11 +363,11 @@ extern "C" int li_paged_attention(const void* q, int q_row_stride, void* out, co
     if (dtype == LI_F32)
         paged_attention_wave_kernel<float><<<grid, 64, 0, stream>>>(
             (const float*)q, q_row_stride, (float*)out, (const float*)kc, (const float*)vc, block_table,
-            max_blocks, seg_of_token, q_start, q_len, ctx_len, nh, nkv, dh, page_size, num_pages, window, scale);
+            max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, nh, nkv, dh, page_size, num_pages, window, scale);
     else if (dtype == LI_BF16)
         paged_attention_wave_kernel<bf16_t><<<grid, 64, 0, stream>>>(
             (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table,
-            max_blocks, seg_of_token, q_start, q_len, ctx_len, nh, nkv, dh, page_size, num_pages, window, scale);
+            max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, nh, nkv, dh, page_size, num_pages, window, scale);
     else return LI_ERR_DTYPE;
     return li_launch_status();
 }

@@ -176,6 +176,100 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
         }
 }
 
+// ------------------------------------------------- bfloat16, few rows (decode)
+// With M <= 64 the product is bound by streaming W once from HBM.  A block
+// owns 16 rows of W (16 output columns); its WAVES waves split K between them
+// in chunks of 128 and add their partial sums through LDS in wave order.  Per
+// chunk a lane loads 64 contiguous bytes of one row of W and the matching
+// pieces of x; v_mfma_f32_16x16x32_bf16 takes W as the row operand and x as the
+// column operand (lane l: row/column l % 16, 8 k-values of k-group l / 16; any
+// assignment of real k to (k-group, slot) is right as long as both operands
+// share it).  The result's register r of lane l is row 4 * (l / 16) + r (an
+// output column n), column l % 16 (an x row m).
+#define SK_CHUNK 128
+
+template <int MT, int WAVES, typename TO>
+__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
+    TO* __restrict__ out, int M, int N, int K, int accumulate) {
+    __shared__ floatx4 red[WAVES][MT][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, r16 = lane & 15;
+    const int n0 = blockIdx.x * 16;
+    const int wr = (n0 + r16 < N) ? n0 + r16 : N - 1;           // rows past the end repeat the last one
+    const bf16_t* wrow = w + (size_t)wr * K + 32 * g;
+    const bf16_t* xrow[MT];
+    bool xok[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = 16 * mt + r16;
+        xok[mt] = m < M;
+        xrow[mt] = x + (size_t)(xok[mt] ? m : 0) * K + 32 * g;
+    }
+    floatx4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+
+    bf16x8 a[4], an[4];
+    auto load_w = [&](int c, bf16x8* dst) {
+        const int kb = c * SK_CHUNK;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            dst[j] = (kb + 32 * g + 8 * j < K) ? *reinterpret_cast<const bf16x8*>(wrow + kb + 8 * j) : zero;
+    };
+    if (wave < nchunks) load_w(wave, a);
+    for (int c = wave; c < nchunks; c += WAVES) {
+        if (c + WAVES < nchunks) load_w(c + WAVES, an);
+        const int kb = c * SK_CHUNK;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            bf16x8 b[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                b[j] = (xok[mt] && kb + 32 * g + 8 * j < K)
+                           ? *reinterpret_cast<const bf16x8*>(xrow[mt] + kb + 8 * j) : zero;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = an[j];
+    }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[wave][mt][lane] = acc[mt];
+    __syncthreads();
+    for (int t = threadIdx.x; t < MT * 64; t += WAVES * 64) {
+        const int mt = t >> 6, l = t & 63;
+        floatx4 s = red[0][mt][l];
+#pragma unroll
+        for (int wv = 1; wv < WAVES; ++wv) {
+            const floatx4 o = red[wv][mt][l];
+            s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
+        }
+        const int m = 16 * mt + (l & 15);
+        if (m >= M) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = n0 + 4 * (l >> 4) + r;
+            if (n < N) epilogue_store(out, (size_t)m * N + n, s[r], bias, n, accumulate);
+        }
+    }
+}
+
+template <typename TO>
+static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
+                          int accumulate, hipStream_t stream) {
+    const int blocks = (N + 15) / 16;
+    const bool many = blocks >= 1024;                 // enough blocks to fill the chip with 4 waves each
+#define LI_SK(MT, WV) gemm_bf16_skinny_kernel<MT, WV, TO><<<blocks, WV * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate)
+    if (M <= 16) { if (many) LI_SK(1, 4); else LI_SK(1, 8); }
+    else if (M <= 32) { if (many) LI_SK(2, 4); else LI_SK(2, 8); }
+    else { if (many) LI_SK(4, 4); else LI_SK(4, 8); }
+#undef LI_SK
+}
+
 extern "C" int li_linear(const void* x, const void* w, const float* bias, void* out, int M, int N,
                          int K, int in_dtype, int out_dtype, int accumulate, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return LI_ERR_SIZE;
@@ -189,6 +283,12 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         dim3 grid((N + BF_BN - 1) / BF_BN, (M + BF_BM - 1) / BF_BM);
         if (grid.y > 65535) return LI_ERR_SIZE;
         const bool aligned = (K % 8) == 0;
+        if (aligned && M <= 64) {
+            if (out_dtype == LI_F32) launch_skinny<float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream);
+            else if (out_dtype == LI_BF16) launch_skinny<bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream);
+            else return LI_ERR_DTYPE;
+            return li_launch_status();
+        }
 #define LI_GEMM(TO, AL) gemm_bf16_kernel<TO, AL><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, accumulate)
         if (out_dtype == LI_F32) { if (aligned) LI_GEMM(float, true); else LI_GEMM(float, false); }
         else if (out_dtype == LI_BF16) { if (aligned) LI_GEMM(bf16_t, true); else LI_GEMM(bf16_t, false); }

@@ -11,7 +11,7 @@ but uploads the tables again for every layer (:993-1007).
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, Hashable, List, Sequence
+from typing import Any, Callable, Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -41,6 +41,13 @@ class AttentionMeta:
     host_q_start: np.ndarray
     host_q_len: np.ndarray
     host_ctx_len: np.ndarray
+    # tokens of segments that bring ONE token (decoding) and the other tokens, as lists of token
+    # numbers; None when all tokens of the batch are of that kind (then no list is needed)
+    single_tokens: Optional[torch.Tensor] = None
+    num_single: int = 0
+    multi_tokens: Optional[torch.Tensor] = None
+    num_multi: int = 0
+    max_single_ctx: int = 0
     extra: Dict[Any, Any] = field(default_factory=dict)    # what kernels derive and keep for the step
 
 
@@ -138,7 +145,10 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     slots = np.array([cache.slot(e.rid) for e in entries], dtype=np.int32)
     want = [int(q_start[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
     want_rows = np.asarray(want, dtype=np.int32)
-    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows]
+    single_mask = q_len[seg_of_token] == 1
+    single = np.nonzero(single_mask)[0].astype(np.int32)
+    multi = np.nonzero(~single_mask)[0].astype(np.int32)
+    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows, single, multi]
     tables, max_blocks = [], []
     for gi in range(len(cache.groups)):
         tabs = [cache.block_table(e.rid, gi) for e in entries]
@@ -155,16 +165,20 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
         parts += [tab, slot_map]
     dev = uploader.upload(parts)
     ctx = StepContext(ws, T, nseg)
-    (ctx.ids, ctx.positions, d_seg, d_qs, d_ql, d_cl, ctx.state_slots, ctx.want_rows) = dev[:8]
+    (ctx.ids, ctx.positions, d_seg, d_qs, d_ql, d_cl, ctx.state_slots, ctx.want_rows,
+     d_single, d_multi) = dev[:10]
     ctx.num_want = len(want)
     ctx.host_state_slots = slots
     ctx.host_q_start, ctx.host_q_len, ctx.host_ctx_len = q_start[:-1], q_len, ctx_len
     for gi in range(len(cache.groups)):
-        d_tab, d_slot = dev[8 + 2 * gi], dev[9 + 2 * gi]
+        d_tab, d_slot = dev[10 + 2 * gi], dev[11 + 2 * gi]
         ctx._slot_maps.append(d_slot)
         ctx._attn.append(AttentionMeta(
             block_table=d_tab, max_blocks=max_blocks[gi], seg_of_token=d_seg, q_start=d_qs,
             q_len=d_ql, ctx_len=d_cl, num_segments=nseg, num_tokens=T,
             max_q_len=int(q_len.max()), max_ctx_len=int(ctx_len.max()),
-            host_q_start=q_start[:-1], host_q_len=q_len, host_ctx_len=ctx_len))
+            host_q_start=q_start[:-1], host_q_len=q_len, host_ctx_len=ctx_len,
+            single_tokens=d_single if len(multi) else None, num_single=len(single),
+            multi_tokens=d_multi if len(single) else None, num_multi=len(multi),
+            max_single_ctx=int(ctx_len[q_len == 1].max()) if len(single) else 0))
     return ctx

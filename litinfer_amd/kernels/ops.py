@@ -38,7 +38,8 @@ _SIGNATURES = {
         "li_linear": [P, P, P, P, I, I, I, I, I, I],
     },
     "attention": {
-        "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
+        "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
+        "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I],
     },
     "sampling": {
         "li_argmax_rows": [P, P, I, I],
@@ -262,12 +263,22 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
 
 
 # ----------------------------------------------------------------- attention
+def _decode_kernel_takes(dtype: torch.dtype, dh: int) -> bool:
+    """The single-query kernel spreads a key's row over dh / (16 bytes) lanes, a power of two."""
+    per = 8 if dtype is torch.bfloat16 else 4
+    return dh % per == 0 and (dh // per) & (dh // per - 1) == 0 and dh // per <= 64
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: torch.Tensor, meta,
-                    nh: int, nkv: int, dh: int, page_size: int, window: int, scale: float) -> None:
+                    nh: int, nkv: int, dh: int, page_size: int, window: int, scale: float,
+                    ws=None) -> None:
     """Causal grouped-query attention of the batch's queries (heads 0..nh-1 of
     qkv's rows) over the paged keys and values; out [T, nh*dh].  Query i of a
     segment stands at position ctx_len - q_len + i and sees the keys at
-    positions <= its own and, with window > 0, closer than `window`."""
+    positions <= its own and, with window > 0, closer than `window`.  Tokens of
+    segments that bring one token go to the split-key decode kernel, the others
+    to the kernel for portions.  `ws` lends the buffers for the splits' partial
+    results."""
     _gpu(qkv, out, k, v, meta.block_table)
     check_attention_sizes(nh, nkv, dh)
     _check_qkv(qkv, nh, dh)
@@ -279,12 +290,38 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
     _chk(bt.dtype is torch.int32 and bt.shape == (meta.num_segments, meta.max_blocks)
          and bt.is_contiguous(), "attention: block table")
     _chk(meta.max_blocks * page_size >= meta.max_ctx_len, "attention: block table too short")
-    if t:
+    _chk(meta.num_single + meta.num_multi == t, "attention: token lists do not cover the batch")
+    if not t:
+        return
+    n_single, n_multi = meta.num_single, meta.num_multi
+    if n_single and not _decode_kernel_takes(qkv.dtype, dh):
+        n_single, n_multi = 0, t                      # every token through the general kernel
+    if n_single:
+        keys = min(meta.max_single_ctx, window) if window > 0 else meta.max_single_ctx
+        nsplit = max(1, min(-(-512 // (n_single * nkv)), -(-keys // 256), 64))
+        acc = ml = None
+        if nsplit > 1:
+            shape_a, shape_m = (n_single, nh, nsplit, dh), (n_single, nh, nsplit, 2)
+            if ws is not None:
+                acc = ws.buffer("attn.part_acc", shape_a, torch.float32)
+                ml = ws.buffer("attn.part_ml", shape_m, torch.float32)
+            else:
+                acc = torch.empty(shape_a, dtype=torch.float32, device=qkv.device)
+                ml = torch.empty(shape_m, dtype=torch.float32, device=qkv.device)
+        lst = meta.single_tokens if n_single < t else None
+        _run("attention", "li_paged_attention_decode", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
+             k.data_ptr(), v.data_ptr(), _DT[qkv.dtype], bt.data_ptr(), meta.max_blocks,
+             0 if lst is None else lst.data_ptr(), n_single, meta.seg_of_token.data_ptr(),
+             meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
+             0 if acc is None else acc.data_ptr(), 0 if ml is None else ml.data_ptr(),
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit)
+    if n_multi:
+        lst = meta.multi_tokens if n_multi < t else None
         _run("attention", "li_paged_attention", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), _DT[qkv.dtype], bt.data_ptr(), meta.max_blocks,
-             meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(),
-             meta.ctx_len.data_ptr(), meta.num_segments, t, meta.max_q_len, meta.max_ctx_len,
-             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale))
+             0 if lst is None else lst.data_ptr(), meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(),
+             meta.q_len.data_ptr(), meta.ctx_len.data_ptr(), meta.num_segments, n_multi, meta.max_q_len,
+             meta.max_ctx_len, nh, nkv, dh, page_size, k.shape[0], int(window), float(scale))
 
 
 # ------------------------------------------------------------------ sampling

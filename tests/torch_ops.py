@@ -87,7 +87,7 @@ def check_attention_sizes(num_heads, num_kv_heads, head_dim):
     assert num_heads % num_kv_heads == 0 and head_dim % 2 == 0
 
 
-def paged_attention(qkv, out, k, v, meta, nh, nkv, dh, page_size, window, scale):
+def paged_attention(qkv, out, k, v, meta, nh, nkv, dh, page_size, window, scale, ws=None):
     g = nh // nkv
     for s in range(meta.num_segments):
         q0, ql, cl = int(meta.host_q_start[s]), int(meta.host_q_len[s]), int(meta.host_ctx_len[s])
