@@ -110,6 +110,27 @@ __device__ __forceinline__ void unpack16(const u32x4& r, float* f) {
     }
 }
 
+// Sum over the LPK lanes that share a key; every one of them gets the total.
+// Steps within a row of 16 lanes are DPP moves inside the vector ALU (swap
+// neighbours, swap pairs, mirror the half row, mirror the row), which keep
+// their place in the instruction stream; only steps across rows go through
+// the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+
+template <int LPK>
+__device__ __forceinline__ float group_sum(float v) {
+    if constexpr (LPK >= 2) v = dpp_add<0xB1>(v);      // quad_perm [1,0,3,2]
+    if constexpr (LPK >= 4) v = dpp_add<0x4E>(v);      // quad_perm [2,3,0,1]
+    if constexpr (LPK >= 8) v = dpp_add<0x141>(v);     // row_half_mirror
+    if constexpr (LPK >= 16) v = dpp_add<0x140>(v);    // row_mirror
+    if constexpr (LPK >= 32) v += __shfl_xor(v, 16, LI_WAVE);
+    if constexpr (LPK >= 64) v += __shfl_xor(v, 32, LI_WAVE);
+    return v;
+}
+
 __device__ __forceinline__ void softmax_merge(float& m, float& l, float* acc, int n, float mo, float lo,
                                               const float* acco) {
     const float mx = fmaxf(m, mo);
@@ -194,8 +215,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
                     float dot = 0.f;
 #pragma unroll
                     for (int j = 0; j < E; ++j) dot = fmaf(qr[h][j], kf[j], dot);
-#pragma unroll
-                    for (int o = 1; o < LPK; o <<= 1) dot += __shfl_xor(dot, o, LI_WAVE);
+                    dot = group_sum<LPK>(dot);
                     sc[u][h] = ok[u] ? dot * scale : -INFINITY;
                 }
             }
@@ -293,6 +313,192 @@ __global__ void attention_merge_kernel(const float* __restrict__ part_acc, const
     }
 }
 
+// ---------------------------------------- single-query tokens, bfloat16, MFMA
+// One WAVE per (token, kv head, split of the keys); up to 16 query heads of the
+// kv head form the rows of the MFMA tiles, so the keys and values are read
+// once for the whole group and nothing is reduced across lanes per key.
+// Per block of 32 keys:
+//   S[16 heads, 32 keys] = Q K^T by v_mfma_f32_16x16x32_bf16 (row operand Q,
+//   column operand K; lane l holds row/column l % 16 and the 8 head dimensions
+//   (DH/4) * (l / 16) + 8 j .. + 7 in step j: both operands share that order);
+//   the result's register r of lane l is head 4 * (l / 16) + r, key l % 16.
+//   Online softmax per head: a row's 16 keys lie in the 16 lanes of one DPP row.
+//   P goes through LDS as bfloat16 to become the row operand of P V.
+//   V[32 keys, DH]: lane (c = l % 16, g = l / 16) loads 8 dimensions 8c .. 8c+7
+//   of the keys 8g .. 8g+7 and transposes them in registers, so MFMA jj yields
+//   the output dimension 8c + jj in column c.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float v) {
+    return fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true)));
+}
+__device__ __forceinline__ float row16_max(float v) {
+    v = dpp_max<0xB1>(v); v = dpp_max<0x4E>(v); v = dpp_max<0x141>(v); v = dpp_max<0x140>(v);
+    return v;
+}
+__device__ __forceinline__ float row16_sum(float v) { return group_sum<16>(v); }
+
+union frag8 { u32x4 raw; bf16x8_t v; };
+
+template <int DH>
+__global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
+    int max_blocks, const int* __restrict__ token_list, const int* __restrict__ seg_of_token,
+    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+    float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv, int page_size,
+    int num_pages, int window, float scale, int nsplit) {
+    constexpr int KS = DH / 32;                 // MFMA steps of Q K^T
+    constexpr int NS = (DH + 127) / 128;        // slabs of 128 output dimensions
+    constexpr int QD = DH / 4;                  // head dimensions owned by one lane group in Q K^T
+    constexpr int PSTRIDE = 40;                 // halves per row of P in LDS (32 keys + pad, 80 bytes)
+    __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * PSTRIDE];
+    const int ti = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+    const int t = token_list ? token_list[ti] : ti;
+    const int G = nh / nkv;
+    const int s = seg_of_token[t];
+    const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
+    const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+    const int nkeys = p - lo + 1;
+    const int per = (((nkeys + nsplit - 1) / nsplit) + 31) & ~31;
+    const int k_begin = lo + split * per;
+    const int k_end = (k_begin + per < p + 1) ? k_begin + per : p + 1;
+    const int* table = block_table + (size_t)s * max_blocks;
+    const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
+    const u32x4 zero4 = {{0u, 0u, 0u, 0u}};
+
+    for (int h0 = 0; h0 < G; h0 += 16) {
+        const int gcount = (G - h0 < 16) ? G - h0 : 16;
+        frag8 qa[KS];
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            qa[j].raw = zero4;
+            if (c < gcount)
+                qa[j].raw = *reinterpret_cast<const u32x4*>(
+                    q + (size_t)t * q_row_stride + (size_t)(kvh * G + h0 + c) * DH + QD * g + 8 * j);
+        }
+        f32x4_t acc[NS][8];
+#pragma unroll
+        for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) acc[ns][jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
+
+        for (int kb = k_begin; kb < k_end; kb += 32) {
+            // ---- S = Q K^T for two tiles of 16 keys
+            f32x4_t sv[2];
+            bool kok[2];
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const int key = kb + 16 * tt + c;
+                kok[tt] = key < k_end;
+                frag8 kf[KS];
+#pragma unroll
+                for (int j = 0; j < KS; ++j) kf[j].raw = zero4;
+                if (kok[tt]) {
+                    const int page = table[key / page_size];
+                    kok[tt] = page >= 0 && page < num_pages;
+                    if (kok[tt]) {
+                        const bf16_t* kp = kc + (((size_t)page * nkv + kvh) * page_size + key % page_size) * DH + QD * g;
+#pragma unroll
+                        for (int j = 0; j < KS; ++j) kf[j].raw = *reinterpret_cast<const u32x4*>(kp + 8 * j);
+                    }
+                }
+                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[j].v, sv[tt], 0, 0, 0);
+            }
+            // ---- V rows of this lane: keys kb + 8g + i, dimensions 128 ns + 8c ..
+            u32x4 vraw[NS][8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int key = kb + 8 * g + i;
+                bool ok = key < k_end;
+                size_t off = 0;
+                if (ok) {
+                    const int page = table[key / page_size];
+                    ok = page >= 0 && page < num_pages;
+                    off = (((size_t)(ok ? page : 0) * nkv + kvh) * page_size + key % page_size) * DH;
+                }
+#pragma unroll
+                for (int ns = 0; ns < NS; ++ns) {
+                    const int d = 128 * ns + 8 * c;
+                    vraw[ns][i] = (ok && d < DH) ? *reinterpret_cast<const u32x4*>(vc + off + d) : zero4;
+                }
+            }
+            // ---- online softmax; lanes whose key is past the end hold -inf
+            float alpha[4], pr[2][4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float s0 = kok[0] ? sv[0][r] * scale : -INFINITY;
+                const float s1 = kok[1] ? sv[1][r] * scale : -INFINITY;
+                const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));     // the block has a key: mx is finite
+                alpha[r] = expf(m[r] - mx);
+                pr[0][r] = expf(s0 - mx);
+                pr[1][r] = expf(s1 - mx);
+                l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];
+                m[r] = mx;
+            }
+            __syncthreads();                                    // readers of the last block's P are done
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = float_to_bf16(pr[tt][r]);
+            __syncthreads();
+            frag8 pa;
+            pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);
+            // ---- O = alpha O + P V
+#pragma unroll
+            for (int ns = 0; ns < NS; ++ns) {
+#pragma unroll
+                for (int jj = 0; jj < 8; ++jj) {
+                    frag8 vf;
+#pragma unroll
+                    for (int ii = 0; ii < 4; ++ii)
+                        vf.raw.w[ii] = __builtin_amdgcn_perm(vraw[ns][2 * ii + 1].w[jj >> 1], vraw[ns][2 * ii].w[jj >> 1],
+                                                             (jj & 1) ? 0x07060302u : 0x05040100u);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[ns][jj][r] *= alpha[r];
+                    acc[ns][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vf.v, acc[ns][jj], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) l[r] = row16_sum(l[r]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int hr = 4 * g + r;
+            if (hr >= gcount) continue;
+            const int head = kvh * G + h0 + hr;
+            if (nsplit == 1) {
+                const float inv = l[r] != 0.f ? 1.0f / l[r] : 0.f;
+                bf16_t* orow = out + (size_t)t * nh * DH + (size_t)head * DH;
+#pragma unroll
+                for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+                    for (int jj = 0; jj < 8; ++jj) {
+                        const int d = 128 * ns + 8 * c + jj;
+                        if (d < DH) orow[d].bits = float_to_bf16(acc[ns][jj][r] * inv);
+                    }
+            } else {
+                const size_t pi = ((size_t)ti * nh + head) * nsplit + split;
+#pragma unroll
+                for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+                    for (int jj = 0; jj < 8; ++jj) {
+                        const int d = 128 * ns + 8 * c + jj;
+                        if (d < DH) part_acc[pi * DH + d] = acc[ns][jj][r];
+                    }
+                if (c == 0) { part_ml[pi * 2] = m[r]; part_ml[pi * 2 + 1] = l[r]; }
+            }
+        }
+    }
+}
+
 template <typename T>
 static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, const T* vc,
                          const int* block_table, int max_blocks, const int* token_list, int n_tokens,
@@ -333,7 +539,7 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
                                          const int* q_start, const int* q_len, const int* ctx_len,
                                          float* part_acc, float* part_ml, int nh, int nkv, int dh,
                                          int page_size, int num_pages, int window, float scale, int nsplit,
-                                         hipStream_t stream) {
+                                         int use_mfma, hipStream_t stream) {
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dh <= 0 || dh > ATT_MAX_DH || page_size <= 0 ||
         max_blocks <= 0)
         return LI_ERR_SIZE;
@@ -342,6 +548,21 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
                                     block_table, max_blocks, token_list, n_tokens, seg_of_token, q_start, q_len,
                                     ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages, window, scale,
                                     nsplit, stream);
+    if (dtype == LI_BF16 && use_mfma) {
+        if (nkv > 65535 || nsplit > 65535 || nsplit < 1) return LI_ERR_SIZE;
+        dim3 grid(n_tokens, nkv, nsplit);
+#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV><<<grid, 64, 0, stream>>>( \
+        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
+        token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
+        scale, nsplit)
+        if (dh == 128) LI_DM(128); else if (dh == 64) LI_DM(64); else return LI_ERR_SIZE;
+#undef LI_DM
+        if (nsplit > 1) {
+            dim3 g2(n_tokens, nh);
+            attention_merge_kernel<bf16_t><<<g2, 64, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit);
+        }
+        return li_launch_status();
+    }
     if (dtype == LI_BF16)
         return launch_decode<bf16_t>((const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc,
                                      (const bf16_t*)vc, block_table, max_blocks, token_list, n_tokens,

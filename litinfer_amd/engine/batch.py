@@ -77,6 +77,9 @@ class StepContext:
     def attention_meta(self, group: int) -> AttentionMeta:
         return self._attn[group]
 
+    def forget_shared(self) -> None:
+        self._shared.clear()
+
     def shared(self, key, make: Callable[[], Any]):
         """Per-step value shared by every part that asks with the same key."""
         if key not in self._shared:
@@ -95,6 +98,7 @@ class BatchUploader:
         self._events = [None, None]
         self._dev = None
         self._turn = 0
+        self.generation = 0          # goes up when the device buffer moves
 
     def upload(self, parts: List[np.ndarray]) -> List[torch.Tensor]:
         offs, total = [], 0
@@ -111,7 +115,8 @@ class BatchUploader:
         elif self._events[i] is not None:
             self._events[i].synchronize()
         if self._dev is None or self._dev.numel() < total:
-            self._dev = torch.empty(total * 2, dtype=torch.int32, device=self.device)
+            self._dev = torch.empty(max(total * 2, 1 << 16), dtype=torch.int32, device=self.device)
+            self.generation += 1
         h = self._host[i].numpy()
         for p, o in zip(parts, offs):
             h[o:o + p.size] = p.reshape(-1)
@@ -127,10 +132,13 @@ class BatchUploader:
         return [self._dev[o:o + p.size].view(p.shape) for p, o in zip(parts, offs)]
 
 
-def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploader") -> StepContext:
+def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploader",
+                  pad_blocks: Optional[Sequence[int]] = None) -> StepContext:
     """Lay out the step's integers (see the module text) for the given entries
     against the cache's current tables, upload them, and return the context.
-    Pages for the entries' tokens must have been reserved."""
+    Pages for the entries' tokens must have been reserved.  `pad_blocks` gives,
+    per page group, a width to pad the block tables to (for steps that are
+    replayed from a recorded graph, whose array shapes must not change)."""
     P = cache.page_size
     nseg = len(entries)
     q_len = np.array([len(e.tokens) for e in entries], dtype=np.int32)
@@ -153,6 +161,8 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     for gi in range(len(cache.groups)):
         tabs = [cache.block_table(e.rid, gi) for e in entries]
         mb = max(1, max(len(t) for t in tabs))
+        if pad_blocks is not None:
+            mb = max(mb, int(pad_blocks[gi]))
         tab = np.full((nseg, mb), -1, dtype=np.int32)
         for i, t in enumerate(tabs):
             tab[i, :len(t)] = t
@@ -180,5 +190,7 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
             host_q_start=q_start[:-1], host_q_len=q_len, host_ctx_len=ctx_len,
             single_tokens=d_single if len(multi) else None, num_single=len(single),
             multi_tokens=d_multi if len(single) else None, num_multi=len(multi),
-            max_single_ctx=int(ctx_len[q_len == 1].max()) if len(single) else 0))
+            # with padded tables the split count must not follow the context either
+            max_single_ctx=(max_blocks[gi] * P if pad_blocks is not None else
+                            int(ctx_len[q_len == 1].max()) if len(single) else 0)))
     return ctx

@@ -50,7 +50,7 @@ class Engine:
     def __init__(self, spec: ModelSpec, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  max_seqs: int = 64, page_order_seed: Optional[int] = None,
-                 config: Any = None):
+                 config: Any = None, use_graphs: bool = True):
         self.spec = spec
         self.config = config
         self.rt = Runtime(torch.device(device), parse_dtype(dtype))
@@ -67,6 +67,12 @@ class Engine:
         self.ws = Workspace(self.rt.device)
         self._uploader = BatchUploader(self.rt.device)
         self.steps_run = 0
+        # decode steps (every request brings one token) are recorded as HIP graphs, one per batch
+        # shape, and replayed: a step is some hundred small launches otherwise
+        self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda"
+        self._graphs: Dict[Any, Any] = {}
+        self._graph_generation = (-1, -1)
+        self.graph_replays = 0
 
     # ---- construction -----------------------------------------------------
     @classmethod
@@ -148,6 +154,8 @@ class Engine:
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of
         the entries and of their `want` lists, or None when nothing is wanted.
+        The tensor may be the output buffer of a recorded step: it is valid until
+        the next step (copy it to keep it).
         Raises StepError for a bad batch and CacheFull when pages or slots do
         not suffice; in both cases the cache is as before."""
         self._validate(entries)
@@ -173,8 +181,11 @@ class Engine:
             for rid in admitted:
                 cache.release(rid)
             raise
-        ctx = self._build_context(entries)
-        logits = self.model.forward(ctx, cache)
+        key = self._graph_key(entries)
+        if key is None:
+            logits = self.model.forward(self._build_context(entries), cache)
+        else:
+            logits = self._forward_graphed(key, self._build_context(entries, pad_blocks=key[2]))
         for e in entries:
             cache.commit(e.rid, len(e.tokens))
         self.steps_run += 1
@@ -185,5 +196,50 @@ class Engine:
         if self.cache.has(rid):
             self.cache.release(rid)
 
-    def _build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        return build_context(self.cache, entries, self.ws, self._uploader)
+    def _build_context(self, entries: Sequence[StepEntry], pad_blocks=None) -> StepContext:
+        return build_context(self.cache, entries, self.ws, self._uploader, pad_blocks)
+
+    # ---- recorded decode steps ----------------------------------------------
+    def _graph_key(self, entries: Sequence[StepEntry]):
+        """(segments, wanted rows, table width per group) of a batch that may be
+        replayed from a graph, else None.  Table widths are rounded up to powers
+        of two so that a graph serves a range of context lengths."""
+        if not self.use_graphs or not self.model.graph_safe:
+            return None
+        if any(len(e.tokens) != 1 for e in entries):
+            return None
+        widths = []
+        for gi in range(len(self.cache.groups)):
+            need = max(len(self.cache.block_table(e.rid, gi)) for e in entries)
+            widths.append(max(16, 1 << (need - 1).bit_length()))
+        return (len(entries), sum(len(e.want) for e in entries), tuple(widths))
+
+    def _forward_graphed(self, key, ctx: StepContext):
+        gen = (self.ws.generation, self._uploader.generation)
+        state = self._graphs.get(key)
+        if state is None or state[0] != "graph" or self._graph_generation != gen:
+            if self._graph_generation != gen:
+                self._graphs.clear()              # a buffer moved: recorded addresses are stale
+                state = None
+            # the first step of a shape runs eagerly (it sizes the buffers), the second is recorded
+            logits = self.model.forward(ctx, self.cache)
+            gen = (self.ws.generation, self._uploader.generation)
+            self._graph_generation = gen
+            if state is None:
+                self._graphs[key] = ("seen",)
+                return logits
+            torch.cuda.synchronize(self.rt.device)
+            ctx.forget_shared()                   # what the eager pass prepared must be prepared in the graph too
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                out = self.model.forward(ctx, self.cache)
+            if (self.ws.generation, self._uploader.generation) != gen:
+                self._graphs.clear()              # recording itself moved a buffer: do not keep it
+                self._graph_generation = (self.ws.generation, self._uploader.generation)
+                return logits
+            self._graphs[key] = ("graph", graph, out)
+            return logits
+        _, graph, out = state
+        graph.replay()
+        self.graph_replays += 1
+        return out

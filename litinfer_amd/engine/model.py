@@ -57,6 +57,10 @@ class Model:
                     stack.append(v)
         return total
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in (self.embedding, *self.layers, self.final_norm, self.head))
+
     # ---- cache ------------------------------------------------------------
     def cache_needs(self) -> Tuple[List[object], List[Optional[int]]]:
         needs = [self.layers[e.layer].cache_need() for e in self.order]

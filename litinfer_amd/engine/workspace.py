@@ -12,6 +12,7 @@ class Workspace:
     def __init__(self, device):
         self.device = torch.device(device)
         self._bufs: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self.generation = 0          # goes up whenever a buffer moves: recorded graphs are stale then
 
     def buffer(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         """A tensor of this shape; its contents are whatever the last user of
@@ -23,4 +24,5 @@ class Workspace:
             cap = n if buf is None else max(n, buf.numel() * 3 // 2)
             buf = torch.empty(cap, dtype=dtype, device=self.device)
             self._bufs[key] = buf
+            self.generation += 1
         return buf[:math.prod(int(s) for s in shape)].view(*shape)

@@ -39,7 +39,7 @@ _SIGNATURES = {
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
-        "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I],
+        "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I],
     },
     "sampling": {
         "li_argmax_rows": [P, P, I, I],
@@ -298,7 +298,13 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         n_single, n_multi = 0, t                      # every token through the general kernel
     if n_single:
         keys = min(meta.max_single_ctx, window) if window > 0 else meta.max_single_ctx
-        nsplit = max(1, min(-(-512 // (n_single * nkv)), -(-keys // 256), 64))
+        # bfloat16 with a head size of 64 or 128: one wave per split on the matrix cores; else one
+        # block of four waves per split on the vector ALU
+        mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
+        if mfma:
+            nsplit = max(1, min(-(-2048 // (n_single * nkv)), -(-keys // 128), 64))
+        else:
+            nsplit = max(1, min(-(-512 // (n_single * nkv)), -(-keys // 256), 64))
         acc = ml = None
         if nsplit > 1:
             shape_a, shape_m = (n_single, nh, nsplit, dh), (n_single, nh, nsplit, 2)
@@ -314,7 +320,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
              0 if lst is None else lst.data_ptr(), n_single, meta.seg_of_token.data_ptr(),
              meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              0 if acc is None else acc.data_ptr(), 0 if ml is None else ml.data_ptr(),
-             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit)
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit, int(mfma))
     if n_multi:
         lst = meta.multi_tokens if n_multi < t else None
         _run("attention", "li_paged_attention", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),

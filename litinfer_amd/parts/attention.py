@@ -22,6 +22,7 @@ from .linear import Linear
 
 
 class GQAttention(Mixer):
+
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         a = spec.args
@@ -41,6 +42,10 @@ class GQAttention(Mixer):
         self.n_kv = self.nkv * self.dh
         self.qkv = None
         self.out = None
+
+    @property
+    def graph_safe(self):
+        return self.position is None or self.position.graph_safe
 
     def cache_need(self):
         return PagedKVNeed(self.nkv, self.dh, self.window)

@@ -70,6 +70,10 @@ class StateNeed:
 
 class Part:
     category = "part"
+    # True if `forward` only launches work whose arguments are device arrays and sizes of the batch
+    # (tokens, segments, table width): then a decode step may be recorded once as a HIP graph and
+    # replayed.  A part that reads the step's host-side arrays must leave this False.
+    graph_safe = False
 
     def __init__(self, spec: PartSpec, rt: Runtime):
         self.spec = spec

@@ -15,6 +15,10 @@ class PreNormBlock(Block):
         self.ffn = build_part("feed_forward", parts["feed_forward"], rt)
         self._all = (self.norm1, self.mixer, self.norm2, self.ffn)
 
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self._all)
+
     def cache_need(self):
         return self.mixer.cache_need()
 

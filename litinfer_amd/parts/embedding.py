@@ -16,6 +16,8 @@ from .linear import Linear
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     category = "embedding"
 
     def __init__(self, spec, rt):
@@ -36,6 +38,8 @@ class TokenEmbedding(Part):
 
 
 class LinearHead(Part):
+    graph_safe = True
+
     category = "head"
 
     def __init__(self, spec, rt):

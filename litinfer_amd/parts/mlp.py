@@ -13,6 +13,8 @@ from .linear import Linear
 
 
 class SwiGLUMLP(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         self.hidden = int(spec.args["hidden_size"])

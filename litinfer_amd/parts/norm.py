@@ -9,6 +9,8 @@ from .base import Norm, register_part
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
         self.size = int(spec.args["size"])

@@ -37,6 +37,8 @@ class Position(Part):
 
 
 class RopeNeox(Position):
+    graph_safe = True
+
     """Half-split rotary encoding (src/ops/rope/op.cpp:13-20, :32-39):
     angle_j = pos / theta^(2j/rotary_dim) in float32; for j < rotary_dim/2 the
     pair (x[j], x[j + rotary_dim/2]) is rotated by angle_j.  The reference

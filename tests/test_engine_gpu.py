@@ -67,3 +67,38 @@ def test_float32_schedules_agree_with_each_other_closely(models, name):
     for kind in ("tail", "chunks", "mixed"):
         for r in reqs:
             assert schedules.rel_err(outs[kind][r], outs["whole"][r].astype(np.float64)) < 5e-6
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_recorded_decode_steps_equal_eager_ones_on_every_replay(models, dt):
+    """Decode steps are recorded as HIP graphs and replayed.  Every replay is
+    compared with an engine that records nothing, with eager steps (portions of
+    another request, a change of the batch's shape) and synchronizations between
+    the replays, and across a change of the block table's width."""
+    from litinfer_amd.engine import StepEntry
+    cfg, page, _ = CASES["B"]
+    d, reqs, ref = models[("B", dt)]
+    a, b, c = reqs["r4"], reqs["r3"], reqs["r5"]           # 100, 70 and 41 tokens
+    engines = [_engine(d, dt, page, 512, use_graphs=g) for g in (True, False)]
+    outs = [[], []]
+    for eng, out in zip(engines, outs):
+        eng.step([StepEntry("a", a[:3], []), StepEntry("b", b[:5], [])])
+        for i in range(60):
+            batch = [StepEntry("a", [a[3 + i]], [0]), StepEntry("b", [b[5 + i]], [0])]
+            out.append(eng.step(batch).clone())
+            torch.cuda.synchronize()
+            if i % 7 == 3 and (i // 7) * 5 + 5 <= len(c):   # eager work between replays
+                lo = (i // 7) * 5
+                out.append(eng.step([StepEntry("c", c[lo:lo + 5], [4])]).clone())
+                last_c = (len(out) - 1, lo + 4)
+            if i == 40:                                    # another shape of batch, once
+                out.append(eng.step([StepEntry("a", [a[44]], [0])]).clone())
+                out.append(eng.step([StepEntry("b", [b[46]], [0])]).clone())
+        out.append(eng.step([StepEntry("a", a[64:70], [5]), StepEntry("b", [b[65]], [0])]).clone())
+    assert engines[0].graph_replays >= 50 and engines[1].graph_replays == 0
+    assert len(engines[0]._graphs) >= 2                    # the table grew past a width: a second graph
+    for x, y in zip(*outs):
+        assert torch.equal(x, y)
+    # and they are right, not only equal: request c was fed in order between the replays
+    at, pos = last_c
+    assert schedules.rel_err(outs[0][at].cpu().numpy()[0], ref["r5"][pos]) < TOL[dt]

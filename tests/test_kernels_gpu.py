@@ -206,6 +206,8 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
     ([(900, 1), (64, 1), (2000, 1)], 12, 1, 64, 16, 300),           # 12 heads in one group, window
     ([(1000, 1), (50, 3), (513, 1)], 4, 2, 16, 8, 0),               # decoding beside a portion
     ([(300, 1), (77, 1)], 6, 3, 80, 16, 0),                         # a head size the split kernel does not take
+    ([(300, 1), (1025, 1), (31, 1)], 40, 2, 64, 16, 0),             # 20 heads in a group: two blocks of MFMA rows
+    ([(33, 1), (32, 1), (1, 1)], 7, 7, 128, 8, 0),                  # one head per group, keys around a block's edge
 ])
 def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     out, ref = _paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=6)
