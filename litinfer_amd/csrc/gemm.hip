@@ -177,97 +177,177 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 }
 
 // ------------------------------------------------- bfloat16, few rows (decode)
-// With M <= 64 the product is bound by streaming W once from HBM.  A block
-// owns 16 rows of W (16 output columns); its WAVES waves split K between them
-// in chunks of 128 and add their partial sums through LDS in wave order.  Per
-// chunk a lane loads 64 contiguous bytes of one row of W and the matching
-// pieces of x; v_mfma_f32_16x16x32_bf16 takes W as the row operand and x as the
-// column operand (lane l: row/column l % 16, 8 k-values of k-group l / 16; any
+// With M <= 64 the product is bound by streaming W once from HBM, and the
+// bandwidth reached is (bytes in flight) / (memory latency): the kernel is
+// built to keep many independent 16-byte loads outstanding.  A block owns NT
+// tiles of 16 rows of W (16 output columns each); its WAVES waves split K
+// between them in chunks of 128 and add their partial sums through LDS in wave
+// order.  The loads of a wave's next chunk are in flight while one chunk is
+// multiplied.  Per chunk a lane loads four 16-byte pieces of one row of W per
+// tile (the four lanes of a row together 64 contiguous bytes an instruction)
+// and the matching pieces of x;
+// v_mfma_f32_16x16x32_bf16 takes W as the row operand and x as the column
+// operand (lane l: row/column l % 16, 8 k-values of k-group l / 16; any
 // assignment of real k to (k-group, slot) is right as long as both operands
 // share it).  The result's register r of lane l is row 4 * (l / 16) + r (an
 // output column n), column l % 16 (an x row m).
+//
+// SWIGLU: W is [gate; up] with N rows each: tile 0 takes gate rows, tile 1 the
+// up rows of the same columns, and out[m, n] = up * gate / (1 + exp(-gate)).
 #define SK_CHUNK 128
 
-template <int MT, int WAVES, typename TO>
-__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-    TO* __restrict__ out, int M, int N, int K, int accumulate) {
-    __shared__ floatx4 red[WAVES][MT][64];
+struct SkinnyArgs {
+    const bf16_t* x;        // [M, K]
+    const bf16_t* w;        // [N, K], or [2 N, K] with SWIGLU
+    const float* bias;      // [N] or null
+    void* out;              // [M, N]
+    int M, N, K, accumulate;
+};
+
+template <int MT, int NT, int WAVES, bool SWIGLU, typename TO>
+__global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs a) {
+    __shared__ floatx4 red[WAVES][MT * NT][64];
+    const int M = a.M, N = a.N, K = a.K;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
-    const int n0 = blockIdx.x * 16;
-    const int wr = (n0 + r16 < N) ? n0 + r16 : N - 1;           // rows past the end repeat the last one
-    const bf16_t* wrow = w + (size_t)wr * K + 32 * g;
+    const int n0 = blockIdx.x * 16 * (SWIGLU ? 1 : NT);
+    const bf16_t* wrow[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        int row;
+        if (SWIGLU) row = ((n0 + r16 < N) ? n0 + r16 : N - 1) + nt * N;      // gate row, up row
+        else row = (n0 + 16 * nt + r16 < N) ? n0 + 16 * nt + r16 : N - 1;    // rows past the end repeat the last
+        wrow[nt] = a.w + (size_t)row * K + 8 * g;
+    }
     const bf16_t* xrow[MT];
     bool xok[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = 16 * mt + r16;
         xok[mt] = m < M;
-        xrow[mt] = x + (size_t)(xok[mt] ? m : 0) * K + 32 * g;
+        xrow[mt] = a.x + (size_t)(xok[mt] ? m : 0) * K + 8 * g;
     }
-    floatx4 acc[MT];
+    floatx4 acc[MT][NT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
 
-    bf16x8 a[4], an[4];
-    auto load_w = [&](int c, bf16x8* dst) {
+    // The memory counter of a wave retires loads in the order they were issued, so waiting for
+    // a chunk's x pieces also waits for every load issued before them.  All loads of a chunk (W
+    // and x) are therefore issued together, one chunk ahead of their use: when chunk c is
+    // multiplied, exactly the loads of chunk c + WAVES are still in flight.  (With 64 rows the x
+    // pieces do not fit a second buffer; then a chunk is loaded and used in one go and the other
+    // waves of the compute unit cover the latency.)
+    constexpr bool AHEAD = MT <= 2;
+    constexpr int NBUF = AHEAD ? 2 : 1;
+    bf16x8 wbuf[NBUF][NT][4], xbuf[NBUF][MT][4];
+    auto load_chunk = [&](int c, bf16x8 (*wd)[4], bf16x8 (*xd)[4]) {
         const int kb = c * SK_CHUNK;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            dst[j] = (kb + 32 * g + 8 * j < K) ? *reinterpret_cast<const bf16x8*>(wrow + kb + 8 * j) : zero;
-    };
-    if (wave < nchunks) load_w(wave, a);
-    for (int c = wave; c < nchunks; c += WAVES) {
-        if (c + WAVES < nchunks) load_w(c + WAVES, an);
-        const int kb = c * SK_CHUNK;
+        for (int j = 0; j < 4; ++j) {
+            const bool in = kb + 8 * g + 32 * j < K;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            bf16x8 b[4];
+            for (int nt = 0; nt < NT; ++nt)
+                wd[nt][j] = in ? *reinterpret_cast<const bf16x8*>(wrow[nt] + kb + 32 * j) : zero;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                b[j] = (xok[mt] && kb + 32 * g + 8 * j < K)
-                           ? *reinterpret_cast<const bf16x8*>(xrow[mt] + kb + 8 * j) : zero;
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j], b[j], acc[mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt)
+                xd[mt][j] = (in && xok[mt]) ? *reinterpret_cast<const bf16x8*>(xrow[mt] + kb + 32 * j) : zero;
         }
+    };
+    auto multiply = [&](bf16x8 (*wa)[4], bf16x8 (*xa)[4]) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) a[j] = an[j];
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[nt][j], xa[mt][j], acc[mt][nt], 0, 0, 0);
+    };
+    if constexpr (AHEAD) {
+        if (wave < nchunks) load_chunk(wave, wbuf[0], xbuf[0]);
+        for (int c = wave; c < nchunks; c += 2 * WAVES) {          // two chunks a turn: buffer numbers are constants
+            if (c + WAVES < nchunks) load_chunk(c + WAVES, wbuf[1], xbuf[1]);
+            multiply(wbuf[0], xbuf[0]);
+            if (c + WAVES >= nchunks) break;
+            if (c + 2 * WAVES < nchunks) load_chunk(c + 2 * WAVES, wbuf[0], xbuf[0]);
+            multiply(wbuf[1], xbuf[1]);
+        }
+    } else {
+        for (int c = wave; c < nchunks; c += WAVES) {
+            load_chunk(c, wbuf[0], xbuf[0]);
+            multiply(wbuf[0], xbuf[0]);
+        }
     }
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) red[wave][mt][lane] = acc[mt];
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) red[wave][mt * NT + nt][lane] = acc[mt][nt];
     __syncthreads();
+    TO* out = (TO*)a.out;
     for (int t = threadIdx.x; t < MT * 64; t += WAVES * 64) {
         const int mt = t >> 6, l = t & 63;
-        floatx4 s = red[0][mt][l];
-#pragma unroll
-        for (int wv = 1; wv < WAVES; ++wv) {
-            const floatx4 o = red[wv][mt][l];
-            s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
-        }
         const int m = 16 * mt + (l & 15);
         if (m >= M) continue;
+        floatx4 s[NT];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int n = n0 + 4 * (l >> 4) + r;
-            if (n < N) epilogue_store(out, (size_t)m * N + n, s[r], bias, n, accumulate);
+        for (int nt = 0; nt < NT; ++nt) {
+            s[nt] = red[0][mt * NT + nt][l];
+#pragma unroll
+            for (int wv = 1; wv < WAVES; ++wv) {
+                const floatx4 o = red[wv][mt * NT + nt][l];
+                s[nt][0] += o[0]; s[nt][1] += o[1]; s[nt][2] += o[2]; s[nt][3] += o[3];
+            }
+        }
+        if constexpr (SWIGLU) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = n0 + 4 * (l >> 4) + r;
+                if (n < N) {
+                    const float gv = s[0][r], uv = s[NT - 1][r];
+                    store_from_float(out + (size_t)m * N + n, uv * (gv / (1.0f + expf(-gv))));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n0 + 16 * nt + 4 * (l >> 4) + r;
+                    if (n < N) epilogue_store(out, (size_t)m * N + n, s[nt][r], a.bias, n, a.accumulate);
+                }
         }
     }
 }
 
-template <typename TO>
-static void launch_skinny(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
-                          int accumulate, hipStream_t stream) {
-    const int blocks = (N + 15) / 16;
-    const bool many = blocks >= 1024;                 // enough blocks to fill the chip with 4 waves each
-#define LI_SK(MT, WV) gemm_bf16_skinny_kernel<MT, WV, TO><<<blocks, WV * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate)
-    if (M <= 16) { if (many) LI_SK(1, 4); else LI_SK(1, 8); }
-    else if (M <= 32) { if (many) LI_SK(2, 4); else LI_SK(2, 8); }
-    else { if (many) LI_SK(4, 4); else LI_SK(4, 8); }
+template <bool SWIGLU, typename TO>
+static void launch_skinny(const SkinnyArgs& a, hipStream_t stream) {
+    const int M = a.M, N = a.N;
+#define LI_SK(MT, NT, WV) gemm_bf16_skinny_kernel<MT, NT, WV, SWIGLU, TO><<<(N + 16 * (SWIGLU ? 1 : NT) - 1) / (16 * (SWIGLU ? 1 : NT)), WV * 64, 0, stream>>>(a)
+    if constexpr (SWIGLU) {
+        if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
+    } else if (N >= 8192) {                                 // many columns: many blocks, two tiles share each piece of x
+        if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
+    } else {                                                // few columns: few blocks, so more waves split K
+        if (M <= 16) LI_SK(1, 1, 16); else if (M <= 32) LI_SK(2, 1, 16); else LI_SK(4, 2, 8);
+    }
 #undef LI_SK
+}
+
+// Few rows (M <= 64), bfloat16, K a multiple of 8.  swiglu: w has 2 N rows ([gate; up]).
+extern "C" int li_linear_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N,
+                                int K, int out_dtype, int accumulate, int swiglu, hipStream_t stream) {
+    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8)) return LI_ERR_SIZE;
+    if (accumulate && out_dtype != LI_F32) return LI_ERR_DTYPE;
+    if (swiglu && (bias || accumulate || out_dtype != LI_BF16)) return LI_ERR_DTYPE;
+    SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, accumulate};
+    if (swiglu) launch_skinny<true, bf16_t>(a, stream);
+    else if (out_dtype == LI_BF16) launch_skinny<false, bf16_t>(a, stream);
+    else if (out_dtype == LI_F32) launch_skinny<false, float>(a, stream);
+    else return LI_ERR_DTYPE;
+    return li_launch_status();
 }
 
 extern "C" int li_linear(const void* x, const void* w, const float* bias, void* out, int M, int N,
@@ -283,12 +363,8 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         dim3 grid((N + BF_BN - 1) / BF_BN, (M + BF_BM - 1) / BF_BM);
         if (grid.y > 65535) return LI_ERR_SIZE;
         const bool aligned = (K % 8) == 0;
-        if (aligned && M <= 64) {
-            if (out_dtype == LI_F32) launch_skinny<float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream);
-            else if (out_dtype == LI_BF16) launch_skinny<bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream);
-            else return LI_ERR_DTYPE;
-            return li_launch_status();
-        }
+        if (aligned && M <= 64)
+            return li_linear_skinny(x, w, bias, out, M, N, K, out_dtype, accumulate, 0, stream);
 #define LI_GEMM(TO, AL) gemm_bf16_kernel<TO, AL><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, accumulate)
         if (out_dtype == LI_F32) { if (aligned) LI_GEMM(float, true); else LI_GEMM(float, false); }
         else if (out_dtype == LI_BF16) { if (aligned) LI_GEMM(bf16_t, true); else LI_GEMM(bf16_t, false); }

@@ -36,6 +36,7 @@ _SIGNATURES = {
     },
     "gemm": {
         "li_linear": [P, P, P, P, I, I, I, I, I, I],
+        "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
@@ -260,6 +261,35 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     if m:
         _run("gemm", "li_linear", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
              out.data_ptr(), m, n, k, _DT[x.dtype], _DT[out.dtype], int(bool(accumulate)))
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def skinny_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
+    """Whether `linear_skinny` takes a product of m rows over k with such a matrix."""
+    return w_dtype is torch.bfloat16 and k % 8 == 0 and 0 < m <= SKINNY_MAX_ROWS
+
+
+def linear_skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                  accumulate: bool = False, swiglu: bool = False) -> None:
+    """The product for few rows (decoding).  swiglu: w is [gate; up] (2N rows)
+    and out[m, n] = up * gate / (1 + exp(-gate)), the activation fused into the
+    product's epilogue."""
+    _gpu(x, w, bias, out)
+    m, k = x.shape
+    n = out.shape[1]
+    _chk(skinny_takes(m, k, w.dtype), "linear_skinny: sizes or dtype not taken")
+    _chk(w.shape == ((2 * n if swiglu else n), k) and out.shape[0] == m, "linear_skinny: shapes do not fit")
+    _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_skinny: contiguous operands")
+    _chk(x.dtype is torch.bfloat16, "linear_skinny: x must be bfloat16")
+    _chk(out.dtype in _DT and (not accumulate or out.dtype is torch.float32), "linear_skinny: out dtype")
+    _chk(not swiglu or (bias is None and not accumulate and out.dtype is torch.bfloat16),
+         "linear_skinny: swiglu takes no bias and no accumulation and writes bfloat16")
+    _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
+         "linear_skinny: bias must be float32 [N]")
+    _run("gemm", "li_linear_skinny", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
+         out.data_ptr(), m, n, k, _DT[out.dtype], int(bool(accumulate)), int(bool(swiglu)))
 
 
 # ----------------------------------------------------------------- attention

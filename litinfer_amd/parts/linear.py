@@ -17,11 +17,21 @@ class Linear:
         self.bias = None if bias is None else rt.vector(bias)
         self.out_features, self.in_features = self.weight.shape
 
-    def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ws=None):
+    def takes_swiglu(self, x: torch.Tensor) -> bool:
+        """Whether the product of these rows can have the SwiGLU activation as its
+        epilogue (few rows, bfloat16)."""
+        return x.dtype is torch.bfloat16 and ops.skinny_takes(x.shape[0], self.in_features, self.weight.dtype)
+
+    def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ws=None,
+                 swiglu: bool = False):
         """out = x W^T + b, or out += ... when `accumulate` (out is float32 then).
-        A matrix that is stored in 32-bit is multiplied in 32-bit also when the
-        activations are bfloat16: they are widened for it, exactly."""
-        if self.weight.dtype is torch.float32 and x.dtype is not torch.float32:
+        With `swiglu` (only where `takes_swiglu`) W is [gate; up] and out gets
+        up * silu(gate).  A matrix that is stored in 32-bit is multiplied in
+        32-bit also when the activations are bfloat16: they are widened for it,
+        exactly."""
+        if swiglu:
+            ops.linear_skinny(x, self.weight, self.bias, out, accumulate, swiglu=True)
+        elif self.weight.dtype is torch.float32 and x.dtype is not torch.float32:
             x32 = ws.buffer("linear.x32", x.shape, torch.float32)
             ops.cast(x, x32)
             if out.dtype is torch.float32:
@@ -31,5 +41,5 @@ class Linear:
                 ops.linear(x32, self.weight, self.bias, y32, False)
                 ops.cast(y32, out)
         else:
-            ops.linear(x, self.weight, self.bias, out, accumulate)
+            ops.linear(x, self.weight, self.bias, out, accumulate)      # few rows go to the skinny kernel inside
         return out

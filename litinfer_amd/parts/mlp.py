@@ -37,10 +37,13 @@ class SwiGLUMLP(FeedForward):
 
     def forward(self, xn, residual, ctx):
         t = xn.shape[0]
-        gu = ctx.ws.buffer("mlp.gate_up", (t, 2 * self.inter), self.rt.dtype)
-        self.gate_up(xn, gu, ws=ctx.ws)
         h = ctx.ws.buffer("mlp.h", (t, self.inter), self.rt.dtype)
-        ops.swiglu(gu, h)
+        if self.gate_up.takes_swiglu(xn):
+            self.gate_up(xn, h, ws=ctx.ws, swiglu=True)        # few rows: the activation is the epilogue
+        else:
+            gu = ctx.ws.buffer("mlp.gate_up", (t, 2 * self.inter), self.rt.dtype)
+            self.gate_up(xn, gu, ws=ctx.ws)
+            ops.swiglu(gu, h)
         self.down(h, residual, accumulate=True, ws=ctx.ws)
 
 

@@ -89,6 +89,40 @@ def test_linear(ops, dtype, mnk, bias, acc):
     assert rel(out, ref) < (4 * math.sqrt(k) * 2.0 ** -24 if out.dtype is torch.float32 else 5e-3)
 
 
+@pytest.mark.parametrize("m,n,k,swiglu,out_dtype,bias,acc", [
+    (1, 16, 8, False, torch.bfloat16, False, False),
+    (8, 4608, 3584, False, torch.bfloat16, True, False),        # decode: qkv + bias
+    (8, 18944, 3584, True, torch.bfloat16, False, False),       # decode: gate/up + swiglu
+    (8, 3584, 18944, False, torch.float32, False, True),        # decode: down + residual
+    (5, 301, 120, False, torch.float32, False, False),          # odd sizes: head
+    (17, 200, 96, True, torch.bfloat16, False, False),
+    (32, 37, 264, False, torch.bfloat16, True, False),
+    (33, 130, 1160, True, torch.bfloat16, False, False),
+    (64, 50, 128, False, torch.float32, True, True),
+    (3, 9000, 64, False, torch.bfloat16, True, False),          # wide output: two tiles a wave
+    (20, 9000, 520, False, torch.bfloat16, False, False),
+])
+def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, acc):
+    g = torch.Generator().manual_seed(12)
+    x = (torch.randn(m, k, generator=g) * 2).to(torch.bfloat16)
+    w = (torch.randn(2 * n if swiglu else n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    b = torch.randn(n, generator=g) if bias else None
+    y = x.double().numpy() @ w.double().numpy().T
+    if swiglu:
+        y = plain_impl.swiglu(y[:, :n], y[:, n:])
+    if b is not None:
+        y = y + b.double().numpy()
+    if acc:
+        base = torch.randn(m, n, generator=g)
+        out = base.to(DEV)
+        y = y + base.double().numpy()
+    else:
+        out = torch.empty(m, n, dtype=out_dtype, device=DEV)
+    assert ops.skinny_takes(m, k, w.dtype)
+    ops.linear_skinny(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, acc, swiglu=swiglu)
+    assert rel(out, y) < (4 * math.sqrt(k) * 2.0 ** -24 if out_dtype is torch.float32 else 5e-3)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_rows_do_not_depend_on_the_batch(ops, dtype):
     g = torch.Generator().manual_seed(3)

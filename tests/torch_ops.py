@@ -83,6 +83,21 @@ def linear(x, w, bias, out, accumulate=False):
         out.copy_(y.to(out.dtype))
 
 
+def linear_skinny(x, w, bias, out, accumulate=False, swiglu=False):
+    y = x.float() @ w.float().T
+    if swiglu:
+        n = out.shape[1]
+        g, u = y[:, :n], y[:, n:]
+        out.copy_((u * (g / (1 + torch.exp(-g)))).to(out.dtype))
+        return
+    if bias is not None:
+        y = y + bias
+    if accumulate:
+        out += y
+    else:
+        out.copy_(y.to(out.dtype))
+
+
 def check_attention_sizes(num_heads, num_kv_heads, head_dim):
     assert num_heads % num_kv_heads == 0 and head_dim % 2 == 0
 
@@ -114,7 +129,7 @@ def argmax_rows(logits, out):
 
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
-       "rope_apply", "kv_store", "rope_kv_store", "linear", "check_attention_sizes",
+       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "check_attention_sizes",
        "paged_attention", "argmax_rows"]
 
 
