@@ -291,25 +291,38 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     }
 }
 
+// Merging the splits of a (token, head), in split order.  The weights exp(m_s - m) are
+// computed once per split by the first lanes, then every thread adds up one output
+// dimension with all its loads independent of each other.
+#define MERGE_MAX_SPLITS 64
+
 template <typename T>
-__global__ void attention_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                       const int* __restrict__ token_list, T* __restrict__ out, int nh,
-                                       int dh, int nsplit) {
+__global__ __launch_bounds__(128) void attention_merge_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int nsplit) {
+    __shared__ float wgt[MERGE_MAX_SPLITS];
+    __shared__ float inv_l;
     const int ti = blockIdx.x, head = blockIdx.y;
     const int t = token_list ? token_list[ti] : ti;
     const size_t base = ((size_t)ti * nh + head) * nsplit;
-    float mx = -INFINITY;
-    for (int sp = 0; sp < nsplit; ++sp) mx = fmaxf(mx, part_ml[(base + sp) * 2]);
-    for (int d = threadIdx.x; d < dh; d += blockDim.x) {
-        float lt = 0.f, at = 0.f;
-        if (mx != -INFINITY) {
-            for (int sp = 0; sp < nsplit; ++sp) {
-                const float f = expf(part_ml[(base + sp) * 2] - mx);
-                lt += part_ml[(base + sp) * 2 + 1] * f;
-                at += part_acc[(base + sp) * dh + d] * f;
-            }
-        }
-        store_from_float(out + (size_t)t * nh * dh + (size_t)head * dh + d, lt != 0.f ? at / lt : 0.f);
+    if (threadIdx.x < 64) {
+        const int sp = threadIdx.x;
+        const float ms = sp < nsplit ? part_ml[(base + sp) * 2] : -INFINITY;
+        const float ls = sp < nsplit ? part_ml[(base + sp) * 2 + 1] : 0.f;
+        const float mx = wave_max(ms);
+        const float f = (mx == -INFINITY) ? 0.f : expf(ms - mx);
+        if (sp < nsplit) wgt[sp] = f;
+        // the sum over splits in split order (one lane adds them up: at most 64 terms)
+        float lt = 0.f;
+        for (int i = 0; i < nsplit; ++i) lt += __shfl(ls * f, i, LI_WAVE);
+        if (sp == 0) inv_l = lt != 0.f ? 1.0f / lt : 0.f;
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < dh; d += 128) {
+        float at = 0.f;
+#pragma unroll 8
+        for (int sp = 0; sp < nsplit; ++sp) at += part_acc[(base + sp) * dh + d] * wgt[sp];
+        store_from_float(out + (size_t)t * nh * dh + (size_t)head * dh + d, at * inv_l);
     }
 }
 
@@ -342,6 +355,8 @@ __device__ __forceinline__ float row16_sum(float v) { return group_sum<16>(v); }
 
 union frag8 { u32x4 raw; bf16x8_t v; };
 
+#define DEC_TABLE_CAP 1024      // pages of one split that fit the kernel's copy of the block table
+
 template <int DH>
 __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
@@ -355,6 +370,7 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     constexpr int QD = DH / 4;                  // head dimensions owned by one lane group in Q K^T
     constexpr int PSTRIDE = 40;                 // halves per row of P in LDS (32 keys + pad, 80 bytes)
     __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * PSTRIDE];
+    __shared__ int pages[DEC_TABLE_CAP];
     const int ti = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
     const int t = token_list ? token_list[ti] : ti;
     const int G = nh / nkv;
@@ -365,9 +381,23 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     const int per = (((nkeys + nsplit - 1) / nsplit) + 31) & ~31;
     const int k_begin = lo + split * per;
     const int k_end = (k_begin + per < p + 1) ? k_begin + per : p + 1;
-    const int* table = block_table + (size_t)s * max_blocks;
     const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
     const u32x4 zero4 = {{0u, 0u, 0u, 0u}};
+    // The block table of this split goes to LDS first: a page number fetched from global
+    // memory in the loop would make every wait for it a wait for all loads issued before.
+    const int first_block = k_begin / page_size;
+    if (k_begin < k_end) {
+        const int nblocks = (k_end - 1) / page_size - first_block + 1;       // the host keeps this <= DEC_TABLE_CAP
+        const int* table = block_table + (size_t)s * max_blocks + first_block;
+        for (int i = lane; i < nblocks && i < DEC_TABLE_CAP; i += 64) pages[i] = table[i];
+    }
+    __syncthreads();
+    auto row_of = [&](int key, bool& ok) -> size_t {       // element offset of the key's row in a cache layer
+        const int blk = key / page_size;
+        const int page = pages[blk - first_block];
+        ok = page >= 0 && page < num_pages;
+        return (((size_t)(ok ? page : 0) * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
+    };
 
     for (int h0 = 0; h0 < G; h0 += 16) {
         const int gcount = (G - h0 < 16) ? G - h0 : 16;
@@ -386,55 +416,56 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
             for (int jj = 0; jj < 8; ++jj) acc[ns][jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
 
-        for (int kb = k_begin; kb < k_end; kb += 32) {
-            // ---- S = Q K^T for two tiles of 16 keys
-            f32x4_t sv[2];
-            bool kok[2];
+        // K of a block: two tiles of 16 keys; lane (c, g) holds key 16 tt + c, dimensions QD g + 8 j ..
+        frag8 kf[2][KS];
+        bool kok[2];
+        auto load_k = [&](int kb) {
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
                 const int key = kb + 16 * tt + c;
                 kok[tt] = key < k_end;
-                frag8 kf[KS];
-#pragma unroll
-                for (int j = 0; j < KS; ++j) kf[j].raw = zero4;
-                if (kok[tt]) {
-                    const int page = table[key / page_size];
-                    kok[tt] = page >= 0 && page < num_pages;
-                    if (kok[tt]) {
-                        const bf16_t* kp = kc + (((size_t)page * nkv + kvh) * page_size + key % page_size) * DH + QD * g;
-#pragma unroll
-                        for (int j = 0; j < KS; ++j) kf[j].raw = *reinterpret_cast<const u32x4*>(kp + 8 * j);
-                    }
-                }
-                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                size_t off = 0;
+                if (kok[tt]) off = row_of(key, kok[tt]);
 #pragma unroll
                 for (int j = 0; j < KS; ++j)
-                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[j].v, sv[tt], 0, 0, 0);
+                    kf[tt][j].raw = kok[tt] ? *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j) : zero4;
             }
-            // ---- V rows of this lane: keys kb + 8g + i, dimensions 128 ns + 8c ..
+        };
+        if (k_begin < k_end) load_k(k_begin);
+        for (int kb = k_begin; kb < k_end; kb += 32) {
+            // ---- V rows of this lane: keys kb + 8g + i, dimensions 128 ns + 8c ..  (issued before
+            // K is waited for, so they stay in flight during Q K^T and the softmax)
             u32x4 vraw[NS][8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int key = kb + 8 * g + i;
                 bool ok = key < k_end;
                 size_t off = 0;
-                if (ok) {
-                    const int page = table[key / page_size];
-                    ok = page >= 0 && page < num_pages;
-                    off = (((size_t)(ok ? page : 0) * nkv + kvh) * page_size + key % page_size) * DH;
-                }
+                if (ok) off = row_of(key, ok);
 #pragma unroll
                 for (int ns = 0; ns < NS; ++ns) {
                     const int d = 128 * ns + 8 * c;
                     vraw[ns][i] = (ok && d < DH) ? *reinterpret_cast<const u32x4*>(vc + off + d) : zero4;
                 }
             }
+            // ---- S = Q K^T
+            f32x4_t sv[2];
+            bool sok[2] = {kok[0], kok[1]};
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0);
+            }
+            // ---- the next block's K: in flight during the softmax and P V
+            if (kb + 32 < k_end) load_k(kb + 32);
             // ---- online softmax; lanes whose key is past the end hold -inf
             float alpha[4], pr[2][4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float s0 = kok[0] ? sv[0][r] * scale : -INFINITY;
-                const float s1 = kok[1] ? sv[1][r] * scale : -INFINITY;
+                const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;
+                const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;
                 const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));     // the block has a key: mx is finite
                 alpha[r] = expf(m[r] - mx);
                 pr[0][r] = expf(s0 - mx);
@@ -526,7 +557,7 @@ static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, cons
 #undef LI_DEC
     if (nsplit > 1) {
         dim3 g2(n_tokens, nh);
-        attention_merge_kernel<T><<<g2, 64, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit);
+        attention_merge_kernel<T><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit);
     }
     return li_launch_status();
 }
@@ -548,8 +579,9 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
                                     block_table, max_blocks, token_list, n_tokens, seg_of_token, q_start, q_len,
                                     ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages, window, scale,
                                     nsplit, stream);
+    if (nsplit > MERGE_MAX_SPLITS) return LI_ERR_SIZE;
     if (dtype == LI_BF16 && use_mfma) {
-        if (nkv > 65535 || nsplit > 65535 || nsplit < 1) return LI_ERR_SIZE;
+        if (nkv > 65535 || nsplit < 1) return LI_ERR_SIZE;
         dim3 grid(n_tokens, nkv, nsplit);
 #define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV><<<grid, 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
@@ -559,7 +591,7 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
 #undef LI_DM
         if (nsplit > 1) {
             dim3 g2(n_tokens, nh);
-            attention_merge_kernel<bf16_t><<<g2, 64, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit);
+            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit);
         }
         return li_launch_status();
     }

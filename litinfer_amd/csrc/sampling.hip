@@ -26,24 +26,51 @@ __device__ __forceinline__ void block_argmax(float& v, int& i, float* sv, int* s
     for (int k = 1; k < SMP_NT / LI_WAVE; ++k) argmax_combine(v, i, sv[k], si[k]);
 }
 
-__global__ __launch_bounds__(SMP_NT) void argmax_rows_kernel(const float* __restrict__ logits,
-                                                             int* __restrict__ out, int V) {
+// Two stages, so that a few rows still use many compute units: stage 1 finds the
+// (maximum, lowest index) of each of ARGMAX_CHUNKS contiguous chunks of a row, stage 2
+// combines a row's chunks.  Ties go to the lower index in both.
+#define ARGMAX_CHUNKS 32
+
+__global__ __launch_bounds__(SMP_NT) void argmax_partial_kernel(const float* __restrict__ logits,
+                                                                float* __restrict__ pv, int* __restrict__ pi,
+                                                                int V, int chunk) {
     __shared__ float sv[SMP_NT / LI_WAVE];
     __shared__ int si[SMP_NT / LI_WAVE];
     const float* row = logits + (size_t)blockIdx.x * V;
+    const int c0 = blockIdx.y * chunk, c1 = (c0 + chunk < V) ? c0 + chunk : V;
     float v = -INFINITY;
     int i = 0x7fffffff;
-    for (int j = threadIdx.x; j < V; j += SMP_NT) {
+    for (int j = c0 + threadIdx.x; j < c1; j += SMP_NT) {
         const float x = row[j];
         if (x > v || i == 0x7fffffff) { v = x; i = j; }   // strictly greater: the first maximum stays
     }
     block_argmax(v, i, sv, si);
+    if (threadIdx.x == 0) { pv[blockIdx.x * gridDim.y + blockIdx.y] = v; pi[blockIdx.x * gridDim.y + blockIdx.y] = i; }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi,
+                                                          int* __restrict__ out, int nchunks) {
+    float v = -INFINITY;
+    int i = 0x7fffffff;
+    for (int c = threadIdx.x; c < nchunks; c += 64) argmax_combine(v, i, pv[blockIdx.x * nchunks + c], pi[blockIdx.x * nchunks + c]);
+#pragma unroll
+    for (int o = LI_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(v, o, LI_WAVE);
+        const int oi = __shfl_xor(i, o, LI_WAVE);
+        argmax_combine(v, i, ov, oi);
+    }
     if (threadIdx.x == 0) out[blockIdx.x] = i;
 }
 
-extern "C" int li_argmax_rows(const float* logits, int* out, int n, int V, hipStream_t stream) {
+// scratch_v, scratch_i: n * ARGMAX_CHUNKS floats / ints
+extern "C" int li_argmax_rows(const float* logits, int* out, float* scratch_v, int* scratch_i, int n, int V,
+                              hipStream_t stream) {
     if (n <= 0 || V <= 0) return LI_ERR_SIZE;
-    argmax_rows_kernel<<<n, SMP_NT, 0, stream>>>(logits, out, V);
+    int nchunks = (V + 4095) / 4096;
+    if (nchunks > ARGMAX_CHUNKS) nchunks = ARGMAX_CHUNKS;
+    const int chunk = (V + nchunks - 1) / nchunks;
+    argmax_partial_kernel<<<dim3(n, nchunks), SMP_NT, 0, stream>>>(logits, scratch_v, scratch_i, V, chunk);
+    argmax_final_kernel<<<n, 64, 0, stream>>>(scratch_v, scratch_i, out, nchunks);
     return li_launch_status();
 }
 

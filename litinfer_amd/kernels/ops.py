@@ -43,7 +43,7 @@ _SIGNATURES = {
         "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I],
     },
     "sampling": {
-        "li_argmax_rows": [P, P, I, I],
+        "li_argmax_rows": [P, P, P, P, I, I],
         "li_sample_rows": [P, P, P, P, P, P, I, I],
     },
 }
@@ -333,6 +333,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
         if mfma:
             nsplit = max(1, min(-(-2048 // (n_single * nkv)), -(-keys // 128), 64))
+            # a split's pages must fit the kernel's copy of the block table (1024 entries)
+            nsplit = max(nsplit, -(-(keys + 64) // (1000 * page_size)))
+            _chk(nsplit <= 64, f"attention: a context of {keys} keys in pages of {page_size} is too "
+                               f"long for the decode kernel")
         else:
             nsplit = max(1, min(-(-512 // (n_single * nkv)), -(-keys // 256), 64))
         acc = ml = None
@@ -361,14 +365,23 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
 
 
 # ------------------------------------------------------------------ sampling
+_argmax_scratch = {}
+
+
 def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
     """out[i] = index of the maximum of row i, the lowest index on ties."""
     _gpu(logits, out)
     _chk(logits.dim() == 2 and logits.dtype is torch.float32 and logits.is_contiguous(), "argmax: logits")
     _chk(out.dtype is torch.int32 and out.numel() == logits.shape[0] and out.is_contiguous(), "argmax: out")
-    if logits.shape[0]:
-        _run("sampling", "li_argmax_rows", logits.data_ptr(), out.data_ptr(), logits.shape[0],
-             logits.shape[1])
+    n = logits.shape[0]
+    if n:
+        key = (logits.device, n)
+        if key not in _argmax_scratch:
+            _argmax_scratch[key] = (torch.empty(n * 32, dtype=torch.float32, device=logits.device),
+                                    torch.empty(n * 32, dtype=torch.int32, device=logits.device))
+        sv, si = _argmax_scratch[key]
+        _run("sampling", "li_argmax_rows", logits.data_ptr(), out.data_ptr(), sv.data_ptr(), si.data_ptr(),
+             n, logits.shape[1])
 
 
 def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
