@@ -530,6 +530,191 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     }
 }
 
+// ------------------------------------------- portions of prompts, bfloat16, MFMA
+// A block takes a tile of up to 16 consecutive tokens of one segment and one kv head; its
+// waves are the query heads of that kv head (up to 8 at a time), so they read the same
+// keys and values at about the same time and share them through the caches.  A wave holds
+// 16 query rows (tokens) of one head and walks the keys in blocks of 32 exactly as the
+// single-query kernel does, with a limit per row: key <= position of the row, and within
+// the window.
+#define PRE_TABLE_CAP 4096
+
+template <int DH>
+__global__ __launch_bounds__(512) void paged_attention_prefill_mfma_kernel(
+    const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
+    int max_blocks, const int* __restrict__ tiles, const int* __restrict__ q_start,
+    const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int page_size,
+    int num_pages, int window, float scale) {
+    constexpr int KS = DH / 32, NS = (DH + 127) / 128, QD = DH / 4, PSTRIDE = 40;
+    __shared__ __attribute__((aligned(16))) uint16_t p_lds_all[8][16 * PSTRIDE];
+    __shared__ int pages[PRE_TABLE_CAP];
+    const int s = tiles[blockIdx.x * 4], t0 = tiles[blockIdx.x * 4 + 1], nrows = tiles[blockIdx.x * 4 + 2];
+    const int kvh = blockIdx.y;
+    const int G = nh / nkv;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int g = lane >> 4, c = lane & 15;
+    uint16_t* p_lds = p_lds_all[wave];
+    const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);           // position of the tile's first token
+    const int p_last = p0 + nrows - 1;
+    const int lo0 = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+    const int k_begin = lo0 & ~31, k_end = p_last + 1;
+    const int first_block = k_begin / page_size;
+    const int nblocks = (k_end - 1) / page_size - first_block + 1;
+    const int* table = block_table + (size_t)s * max_blocks + first_block;
+    const bool in_lds = nblocks <= PRE_TABLE_CAP;
+    if (in_lds)
+        for (int i = threadIdx.x; i < nblocks; i += blockDim.x) pages[i] = table[i];
+    __syncthreads();
+    const u32x4 zero4 = {{0u, 0u, 0u, 0u}};
+    auto row_of = [&](int key, bool& ok) -> size_t {
+        const int blk = key / page_size;
+        const int page = in_lds ? pages[blk - first_block] : table[blk - first_block];
+        ok = page >= 0 && page < num_pages;
+        return (((size_t)(ok ? page : 0) * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
+    };
+    int prow[4], lrow[4];                       // last and first visible key of this lane's four rows
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * g + r;
+        prow[r] = (row < nrows) ? p0 + row : -1;
+        lrow[r] = (window > 0 && prow[r] - window + 1 > 0) ? prow[r] - window + 1 : 0;
+    }
+
+    for (int hw = wave; hw < G; hw += nwaves) {
+        const int head = kvh * G + hw;
+        frag8 qa[KS];
+#pragma unroll
+        for (int j = 0; j < KS; ++j)
+            qa[j].raw = (c < nrows) ? *reinterpret_cast<const u32x4*>(
+                            q + (size_t)(t0 + c) * q_row_stride + (size_t)head * DH + QD * g + 8 * j) : zero4;
+        f32x4_t acc[NS][8];
+#pragma unroll
+        for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) acc[ns][jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
+        frag8 kf[2][KS];
+        bool kok[2];
+        auto load_k = [&](int kb) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                const int key = kb + 16 * tt + c;
+                kok[tt] = key < k_end && key >= lo0;
+                size_t off = 0;
+                if (kok[tt]) off = row_of(key, kok[tt]);
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+                    kf[tt][j].raw = kok[tt] ? *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j) : zero4;
+            }
+        };
+        load_k(k_begin);
+        for (int kb = k_begin; kb < k_end; kb += 32) {
+            u32x4 vraw[NS][8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int key = kb + 8 * g + i;
+                bool ok = key < k_end && key >= lo0;
+                size_t off = 0;
+                if (ok) off = row_of(key, ok);
+#pragma unroll
+                for (int ns = 0; ns < NS; ++ns) {
+                    const int d = 128 * ns + 8 * c;
+                    vraw[ns][i] = (ok && d < DH) ? *reinterpret_cast<const u32x4*>(vc + off + d) : zero4;
+                }
+            }
+            f32x4_t sv[2];
+            const bool sok[2] = {kok[0], kok[1]};
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < KS; ++j)
+                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0);
+            }
+            if (kb + 32 < k_end) load_k(kb + 32);
+            float alpha[4], pr[2][4];
+            const int key0 = kb + c, key1 = kb + 16 + c;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float s0 = (sok[0] && key0 <= prow[r] && key0 >= lrow[r]) ? sv[0][r] * scale : -INFINITY;
+                const float s1 = (sok[1] && key1 <= prow[r] && key1 >= lrow[r]) ? sv[1][r] * scale : -INFINITY;
+                const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));
+                const float ms = (mx == -INFINITY) ? 0.f : mx;       // a row may see no key yet
+                alpha[r] = expf(m[r] - ms);
+                pr[0][r] = expf(s0 - ms);
+                pr[1][r] = expf(s1 - ms);
+                l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];
+                m[r] = mx;
+            }
+            // P through this wave's own piece of LDS: a wave's LDS operations run in order
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = float_to_bf16(pr[tt][r]);
+            __builtin_amdgcn_wave_barrier();
+            frag8 pa;
+            pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int ns = 0; ns < NS; ++ns) {
+#pragma unroll
+                for (int jj = 0; jj < 8; ++jj) {
+                    frag8 vf;
+#pragma unroll
+                    for (int ii = 0; ii < 4; ++ii)
+                        vf.raw.w[ii] = __builtin_amdgcn_perm(vraw[ns][2 * ii + 1].w[jj >> 1], vraw[ns][2 * ii].w[jj >> 1],
+                                                             (jj & 1) ? 0x07060302u : 0x05040100u);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[ns][jj][r] *= alpha[r];
+                    acc[ns][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vf.v, acc[ns][jj], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float lt = row16_sum(l[r]);
+            const int row = 4 * g + r;
+            if (row >= nrows) continue;
+            const float inv = lt != 0.f ? 1.0f / lt : 0.f;
+            bf16_t* orow = out + (size_t)(t0 + row) * nh * DH + (size_t)head * DH;
+#pragma unroll
+            for (int ns = 0; ns < NS; ++ns) {
+                const int d = 128 * ns + 8 * c;
+                if (d < DH) {
+                    u32x4 o;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        o.w[i] = (uint32_t)float_to_bf16(acc[ns][2 * i][r] * inv) |
+                                 ((uint32_t)float_to_bf16(acc[ns][2 * i + 1][r] * inv) << 16);
+                    *reinterpret_cast<u32x4*>(orow + d) = o;
+                }
+            }
+        }
+    }
+}
+
+// tiles: int [ntiles, 4] = (segment, first token of the tile in the batch, rows <= 16, unused)
+extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void* out, const void* kc,
+                                          const void* vc, const int* block_table, int max_blocks,
+                                          const int* tiles, int ntiles, const int* q_start, const int* q_len,
+                                          const int* ctx_len, int nh, int nkv, int dh, int page_size,
+                                          int num_pages, int window, float scale, hipStream_t stream) {
+    if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || page_size <= 0 || max_blocks <= 0)
+        return LI_ERR_SIZE;
+    const int G = nh / nkv;
+    const int waves = G < 8 ? G : 8;        // more heads than waves: a wave takes several in turn
+    dim3 grid(ntiles, nkv);
+#define LI_PRE(DHV) paged_attention_prefill_mfma_kernel<DHV><<<grid, waves * 64, 0, stream>>>( \
+        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
+        tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale)
+    if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
+#undef LI_PRE
+    return li_launch_status();
+}
+
 template <typename T>
 static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, const T* vc,
                          const int* block_table, int max_blocks, const int* token_list, int n_tokens,

@@ -47,6 +47,10 @@ class AttentionMeta:
     num_single: int = 0
     multi_tokens: Optional[torch.Tensor] = None
     num_multi: int = 0
+    # the tokens of segments with several tokens, cut into tiles of up to 16 consecutive tokens
+    # of one segment: int32 [tiles, 4] = (segment, first token, tokens, 0)
+    tiles: Optional[torch.Tensor] = None
+    num_tiles: int = 0
     max_single_ctx: int = 0
     extra: Dict[Any, Any] = field(default_factory=dict)    # what kernels derive and keep for the step
 
@@ -156,7 +160,10 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     single_mask = q_len[seg_of_token] == 1
     single = np.nonzero(single_mask)[0].astype(np.int32)
     multi = np.nonzero(~single_mask)[0].astype(np.int32)
-    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows, single, multi]
+    tile_rows = [(i, int(q_start[i]) + a, min(16, int(q_len[i]) - a), 0)
+                 for i in range(nseg) if q_len[i] > 1 for a in range(0, int(q_len[i]), 16)]
+    tiles = np.asarray(tile_rows, dtype=np.int32).reshape(-1, 4)
+    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows, single, multi, tiles]
     tables, max_blocks = [], []
     for gi in range(len(cache.groups)):
         tabs = [cache.block_table(e.rid, gi) for e in entries]
@@ -176,12 +183,12 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     dev = uploader.upload(parts)
     ctx = StepContext(ws, T, nseg)
     (ctx.ids, ctx.positions, d_seg, d_qs, d_ql, d_cl, ctx.state_slots, ctx.want_rows,
-     d_single, d_multi) = dev[:10]
+     d_single, d_multi, d_tiles) = dev[:11]
     ctx.num_want = len(want)
     ctx.host_state_slots = slots
     ctx.host_q_start, ctx.host_q_len, ctx.host_ctx_len = q_start[:-1], q_len, ctx_len
     for gi in range(len(cache.groups)):
-        d_tab, d_slot = dev[10 + 2 * gi], dev[11 + 2 * gi]
+        d_tab, d_slot = dev[11 + 2 * gi], dev[12 + 2 * gi]
         ctx._slot_maps.append(d_slot)
         ctx._attn.append(AttentionMeta(
             block_table=d_tab, max_blocks=max_blocks[gi], seg_of_token=d_seg, q_start=d_qs,
@@ -190,6 +197,7 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
             host_q_start=q_start[:-1], host_q_len=q_len, host_ctx_len=ctx_len,
             single_tokens=d_single if len(multi) else None, num_single=len(single),
             multi_tokens=d_multi if len(single) else None, num_multi=len(multi),
+            tiles=d_tiles, num_tiles=len(tile_rows),
             # with padded tables the split count must not follow the context either
             max_single_ctx=(max_blocks[gi] * P if pad_blocks is not None else
                             int(ctx_len[q_len == 1].max()) if len(single) else 0)))

@@ -40,6 +40,7 @@ _SIGNATURES = {
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
+        "li_paged_attention_prefill": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F],
         "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I],
     },
     "sampling": {
@@ -355,7 +356,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
              meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              0 if acc is None else acc.data_ptr(), 0 if ml is None else ml.data_ptr(),
              nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit, int(mfma))
-    if n_multi:
+    if n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles and n_multi == meta.num_multi:
+        _run("attention", "li_paged_attention_prefill", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
+             k.data_ptr(), v.data_ptr(), bt.data_ptr(), meta.max_blocks, meta.tiles.data_ptr(),
+             meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale))
+    elif n_multi:
         lst = meta.multi_tokens if n_multi < t else None
         _run("attention", "li_paged_attention", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), _DT[qkv.dtype], bt.data_ptr(), meta.max_blocks,

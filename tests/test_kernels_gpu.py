@@ -212,6 +212,10 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
                          host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len,
                          single_tokens=dev(single) if len(multi) else None, num_single=len(single),
                          multi_tokens=dev(multi) if len(single) else None, num_multi=len(multi),
+                         tiles=dev(np.asarray([(i, int(q_start[i]) + a, min(16, int(q_len[i]) - a), 0)
+                                               for i in range(nseg) if q_len[i] > 1
+                                               for a in range(0, int(q_len[i]), 16)], dtype=np.int32).reshape(-1, 4)),
+                         num_tiles=sum(-(-int(n) // 16) for n in q_len if n > 1),
                          max_single_ctx=int(ctx_len[q_len == 1].max()) if len(single) else 0)
     out = torch.empty(T, nh * dh, dtype=dtype, device=DEV)
     scale = 1.0 / math.sqrt(dh)
@@ -242,6 +246,9 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
     ([(300, 1), (77, 1)], 6, 3, 80, 16, 0),                         # a head size the split kernel does not take
     ([(300, 1), (1025, 1), (31, 1)], 40, 2, 64, 16, 0),             # 20 heads in a group: two blocks of MFMA rows
     ([(33, 1), (32, 1), (1, 1)], 7, 7, 128, 8, 0),                  # one head per group, keys around a block's edge
+    ([(700, 700), (40, 3), (513, 1), (300, 17)], 28, 4, 128, 16, 0),    # portions on the matrix cores
+    ([(257, 100), (90, 90), (64, 33)], 20, 2, 64, 8, 50),           # 10 heads a group (two turns of waves), window
+    ([(2, 2), (17, 16), (33, 2)], 3, 3, 128, 16, 0),
 ])
 def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     out, ref = _paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=6)
