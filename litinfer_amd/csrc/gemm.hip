@@ -176,6 +176,158 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
         }
 }
 
+// ---------------------------------------------- bfloat16, many rows (prompts)
+// With many rows the product is bound by the matrix cores and, before them, by
+// how often an operand byte has to be read from LDS: a wave's tile of WM x WN
+// needs (WM + WN) * BK operand elements for WM * WN * BK multiply-adds, so the
+// tiles are made large.  Block tile BM x BN, 4 waves as 2 x 2, wave tile
+// BM/2 x BN/2 made of MFMA 32x32x16 tiles, K in steps of 64.  Two LDS stages:
+// the global loads of the next K step are in flight (in registers) while this
+// step is multiplied from LDS, then written to the other stage; one barrier a
+// step.  A row of a stage is 64 elements = 128 bytes = 8 chunks of 16 bytes;
+// chunk c of row r lies at position c ^ ((r >> 1) & 7), which spreads the 16
+// rows that one fragment read touches over all banks.
+template <int BM, int BN, int BK, typename TO>
+__global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __restrict__ x,
+                                                             const bf16_t* __restrict__ w,
+                                                             const float* __restrict__ bias,
+                                                             TO* __restrict__ out, int M, int N, int K,
+                                                             int accumulate) {
+    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    constexpr int CPR = BK / 8;                                   // 16-byte chunks in a row of a stage
+    constexpr int WRAP = 128 / BK;                                // rows that fill all 64 banks once
+    constexpr int CA = BM * CPR / 256, CB = BN * CPR / 256;       // chunks per thread and stage
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    uint16_t* As = lds;                                           // [2][BM][BK]
+    uint16_t* Bs = lds + 2 * BM * BK;                             // [2][BN][BK]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    // Blocks go to the 8 XCDs in turn (block b runs on XCD b % 8), and each XCD has an L2 of its
+    // own.  The tiles are dealt so that the ~32 blocks an XCD runs at one time form a patch of
+    // all row panels x a few column panels: a column panel of W is then read from HBM by one
+    // XCD only, by blocks that run together, and x is read again per patch from the caches.
+    const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
+    const int gn = mtiles >= 32 ? 1 : 32 / mtiles;                // column panels of a patch
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int patch = idx / (mtiles * gn), within = idx % (mtiles * gn);
+    const int mt = within % mtiles, nt = ((patch * gn) + within / mtiles) * 8 + xcd;
+    if (nt >= ntiles) return;
+    const int m0 = mt * BM, n0 = nt * BN;
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    auto slot = [](int row, int c) { return row * BK + ((c ^ ((row / WRAP) & (CPR - 1))) << 3); };
+    // Global loads carry no branches: a row past the end is read as the last row (its products
+    // land in output rows that are not stored), and only a K step that reaches past K is
+    // masked, chunk by chunk.
+    bf16x8 ra[CA], rb[CB];
+    size_t oa[CA], ob[CB];
+#pragma unroll
+    for (int i = 0; i < CA; ++i) {
+        const int qd = tid + 256 * i, row = qd / CPR, c = qd % CPR;
+        oa[i] = (size_t)((m0 + row < M) ? m0 + row : M - 1) * K + 8 * c;
+    }
+#pragma unroll
+    for (int i = 0; i < CB; ++i) {
+        const int qd = tid + 256 * i, row = qd / CPR, c = qd % CPR;
+        ob[i] = (size_t)((n0 + row < N) ? n0 + row : N - 1) * K + 8 * c;
+    }
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#define LI_GLOAD(k0)                                                                                      \
+    {                                                                                                     \
+        const bool full_ = (k0) + BK <= K;                                                                \
+        _Pragma("unroll") for (int i = 0; i < CA; ++i)                                                    \
+            ra[i] = (full_ || (k0) + 8 * ((tid + 256 * i) % CPR) < K)                                     \
+                        ? *reinterpret_cast<const bf16x8*>(x + oa[i] + (k0)) : zero8;                     \
+        _Pragma("unroll") for (int i = 0; i < CB; ++i)                                                    \
+            rb[i] = (full_ || (k0) + 8 * ((tid + 256 * i) % CPR) < K)                                     \
+                        ? *reinterpret_cast<const bf16x8*>(w + ob[i] + (k0)) : zero8;                     \
+    }
+#define LI_LSTORE(stage)                                                                                  \
+    {                                                                                                     \
+        _Pragma("unroll") for (int i = 0; i < CA; ++i) {                                                  \
+            const int qd = tid + 256 * i, row = qd / CPR, c = qd % CPR;                                   \
+            *reinterpret_cast<bf16x8*>(&As[(stage) * BM * BK + slot(row, c)]) = ra[i];                    \
+        }                                                                                                 \
+        _Pragma("unroll") for (int i = 0; i < CB; ++i) {                                                  \
+            const int qd = tid + 256 * i, row = qd / CPR, c = qd % CPR;                                   \
+            *reinterpret_cast<bf16x8*>(&Bs[(stage) * BN * BK + slot(row, c)]) = rb[i];                    \
+        }                                                                                                 \
+    }
+    const int frow = lane & 31, fh = lane >> 5;
+    const int nk = (K + BK - 1) / BK;
+    // fragments of K sub-step ks + 1 are read from LDS before the MFMAs of sub-step ks are
+    // issued, so the reads' latency passes while the matrix cores work
+    bf16x8 af[2][TM], bfr[2][TN];
+#define LI_FREAD(stage, ks, buf)                                                                          \
+    {                                                                                                     \
+        const int c_ = 2 * (ks) + fh;                                                                     \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                    \
+            af[buf][i] = *reinterpret_cast<const bf16x8*>(&As[(stage) * BM * BK + slot(wm + 32 * i + frow, c_)]); \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                    \
+            bfr[buf][j] = *reinterpret_cast<const bf16x8*>(&Bs[(stage) * BN * BK + slot(wn + 32 * j + frow, c_)]); \
+    }
+    LI_GLOAD(0)
+    LI_LSTORE(0)
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int stage = kt & 1;
+        if (kt + 1 < nk) LI_GLOAD((kt + 1) * BK)
+        LI_FREAD(stage, 0, 0)
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            if (ks + 1 < BK / 16) LI_FREAD(stage, ks + 1, (ks + 1) & 1)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) LI_LSTORE(stage ^ 1)
+        __syncthreads();
+    }
+#undef LI_FREAD
+#undef LI_GLOAD
+#undef LI_LSTORE
+    const int ccol = lane & 31, crow = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = n0 + wn + 32 * j + ccol;
+            if (col >= N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm + 32 * i + 8 * (r >> 2) + crow + (r & 3);
+                if (row < M) epilogue_store(out, (size_t)row * N + col, acc[i][j][r], bias, col, accumulate);
+            }
+        }
+}
+
+template <int BM, int BN, int BK, typename TO>
+static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
+                      int accumulate, hipStream_t stream) {
+    const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
+    const long gn = mtiles >= 32 ? 1 : 32 / mtiles;
+    const long per_xcd = ((ntiles + 7) / 8 + gn - 1) / gn * gn * mtiles;     // whole patches
+    if (per_xcd * 8 > 0x7fffffffL) return LI_ERR_SIZE;
+    dim3 grid((unsigned)(per_xcd * 8));
+    constexpr int lds_bytes = 2 * (BM + BN) * BK * 2;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)gemm_bf16_big_kernel<BM, BN, BK, TO>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+            return LI_ERR_LAUNCH;
+        configured = true;
+    }
+    gemm_bf16_big_kernel<BM, BN, BK, TO><<<grid, 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
+    return li_launch_status();
+}
+
 // ------------------------------------------------- bfloat16, few rows (decode)
 // With M <= 64 the product is bound by streaming W once from HBM, and the
 // bandwidth reached is (bytes in flight) / (memory latency): the kernel is
@@ -365,6 +517,18 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         const bool aligned = (K % 8) == 0;
         if (aligned && M <= 64)
             return li_linear_skinny(x, w, bias, out, M, N, K, out_dtype, accumulate, 0, stream);
+        if (aligned && M > 64) {
+            // the largest tile that still gives every compute unit a block
+            const long blocks256 = (long)((N + 255) / 256) * ((M + 255) / 256);
+#define LI_BIG(BM, BN, BK) (out_dtype == LI_F32 ? launch_big<BM, BN, BK, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
+                                            : launch_big<BM, BN, BK, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
+            if (out_dtype != LI_F32 && out_dtype != LI_BF16) return LI_ERR_DTYPE;
+            // measured at M = 2048: 256 x 256 tiles win where they still give every compute unit
+            // two blocks' worth of work, 128 x 128 tiles (three blocks a compute unit) elsewhere
+            if (blocks256 >= 512) return LI_BIG(256, 256, 64);
+            return LI_BIG(128, 128, 64);
+#undef LI_BIG
+        }
 #define LI_GEMM(TO, AL) gemm_bf16_kernel<TO, AL><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, accumulate)
         if (out_dtype == LI_F32) { if (aligned) LI_GEMM(float, true); else LI_GEMM(float, false); }
         else if (out_dtype == LI_BF16) { if (aligned) LI_GEMM(bf16_t, true); else LI_GEMM(bf16_t, false); }
