@@ -549,7 +549,9 @@ __global__ __launch_bounds__(512) void paged_attention_prefill_mfma_kernel(
     constexpr int KS = DH / 32, NS = (DH + 127) / 128, QD = DH / 4, PSTRIDE = 40;
     __shared__ __attribute__((aligned(16))) uint16_t p_lds_all[8][16 * PSTRIDE];
     __shared__ int pages[PRE_TABLE_CAP];
-    const int s = tiles[blockIdx.x * 4], t0 = tiles[blockIdx.x * 4 + 1], nrows = tiles[blockIdx.x * 4 + 2];
+    // the last tiles of a long segment have the most keys: they are started first
+    const int tile = gridDim.x - 1 - blockIdx.x;
+    const int s = tiles[tile * 4], t0 = tiles[tile * 4 + 1], nrows = tiles[tile * 4 + 2];
     const int kvh = blockIdx.y;
     const int G = nh / nkv;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;

@@ -29,25 +29,41 @@ extern "C" int li_embedding(const int* ids, const void* table, int table_dtype, 
 }
 
 // ------------------------------------------------------------------ rmsnorm
-// y = w * x * rsqrt(mean(x^2) + eps), eps inside the root; one block per row.
+// y = w * x * rsqrt(mean(x^2) + eps), eps inside the root; one block per row.  The row is
+// read once and kept in registers (up to RN_PER elements a thread); longer rows are read again.
+#define RN_NT 1024
+#define RN_PER 8
+
 template <typename TI, typename TO>
-__global__ void rmsnorm_kernel(const TI* __restrict__ x, const float* __restrict__ w, float eps,
-                               TO* __restrict__ out, int H) {
-    __shared__ float red[256 / LI_WAVE];
+__global__ __launch_bounds__(RN_NT) void rmsnorm_kernel(const TI* __restrict__ x, const float* __restrict__ w,
+                                                         float eps, TO* __restrict__ out, int H) {
+    __shared__ float red[RN_NT / LI_WAVE];
     const TI* row = x + (size_t)blockIdx.x * H;
     TO* o = out + (size_t)blockIdx.x * H;
+    float v[RN_PER];
     float ss = 0.f;
-    for (int j = threadIdx.x; j < H; j += 256) { float v = load_as_float(row + j); ss += v * v; }
-    ss = block_sum<256>(ss, red);
+#pragma unroll
+    for (int i = 0; i < RN_PER; ++i) {
+        const int j = threadIdx.x + i * RN_NT;
+        v[i] = (j < H) ? load_as_float(row + j) : 0.f;
+        ss += v[i] * v[i];
+    }
+    for (int j = threadIdx.x + RN_PER * RN_NT; j < H; j += RN_NT) { const float t = load_as_float(row + j); ss += t * t; }
+    ss = block_sum<RN_NT>(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)H + eps);
-    for (int j = threadIdx.x; j < H; j += 256)
+#pragma unroll
+    for (int i = 0; i < RN_PER; ++i) {
+        const int j = threadIdx.x + i * RN_NT;
+        if (j < H) store_from_float(o + j, w[j] * v[i] * inv);
+    }
+    for (int j = threadIdx.x + RN_PER * RN_NT; j < H; j += RN_NT)
         store_from_float(o + j, w[j] * load_as_float(row + j) * inv);
 }
 
 extern "C" int li_rmsnorm(const void* x, int x_dtype, const float* w, float eps, void* out,
                           int out_dtype, int T, int H, hipStream_t stream) {
     if (T <= 0 || H <= 0) return LI_ERR_SIZE;
-#define LI_NORM(TI, TO) rmsnorm_kernel<TI, TO><<<T, 256, 0, stream>>>((const TI*)x, w, eps, (TO*)out, H)
+#define LI_NORM(TI, TO) rmsnorm_kernel<TI, TO><<<T, RN_NT, 0, stream>>>((const TI*)x, w, eps, (TO*)out, H)
     if (x_dtype == LI_F32 && out_dtype == LI_F32) LI_NORM(float, float);
     else if (x_dtype == LI_F32 && out_dtype == LI_BF16) LI_NORM(float, bf16_t);
     else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) LI_NORM(bf16_t, bf16_t);

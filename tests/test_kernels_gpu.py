@@ -330,3 +330,63 @@ def test_gather_and_cast(ops):
     f = torch.empty(10, 37, device=DEV)
     ops.cast(b, f)
     assert torch.equal(f.cpu(), x.to(torch.bfloat16).float())
+
+
+def _sample(ops, logits, temperature, top_k, top_p, u):
+    n = logits.shape[0]
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    f = lambda v, dt: torch.tensor(v, dtype=dt, device=DEV)
+    ops.sample_rows(logits.to(DEV), f(temperature, torch.float32), f(top_k, torch.int32),
+                    f(top_p, torch.float32), f(u, torch.float32), out)
+    return out.cpu().tolist()
+
+
+def _pick_is_right(row, temperature, top_k, top_p, u, pick, slack=2e-5):
+    """The kernel sums in float32 in another order than the plain sampler: the
+    pick is right if the uniform number lies within its interval of the CDF,
+    give or take the rounding of the sums."""
+    ids, p = plain_impl.sampling_candidates(row, temperature, top_k, top_p)
+    assert pick in ids.tolist(), f"token {pick} is not among the candidates"
+    cum = np.cumsum(p)
+    i = ids.tolist().index(pick)
+    lo = cum[i - 1] if i else 0.0
+    return lo - slack <= u <= cum[i] + slack
+
+
+@pytest.mark.parametrize("vocab", [8, 301, 4096, 152064])
+def test_sample_rows_against_the_plain_sampler(ops, vocab):
+    g = torch.Generator().manual_seed(13)
+    n = 12
+    logits = torch.randn(n, vocab, generator=g) * 3
+    logits[1, : min(5, vocab)] = 7.0                       # equal maxima: ties go by index
+    temperature = [0.0, 0.7, 1.0, 1.3, 0.8, 1.0, 0.5, 2.0, 1.0, 1.0, 0.9, 1.0]
+    top_k = [0, 3, 0, 0, 50, 1, 0, 7, vocab, 0, 5, 2]
+    top_p = [1.0, 1.0, 0.9, 0.5, 0.8, 0.3, 1.0, 0.95, 1.0, 0.01, 0.99, 1.0]
+    u = torch.rand(n, generator=g).tolist()
+    picks = _sample(ops, logits, temperature, top_k, top_p, u)
+    rows = logits.double().numpy()
+    assert picks[0] == plain_impl.argmax_first(rows[0])                    # temperature 0: greedy
+    assert picks[5] == plain_impl.argmax_first(rows[5])                    # top_k 1
+    assert picks[9] == plain_impl.argmax_first(rows[9])                    # a tiny top_p keeps the maximum only
+    for r in range(1, n):
+        assert _pick_is_right(rows[r], temperature[r], top_k[r], top_p[r], u[r], picks[r]), r
+    # exact agreement wherever the uniform number is not at an interval's edge
+    same = sum(picks[r] == plain_impl.sample_with_uniform(rows[r], temperature[r], top_k[r], top_p[r], u[r])
+               for r in range(n))
+    assert same >= n - 1
+
+
+def test_sample_rows_frequencies_and_ties(ops):
+    lg = torch.tensor([[2.0, 1.0, 3.0, 3.0, -1.0, 0.5, 2.5, 0.0]])
+    n = 4000
+    g = torch.Generator().manual_seed(14)
+    u = torch.rand(n, generator=g).tolist()
+    picks = _sample(ops, lg.repeat(n, 1), [1.0] * n, [0] * n, [1.0] * n, u)
+    freq = np.bincount(picks, minlength=8) / n
+    want = np.exp(lg[0].double().numpy())
+    assert np.abs(freq - want / want.sum()).max() < 0.03
+    # top_k = 1 with two equal maxima: the lower index; top_k = 3: ids 2, 3 and 6 only
+    assert set(_sample(ops, lg.repeat(50, 1), [1.0] * 50, [1] * 50, [1.0] * 50, u[:50])) == {2}
+    assert set(_sample(ops, lg.repeat(500, 1), [1.0] * 500, [3] * 500, [1.0] * 500, u[:500])) == {2, 3, 6}
+    # top_p = 0.5: the shortest prefix reaching half the mass is {2, 3}
+    assert set(_sample(ops, lg.repeat(500, 1), [1.0] * 500, [0] * 500, [0.5] * 500, u[:500])) == {2, 3}
