@@ -9,6 +9,7 @@ import torch
 from ..config.spec import ModelSpec, PartSpec
 from ..kernels import ops
 from ..parts.base import Runtime, build_part
+from ..parts.stream import ResidualStream
 from ..weights.loader import ParamSpec
 
 
@@ -74,8 +75,10 @@ class Model:
         h = self.spec.hidden_size
         x = ctx.ws.buffer("model.residual", (ctx.num_tokens, h), torch.float32)
         self.embedding.forward(ctx.ids, x)
+        stream = ResidualStream(x, ctx.ws)
         for i, e in enumerate(self.order):
-            self.layers[e.layer].forward(x, ctx, cache.view(i))
+            self.layers[e.layer].forward(stream, ctx, cache.view(i))
+        x = stream.tensor()
         if ctx.num_want == 0:
             return None
         rows = ctx.ws.buffer("model.rows", (ctx.num_want, h), torch.float32)

@@ -2,6 +2,7 @@ from .base import (Block, FeedForward, Mixer, Norm, PagedKVNeed, Part, Runtime, 
                    build_part, register_part)
 from .position import Position, RopeNeox
 from .linear import Linear
+from .stream import ResidualStream
 from .norm import RMSNorm
 from .attention import GQAttention
 from .mlp import SwiGLUMLP
@@ -9,5 +10,5 @@ from .block import PreNormBlock
 from .embedding import LinearHead, TokenEmbedding
 
 __all__ = ["Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "Part", "Runtime", "StateNeed",
-           "build_part", "register_part", "Position", "RopeNeox", "Linear", "RMSNorm",
+           "build_part", "register_part", "Position", "RopeNeox", "Linear", "ResidualStream", "RMSNorm",
            "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding"]

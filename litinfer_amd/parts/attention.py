@@ -92,7 +92,7 @@ class GQAttention(Mixer):
         attn = ctx.ws.buffer("attn.out", (t, self.n_q), self.rt.dtype)
         ops.paged_attention(qkv, attn, cache.k, cache.v, ctx.attention_meta(cache.group),
                             self.nh, self.nkv, self.dh, cache.page_size, self.window, self.scale, ws=ctx.ws)
-        self.out(attn, residual, accumulate=True, ws=ctx.ws)
+        residual.add_linear(self.out, attn)
 
 
 register_part("mixer", "gqa_attention", GQAttention)

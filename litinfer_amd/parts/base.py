@@ -8,16 +8,19 @@ here.
 
 Interfaces (T = tokens of the step, H = hidden size):
 
-* Norm.forward(x [T, H] float32) -> [T, H] in the activation dtype.
+* Norm.forward(x [T, H] float32, out) -> out [T, H] in the activation dtype.
 * Mixer.cache_need() -> PagedKVNeed | StateNeed | None;
-  Mixer.forward(xn [T, H], residual [T, H] float32, ctx, cache): ADDS its
-  output to `residual` in 32-bit.  `cache` is the CacheView of the entry of the
-  execution order that is running; `cache.owned` is False when the entry reads
-  another entry's cache and must write nothing.
-* FeedForward.forward(xn, residual): adds its output to `residual`.
+  Mixer.forward(xn [T, H], residual, ctx, cache): ADDS its output to the
+  residual stream in 32-bit.  `residual` is a `ResidualStream`
+  (parts/stream.py): `residual.add_linear(linear, h)` adds h W^T + b, and
+  `residual.tensor()` is the float32 tensor [T, H] itself for a part that adds
+  in its own way.  `cache` is the CacheView of the entry of the execution order
+  that is running; `cache.owned` is False when the entry reads another entry's
+  cache and must write nothing.
+* FeedForward.forward(xn, residual, ctx): adds its output to the stream.
 * Position: prepares per-step tables and rotates (or otherwise encodes) the
   mixer's queries and keys; see `parts/position.py`.
-* Block.forward(x [T, H] float32 residual stream, ctx, cache).
+* Block.forward(stream, ctx, cache): runs its parts on the `ResidualStream`.
 """
 from __future__ import annotations
 

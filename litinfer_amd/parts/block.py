@@ -1,6 +1,7 @@
 """The pre-norm arrangement of a layer's parts
 (src/llaisys/models/qwen2.cpp:272-317): x += mixer(norm1(x)); x += ffn(norm2(x)).
-The residual stream x is float32; mixer and feed-forward add into it."""
+The residual stream x is float32; mixer and feed-forward add into it through
+the `ResidualStream` they are given."""
 from __future__ import annotations
 
 from .base import Block, build_part, register_part
@@ -32,12 +33,12 @@ class PreNormBlock(Block):
         for p in self._all:
             p.load_params(get)
 
-    def forward(self, x, ctx, cache):
-        xn = ctx.ws.buffer("block.xn", x.shape, self.rt.dtype)
-        self.norm1.forward(x, xn)
-        self.mixer.forward(xn, x, ctx, cache)
-        self.norm2.forward(x, xn)
-        self.ffn.forward(xn, x, ctx)
+    def forward(self, stream, ctx, cache):
+        xn = ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype)
+        stream.normed(self.norm1, xn)
+        self.mixer.forward(xn, stream, ctx, cache)
+        stream.normed(self.norm2, xn)
+        self.ffn.forward(xn, stream, ctx)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -44,7 +44,7 @@ class SwiGLUMLP(FeedForward):
             gu = ctx.ws.buffer("mlp.gate_up", (t, 2 * self.inter), self.rt.dtype)
             self.gate_up(xn, gu, ws=ctx.ws)
             ops.swiglu(gu, h)
-        self.down(h, residual, accumulate=True, ws=ctx.ws)
+        residual.add_linear(self.down, h)
 
 
 register_part("feed_forward", "swiglu_mlp", SwiGLUMLP)

@@ -16,7 +16,7 @@ from litinfer_amd.config import ExecEntry, LayerSpec, ModelSpec, PartSpec, Qwen2
 from litinfer_amd.engine import Engine, StepEntry, StepError
 from litinfer_amd.engine.batch import BatchUploader, build_context
 from litinfer_amd.engine.workspace import Workspace
-from litinfer_amd.parts import Mixer, Runtime, StateNeed, build_part, register_part
+from litinfer_amd.parts import Mixer, ResidualStream, Runtime, StateNeed, build_part, register_part
 from litinfer_amd.weights import ParamSpec
 from tiny_configs import TINY_A, TINY_B, TINY_C
 
@@ -189,7 +189,7 @@ def test_feed_forward_part_alone(device):
     res = torch.randn(t, h, generator=g)
     out = res.clone().to(device)
     ctx = type("Ctx", (), {"ws": Workspace(device)})()
-    part.forward(x.to(device), out, ctx)
+    part.forward(x.to(device), ResidualStream(out, ctx.ws), ctx)
     xd = x.double().numpy()
     d = {k: v.double().numpy() for k, v in ws.items()}
     ref = res.double().numpy() + P.swiglu(xd @ d["f.gate_proj.weight"].T, xd @ d["f.up_proj.weight"].T) @ d["f.down_proj.weight"].T
@@ -223,7 +223,7 @@ def _mixer_case(device, window, cache_steps):
         ctx = build_context(cache, entries, wsp, up)
         x = torch.cat([xs[r][done[r]:done[r] + n] for r, n in step]).to(device)
         res = torch.zeros(x.shape[0], h, device=device)
-        mixer.forward(x, res, ctx, cache.view(0))
+        mixer.forward(x, ResidualStream(res, wsp), ctx, cache.view(0))
         o = 0
         for r, n in step:
             got[r].append(res[o:o + n].cpu().numpy())
@@ -331,6 +331,7 @@ class ToyStateMixer(Mixer):
         self.w = get(self.prefix + "w").to(torch.float32).to(self.rt.device)
 
     def forward(self, xn, residual, ctx, cache):
+        residual = residual.tensor()
         for s in range(ctx.num_segments):
             q0, n, slot = int(ctx.host_q_start[s]), int(ctx.host_q_len[s]), int(ctx.host_state_slots[s])
             state = cache.state[slot]
