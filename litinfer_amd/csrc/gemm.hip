@@ -346,21 +346,14 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
 //
 // SWIGLU: W is [gate; up] with N rows each: tile 0 takes gate rows, tile 1 the
 // up rows of the same columns, and out[m, n] = up * gate / (1 + exp(-gate)).
-//
-// A product with few output columns has few blocks of 16 columns; to give every
-// compute unit an equal share of W such a product is also cut along K over
-// gridDim.y.  Each part then writes its plain partial sums as float32
-// [part, M, N]; `skinny_finish_kernel` adds the parts in part order, so the
-// result does not depend on timing.
 #define SK_CHUNK 128
 
 struct SkinnyArgs {
     const bf16_t* x;        // [M, K]
     const bf16_t* w;        // [N, K], or [2 N, K] with SWIGLU
     const float* bias;      // [N] or null
-    void* out;              // [M, N]; with parts > 1: float [parts, M, N] of partial sums
+    void* out;              // [M, N]
     int M, N, K, accumulate;
-    int parts;              // K is cut into this many parts over gridDim.y (1: the whole K in one block)
 };
 
 template <int MT, int NT, int WAVES, bool SWIGLU, typename TO>
@@ -396,10 +389,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    const int all_chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
-    const int per_part = (all_chunks + a.parts - 1) / a.parts;
-    const int c_lo = blockIdx.y * per_part;                       // this block's chunks: c_lo .. nchunks - 1
-    const int nchunks = (c_lo + per_part < all_chunks) ? c_lo + per_part : all_chunks;
+    const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
 
     // The memory counter of a wave retires loads in the order they were issued, so waiting for
     // a chunk's x pieces also waits for every load issued before them.  All loads of a chunk (W
@@ -457,8 +447,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
         __builtin_amdgcn_wave_barrier();
     };
     if constexpr (AHEAD) {
-        if (c_lo + wave < nchunks) load_chunk(c_lo + wave, wbuf[0], xbuf[0]);
-        for (int c = c_lo + wave; c < nchunks; c += 2 * WAVES) {   // two chunks a turn: buffer numbers are constants
+        if (wave < nchunks) load_chunk(wave, wbuf[0], xbuf[0]);
+        for (int c = wave; c < nchunks; c += 2 * WAVES) {          // two chunks a turn: buffer numbers are constants
             if (c + WAVES < nchunks) load_chunk(c + WAVES, wbuf[1], xbuf[1]);
             multiply(wbuf[0], xbuf[0]);
             if (c + WAVES >= nchunks) break;
@@ -466,7 +456,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
             multiply(wbuf[1], xbuf[1]);
         }
     } else {
-        for (int c = c_lo + wave; c < nchunks; c += WAVES) {
+        for (int c = wave; c < nchunks; c += WAVES) {
             load_chunk(c, wbuf[0], xbuf[0]);
             multiply(wbuf[0], xbuf[0]);
         }
@@ -491,16 +481,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 s[nt][0] += o[0]; s[nt][1] += o[1]; s[nt][2] += o[2]; s[nt][3] += o[3];
             }
         }
-        if (a.parts > 1) {                                   // plain partial sums; the finish kernel does the rest
-            float* part = (float*)a.out + (size_t)blockIdx.y * M * N;
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int n = n0 + 16 * nt + 4 * (l >> 4) + r;
-                    if (n < N) part[(size_t)m * N + n] = s[nt][r];
-                }
-        } else if constexpr (SWIGLU) {
+        if constexpr (SWIGLU) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int n = n0 + 4 * (l >> 4) + r;
@@ -524,10 +505,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
 template <bool SWIGLU, typename TO>
 static void launch_skinny(const SkinnyArgs& a, hipStream_t stream) {
     const int M = a.M, N = a.N;
-#define LI_SK(MT, NT, WV) gemm_bf16_skinny_kernel<MT, NT, WV, SWIGLU, TO><<<dim3((N + 16 * (SWIGLU ? 1 : NT) - 1) / (16 * (SWIGLU ? 1 : NT)), a.parts), WV * 64, 0, stream>>>(a)
-    if (a.parts > 1) {                                      // K cut over blocks: four waves a block
-        if constexpr (!SWIGLU) { if (M <= 16) LI_SK(1, 1, 4); else if (M <= 32) LI_SK(2, 1, 4); else LI_SK(4, 2, 8); }
-    } else if constexpr (SWIGLU) {
+#define LI_SK(MT, NT, WV) gemm_bf16_skinny_kernel<MT, NT, WV, SWIGLU, TO><<<(N + 16 * (SWIGLU ? 1 : NT) - 1) / (16 * (SWIGLU ? 1 : NT)), WV * 64, 0, stream>>>(a)
+    if constexpr (SWIGLU) {
         if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
     } else if (N >= 8192) {                                 // many columns: many blocks, two tiles share each piece of x
         if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
@@ -537,77 +516,13 @@ static void launch_skinny(const SkinnyArgs& a, hipStream_t stream) {
 #undef LI_SK
 }
 
-// out = out + bias + sum over parts of partial[part], then (when norm_w is given)
-// xn = norm_w * out / sqrt(mean(out^2) + eps): the end of a product cut along K, the residual
-// add and the RMSNorm that follows it, in one pass over the row.  One block per row.
-#define FIN_NT 1024
-#define FIN_PER 8
-
-template <typename TO>
-__global__ __launch_bounds__(FIN_NT) void skinny_finish_kernel(const float* __restrict__ partial, int parts,
-                                                               const float* __restrict__ bias,
-                                                               float* __restrict__ residual,
-                                                               const float* __restrict__ norm_w, float eps,
-                                                               TO* __restrict__ xn, int M, int N) {
-    __shared__ float red[FIN_NT / LI_WAVE];
-    const int m = blockIdx.x;
-    float* row = residual + (size_t)m * N;
-    float v[FIN_PER];
-    float ss = 0.f;
-    auto value = [&](int n) {
-        float sum = partial[(size_t)m * N + n];
-        for (int p = 1; p < parts; ++p) sum += partial[((size_t)p * M + m) * N + n];      // part order
-        if (bias) sum += bias[n];
-        return row[n] + sum;
-    };
-#pragma unroll
-    for (int i = 0; i < FIN_PER; ++i) {
-        const int n = threadIdx.x + i * FIN_NT;
-        v[i] = 0.f;
-        if (n < N) { v[i] = value(n); row[n] = v[i]; }
-        ss += v[i] * v[i];
-    }
-    for (int n = threadIdx.x + FIN_PER * FIN_NT; n < N; n += FIN_NT) {
-        const float t = value(n);
-        row[n] = t;
-        ss += t * t;
-    }
-    if (!norm_w) return;
-    ss = block_sum<FIN_NT>(ss, red);                 // (the barrier inside also orders the row's writes)
-    const float inv = 1.0f / sqrtf(ss / (float)N + eps);
-    TO* o = xn + (size_t)m * N;
-#pragma unroll
-    for (int i = 0; i < FIN_PER; ++i) {
-        const int n = threadIdx.x + i * FIN_NT;
-        if (n < N) store_from_float(o + n, norm_w[n] * v[i] * inv);
-    }
-    for (int n = threadIdx.x + FIN_PER * FIN_NT; n < N; n += FIN_NT)
-        store_from_float(o + n, norm_w[n] * row[n] * inv);
-}
-
-extern "C" int li_skinny_finish(const float* partial, int parts, const float* bias, float* residual,
-                                const float* norm_w, float eps, void* xn, int xn_dtype, int M, int N,
-                                hipStream_t stream) {
-    if (M <= 0 || N <= 0 || parts < 1) return LI_ERR_SIZE;
-    if (norm_w && xn_dtype == LI_F32)
-        skinny_finish_kernel<float><<<M, FIN_NT, 0, stream>>>(partial, parts, bias, residual, norm_w, eps, (float*)xn, M, N);
-    else if (!norm_w || xn_dtype == LI_BF16)
-        skinny_finish_kernel<bf16_t><<<M, FIN_NT, 0, stream>>>(partial, parts, bias, residual, norm_w, eps, (bf16_t*)xn, M, N);
-    else return LI_ERR_DTYPE;
-    return li_launch_status();
-}
-
 // Few rows (M <= 64), bfloat16, K a multiple of 8.  swiglu: w has 2 N rows ([gate; up]).
-// parts > 1: K is cut into parts over blocks and out is float32 [parts, M, N] of partial sums
-// (no bias, no accumulation: li_skinny_finish does those).
 extern "C" int li_linear_skinny(const void* x, const void* w, const float* bias, void* out, int M, int N,
-                                int K, int out_dtype, int accumulate, int swiglu, int parts,
-                                hipStream_t stream) {
+                                int K, int out_dtype, int accumulate, int swiglu, hipStream_t stream) {
     if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8)) return LI_ERR_SIZE;
     if (accumulate && out_dtype != LI_F32) return LI_ERR_DTYPE;
     if (swiglu && (bias || accumulate || out_dtype != LI_BF16)) return LI_ERR_DTYPE;
-    if (parts < 1 || parts > 64 || (parts > 1 && (swiglu || bias || accumulate || out_dtype != LI_F32))) return LI_ERR_SIZE;
-    SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, accumulate, parts};
+    SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, accumulate};
     if (swiglu) launch_skinny<true, bf16_t>(a, stream);
     else if (out_dtype == LI_BF16) launch_skinny<false, bf16_t>(a, stream);
     else if (out_dtype == LI_F32) launch_skinny<false, float>(a, stream);
@@ -629,7 +544,7 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         if (grid.y > 65535) return LI_ERR_SIZE;
         const bool aligned = (K % 8) == 0;
         if (aligned && M <= 64)
-            return li_linear_skinny(x, w, bias, out, M, N, K, out_dtype, accumulate, 0, 1, stream);
+            return li_linear_skinny(x, w, bias, out, M, N, K, out_dtype, accumulate, 0, stream);
         if (aligned && M > 64) {
             // the largest tile that still gives every compute unit a block
             const long blocks256 = (long)((N + 255) / 256) * ((M + 255) / 256);

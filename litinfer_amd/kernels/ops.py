@@ -36,8 +36,7 @@ _SIGNATURES = {
     },
     "gemm": {
         "li_linear": [P, P, P, P, I, I, I, I, I, I],
-        "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I, I],
-        "li_skinny_finish": [P, I, P, P, P, F, P, I, I, I],
+        "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
@@ -274,54 +273,24 @@ def skinny_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
 
 
 def linear_skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                  accumulate: bool = False, swiglu: bool = False, parts: int = 1) -> None:
+                  accumulate: bool = False, swiglu: bool = False) -> None:
     """The product for few rows (decoding).  swiglu: w is [gate; up] (2N rows)
     and out[m, n] = up * gate / (1 + exp(-gate)), the activation fused into the
-    product's epilogue.  parts > 1: K is cut into that many parts over blocks
-    and `out` is float32 [parts, M, N] of partial sums, to be added up by
-    `skinny_finish` (no bias, no accumulation here)."""
+    product's epilogue."""
     _gpu(x, w, bias, out)
     m, k = x.shape
-    n = out.shape[-1]
+    n = out.shape[1]
     _chk(skinny_takes(m, k, w.dtype), "linear_skinny: sizes or dtype not taken")
-    _chk(w.shape == ((2 * n if swiglu else n), k), "linear_skinny: shapes do not fit")
+    _chk(w.shape == ((2 * n if swiglu else n), k) and out.shape[0] == m, "linear_skinny: shapes do not fit")
     _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_skinny: contiguous operands")
     _chk(x.dtype is torch.bfloat16, "linear_skinny: x must be bfloat16")
-    if parts > 1:
-        _chk(out.shape == (parts, m, n) and out.dtype is torch.float32 and bias is None and not accumulate
-             and not swiglu and parts <= 64, "linear_skinny: partial sums are float32 [parts, M, N], plain")
-    else:
-        _chk(out.shape == (m, n), "linear_skinny: out shape")
     _chk(out.dtype in _DT and (not accumulate or out.dtype is torch.float32), "linear_skinny: out dtype")
     _chk(not swiglu or (bias is None and not accumulate and out.dtype is torch.bfloat16),
          "linear_skinny: swiglu takes no bias and no accumulation and writes bfloat16")
     _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
          "linear_skinny: bias must be float32 [N]")
     _run("gemm", "li_linear_skinny", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
-         out.data_ptr(), m, n, k, _DT[out.dtype], int(bool(accumulate)), int(bool(swiglu)), int(parts))
-
-
-def skinny_finish(partial: torch.Tensor, bias: Optional[torch.Tensor], residual: torch.Tensor,
-                  norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 0.0,
-                  xn: Optional[torch.Tensor] = None) -> None:
-    """residual += bias + sum over parts of partial[part] (in part order); with
-    norm_weight also xn = norm_weight * residual / sqrt(mean(residual^2) + eps):
-    the end of a product cut along K, the residual add and the RMSNorm that
-    follows, in one pass."""
-    _gpu(partial, bias, residual, norm_weight, xn)
-    _chk(partial.dim() == 3 and partial.dtype is torch.float32 and partial.is_contiguous(), "skinny_finish: partial")
-    parts, m, n = partial.shape
-    _chk(residual.shape == (m, n) and residual.dtype is torch.float32 and residual.is_contiguous(),
-         "skinny_finish: residual must be float32 [M, N]")
-    _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
-         "skinny_finish: bias")
-    if norm_weight is not None:
-        _chk(norm_weight.dtype is torch.float32 and norm_weight.numel() == n and norm_weight.is_contiguous()
-             and xn is not None and xn.shape == (m, n) and xn.is_contiguous() and xn.dtype in _DT,
-             "skinny_finish: norm weight [N] float32 and xn [M, N]")
-    _run("gemm", "li_skinny_finish", partial.data_ptr(), parts, 0 if bias is None else bias.data_ptr(),
-         residual.data_ptr(), 0 if norm_weight is None else norm_weight.data_ptr(), float(norm_eps),
-         0 if xn is None else xn.data_ptr(), _DT[xn.dtype] if xn is not None else 0, m, n)
+         out.data_ptr(), m, n, k, _DT[out.dtype], int(bool(accumulate)), int(bool(swiglu)))
 
 
 # ----------------------------------------------------------------- attention

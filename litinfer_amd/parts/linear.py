@@ -10,12 +10,6 @@ import torch
 from ..kernels import ops
 
 
-# Products with fewer blocks of 16 output columns than this are cut along K over blocks.  Measured
-# on MI355X at the 7B layer sizes the cut does not pay (the finish kernel costs what the better
-# balance gains), so it is off (0); tests switch it on to cover the path.
-SPLIT_BELOW_BLOCKS = 0
-
-
 class Linear:
     def __init__(self, rt, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
         self.rt = rt
@@ -27,20 +21,6 @@ class Linear:
         """Whether the product of these rows can have the SwiGLU activation as its
         epilogue (few rows, bfloat16)."""
         return x.dtype is torch.bfloat16 and ops.skinny_takes(x.shape[0], self.in_features, self.weight.dtype)
-
-    def split_parts(self, x: torch.Tensor) -> int:
-        """Into how many parts along K the product of these rows should be cut
-        over blocks (1: not at all).  Worth it for few rows and few output
-        columns: 16 columns make a block, and with fewer blocks than would
-        occupy the chip every compute unit gets an equal share only if K is cut."""
-        if x.dtype is not torch.bfloat16 or x.shape[0] > 32 or \
-                not ops.skinny_takes(x.shape[0], self.in_features, self.weight.dtype):
-            return 1
-        blocks = -(-self.out_features // 16)
-        chunks = -(-self.in_features // 128)
-        if blocks >= SPLIT_BELOW_BLOCKS or chunks < 8:
-            return 1
-        return max(1, min(8, chunks // 4, -(-1536 // blocks)))
 
     def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ws=None,
                  swiglu: bool = False):

@@ -10,7 +10,6 @@ from .base import Norm, register_part
 
 class RMSNorm(Norm):
     graph_safe = True
-    fusable_rmsnorm = True       # y = weight * x / sqrt(mean(x^2) + eps): a kernel may compute it from weight and eps
 
     def __init__(self, spec, rt):
         super().__init__(spec, rt)

@@ -123,36 +123,6 @@ def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, 
     assert rel(out, y) < (4 * math.sqrt(k) * 2.0 ** -24 if out_dtype is torch.float32 else 5e-3)
 
 
-@pytest.mark.parametrize("m,n,k,parts,bias,norm", [
-    (8, 3584, 18944, 7, False, True),       # decode: down product cut along K, residual add, next norm
-    (8, 3584, 3584, 7, False, True),
-    (1, 96, 1032, 3, True, True), (17, 37, 264, 2, True, False), (32, 200, 2056, 8, False, True),
-    (5, 9000, 1024, 4, False, True),        # a row longer than one pass of the finish kernel keeps in registers
-])
-def test_product_cut_along_k_and_its_finish(ops, m, n, k, parts, bias, norm):
-    g = torch.Generator().manual_seed(15)
-    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
-    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
-    b = torch.randn(n, generator=g) if bias else None
-    base = torch.randn(m, n, generator=g)
-    nw = 1 + 0.1 * torch.randn(n, generator=g)
-    partial = torch.empty(parts, m, n, device=DEV)
-    ops.linear_skinny(x.to(DEV), w.to(DEV), None, partial, parts=parts)
-    res = base.to(DEV)
-    xn = torch.empty(m, n, dtype=torch.bfloat16, device=DEV) if norm else None
-    ops.skinny_finish(partial, None if b is None else b.to(DEV), res, nw.to(DEV) if norm else None, 1e-5, xn)
-    want = base.double().numpy() + x.double().numpy() @ w.double().numpy().T
-    if b is not None:
-        want = want + b.double().numpy()
-    assert rel(res, want) < 4 * math.sqrt(k) * 2.0 ** -24
-    if norm:
-        assert rel(xn, plain_impl.rms_norm(want, nw.double().numpy(), 1e-5)) < 8e-3
-    # the sum over the parts does not depend on timing: twice the same bits
-    partial2 = torch.empty_like(partial)
-    ops.linear_skinny(x.to(DEV), w.to(DEV), None, partial2, parts=parts)
-    assert torch.equal(partial, partial2)
-
-
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_rows_do_not_depend_on_the_batch(ops, dtype):
     g = torch.Generator().manual_seed(3)

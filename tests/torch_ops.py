@@ -83,23 +83,7 @@ def linear(x, w, bias, out, accumulate=False):
         out.copy_(y.to(out.dtype))
 
 
-def skinny_finish(partial, bias, residual, norm_weight=None, norm_eps=0.0, xn=None):
-    s = partial.sum(0)
-    if bias is not None:
-        s = s + bias
-    residual += s
-    if norm_weight is not None:
-        rmsnorm(residual, norm_weight, norm_eps, xn)
-
-
-def linear_skinny(x, w, bias, out, accumulate=False, swiglu=False, parts=1):
-    if parts > 1:
-        k = x.shape[1]
-        chunks = -(-k // 128)
-        per = -(-chunks // parts) * 128
-        for p in range(parts):
-            out[p] = x[:, p * per:(p + 1) * per].float() @ w[:, p * per:(p + 1) * per].float().T
-        return
+def linear_skinny(x, w, bias, out, accumulate=False, swiglu=False):
     y = x.float() @ w.float().T
     if swiglu:
         n = out.shape[1]
@@ -145,7 +129,7 @@ def argmax_rows(logits, out):
 
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
-       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "skinny_finish", "check_attention_sizes",
+       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "check_attention_sizes",
        "paged_attention", "argmax_rows"]
 
 
