@@ -293,19 +293,247 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
 #undef LI_FREAD
 #undef LI_GLOAD
 #undef LI_LSTORE
+    // Epilogue through LDS: a wave puts a band of 32 rows of its tile into a piece of LDS of its
+    // own and takes it out again row by row, 8 consecutive columns a lane, so that the stores
+    // (and the loads of what is added to) are whole 16-byte pieces, 16 lanes to a row.
+    __syncthreads();                               // the main loop's LDS is free now
+    constexpr int ESTRIDE = WN + 4;                // floats per row of a band (pad against bank conflicts)
+    float* band = reinterpret_cast<float*>(lds) + wave * 32 * ESTRIDE;
     const int ccol = lane & 31, crow = (lane >> 5) * 4;
+    constexpr int LPR = WN / 8;                    // lanes that take one row of the band out (8 columns each)
+    constexpr int RPP = 64 / LPR;                  // rows per pass of the wave
+    const int erow = lane / LPR, ecol = (lane % LPR) * 8;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 32 * j + ccol] = acc[i][j][r];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int pass = 0; pass < 32 / RPP; ++pass) {
+            const int row = m0 + wm + 32 * i + RPP * pass + erow;
+            if (row >= M) continue;
+            {
+                const int col = n0 + wn + ecol;
+                if (col >= N) continue;
+                const float* src = &band[(RPP * pass + erow) * ESTRIDE + ecol];
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = src[e];
+                const size_t idx = (size_t)row * N + col;
+                if (col + 8 <= N && (N % 8) == 0) {               // whole pieces: wide loads and stores
+                    if (bias) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) v[e] += bias[col + e];
+                    }
+                    if constexpr (sizeof(TO) == 4) {
+                        float4* o = reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + idx);
+                        if (accumulate) {
+                            const float4 a0 = o[0], a1 = o[1];
+                            v[0] += a0.x; v[1] += a0.y; v[2] += a0.z; v[3] += a0.w;
+                            v[4] += a1.x; v[5] += a1.y; v[6] += a1.z; v[7] += a1.w;
+                        }
+                        o[0] = float4{v[0], v[1], v[2], v[3]};
+                        o[1] = float4{v[4], v[5], v[6], v[7]};
+                    } else {
+                        chunk16 o;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            o.w[e] = (uint32_t)float_to_bf16(v[2 * e]) | ((uint32_t)float_to_bf16(v[2 * e + 1]) << 16);
+                        *reinterpret_cast<chunk16*>(reinterpret_cast<uint16_t*>(out) + idx) = o;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (col + e < N) epilogue_store(out, idx + e, v[e], bias, col + e, accumulate);
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------- bfloat16, many rows, loads straight into LDS
+// The same tiling with the global loads going straight into LDS
+// (global_load_lds_dwordx4: lane i's 16 bytes land at the wave's LDS base + 16 i),
+// which needs no staging registers, so DMA_STAGES - 1 steps of K are in flight
+// while one is multiplied: the latency of a load is several steps long.  The
+// compiler does not track these loads' completion; `s_waitcnt vmcnt(n)` is
+// placed by hand: a wave's loads retire in order, so allowing the loads of the
+// younger steps to stay outstanding waits exactly for the oldest step, and the
+// barrier after it makes that true for the loads of all four waves.
+// Needs K to be a multiple of the step (a load cannot be masked to zeros).  Tiles: 256 x 256
+// with steps of 32 (each operand byte read from LDS feeds twice the multiply-adds of the
+// 128 x 128 tile, which is bound by LDS bandwidth), or 128 x 128 with steps of 64 where the
+// larger tile would leave compute units without a block.
+#define DMA_STAGES 4
+#define LI_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
+#define LI_LOAD_TO_LDS(gptr, lptr)                                                                        \
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),              \
+                                     (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+template <int BM, int BN, int BK, typename TO>
+__global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x,
+                                                             const bf16_t* __restrict__ w,
+                                                             const float* __restrict__ bias,
+                                                             TO* __restrict__ out, int M, int N, int K,
+                                                             int accumulate) {
+    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    constexpr int CPR = BK / 8, WRAP = 128 / BK;                 // chunks in a row; rows that fill all banks once
+    constexpr int RPI = 64 / CPR;                                // rows one load instruction of a wave covers
+    constexpr int IA = BM / 4 / RPI, IB = BN / 4 / RPI;          // load instructions per wave and step for A and B
+    constexpr int STAGE = (BM + BN) * BK;                        // elements of a stage: A rows then B rows
+    constexpr int LPW = IA + IB;                                 // loads a wave issues per step
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
+    const int gn = mtiles >= 32 ? 1 : 32 / mtiles;               // see gemm_bf16_big_kernel: patches per XCD
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    const int patch = idx / (mtiles * gn), within = idx % (mtiles * gn);
+    const int mt = within % mtiles, nt = ((patch * gn) + within / mtiles) * 8 + xcd;
+    if (nt >= ntiles) return;
+    const int m0 = mt * BM, n0 = nt * BN;
+    floatx16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int col = n0 + wn + 32 * j + ccol;
-            if (col >= N) continue;
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm + 32 * i + 8 * (r >> 2) + crow + (r & 3);
-                if (row < M) epilogue_store(out, (size_t)row * N + col, acc[i][j][r], bias, col, accumulate);
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    // chunk c of row r lies at position c ^ ((r / WRAP) % CPR) of the row's CPR positions
+    auto slot = [](int row, int c) { return row * BK + ((c ^ ((row / WRAP) & (CPR - 1))) << 3); };
+    // this lane's part of a step: a wave takes BM / 4 rows of A and BN / 4 rows of B; one
+    // instruction covers RPI rows, lane -> row lane / CPR, position lane % CPR
+    const bf16_t* ga[IA];
+    const bf16_t* gb[IB];
+#pragma unroll
+    for (int i = 0; i < IA; ++i) {
+        const int row = (BM / 4) * wave + RPI * i + lane / CPR, c = (lane % CPR) ^ ((row / WRAP) & (CPR - 1));
+        ga[i] = x + (size_t)((m0 + row < M) ? m0 + row : M - 1) * K + 8 * c;     // rows past the end: the last row
+    }
+#pragma unroll
+    for (int i = 0; i < IB; ++i) {
+        const int row = (BN / 4) * wave + RPI * i + lane / CPR, c = (lane % CPR) ^ ((row / WRAP) & (CPR - 1));
+        gb[i] = w + (size_t)((n0 + row < N) ? n0 + row : N - 1) * K + 8 * c;
+    }
+    auto issue = [&](int kt) {
+        uint16_t* st = lds + (kt % DMA_STAGES) * STAGE;
+#pragma unroll
+        for (int i = 0; i < IA; ++i) LI_LOAD_TO_LDS(ga[i] + (size_t)kt * BK, st + ((BM / 4) * wave + RPI * i) * BK);
+#pragma unroll
+        for (int i = 0; i < IB; ++i) LI_LOAD_TO_LDS(gb[i] + (size_t)kt * BK, st + BM * BK + ((BN / 4) * wave + RPI * i) * BK);
+    };
+    const int frow = lane & 31, fh = lane >> 5;
+    const int nk = K / BK;
+#pragma unroll
+    for (int p = 0; p < DMA_STAGES - 1; ++p)
+        if (p < nk) issue(p);
+    for (int kt = 0; kt < nk; ++kt) {
+        // loads of the steps after kt that this wave has issued: at most DMA_STAGES - 2 steps here
+        const int younger = (nk - 1 - kt < DMA_STAGES - 2) ? nk - 1 - kt : DMA_STAGES - 2;
+        if (younger >= 2) LI_VMCNT(2 * LPW); else if (younger == 1) LI_VMCNT(LPW); else LI_VMCNT(0);
+        __builtin_amdgcn_s_barrier();              // step kt is in LDS for all waves; step kt - 1 is read by all
+        asm volatile("" ::: "memory");
+        if (kt + DMA_STAGES - 1 < nk) issue(kt + DMA_STAGES - 1);      // into the stage step kt - 1 was in
+        const uint16_t* As = lds + (kt % DMA_STAGES) * STAGE;
+        const uint16_t* Bs = As + BM * BK;
+        bf16x8 af[2][TM], bfr[2][TN];
+#define LI_FREAD(ks, buf)                                                                                  \
+    {                                                                                                     \
+        const int c_ = 2 * (ks) + fh;                                                                     \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                    \
+            af[buf][i] = *reinterpret_cast<const bf16x8*>(&As[slot(wm + 32 * i + frow, c_)]);             \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                    \
+            bfr[buf][j] = *reinterpret_cast<const bf16x8*>(&Bs[slot(wn + 32 * j + frow, c_)]);            \
+    }
+        LI_FREAD(0, 0)
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            if (ks + 1 < BK / 16) LI_FREAD(ks + 1, (ks + 1) & 1)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
+        }
+#undef LI_FREAD
+        asm volatile("" ::: "memory");
+    }
+    __syncthreads();                               // the main loop's LDS is free now
+    constexpr int ESTRIDE = WN + 4;
+    float* band = reinterpret_cast<float*>(lds) + wave * 32 * ESTRIDE;
+    const int ccol = lane & 31, crow = (lane >> 5) * 4;
+    constexpr int LPR = WN / 8, RPP = 64 / LPR;
+    const int erow = lane / LPR, ecol = (lane % LPR) * 8;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 32 * j + ccol] = acc[i][j][r];
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int pass = 0; pass < 32 / RPP; ++pass) {
+            const int row = m0 + wm + 32 * i + RPP * pass + erow;
+            const int col = n0 + wn + ecol;
+            if (row >= M || col >= N) continue;
+            const float* src = &band[(RPP * pass + erow) * ESTRIDE + ecol];
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = src[e];
+            const size_t o_idx = (size_t)row * N + col;
+            if (col + 8 <= N && (N % 8) == 0) {
+                if (bias) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v[e] += bias[col + e];
+                }
+                if constexpr (sizeof(TO) == 4) {
+                    float4* o = reinterpret_cast<float4*>(reinterpret_cast<float*>(out) + o_idx);
+                    if (accumulate) {
+                        const float4 a0 = o[0], a1 = o[1];
+                        v[0] += a0.x; v[1] += a0.y; v[2] += a0.z; v[3] += a0.w;
+                        v[4] += a1.x; v[5] += a1.y; v[6] += a1.z; v[7] += a1.w;
+                    }
+                    o[0] = float4{v[0], v[1], v[2], v[3]};
+                    o[1] = float4{v[4], v[5], v[6], v[7]};
+                } else {
+                    chunk16 o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        o.w[e] = (uint32_t)float_to_bf16(v[2 * e]) | ((uint32_t)float_to_bf16(v[2 * e + 1]) << 16);
+                    *reinterpret_cast<chunk16*>(reinterpret_cast<uint16_t*>(out) + o_idx) = o;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (col + e < N) epilogue_store(out, o_idx + e, v[e], bias, col + e, accumulate);
             }
         }
+    }
+}
+
+template <int BM, int BN, int BK, typename TO>
+static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
+                      int accumulate, hipStream_t stream) {
+    const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
+    const long gn = mtiles >= 32 ? 1 : 32 / mtiles;
+    const long per_xcd = ((ntiles + 7) / 8 + gn - 1) / gn * gn * mtiles;
+    if (per_xcd * 8 > 0x7fffffffL) return LI_ERR_SIZE;
+    constexpr int lds_bytes = DMA_STAGES * (BM + BN) * BK * 2;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, BK, TO>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
+            return LI_ERR_LAUNCH;
+        configured = true;
+    }
+    gemm_bf16_dma_kernel<BM, BN, BK, TO><<<dim3((unsigned)(per_xcd * 8)), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
+    return li_launch_status();
 }
 
 template <int BM, int BN, int BK, typename TO>
@@ -551,10 +779,16 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
 #define LI_BIG(BM, BN, BK) (out_dtype == LI_F32 ? launch_big<BM, BN, BK, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                             : launch_big<BM, BN, BK, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
             if (out_dtype != LI_F32 && out_dtype != LI_BF16) return LI_ERR_DTYPE;
-            // measured at M = 2048: 256 x 256 tiles win where they still give every compute unit
-            // two blocks' worth of work, 128 x 128 tiles (three blocks a compute unit) elsewhere
-            if (blocks256 >= 512) return LI_BIG(256, 256, 64);
-            return LI_BIG(128, 128, 64);
+#define LI_DMA(BM, BN, BK) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
+                                               : launch_dma<BM, BN, BK, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
+            // measured at the 7B layer sizes: 256 x 256 tiles win where they still give every
+            // compute unit two blocks' worth of work, 128 x 128 tiles elsewhere and for fewer rows
+            if (K % 64 == 0 && K >= 64 * DMA_STAGES) {
+                if (blocks256 >= 512) return LI_DMA(256, 256, 32);
+                return LI_DMA(128, 128, 64);
+            }
+#undef LI_DMA
+            return LI_BIG(128, 128, 64);             // K not a multiple of 64: loads staged in registers
 #undef LI_BIG
         }
 #define LI_GEMM(TO, AL) gemm_bf16_kernel<TO, AL><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)w, bias, (TO*)out, M, N, K, accumulate)
