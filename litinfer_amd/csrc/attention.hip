@@ -355,6 +355,12 @@ __device__ __forceinline__ float row16_sum(float v) { return group_sum<16>(v); }
 
 union frag8 { u32x4 raw; bf16x8_t v; };
 
+// Loads in these kernels are never conditional: a load under a branch is waited for at once,
+// and so is one whose result is replaced by zeros right away.  A key that must not be read is
+// replaced by the nearest one of the same request that may (its score is masked to -inf, so its
+// probability is exactly 0 and the finite value it brings adds nothing); a lane without a head or
+// a dimension of its own repeats a neighbour's work and stores nothing.
+
 #define DEC_TABLE_CAP 1024      // pages of one split that fit the kernel's copy of the block table
 
 template <int DH>
@@ -382,7 +388,6 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     const int k_begin = lo + split * per;
     const int k_end = (k_begin + per < p + 1) ? k_begin + per : p + 1;
     const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
-    const u32x4 zero4 = {{0u, 0u, 0u, 0u}};
     // The block table of this split goes to LDS first: a page number fetched from global
     // memory in the loop would make every wait for it a wait for all loads issued before.
     const int first_block = k_begin / page_size;
@@ -393,22 +398,22 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     }
     __syncthreads();
     auto row_of = [&](int key, bool& ok) -> size_t {       // element offset of the key's row in a cache layer
+        ok = key < k_end;
+        key = ok ? key : k_end - 1;                        // (only called when k_begin < k_end)
         const int blk = key / page_size;
-        const int page = pages[blk - first_block];
-        ok = page >= 0 && page < num_pages;
-        return (((size_t)(ok ? page : 0) * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
+        int page = pages[blk - first_block];
+        ok = ok && page >= 0 && page < num_pages;
+        page = page < 0 ? 0 : (page >= num_pages ? num_pages - 1 : page);
+        return (((size_t)page * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
     };
 
     for (int h0 = 0; h0 < G; h0 += 16) {
         const int gcount = (G - h0 < 16) ? G - h0 : 16;
         frag8 qa[KS];
 #pragma unroll
-        for (int j = 0; j < KS; ++j) {
-            qa[j].raw = zero4;
-            if (c < gcount)
-                qa[j].raw = *reinterpret_cast<const u32x4*>(
-                    q + (size_t)t * q_row_stride + (size_t)(kvh * G + h0 + c) * DH + QD * g + 8 * j);
-        }
+        for (int j = 0; j < KS; ++j)
+            qa[j].raw = *reinterpret_cast<const u32x4*>(
+                q + (size_t)t * q_row_stride + (size_t)(kvh * G + h0 + (c < gcount ? c : gcount - 1)) * DH + QD * g + 8 * j);
         f32x4_t acc[NS][8];
 #pragma unroll
         for (int ns = 0; ns < NS; ++ns)
@@ -422,13 +427,10 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
         auto load_k = [&](int kb) {
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
-                const int key = kb + 16 * tt + c;
-                kok[tt] = key < k_end;
-                size_t off = 0;
-                if (kok[tt]) off = row_of(key, kok[tt]);
+                const size_t off = row_of(kb + 16 * tt + c, kok[tt]);
 #pragma unroll
                 for (int j = 0; j < KS; ++j)
-                    kf[tt][j].raw = kok[tt] ? *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j) : zero4;
+                    kf[tt][j].raw = *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j);
             }
         };
         if (k_begin < k_end) load_k(k_begin);
@@ -438,14 +440,12 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
             u32x4 vraw[NS][8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int key = kb + 8 * g + i;
-                bool ok = key < k_end;
-                size_t off = 0;
-                if (ok) off = row_of(key, ok);
+                bool ok;
+                const size_t off = row_of(kb + 8 * g + i, ok);
 #pragma unroll
                 for (int ns = 0; ns < NS; ++ns) {
                     const int d = 128 * ns + 8 * c;
-                    vraw[ns][i] = (ok && d < DH) ? *reinterpret_cast<const u32x4*>(vc + off + d) : zero4;
+                    vraw[ns][i] = *reinterpret_cast<const u32x4*>(vc + off + (d < DH ? d : DH - 8));
                 }
             }
             // ---- S = Q K^T
@@ -531,189 +531,234 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
 }
 
 // ------------------------------------------- portions of prompts, bfloat16, MFMA
-// A block takes a tile of up to 16 consecutive tokens of one segment and one kv head; its
-// waves are the query heads of that kv head (up to 8 at a time), so they read the same
-// keys and values at about the same time and share them through the caches.  A wave holds
-// 16 query rows (tokens) of one head and walks the keys in blocks of 32 exactly as the
-// single-query kernel does, with a limit per row: key <= position of the row, and within
-// the window.
-#define PRE_TABLE_CAP 4096
+// A block takes a tile of up to 32 consecutive tokens of one segment and one kv head; its
+// waves are query heads of that kv head (PRE_WAVES at a time; blockIdx.z picks which), so
+// the keys and values of a block of 32 keys are fetched once, into LDS, for all of them.
+//
+// A wave holds 32 queries of one head and works with the TRANSPOSED score tile
+// S^T[key, query] = K Q^T (v_mfma_f32_32x32x16_bf16; row operand K from LDS, column operand
+// Q in registers; lane l: row/column l % 32 and the 64 head dimensions 64 * (l / 32) ..): in
+// the result a lane holds 16 keys of ITS query (register r: key 8 (r / 4) + 4 (l / 32) + r % 4),
+// so the softmax over keys is arithmetic inside a lane plus one exchange with lane l ^ 32.
+// These registers, rounded to bfloat16, are already the column operand of
+// O^T[d, query] = V^T P^T: MFMA step s takes registers 8 s .. 8 s + 7, i.e. the keys
+// {16 s + 4 h + i, 16 s + 8 + 4 h + i : i < 4} for lane half h.  The row operand V^T wants those
+// same keys next to each other for one dimension d: the values are transposed in registers
+// when they are put into LDS (8 keys x 8 dimensions a thread), in that key order.
+#define PRE_TABLE_CAP 8192
+#define PRE_WAVES 4
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 template <int DH>
-__global__ __launch_bounds__(512) void paged_attention_prefill_mfma_kernel(
+__global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ tiles, const int* __restrict__ q_start,
     const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int page_size,
     int num_pages, int window, float scale) {
-    constexpr int KS = DH / 32, NS = (DH + 127) / 128, QD = DH / 4, PSTRIDE = 40;
-    __shared__ __attribute__((aligned(16))) uint16_t p_lds_all[8][16 * PSTRIDE];
+    constexpr int KS = DH / 16;                 // MFMA steps of K Q^T (16 head dimensions each)
+    constexpr int HD = DH / 2;                  // head dimensions owned by one lane half
+    constexpr int DT = DH / 32;                 // tiles of 32 output dimensions
+    constexpr int CPR = DH / 8;                 // 16-byte chunks in a row of K
+    constexpr int NT = PRE_WAVES * 64;
+    constexpr int VS = 40;                      // row stride of Vt in elements: 32 key positions and a pad that spreads the banks
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][32 * DH];      // [key][dimension], chunks swizzled by key
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[2][DH * VS];      // [dimension][key position]
     __shared__ int pages[PRE_TABLE_CAP];
     // the last tiles of a long segment have the most keys: they are started first
     const int tile = gridDim.x - 1 - blockIdx.x;
     const int s = tiles[tile * 4], t0 = tiles[tile * 4 + 1], nrows = tiles[tile * 4 + 2];
     const int kvh = blockIdx.y;
     const int G = nh / nkv;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-    const int g = lane >> 4, c = lane & 15;
-    uint16_t* p_lds = p_lds_all[wave];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hw = blockIdx.z * PRE_WAVES + wave;       // this wave's head within the group
+    const bool active = hw < G;                         // (idle waves still help to fetch and keep the barriers)
+    const int head = kvh * G + (active ? hw : 0);
+    const int ql = lane & 31, h = lane >> 5;
     const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);           // position of the tile's first token
     const int p_last = p0 + nrows - 1;
     const int lo0 = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
     const int k_begin = lo0 & ~31, k_end = p_last + 1;
-    const int first_block = k_begin / page_size;
-    const int nblocks = (k_end - 1) / page_size - first_block + 1;
+    const int first_block = lo0 / page_size;
+    const int nblocks = (k_end - 1) / page_size - first_block + 1;     // <= PRE_TABLE_CAP (checked by the host)
     const int* table = block_table + (size_t)s * max_blocks + first_block;
-    const bool in_lds = nblocks <= PRE_TABLE_CAP;
-    if (in_lds)
-        for (int i = threadIdx.x; i < nblocks; i += blockDim.x) pages[i] = table[i];
+    for (int i = tid; i < nblocks; i += NT) pages[i] = table[i];
     __syncthreads();
-    const u32x4 zero4 = {{0u, 0u, 0u, 0u}};
-    auto row_of = [&](int key, bool& ok) -> size_t {
-        const int blk = key / page_size;
-        const int page = in_lds ? pages[blk - first_block] : table[blk - first_block];
-        ok = page >= 0 && page < num_pages;
-        return (((size_t)(ok ? page : 0) * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
+    // Element offset of a key's row in a cache layer; a key outside the tile's range gives the
+    // nearest key inside it (its scores are masked below).
+    const float inv_page = 1.0f / (float)page_size;
+    auto row_of = [&](int key) -> size_t {
+        key = key < lo0 ? lo0 : (key >= k_end ? k_end - 1 : key);
+        const int blk = (int)(((float)key + 0.5f) * inv_page);       // key / page_size, exact below 2^21 (checked by the host)
+        int page = pages[blk - first_block];
+        page = page < 0 ? 0 : (page >= num_pages ? num_pages - 1 : page);
+        return (((size_t)page * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
     };
-    int prow[4], lrow[4];                       // last and first visible key of this lane's four rows
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int row = 4 * g + r;
-        prow[r] = (row < nrows) ? p0 + row : -1;
-        lrow[r] = (window > 0 && prow[r] - window + 1 > 0) ? prow[r] - window + 1 : 0;
+    // ---- fetching a block of 32 keys.  K: 16-byte chunks tid, tid + NT, ...  V: units of two
+    // neighbouring key positions x 8 dimensions; position p of the key order holds the key
+    // 16 (p / 16) + 4 ((p / 8) % 2) + (p % 8 < 4 ? p % 8 : p % 8 + 4).
+    constexpr int KCH = (32 * CPR + NT - 1) / NT;
+    constexpr int VU = 16 * CPR, VCH = (VU + NT - 1) / NT;
+    u32x4 kreg[KCH], vreg[VCH][2];
+#define LI_PRE_FETCH(kb)                                                                             \
+    {                                                                                                \
+        _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                            \
+            int ch = tid + i * NT;                                                                   \
+            ch = ch < 32 * CPR ? ch : 32 * CPR - 1;                                                  \
+            const size_t off = row_of((kb) + ch / CPR);                                               \
+            kreg[i] = *reinterpret_cast<const u32x4*>(kc + off + 8 * (ch % CPR));                    \
+        }                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                            \
+            int u = tid + i * NT;                                                                    \
+            u = u < VU ? u : VU - 1;                                                                 \
+            const int dg = (u & 3) + 4 * (u >> 6), pp = (u >> 2) & 15, pc = pp >> 2, ip = 2 * (pp & 3); \
+            const int key = (kb) + 16 * (pc >> 1) + 4 * (pc & 1) + (ip < 4 ? ip : ip + 4);           \
+            const size_t o0 = row_of(key), o1 = row_of(key + 1);                                     \
+            vreg[i][0] = *reinterpret_cast<const u32x4*>(vc + o0 + 8 * dg);                          \
+            vreg[i][1] = *reinterpret_cast<const u32x4*>(vc + o1 + 8 * dg);                          \
+        }                                                                                            \
     }
+#define LI_PRE_STASH(stage)                                                                          \
+    {                                                                                                \
+        _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                            \
+            const int ch = tid + i * NT;                                                             \
+            if (ch < 32 * CPR) {                                                                     \
+                const int key = ch / CPR, c = ch % CPR;                                              \
+                *reinterpret_cast<u32x4*>(&Ks[stage][key * DH + ((c ^ (key & (CPR - 1))) << 3)]) =   \
+                    kreg[i];                                                                         \
+            }                                                                                        \
+        }                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                            \
+            const int u = tid + i * NT;                                                              \
+            if (u < VU) {                                                                            \
+                const int dg = (u & 3) + 4 * (u >> 6), pp = (u >> 2) & 15;                           \
+                const u32x4 v0 = vreg[i][0], v1 = vreg[i][1];                                        \
+                _Pragma("unroll") for (int jj = 0; jj < 8; ++jj)                                     \
+                    *reinterpret_cast<uint32_t*>(&Vt[stage][(8 * dg + jj) * VS + 2 * pp]) =          \
+                        __builtin_amdgcn_perm(v1.w[jj >> 1], v0.w[jj >> 1], (jj & 1) ? 0x07060302u : 0x05040100u); \
+            }                                                                                        \
+        }                                                                                            \
+    }
+    // ---- this wave's queries
+    frag8 qf[KS];
+    {
+        const bf16_t* qrow = q + (size_t)(t0 + (ql < nrows ? ql : nrows - 1)) * q_row_stride + (size_t)head * DH + HD * h;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) qf[st].raw = *reinterpret_cast<const u32x4*>(qrow + 8 * st);
+    }
+    const int pq = (ql < nrows) ? p0 + ql : -1;                              // last visible key of this lane's query
+    const int lq = (window > 0 && pq - window + 1 > 0) ? pq - window + 1 : 0;
+    const float scale2 = scale * 1.44269504088896341f;                       // scores in units of log 2
+    f32x16_t acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
 
-    for (int hw = wave; hw < G; hw += nwaves) {
-        const int head = kvh * G + hw;
-        frag8 qa[KS];
+    LI_PRE_FETCH(k_begin);
+    LI_PRE_STASH(0);
+    __syncthreads();
+    int stage = 0;
+    for (int kb = k_begin; kb < k_end; kb += 32, stage ^= 1) {
+        const bool more = kb + 32 < k_end;
+        if (more) LI_PRE_FETCH(kb + 32);              // in flight while this block is worked on
+        if (active) {
+            // ---- S^T = K Q^T
+            f32x16_t sv;
 #pragma unroll
-        for (int j = 0; j < KS; ++j)
-            qa[j].raw = (c < nrows) ? *reinterpret_cast<const u32x4*>(
-                            q + (size_t)(t0 + c) * q_row_stride + (size_t)head * DH + QD * g + 8 * j) : zero4;
-        f32x4_t acc[NS][8];
+            for (int r = 0; r < 16; ++r) sv[r] = 0.f;
 #pragma unroll
-        for (int ns = 0; ns < NS; ++ns)
-#pragma unroll
-            for (int jj = 0; jj < 8; ++jj) acc[ns][jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
-        frag8 kf[2][KS];
-        bool kok[2];
-        auto load_k = [&](int kb) {
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const int key = kb + 16 * tt + c;
-                kok[tt] = key < k_end && key >= lo0;
-                size_t off = 0;
-                if (kok[tt]) off = row_of(key, kok[tt]);
-#pragma unroll
-                for (int j = 0; j < KS; ++j)
-                    kf[tt][j].raw = kok[tt] ? *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j) : zero4;
+            for (int st = 0; st < KS; ++st) {
+                frag8 kf;
+                const int c = (HD / 8) * h + st;
+                kf.raw = *reinterpret_cast<const u32x4*>(&Ks[stage][ql * DH + ((c ^ (ql & (CPR - 1))) << 3)]);
+                sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[st].v, sv, 0, 0, 0);
             }
-        };
-        load_k(k_begin);
-        for (int kb = k_begin; kb < k_end; kb += 32) {
-            u32x4 vraw[NS][8];
+            // ---- softmax over the keys of this lane's query.  The running maximum m is only moved
+            // (and the sums so far rescaled, for the whole wave) when some query's scores pass it by
+            // more than 2^8: until then the exponentials are taken against the older maximum, which
+            // changes no result (numerator and denominator carry the same factor) and stays far
+            // inside the range of float and bfloat16.
+            float mx = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int key = kb + 8 * g + i;
-                bool ok = key < k_end && key >= lo0;
-                size_t off = 0;
-                if (ok) off = row_of(key, ok);
-#pragma unroll
-                for (int ns = 0; ns < NS; ++ns) {
-                    const int d = 128 * ns + 8 * c;
-                    vraw[ns][i] = (ok && d < DH) ? *reinterpret_cast<const u32x4*>(vc + off + d) : zero4;
-                }
+            for (int r = 0; r < 16; ++r) {
+                const int key = kb + 8 * (r >> 2) + 4 * h + (r & 3);
+                sv[r] = (key <= pq && key >= lq) ? sv[r] * scale2 : -INFINITY;
+                mx = fmaxf(mx, sv[r]);
             }
-            f32x4_t sv[2];
-            const bool sok[2] = {kok[0], kok[1]};
+            mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
+            if (__any(mx > m + 8.0f)) {
+                const float mn = fmaxf(m, mx);
+                const float alpha = (mn == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - mn);   // (m = -inf: nothing summed yet)
+                l *= alpha;
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int j = 0; j < KS; ++j)
-                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0);
+                    for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
+                m = mn;
             }
-            if (kb + 32 < k_end) load_k(kb + 32);
-            float alpha[4], pr[2][4];
-            const int key0 = kb + c, key1 = kb + 16 + c;
+            const float ms = (m == -INFINITY) ? 0.f : m;         // a query may see no key yet
+            float ps = 0.f;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float s0 = (sok[0] && key0 <= prow[r] && key0 >= lrow[r]) ? sv[0][r] * scale : -INFINITY;
-                const float s1 = (sok[1] && key1 <= prow[r] && key1 >= lrow[r]) ? sv[1][r] * scale : -INFINITY;
-                const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));
-                const float ms = (mx == -INFINITY) ? 0.f : mx;       // a row may see no key yet
-                alpha[r] = expf(m[r] - ms);
-                pr[0][r] = expf(s0 - ms);
-                pr[1][r] = expf(s1 - ms);
-                l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];
-                m[r] = mx;
-            }
-            // P through this wave's own piece of LDS: a wave's LDS operations run in order
-            __builtin_amdgcn_wave_barrier();
+            for (int r = 0; r < 16; ++r) { sv[r] = __builtin_amdgcn_exp2f(sv[r] - ms); ps += sv[r]; }
+            l += ps;
+            frag8 pf[2];
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
+            for (int st = 0; st < 2; ++st)
 #pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = float_to_bf16(pr[tt][r]);
-            __builtin_amdgcn_wave_barrier();
-            frag8 pa;
-            pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);
-            __builtin_amdgcn_wave_barrier();
+                for (int i = 0; i < 4; ++i) pf[st].raw.w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
+            // ---- O^T += V^T P^T
 #pragma unroll
-            for (int ns = 0; ns < NS; ++ns) {
+            for (int dt = 0; dt < DT; ++dt) {
+                const int d = 32 * dt + ql;
 #pragma unroll
-                for (int jj = 0; jj < 8; ++jj) {
+                for (int st = 0; st < 2; ++st) {
                     frag8 vf;
-#pragma unroll
-                    for (int ii = 0; ii < 4; ++ii)
-                        vf.raw.w[ii] = __builtin_amdgcn_perm(vraw[ns][2 * ii + 1].w[jj >> 1], vraw[ns][2 * ii].w[jj >> 1],
-                                                             (jj & 1) ? 0x07060302u : 0x05040100u);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[ns][jj][r] *= alpha[r];
-                    acc[ns][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vf.v, acc[ns][jj], 0, 0, 0);
+                    vf.raw = *reinterpret_cast<const u32x4*>(&Vt[stage][d * VS + ((2 * st + h) << 3)]);
+                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
                 }
             }
         }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float lt = row16_sum(l[r]);
-            const int row = 4 * g + r;
-            if (row >= nrows) continue;
-            const float inv = lt != 0.f ? 1.0f / lt : 0.f;
-            bf16_t* orow = out + (size_t)(t0 + row) * nh * DH + (size_t)head * DH;
-#pragma unroll
-            for (int ns = 0; ns < NS; ++ns) {
-                const int d = 128 * ns + 8 * c;
-                if (d < DH) {
-                    u32x4 o;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        o.w[i] = (uint32_t)float_to_bf16(acc[ns][2 * i][r] * inv) |
-                                 ((uint32_t)float_to_bf16(acc[ns][2 * i + 1][r] * inv) << 16);
-                    *reinterpret_cast<u32x4*>(orow + d) = o;
-                }
-            }
-        }
+        if (more) LI_PRE_STASH(stage ^ 1);
+        __syncthreads();
     }
+    if (!active || ql >= nrows) return;
+    l += __shfl_xor(l, 32, LI_WAVE);               // (both halves of a query are past the return together)
+    const float inv = l != 0.f ? 1.0f / l : 0.f;
+    bf16_t* orow = out + (size_t)(t0 + ql) * nh * DH + (size_t)head * DH;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {           // registers 4 rg .. 4 rg + 3: dimensions 32 dt + 8 rg + 4 h ..
+            uint32_t w0 = pack2_bf16(acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv);
+            uint32_t w1 = pack2_bf16(acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv);
+            uint32_t* dst = reinterpret_cast<uint32_t*>(orow + 32 * dt + 8 * rg + 4 * h);
+            dst[0] = w0;
+            dst[1] = w1;
+        }
 }
 
-// tiles: int [ntiles, 4] = (segment, first token of the tile in the batch, rows <= 16, unused)
+// tiles: int [ntiles, 4] = (segment, first token of the tile in the batch, rows <= 32, unused)
 extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void* out, const void* kc,
                                           const void* vc, const int* block_table, int max_blocks,
                                           const int* tiles, int ntiles, const int* q_start, const int* q_len,
                                           const int* ctx_len, int nh, int nkv, int dh, int page_size,
                                           int num_pages, int window, float scale, hipStream_t stream) {
-    if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || page_size <= 0 || max_blocks <= 0)
+    if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || page_size <= 0 || max_blocks <= 0 ||
+        max_blocks > PRE_TABLE_CAP || (long long)max_blocks * page_size > (1ll << 21))
         return LI_ERR_SIZE;
     const int G = nh / nkv;
-    const int waves = G < 8 ? G : 8;        // more heads than waves: a wave takes several in turn
-    dim3 grid(ntiles, nkv);
-#define LI_PRE(DHV) paged_attention_prefill_mfma_kernel<DHV><<<grid, waves * 64, 0, stream>>>( \
+    const int parts = (G + PRE_WAVES - 1) / PRE_WAVES;
+    if (parts > 65535) return LI_ERR_SIZE;
+    dim3 grid(ntiles, nkv, parts);
+#define LI_PRE(DHV) paged_attention_prefill_mfma_kernel<DHV><<<grid, PRE_WAVES * 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
         tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale)
     if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
 #undef LI_PRE
+#undef LI_PRE_FETCH
+#undef LI_PRE_STASH
     return li_launch_status();
 }
 

@@ -20,12 +20,16 @@ __device__ __forceinline__ float bf16_to_float(uint16_t b) {
     return __uint_as_float(((uint32_t)b) << 16);
 }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN (v_cvt_pk_bf16_f32, one instruction for one or two values)
 __device__ __forceinline__ uint16_t float_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+
+typedef __bf16 li_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float li_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {      // lo in bits 0..15
+    li_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, li_bf16x2));
 }
 
 __device__ __forceinline__ float load_as_float(const float* p) { return *p; }

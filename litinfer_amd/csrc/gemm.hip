@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
                         chunk16 o;
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
-                            o.w[e] = (uint32_t)float_to_bf16(v[2 * e]) | ((uint32_t)float_to_bf16(v[2 * e + 1]) << 16);
+                            o.w[e] = pack2_bf16(v[2 * e], v[2 * e + 1]);
                         *reinterpret_cast<chunk16*>(reinterpret_cast<uint16_t*>(out) + idx) = o;
                     }
                 } else {
@@ -505,7 +505,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                     chunk16 o;
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
-                        o.w[e] = (uint32_t)float_to_bf16(v[2 * e]) | ((uint32_t)float_to_bf16(v[2 * e + 1]) << 16);
+                        o.w[e] = pack2_bf16(v[2 * e], v[2 * e + 1]);
                     *reinterpret_cast<chunk16*>(reinterpret_cast<uint16_t*>(out) + o_idx) = o;
                 }
             } else {

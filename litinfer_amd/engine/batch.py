@@ -47,7 +47,7 @@ class AttentionMeta:
     num_single: int = 0
     multi_tokens: Optional[torch.Tensor] = None
     num_multi: int = 0
-    # the tokens of segments with several tokens, cut into tiles of up to 16 consecutive tokens
+    # the tokens of segments with several tokens, cut into tiles of up to 32 consecutive tokens
     # of one segment: int32 [tiles, 4] = (segment, first token, tokens, 0)
     tiles: Optional[torch.Tensor] = None
     num_tiles: int = 0
@@ -160,8 +160,8 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     single_mask = q_len[seg_of_token] == 1
     single = np.nonzero(single_mask)[0].astype(np.int32)
     multi = np.nonzero(~single_mask)[0].astype(np.int32)
-    tile_rows = [(i, int(q_start[i]) + a, min(16, int(q_len[i]) - a), 0)
-                 for i in range(nseg) if q_len[i] > 1 for a in range(0, int(q_len[i]), 16)]
+    tile_rows = [(i, int(q_start[i]) + a, min(32, int(q_len[i]) - a), 0)
+                 for i in range(nseg) if q_len[i] > 1 for a in range(0, int(q_len[i]), 32)]
     tiles = np.asarray(tile_rows, dtype=np.int32).reshape(-1, 4)
     parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows, single, multi, tiles]
     tables, max_blocks = [], []

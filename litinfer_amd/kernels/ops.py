@@ -356,7 +356,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
              meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              0 if acc is None else acc.data_ptr(), 0 if ml is None else ml.data_ptr(),
              nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit, int(mfma))
-    if n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles and n_multi == meta.num_multi:
+    # the matrix-core kernel for portions keeps a tile's pages in LDS (8192 entries) and divides
+    # positions by the page size in float, exact below 2^21 keys; longer tables take the general kernel
+    if (n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles
+            and n_multi == meta.num_multi and meta.max_blocks <= 8192 and meta.max_blocks * page_size <= 1 << 21):
         _run("attention", "li_paged_attention_prefill", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), bt.data_ptr(), meta.max_blocks, meta.tiles.data_ptr(),
              meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),

@@ -212,10 +212,10 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
                          host_q_start=q_start, host_q_len=q_len, host_ctx_len=ctx_len,
                          single_tokens=dev(single) if len(multi) else None, num_single=len(single),
                          multi_tokens=dev(multi) if len(single) else None, num_multi=len(multi),
-                         tiles=dev(np.asarray([(i, int(q_start[i]) + a, min(16, int(q_len[i]) - a), 0)
+                         tiles=dev(np.asarray([(i, int(q_start[i]) + a, min(32, int(q_len[i]) - a), 0)
                                                for i in range(nseg) if q_len[i] > 1
-                                               for a in range(0, int(q_len[i]), 16)], dtype=np.int32).reshape(-1, 4)),
-                         num_tiles=sum(-(-int(n) // 16) for n in q_len if n > 1),
+                                               for a in range(0, int(q_len[i]), 32)], dtype=np.int32).reshape(-1, 4)),
+                         num_tiles=sum(-(-int(n) // 32) for n in q_len if n > 1),
                          max_single_ctx=int(ctx_len[q_len == 1].max()) if len(single) else 0)
     out = torch.empty(T, nh * dh, dtype=dtype, device=DEV)
     scale = 1.0 / math.sqrt(dh)
