@@ -646,8 +646,9 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
 #pragma unroll
         for (int st = 0; st < KS; ++st) qf[st].raw = *reinterpret_cast<const u32x4*>(qrow + 8 * st);
     }
-    const int pq = (ql < nrows) ? p0 + ql : -1;                              // last visible key of this lane's query
+    const int pq = p0 + (ql < nrows ? ql : nrows - 1);       // last visible key of this lane's query (lanes past the tile repeat its last row)
     const int lq = (window > 0 && pq - window + 1 > 0) ? pq - window + 1 : 0;
+    const int l_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
     const float scale2 = scale * 1.44269504088896341f;                       // scores in units of log 2
     f32x16_t acc[DT];
 #pragma unroll
@@ -680,14 +681,18 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
             // more than 2^8: until then the exponentials are taken against the older maximum, which
             // changes no result (numerator and denominator carry the same factor) and stays far
             // inside the range of float and bfloat16.
-            float mx = -INFINITY;
+            // A block that every query of the tile sees whole (most are) needs no masks.
+            if (!(kb + 31 <= p0 && kb >= l_last)) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int key = kb + 8 * (r >> 2) + 4 * h + (r & 3);
-                sv[r] = (key <= pq && key >= lq) ? sv[r] * scale2 : -INFINITY;
-                mx = fmaxf(mx, sv[r]);
+                for (int r = 0; r < 16; ++r) {
+                    const int key = kb + 8 * (r >> 2) + 4 * h + (r & 3);
+                    sv[r] = (key <= pq && key >= lq) ? sv[r] : -INFINITY;
+                }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
+            float mx = fmaxf(sv[0], sv[1]);
+#pragma unroll
+            for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(sv[r], sv[r + 1]));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE)) * scale2;       // (scale2 > 0)
             if (__any(mx > m + 8.0f)) {
                 const float mn = fmaxf(m, mx);
                 const float alpha = (mn == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - mn);   // (m = -inf: nothing summed yet)
@@ -701,7 +706,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
             const float ms = (m == -INFINITY) ? 0.f : m;         // a query may see no key yet
             float ps = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) { sv[r] = __builtin_amdgcn_exp2f(sv[r] - ms); ps += sv[r]; }
+            for (int r = 0; r < 16; ++r) { sv[r] = __builtin_amdgcn_exp2f(fmaf(sv[r], scale2, -ms)); ps += sv[r]; }
             l += ps;
             frag8 pf[2];
 #pragma unroll
@@ -746,7 +751,7 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
                                           const int* ctx_len, int nh, int nkv, int dh, int page_size,
                                           int num_pages, int window, float scale, hipStream_t stream) {
     if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || page_size <= 0 || max_blocks <= 0 ||
-        max_blocks > PRE_TABLE_CAP || (long long)max_blocks * page_size > (1ll << 21))
+        max_blocks > PRE_TABLE_CAP || (long long)max_blocks * page_size > (1ll << 21) || !(scale > 0.f))
         return LI_ERR_SIZE;
     const int G = nh / nkv;
     const int parts = (G + PRE_WAVES - 1) / PRE_WAVES;

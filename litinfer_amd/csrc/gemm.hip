@@ -358,23 +358,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
 // ------------------------------- bfloat16, many rows, loads straight into LDS
 // The same tiling with the global loads going straight into LDS
 // (global_load_lds_dwordx4: lane i's 16 bytes land at the wave's LDS base + 16 i),
-// which needs no staging registers, so DMA_STAGES - 1 steps of K are in flight
-// while one is multiplied: the latency of a load is several steps long.  The
+// which needs no staging registers, so all stages but the one being multiplied are
+// in flight: the latency of a load is long against a step.  The
 // compiler does not track these loads' completion; `s_waitcnt vmcnt(n)` is
 // placed by hand: a wave's loads retire in order, so allowing the loads of the
 // younger steps to stay outstanding waits exactly for the oldest step, and the
 // barrier after it makes that true for the loads of all four waves.
-// Needs K to be a multiple of the step (a load cannot be masked to zeros).  Tiles: 256 x 256
-// with steps of 32 (each operand byte read from LDS feeds twice the multiply-adds of the
-// 128 x 128 tile, which is bound by LDS bandwidth), or 128 x 128 with steps of 64 where the
-// larger tile would leave compute units without a block.
-#define DMA_STAGES 4
+// Needs K to be a multiple of the step (a load cannot be masked to zeros).  A step is 64
+// columns, so that a row of a stage is one whole 128-byte line of the caches.  Tiles: 256 x 256
+// with two stages, 256 x 128 with three, 128 x 128 with four (what fits the 160 KB of LDS).
 #define LI_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 #define LI_LOAD_TO_LDS(gptr, lptr)                                                                        \
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),              \
                                      (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
-template <int BM, int BN, int BK, typename TO>
+template <int BM, int BN, int BK, int NSTAGE, typename TO>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x,
                                                              const bf16_t* __restrict__ w,
                                                              const float* __restrict__ bias,
@@ -420,7 +418,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
         gb[i] = w + (size_t)((n0 + row < N) ? n0 + row : N - 1) * K + 8 * c;
     }
     auto issue = [&](int kt) {
-        uint16_t* st = lds + (kt % DMA_STAGES) * STAGE;
+        uint16_t* st = lds + (kt % NSTAGE) * STAGE;
 #pragma unroll
         for (int i = 0; i < IA; ++i) LI_LOAD_TO_LDS(ga[i] + (size_t)kt * BK, st + ((BM / 4) * wave + RPI * i) * BK);
 #pragma unroll
@@ -428,40 +426,68 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     };
     const int frow = lane & 31, fh = lane >> 5;
     const int nk = K / BK;
+    constexpr int KS = BK / 16;                    // MFMA steps of a stage (even)
+    // Order of a step: the MFMAs of stage kt run while the fragments of its next 16 columns are
+    // read; in the middle of the stage's LAST 16 columns the wave waits for stage kt + 1 (loaded
+    // long before), meets the others at the barrier, starts the load of stage kt + NSTAGE into
+    // the stage all waves have just finished reading, and reads the first fragments of stage
+    // kt + 1, so that the barrier and the latency of LDS fall under the remaining MFMAs.
 #pragma unroll
-    for (int p = 0; p < DMA_STAGES - 1; ++p)
+    for (int p = 0; p < NSTAGE; ++p)
         if (p < nk) issue(p);
-    for (int kt = 0; kt < nk; ++kt) {
-        // loads of the steps after kt that this wave has issued: at most DMA_STAGES - 2 steps here
-        const int younger = (nk - 1 - kt < DMA_STAGES - 2) ? nk - 1 - kt : DMA_STAGES - 2;
-        if (younger >= 2) LI_VMCNT(2 * LPW); else if (younger == 1) LI_VMCNT(LPW); else LI_VMCNT(0);
-        __builtin_amdgcn_s_barrier();              // step kt is in LDS for all waves; step kt - 1 is read by all
-        asm volatile("" ::: "memory");
-        if (kt + DMA_STAGES - 1 < nk) issue(kt + DMA_STAGES - 1);      // into the stage step kt - 1 was in
-        const uint16_t* As = lds + (kt % DMA_STAGES) * STAGE;
-        const uint16_t* Bs = As + BM * BK;
-        bf16x8 af[2][TM], bfr[2][TN];
-#define LI_FREAD(ks, buf)                                                                                  \
+    bf16x8 af[2][TM], bfr[2][TN];
+#define LI_FREAD(stage_, ks, buf)                                                                          \
     {                                                                                                     \
+        const uint16_t* As_ = lds + (stage_) * STAGE;                                                     \
+        const uint16_t* Bs_ = As_ + BM * BK;                                                              \
         const int c_ = 2 * (ks) + fh;                                                                     \
         _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                    \
-            af[buf][i] = *reinterpret_cast<const bf16x8*>(&As[slot(wm + 32 * i + frow, c_)]);             \
+            af[buf][i] = *reinterpret_cast<const bf16x8*>(&As_[slot(wm + 32 * i + frow, c_)]);            \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                    \
-            bfr[buf][j] = *reinterpret_cast<const bf16x8*>(&Bs[slot(wn + 32 * j + frow, c_)]);            \
+            bfr[buf][j] = *reinterpret_cast<const bf16x8*>(&Bs_[slot(wn + 32 * j + frow, c_)]);           \
     }
-        LI_FREAD(0, 0)
+#define LI_WAIT_YOUNGER(y)                                                                                 \
+    { if ((y) >= 3) LI_VMCNT(3 * LPW); else if ((y) == 2) LI_VMCNT(2 * LPW); else if ((y) == 1) LI_VMCNT(LPW); else LI_VMCNT(0); }
+    {
+        const int younger = nk - 1 < NSTAGE - 1 ? nk - 1 : NSTAGE - 1;     // loads of later stages in flight
+        LI_WAIT_YOUNGER(younger)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        LI_FREAD(0, 0, 0)
+    }
+    for (int kt = 0; kt < nk; ++kt) {
+        const int stage = kt % NSTAGE;
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            if (ks + 1 < BK / 16) LI_FREAD(ks + 1, (ks + 1) & 1)
+        for (int ks = 0; ks < KS - 1; ++ks) {
+            LI_FREAD(stage, ks + 1, (ks + 1) & 1)
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
         }
-#undef LI_FREAD
-        asm volatile("" ::: "memory");
+        constexpr int BL = (KS - 1) & 1;           // = 1: the fragments of the last 16 columns
+#pragma unroll
+        for (int i = 0; i < TM / 2; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][i], bfr[BL][j], acc[i][j], 0, 0, 0);
+        if (kt + 1 < nk) {
+            const int younger = nk - 2 - kt < NSTAGE - 2 ? nk - 2 - kt : NSTAGE - 2;
+            LI_WAIT_YOUNGER(younger)
+            __builtin_amdgcn_s_barrier();          // stage kt + 1 is in LDS for all waves; stage kt is read by all
+            asm volatile("" ::: "memory");
+            if (kt + NSTAGE < nk) issue(kt + NSTAGE);          // into the stage of step kt
+            LI_FREAD((kt + 1) % NSTAGE, 0, 0)
+        }
+#pragma unroll
+        for (int i = TM / 2; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][i], bfr[BL][j], acc[i][j], 0, 0, 0);
     }
+#undef LI_FREAD
+#undef LI_WAIT_YOUNGER
     __syncthreads();                               // the main loop's LDS is free now
     constexpr int ESTRIDE = WN + 4;
     float* band = reinterpret_cast<float*>(lds) + wave * 32 * ESTRIDE;
@@ -517,22 +543,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     }
 }
 
-template <int BM, int BN, int BK, typename TO>
+template <int BM, int BN, int BK, int NSTAGE, typename TO>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
     const long gn = mtiles >= 32 ? 1 : 32 / mtiles;
     const long per_xcd = ((ntiles + 7) / 8 + gn - 1) / gn * gn * mtiles;
     if (per_xcd * 8 > 0x7fffffffL) return LI_ERR_SIZE;
-    constexpr int lds_bytes = DMA_STAGES * (BM + BN) * BK * 2;
+    constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, BK, TO>,
+        if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, TO>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
             return LI_ERR_LAUNCH;
         configured = true;
     }
-    gemm_bf16_dma_kernel<BM, BN, BK, TO><<<dim3((unsigned)(per_xcd * 8)), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
+    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, TO><<<dim3((unsigned)(per_xcd * 8)), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
     return li_launch_status();
 }
 
@@ -779,13 +805,20 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
 #define LI_BIG(BM, BN, BK) (out_dtype == LI_F32 ? launch_big<BM, BN, BK, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                             : launch_big<BM, BN, BK, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
             if (out_dtype != LI_F32 && out_dtype != LI_BF16) return LI_ERR_DTYPE;
-#define LI_DMA(BM, BN, BK) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
-                                               : launch_dma<BM, BN, BK, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
-            // measured at the 7B layer sizes: 256 x 256 tiles win where they still give every
-            // compute unit two blocks' worth of work, 128 x 128 tiles elsewhere and for fewer rows
-            if (K % 64 == 0 && K >= 64 * DMA_STAGES) {
-                if (blocks256 >= 512) return LI_DMA(256, 256, 32);
-                return LI_DMA(128, 128, 64);
+#define LI_DMA(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
+                                               : launch_dma<BM, BN, BK, NS, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
+            // Three tilings; the one with the least (rounds of blocks over the 256 compute units) x
+            // (area of a tile) / (its measured relative speed) is taken: large tiles are the fastest
+            // per multiply-add but leave compute units idle when the matrix has few of them.
+            if (K % 64 == 0) {
+                auto cost = [&](int bm, int bn, double speed) {
+                    const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+                    return (double)((tiles + 255) / 256) * bm * bn / speed;
+                };
+                const double c_large = cost(256, 256, 1.0), c_mid = cost(256, 128, 0.95), c_small = cost(128, 128, 0.8);
+                if (c_large <= c_mid && c_large <= c_small) return LI_DMA(256, 256, 64, 2);
+                if (c_mid <= c_small) return LI_DMA(256, 128, 64, 3);
+                return LI_DMA(128, 128, 64, 4);
             }
 #undef LI_DMA
             return LI_BIG(128, 128, 64);             // K not a multiple of 64: loads staged in registers

@@ -28,6 +28,11 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-result"]          # no fast-math: the 32-bit path needs exact expf/sinf/cosf
 
+# The attention kernels multiply their matrix-core accumulators by the softmax's rescaling factors:
+# with the accumulators in ordinary vector registers this needs no copies to and from the
+# accumulation registers (and fewer registers in all).
+MODULE_FLAGS = {"attention": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
 MODULES = ("elementwise", "gemm", "attention", "sampling")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -55,7 +60,7 @@ def _digest(module: str) -> str:
     for p in [CSRC / f"{module}.hip", *_headers()]:
         h.update(p.name.encode())
         h.update(p.read_bytes())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + MODULE_FLAGS.get(module, [])).encode())
     return h.hexdigest()[:16]
 
 
@@ -109,7 +114,7 @@ def compile_module(module: str, verbose: bool = True) -> Path:
     out_dir = _writable_dir()
     out = out_dir / lib_name(module)
     tmp = out_dir / f".{out.name}.{os.getpid()}.tmp"
-    cmd = [_hipcc(), *FLAGS, f"-I{CSRC}", str(src), "-o", str(tmp)]
+    cmd = [_hipcc(), *FLAGS, *MODULE_FLAGS.get(module, []), f"-I{CSRC}", str(src), "-o", str(tmp)]
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())     # hipcc wants a HOME it can look into
     t0 = time.time()
