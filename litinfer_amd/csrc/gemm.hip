@@ -372,7 +372,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),              \
                                      (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
-template <int BM, int BN, int BK, int NSTAGE, typename TO>
+template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x,
                                                              const bf16_t* __restrict__ w,
                                                              const float* __restrict__ bias,
@@ -415,7 +415,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #pragma unroll
     for (int i = 0; i < IB; ++i) {
         const int row = (BN / 4) * wave + RPI * i + lane / CPR, c = (lane % CPR) ^ ((row / WRAP) & (CPR - 1));
-        gb[i] = w + (size_t)((n0 + row < N) ? n0 + row : N - 1) * K + 8 * c;
+        int wrow = n0 + row;
+        if constexpr (SWIGLU) {
+            // w is [gate; up] with N / 2 rows each.  The tile's rows alternate in blocks of 32: 32
+            // gate rows, the 32 up rows of the same outputs, the next 32 gate rows, ..., so that an
+            // accumulator tile and its neighbour hold the two factors of one output tile.
+            const int half = N / 2, blk = row / 32;
+            const int o = n0 / 2 + (blk / 2) * 32 + row % 32;
+            wrow = (o < half ? o : half - 1) + (blk & 1) * half;
+        }
+        gb[i] = w + (size_t)(wrow < N ? wrow : N - 1) * K + 8 * c;
     }
     auto issue = [&](int kt) {
         uint16_t* st = lds + (kt % NSTAGE) * STAGE;
@@ -489,31 +498,43 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #undef LI_FREAD
 #undef LI_WAIT_YOUNGER
     __syncthreads();                               // the main loop's LDS is free now
-    constexpr int ESTRIDE = WN + 4;
+    constexpr int EW = SWIGLU ? WN / 2 : WN;        // output columns of a wave
+    constexpr int ESTRIDE = EW + 4;
     float* band = reinterpret_cast<float*>(lds) + wave * 32 * ESTRIDE;
     const int ccol = lane & 31, crow = (lane >> 5) * 4;
-    constexpr int LPR = WN / 8, RPP = 64 / LPR;
+    constexpr int LPR = EW / 8, RPP = 64 / LPR;
     const int erow = lane / LPR, ecol = (lane % LPR) * 8;
+    const int NO = SWIGLU ? N / 2 : N;             // columns of out
+    const int col = (SWIGLU ? (n0 + wn) / 2 : n0 + wn) + ecol;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         __builtin_amdgcn_wave_barrier();
+        if constexpr (SWIGLU) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+            for (int j = 0; j < TN; j += 2)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 32 * j + ccol] = acc[i][j][r];
+                for (int r = 0; r < 16; ++r) {
+                    const float gv = acc[i][j][r], uv = acc[i][j + 1][r];
+                    band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 16 * j + ccol] = uv * (gv / (1.0f + expf(-gv)));
+                }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 32 * j + ccol] = acc[i][j][r];
+        }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int pass = 0; pass < 32 / RPP; ++pass) {
             const int row = m0 + wm + 32 * i + RPP * pass + erow;
-            const int col = n0 + wn + ecol;
-            if (row >= M || col >= N) continue;
+            if (row >= M || col >= NO) continue;
             const float* src = &band[(RPP * pass + erow) * ESTRIDE + ecol];
             float v[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = src[e];
-            const size_t o_idx = (size_t)row * N + col;
-            if (col + 8 <= N && (N % 8) == 0) {
+            const size_t o_idx = (size_t)row * NO + col;
+            if (col + 8 <= NO && (NO % 8) == 0) {
                 if (bias) {
 #pragma unroll
                     for (int e = 0; e < 8; ++e) v[e] += bias[col + e];
@@ -537,13 +558,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    if (col + e < N) epilogue_store(out, o_idx + e, v[e], bias, col + e, accumulate);
+                    if (col + e < NO) epilogue_store(out, o_idx + e, v[e], bias, col + e, accumulate);
             }
         }
     }
 }
 
-template <int BM, int BN, int BK, int NSTAGE, typename TO>
+template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
@@ -553,12 +574,12 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
     constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, TO>,
+        if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
             return LI_ERR_LAUNCH;
         configured = true;
     }
-    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, TO><<<dim3((unsigned)(per_xcd * 8)), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
+    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO><<<dim3((unsigned)(per_xcd * 8)), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
     return li_launch_status();
 }
 
@@ -800,13 +821,11 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         if (aligned && M <= 64)
             return li_linear_skinny(x, w, bias, out, M, N, K, out_dtype, accumulate, 0, stream);
         if (aligned && M > 64) {
-            // the largest tile that still gives every compute unit a block
-            const long blocks256 = (long)((N + 255) / 256) * ((M + 255) / 256);
 #define LI_BIG(BM, BN, BK) (out_dtype == LI_F32 ? launch_big<BM, BN, BK, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                             : launch_big<BM, BN, BK, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
             if (out_dtype != LI_F32 && out_dtype != LI_BF16) return LI_ERR_DTYPE;
-#define LI_DMA(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
-                                               : launch_dma<BM, BN, BK, NS, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
+#define LI_DMA(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, false, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
+                                               : launch_dma<BM, BN, BK, NS, false, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
             // Three tilings; the one with the least (rounds of blocks over the 256 compute units) x
             // (area of a tile) / (its measured relative speed) is taken: large tiles are the fastest
             // per multiply-add but leave compute units idle when the matrix has few of them.
@@ -831,4 +850,25 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
 #undef LI_GEMM
     } else return LI_ERR_DTYPE;
     return li_launch_status();
+}
+
+// out[m, n] = up * gate / (1 + exp(-gate)) with [gate, up] = x w^T, w = [gate; up] of I rows each:
+// the activation as the product's epilogue, so the 2 I columns never go to memory.  bfloat16;
+// K a multiple of 8 for up to 64 rows, a multiple of 64 above.
+extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, int I, int K,
+                                hipStream_t stream) {
+    if (M <= 0 || I <= 0 || K <= 0 || I > 0x3fffffff) return LI_ERR_SIZE;
+    if (M <= 64) return li_linear_skinny(x, w, nullptr, out, M, I, K, LI_BF16, 0, 1, stream);
+    if (K % 64) return LI_ERR_SIZE;
+    const int N = 2 * I;
+    auto cost = [&](int bm, int bn, double speed) {
+        const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+        return (double)((tiles + 255) / 256) * bm * bn / speed;
+    };
+#define LI_DMA(BM, BN, BK, NS) launch_dma<BM, BN, BK, NS, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream)
+    const double c_large = cost(256, 256, 1.0), c_mid = cost(256, 128, 0.95), c_small = cost(128, 128, 0.8);
+    if (c_large <= c_mid && c_large <= c_small) return LI_DMA(256, 256, 64, 2);
+    if (c_mid <= c_small) return LI_DMA(256, 128, 64, 3);
+    return LI_DMA(128, 128, 64, 4);
+#undef LI_DMA
 }

@@ -37,6 +37,7 @@ _SIGNATURES = {
     "gemm": {
         "li_linear": [P, P, P, P, I, I, I, I, I, I],
         "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
+        "li_linear_swiglu": [P, P, P, I, I, I],
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
@@ -291,6 +292,25 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
          "linear_skinny: bias must be float32 [N]")
     _run("gemm", "li_linear_skinny", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
          out.data_ptr(), m, n, k, _DT[out.dtype], int(bool(accumulate)), int(bool(swiglu)))
+
+
+def swiglu_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
+    """Whether `linear_swiglu` takes a product of m rows over k with such a matrix."""
+    return w_dtype is torch.bfloat16 and m > 0 and (k % 8 == 0 if m <= SKINNY_MAX_ROWS else k % 64 == 0)
+
+
+def linear_swiglu(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[m, n] = up * gate / (1 + exp(-gate)) with [gate, up] = x w^T, w = [gate; up]
+    (2 N rows): the activation in the product's epilogue, from the product's float32 sums."""
+    _gpu(x, w, out)
+    _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear_swiglu: needs matrices")
+    m, k = x.shape
+    n = out.shape[1]
+    _chk(swiglu_takes(m, k, w.dtype), "linear_swiglu: sizes or dtype not taken")
+    _chk(w.shape == (2 * n, k) and out.shape[0] == m, "linear_swiglu: shapes do not fit")
+    _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_swiglu: contiguous operands")
+    _chk(x.dtype is torch.bfloat16 and out.dtype is torch.bfloat16, "linear_swiglu: x and out must be bfloat16")
+    _run("gemm", "li_linear_swiglu", x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k)
 
 
 # ----------------------------------------------------------------- attention

@@ -19,8 +19,9 @@ class Linear:
 
     def takes_swiglu(self, x: torch.Tensor) -> bool:
         """Whether the product of these rows can have the SwiGLU activation as its
-        epilogue (few rows, bfloat16)."""
-        return x.dtype is torch.bfloat16 and ops.skinny_takes(x.shape[0], self.in_features, self.weight.dtype)
+        epilogue (bfloat16, no bias, a width the kernels take)."""
+        return (x.dtype is torch.bfloat16 and self.bias is None
+                and ops.swiglu_takes(x.shape[0], self.in_features, self.weight.dtype))
 
     def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ws=None,
                  swiglu: bool = False):
@@ -30,7 +31,7 @@ class Linear:
         32-bit also when the activations are bfloat16: they are widened for it,
         exactly."""
         if swiglu:
-            ops.linear_skinny(x, self.weight, self.bias, out, accumulate, swiglu=True)
+            ops.linear_swiglu(x, self.weight, out)
         elif self.weight.dtype is torch.float32 and x.dtype is not torch.float32:
             x32 = ws.buffer("linear.x32", x.shape, torch.float32)
             ops.cast(x, x32)

@@ -123,6 +123,38 @@ def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, 
     assert rel(out, y) < (4 * math.sqrt(k) * 2.0 ** -24 if out_dtype is torch.float32 else 5e-3)
 
 
+@pytest.mark.parametrize("m,n,k", [
+    (8, 200, 96),                # few rows: the decode kernel
+    (65, 32, 64),                # one tile, one step of K
+    (100, 200, 128),             # an output width that is no multiple of 32
+    (300, 1000, 192),            # several tiles both ways, ragged edges
+    (700, 4700, 256),            # enough tiles for the largest tiling
+    (2048, 18944, 128),
+])
+def test_linear_with_swiglu_epilogue(ops, m, n, k):
+    g = torch.Generator().manual_seed(14)
+    x = (torch.randn(m, k, generator=g) * 2).to(torch.bfloat16)
+    w = (torch.randn(2 * n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    y = x.double().numpy() @ w.double().numpy().T
+    y = plain_impl.swiglu(y[:, :n], y[:, n:])
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert ops.swiglu_takes(m, k, w.dtype)
+    ops.linear_swiglu(x.to(DEV), w.to(DEV), out)
+    assert rel(out, y) < 5e-3
+    # a gate far from zero either way and single outputs that stand out
+    w2 = torch.zeros(2 * n, k)
+    w2[3, 0] = 30.0; w2[n + 3, 0] = 1.0          # silu(+large) * up
+    w2[5, 0] = -30.0; w2[n + 5, 0] = 1.0         # silu(-large) -> 0
+    w2[n - 1, 1] = 1.0; w2[2 * n - 1, 1] = 2.0   # the last output
+    x2 = torch.zeros(m, k); x2[:, 0] = 1.0; x2[m - 1, 1] = 3.0
+    ops.linear_swiglu(x2.to(torch.bfloat16).to(DEV), w2.to(torch.bfloat16).to(DEV), out)
+    o = out.float().cpu()
+    assert abs(o[0, 3].item() - 30.0) < 0.2 and abs(o[0, 5].item()) < 1e-9
+    want_last = 2.0 * 3.0 * (3.0 / (1 + math.exp(-3.0)))
+    assert abs(o[m - 1, n - 1].item() - want_last) < 0.1 and o[0, n - 1].item() == 0.0
+    assert torch.count_nonzero(o).item() <= 2 * m + 1
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_rows_do_not_depend_on_the_batch(ops, dtype):
     g = torch.Generator().manual_seed(3)

@@ -124,12 +124,20 @@ def paged_attention(qkv, out, k, v, meta, nh, nkv, dh, page_size, window, scale,
                 out[q0 + i, h * dh:(h + 1) * dh] = (w @ vv).to(out.dtype)
 
 
+def swiglu_takes(m, k, w_dtype):
+    return w_dtype is torch.bfloat16 and m > 0 and (k % 8 == 0 if m <= 64 else k % 64 == 0)
+
+
+def linear_swiglu(x, w, out):
+    linear_skinny(x, w, None, out, False, swiglu=True)
+
+
 def argmax_rows(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
-       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "check_attention_sizes",
+       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "check_attention_sizes",
        "paged_attention", "argmax_rows"]
 
 
