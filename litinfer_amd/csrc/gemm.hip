@@ -378,6 +378,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                                                              const float* __restrict__ bias,
                                                              TO* __restrict__ out, int M, int N, int K,
                                                              int accumulate) {
+    // gridDim.y > 1: block (., y) multiplies the y-th part of K and writes its sums to the y-th
+    // [M, N] matrix behind `out` (float, no bias, no accumulation); splitk_reduce_kernel adds them
     constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
     constexpr int CPR = BK / 8, WRAP = 128 / BK;                 // chunks in a row; rows that fill all banks once
     constexpr int RPI = 64 / CPR;                                // rows one load instruction of a wave covers
@@ -434,7 +436,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
         for (int i = 0; i < IB; ++i) LI_LOAD_TO_LDS(gb[i] + (size_t)kt * BK, st + BM * BK + ((BN / 4) * wave + RPI * i) * BK);
     };
     const int frow = lane & 31, fh = lane >> 5;
-    const int nk = K / BK;
+    const int kt_first = (int)((long)(K / BK) * blockIdx.y / gridDim.y);
+    const int nk = (int)((long)(K / BK) * (blockIdx.y + 1) / gridDim.y) - kt_first;
+    out += (size_t)blockIdx.y * M * (SWIGLU ? N / 2 : N);
+#pragma unroll
+    for (int i = 0; i < IA; ++i) ga[i] += (size_t)kt_first * BK;
+#pragma unroll
+    for (int i = 0; i < IB; ++i) gb[i] += (size_t)kt_first * BK;
     constexpr int KS = BK / 16;                    // MFMA steps of a stage (even)
     // Order of a step: the MFMAs of stage kt run while the fragments of its next 16 columns are
     // read; in the middle of the stage's LAST 16 columns the wave waits for stage kt + 1 (loaded
@@ -566,11 +574,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 
 template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
-                      int accumulate, hipStream_t stream) {
+                      int accumulate, hipStream_t stream, int nsplit = 1) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
     const long gn = mtiles >= 32 ? 1 : 32 / mtiles;
     const long per_xcd = ((ntiles + 7) / 8 + gn - 1) / gn * gn * mtiles;
-    if (per_xcd * 8 > 0x7fffffffL) return LI_ERR_SIZE;
+    if (per_xcd * 8 > 0x7fffffffL || nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
     constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool configured = false;
     if (!configured) {
@@ -579,8 +587,19 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
             return LI_ERR_LAUNCH;
         configured = true;
     }
-    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO><<<dim3((unsigned)(per_xcd * 8)), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
+    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO><<<dim3((unsigned)(per_xcd * 8), nsplit), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
     return li_launch_status();
+}
+
+// out (+)= sum over the parts, in the order of the parts, + bias
+template <typename TO>
+__global__ void splitk_reduce_kernel(const float* __restrict__ part, int nsplit, size_t mn, int N,
+                                     const float* __restrict__ bias, TO* __restrict__ out, int accumulate) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= mn) return;
+    float v = part[i];
+    for (int s = 1; s < nsplit; ++s) v += part[(size_t)s * mn + i];
+    epilogue_store(out, i, v, bias, (int)(i % N), accumulate);
 }
 
 template <int BM, int BN, int BK, typename TO>
@@ -805,8 +824,39 @@ extern "C" int li_linear_skinny(const void* x, const void* w, const float* bias,
     return li_launch_status();
 }
 
+// Between 33 and 64 rows (a large decoding batch) the product is still bound by streaming W, but
+// x is too large to be read again by every block of a few columns: tiles of 64 rows with the
+// loads straight into LDS, and, where the matrix has too few such tiles to fill the chip, K cut
+// into parts whose sums go to `work` and are added up in a fixed order.  Returns -1 when it does
+// not take the call.
+static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, void* out, int M, int N,
+                           int K, int out_dtype, int accumulate, void* work, long work_bytes,
+                           hipStream_t stream) {
+    if (M <= 32 || M > 64 || K % 64 || (out_dtype != LI_F32 && out_dtype != LI_BF16)) return -1;
+#define LI_MID(BN, NS, TO, dst, b, acc, split) launch_dma<64, BN, 64, NS, false, TO>(x, w, b, (TO*)(dst), M, N, K, acc, stream, split)
+    if ((N + 255) / 256 >= 128)
+        return out_dtype == LI_F32 ? LI_MID(256, 3, float, out, bias, accumulate, 1) : LI_MID(256, 3, bf16_t, out, bias, accumulate, 1);
+    const int tiles = (N + 127) / 128;
+    if (tiles >= 128)
+        return out_dtype == LI_F32 ? LI_MID(128, 4, float, out, bias, accumulate, 1) : LI_MID(128, 4, bf16_t, out, bias, accumulate, 1);
+    int nsplit = 256 / tiles;
+    if (nsplit > 8) nsplit = 8;
+    if (nsplit > K / 64 / 8) nsplit = K / 64 / 8;              // at least 8 steps a part
+    const size_t mn = (size_t)M * N;
+    if (nsplit < 2 || !work || (size_t)work_bytes < (size_t)nsplit * mn * sizeof(float)) return -1;
+    const int rc = LI_MID(128, 4, float, work, nullptr, 0, nsplit);
+    if (rc != LI_OK) return rc;
+#undef LI_MID
+    const unsigned blocks = (unsigned)((mn + 255) / 256);
+    if (out_dtype == LI_F32) splitk_reduce_kernel<float><<<blocks, 256, 0, stream>>>((const float*)work, nsplit, mn, N, bias, (float*)out, accumulate);
+    else splitk_reduce_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const float*)work, nsplit, mn, N, bias, (bf16_t*)out, accumulate);
+    return li_launch_status();
+}
+
+// `work` (may be null): device memory of work_bytes for the partial sums of a product cut along K.
 extern "C" int li_linear(const void* x, const void* w, const float* bias, void* out, int M, int N,
-                         int K, int in_dtype, int out_dtype, int accumulate, hipStream_t stream) {
+                         int K, int in_dtype, int out_dtype, int accumulate, void* work, long work_bytes,
+                         hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0) return LI_ERR_SIZE;
     if (accumulate && out_dtype != LI_F32) return LI_ERR_DTYPE;
     if (in_dtype == LI_F32) {
@@ -818,8 +868,12 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         dim3 grid((N + BF_BN - 1) / BF_BN, (M + BF_BM - 1) / BF_BM);
         if (grid.y > 65535) return LI_ERR_SIZE;
         const bool aligned = (K % 8) == 0;
-        if (aligned && M <= 64)
+        if (aligned && M <= 64) {
+            const int rc = linear_mid_rows((const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, out_dtype,
+                                           accumulate, work, work_bytes, stream);
+            if (rc >= 0) return rc;
             return li_linear_skinny(x, w, bias, out, M, N, K, out_dtype, accumulate, 0, stream);
+        }
         if (aligned && M > 64) {
 #define LI_BIG(BM, BN, BK) (out_dtype == LI_F32 ? launch_big<BM, BN, BK, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                             : launch_big<BM, BN, BK, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
@@ -858,9 +912,15 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
 extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, int I, int K,
                                 hipStream_t stream) {
     if (M <= 0 || I <= 0 || K <= 0 || I > 0x3fffffff) return LI_ERR_SIZE;
+    const int N = 2 * I;
+    if (M > 32 && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
+        if ((N + 255) / 256 >= 128)
+            return launch_dma<64, 256, 64, 3, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
+        if ((N + 127) / 128 >= 128)
+            return launch_dma<64, 128, 64, 4, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
+    }
     if (M <= 64) return li_linear_skinny(x, w, nullptr, out, M, I, K, LI_BF16, 0, 1, stream);
     if (K % 64) return LI_ERR_SIZE;
-    const int N = 2 * I;
     auto cost = [&](int bm, int bn, double speed) {
         const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
         return (double)((tiles + 255) / 256) * bm * bn / speed;

@@ -35,7 +35,7 @@ _SIGNATURES = {
         "li_rope_kv_store": [P, I, I, I, I, I, I, P, P, P, P, P, I, I, I],
     },
     "gemm": {
-        "li_linear": [P, P, P, P, I, I, I, I, I, I],
+        "li_linear": [P, P, P, P, I, I, I, I, I, I, P, L],
         "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
         "li_linear_swiglu": [P, P, P, I, I, I],
     },
@@ -243,11 +243,17 @@ def rope_kv_store(qkv: torch.Tensor, nh: int, nkv: int, dh: int, rotary_dim: int
 
 
 # ---------------------------------------------------------------------- gemm
+SKINNY_MAX_ROWS = 64
+SPLITK_MAX_PARTS = 8
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-           accumulate: bool = False) -> None:
+           accumulate: bool = False, ws=None) -> None:
     """out = x w^T + bias, or out += x w^T + bias when `accumulate`.
     x [M, K] and w [N, K] of one dtype (float32 or bfloat16); out [M, N] of that
-    dtype or float32; accumulation of the product is float32."""
+    dtype or float32; accumulation of the product is float32.  `ws` lends the
+    memory for partial sums where the kernel cuts K into parts (33 to 64 rows
+    against a matrix of few columns); without it such a product takes a slower kernel."""
     _gpu(x, w, bias, out)
     _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear: needs matrices")
     m, k = x.shape
@@ -261,11 +267,13 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
          "linear: bias must be float32 [N]")
     if m:
+        work, work_bytes = 0, 0
+        if ws is not None and x.dtype is torch.bfloat16 and SKINNY_MAX_ROWS // 2 < m <= SKINNY_MAX_ROWS:
+            buf = ws.buffer("gemm.parts", (SPLITK_MAX_PARTS * SKINNY_MAX_ROWS * n,), torch.float32)
+            work, work_bytes = buf.data_ptr(), buf.numel() * 4
         _run("gemm", "li_linear", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
-             out.data_ptr(), m, n, k, _DT[x.dtype], _DT[out.dtype], int(bool(accumulate)))
+             out.data_ptr(), m, n, k, _DT[x.dtype], _DT[out.dtype], int(bool(accumulate)), work, work_bytes)
 
-
-SKINNY_MAX_ROWS = 64
 
 
 def skinny_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:

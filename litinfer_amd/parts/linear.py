@@ -36,11 +36,11 @@ class Linear:
             x32 = ws.buffer("linear.x32", x.shape, torch.float32)
             ops.cast(x, x32)
             if out.dtype is torch.float32:
-                ops.linear(x32, self.weight, self.bias, out, accumulate)
+                ops.linear(x32, self.weight, self.bias, out, accumulate, ws=ws)
             else:
                 y32 = ws.buffer("linear.y32", out.shape, torch.float32)
                 ops.linear(x32, self.weight, self.bias, y32, False)
                 ops.cast(y32, out)
         else:
-            ops.linear(x, self.weight, self.bias, out, accumulate)      # few rows go to the skinny kernel inside
+            ops.linear(x, self.weight, self.bias, out, accumulate, ws=ws)      # few rows go to their own kernels inside
         return out

@@ -123,8 +123,46 @@ def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, 
     assert rel(out, y) < (4 * math.sqrt(k) * 2.0 ** -24 if out_dtype is torch.float32 else 5e-3)
 
 
+class _Lender:
+    """Stands in for the engine's workspace."""
+    def buffer(self, name, shape, dtype):
+        return torch.empty(*shape, dtype=dtype, device=DEV)
+
+
+@pytest.mark.parametrize("m,n,k,out_dtype,bias,acc", [
+    (33, 200, 1024, torch.float32, True, True),          # K in parts: few tiles
+    (64, 3584, 3584, torch.float32, False, True),
+    (48, 300, 18944, torch.bfloat16, True, False),
+    (64, 136, 512, torch.bfloat16, False, False),        # too short a K for parts
+    (40, 20000, 128, torch.float32, True, False),        # many tiles of 128 columns
+    (64, 37000, 64, torch.bfloat16, False, False),       # many tiles of 256 columns
+])
+def test_linear_between_33_and_64_rows(ops, m, n, k, out_dtype, bias, acc):
+    g = torch.Generator().manual_seed(15)
+    x = (torch.randn(m, k, generator=g) * 2).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    b = torch.randn(n, generator=g) if bias else None
+    y = x.double().numpy() @ w.double().numpy().T
+    if b is not None:
+        y = y + b.double().numpy()
+    if acc:
+        base = torch.randn(m, n, generator=g)
+        y = y + base.double().numpy()
+    outs = []
+    for ws in (_Lender(), None):                         # with and without memory for partial sums
+        out = base.to(DEV) if acc else torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+        ops.linear(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, acc, ws=ws)
+        assert rel(out, y) < (4 * math.sqrt(k) * 2.0 ** -24 if out_dtype is torch.float32 else 5e-3)
+        outs.append(out)
+    again = base.to(DEV) if acc else torch.empty(m, n, dtype=out_dtype, device=DEV)
+    ops.linear(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), again, acc, ws=_Lender())
+    assert torch.equal(again, outs[0])                   # the parts are added in a fixed order
+
+
 @pytest.mark.parametrize("m,n,k", [
     (8, 200, 96),                # few rows: the decode kernel
+    (40, 20000, 128),            # 33 to 64 rows: tiles of 64 rows
+    (64, 9500, 192),
     (65, 32, 64),                # one tile, one step of K
     (100, 200, 128),             # an output width that is no multiple of 32
     (300, 1000, 192),            # several tiles both ways, ragged edges

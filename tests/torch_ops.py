@@ -73,7 +73,7 @@ def rope_kv_store(qkv, nh, nkv, dh, rotary_dim, cos, sin, slot_map, k, v, page_s
     kv_store(qkv, nh, nkv, dh, slot_map, k, v, page_size)
 
 
-def linear(x, w, bias, out, accumulate=False):
+def linear(x, w, bias, out, accumulate=False, ws=None):
     y = x.float() @ w.float().T
     if bias is not None:
         y = y + bias
