@@ -16,7 +16,7 @@ from litinfer_amd.config import ExecEntry, LayerSpec, ModelSpec, PartSpec, Qwen2
 from litinfer_amd.engine import Engine, StepEntry, StepError
 from litinfer_amd.engine.batch import BatchUploader, build_context
 from litinfer_amd.engine.workspace import Workspace
-from litinfer_amd.parts import Mixer, ResidualStream, Runtime, StateNeed, build_part, register_part
+from litinfer_amd.parts import FeedForward, Mixer, Position, ResidualStream, Runtime, StateNeed, build_part, register_part
 from litinfer_amd.weights import ParamSpec
 from tiny_configs import TINY_A, TINY_B, TINY_C
 
@@ -393,3 +393,122 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, device
         out = schedules.run(eng, reqs, getattr(schedules, kind)(reqs))
         assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind   # slots reused, state zeroed
     eng.cache.check_invariants()
+
+
+# --------- a toy feed-forward with routing and a toy position encoding, defined here
+class ToyRoutedFFN(FeedForward):
+    """y = W2_e relu(W1_e xn) with e = argmax(router xn), one expert per token.
+    Written with torch: it is a toy that shows the interface, not a kernel."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.h, self.inner, self.experts = (spec.args[k] for k in ("hidden_size", "inner", "experts"))
+
+    def expected_params(self):
+        p = self.prefix
+        out = {p + "router.weight": ParamSpec((self.experts, self.h))}
+        for e in range(self.experts):
+            out[p + f"experts.{e}.w1"] = ParamSpec((self.inner, self.h))
+            out[p + f"experts.{e}.w2"] = ParamSpec((self.h, self.inner))
+        return out
+
+    def load_params(self, get):
+        f = lambda n: get(self.prefix + n).to(torch.float32).to(self.rt.device)
+        self.router = f("router.weight")
+        self.w1 = torch.stack([f(f"experts.{e}.w1") for e in range(self.experts)])
+        self.w2 = torch.stack([f(f"experts.{e}.w2") for e in range(self.experts)])
+
+    def forward(self, xn, residual, ctx):
+        x = xn.float()
+        choice = torch.argmax(x @ self.router.T, dim=-1)               # router logits in 32-bit
+        hidden = torch.relu(torch.einsum("th,tih->ti", x, self.w1[choice]))
+        residual.tensor().add_(torch.einsum("ti,thi->th", hidden, self.w2[choice]))
+
+
+class ToyPairRope(Position):
+    """Rotary encoding over NEIGHBOURING pairs (2j, 2j+1), unlike the half-split
+    pairing of the architecture: another position encoding behind the same interface."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.dh, self.theta = spec.args["head_dim"], spec.args["theta"]
+
+    def key(self):
+        return ("toy_pair_rope", self.dh, self.theta)
+
+    def tables(self, ctx):
+        def make():
+            j = torch.arange(self.dh // 2, dtype=torch.float32, device=ctx.positions.device)
+            ang = ctx.positions.float()[:, None] / (self.theta ** (2 * j / self.dh))
+            return torch.cos(ang), torch.sin(ang)
+        return ctx.shared(self.key(), make)
+
+    def apply(self, qkv, n_heads_total, head_dim, ctx):
+        cos, sin = self.tables(ctx)
+        x = qkv[:, :n_heads_total * head_dim].float().reshape(qkv.shape[0], n_heads_total, head_dim // 2, 2)
+        a, b = x[..., 0], x[..., 1]
+        c, s = cos[:, None, :], sin[:, None, :]
+        y = torch.stack([a * c - b * s, b * c + a * s], dim=-1).reshape(qkv.shape[0], -1)
+        qkv[:, :n_heads_total * head_dim] = y.to(qkv.dtype)
+
+
+def _routed_spec(c: ToyConfig) -> ModelSpec:
+    base = qwen2_model_spec(c.inner)
+    l0 = base.layers[0]
+    mixer = l0.parts["mixer"]
+    pair = PartSpec("toy_pair_rope", "", {"head_dim": c.inner.head_dim, "theta": c.inner.rope_theta})
+    toy = LayerSpec("prenorm", dict(
+        l0.parts,
+        mixer=PartSpec(mixer.kind, mixer.prefix, dict(mixer.args, position=pair)),
+        feed_forward=PartSpec("toy_routed", "model.layers.0.moe.",
+                              {"hidden_size": c.hidden_size, "inner": 24, "experts": 3})))
+    return replace(base, architecture="ToyRoutedLM", layers=(toy,) + base.layers[1:])
+
+
+def test_a_toy_routed_feed_forward_and_another_position_encoding(tmp_path, device):
+    register_part("feed_forward", "toy_routed", ToyRoutedFFN)
+    register_part("position", "toy_pair_rope", ToyPairRope)
+    register_architecture("ToyRoutedLM", ToyConfig.from_dict, _routed_spec)
+    cfg = dict(TINY_A, architectures=["ToyRoutedLM"], toy_decay=0.0)
+    d = helpers.make_model(tmp_path, cfg, 8)
+    pcfg, w = P.load_folder(d)
+    assert "model.layers.0.moe.experts.2.w2" in w and "model.layers.0.mlp.down_proj.weight" not in w
+    nh, nkv, dh = pcfg["num_attention_heads"], pcfg["num_key_value_heads"], P.head_dim_of(pcfg)
+
+    def pair_rope(x, pos, theta):
+        j = np.arange(dh // 2)
+        ang = np.asarray(pos, dtype=np.float64)[:, None] / (theta ** (2 * j / dh))
+        c, s = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+        a, b = x[..., 0::2], x[..., 1::2]
+        y = np.empty_like(x)
+        y[..., 0::2], y[..., 1::2] = a * c - b * s, b * c + a * s
+        return y
+
+    used = set()
+
+    def plain(ids):
+        t = len(ids)
+        pos = np.arange(t)
+        x = P.embedding(ids, w["model.embed_tokens.weight"])
+        p = "model.layers.0."
+        xn = P.rms_norm(x, w[p + "input_layernorm.weight"], 1e-6)
+        proj = lambda n: P.linear(xn, w[p + f"self_attn.{n}_proj.weight"], w[p + f"self_attn.{n}_proj.bias"])
+        q = pair_rope(proj("q").reshape(t, nh, dh), pos, pcfg["rope_theta"])
+        k = pair_rope(proj("k").reshape(t, nkv, dh), pos, pcfg["rope_theta"])
+        a = P.attention(q, k, proj("v").reshape(t, nkv, dh), pos, pos, 1 / math.sqrt(dh))
+        x = x + P.linear(a.reshape(t, nh * dh), w[p + "self_attn.o_proj.weight"])
+        xn = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-6)
+        choice = np.argmax(xn @ w[p + "moe.router.weight"].T, axis=-1)
+        used.update(choice.tolist())
+        y = np.stack([w[p + f"moe.experts.{e}.w2"] @ np.maximum(w[p + f"moe.experts.{e}.w1"] @ v, 0)
+                      for e, v in zip(choice, xn)])
+        x, _ = P.decoder_layer(x + y, pos, w, "model.layers.1.", pcfg, 0)
+        return P.rms_norm(x, w["model.norm.weight"], 1e-6) @ w["model.embed_tokens.weight"].T
+
+    reqs = helpers.random_requests(256, [33, 18, 5, 26], 9)
+    ref = {r: plain(np.asarray(t)) for r, t in reqs.items()}
+    assert len(used) > 1                                   # the router does choose
+    eng = engine_for(d, device)
+    for kind in ("whole", "tail", "chunks", "mixed"):
+        out = schedules.run(eng, reqs, getattr(schedules, kind)(reqs))
+        assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind
