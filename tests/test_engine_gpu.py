@@ -7,11 +7,13 @@ import torch
 
 import helpers
 import schedules
-from tiny_configs import TINY_A, TINY_A_PAGE, TINY_B, TINY_B_PAGE, TINY_C, TINY_C_PAGE
+from tiny_configs import (TINY_A, TINY_A_PAGE, TINY_B, TINY_B_PAGE, TINY_C, TINY_C_PAGE, TINY_D, TINY_D_PAGE,
+                          TINY_E, TINY_E_PAGE)
 
 pytestmark = pytest.mark.gpu
 
-CASES = {"A": (TINY_A, TINY_A_PAGE, 0), "B": (TINY_B, TINY_B_PAGE, 1), "C": (TINY_C, TINY_C_PAGE, 2)}
+CASES = {"A": (TINY_A, TINY_A_PAGE, 0), "B": (TINY_B, TINY_B_PAGE, 1), "C": (TINY_C, TINY_C_PAGE, 2),
+         "D": (TINY_D, TINY_D_PAGE, 3), "E": (TINY_E, TINY_E_PAGE, 4)}
 LENGTHS = [5, 17, 33, 70, 100, 41, 64, 2, 1]
 # float32: rounding of a different summation order only.  bfloat16: weights are
 # bfloat16 on both sides (the plain side computes in float64 from the stored
