@@ -4,7 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
 
 A "step" is one decode step of the whole batch through the engine's step
-function plus greedy sampling, the next tokens fed back.  Weights are random
+function plus greedy sampling, the next tokens fed back (on the device: the
+host reads each step's tokens while the next step runs, as the scheduler does
+with lookahead).  Weights are random
 (drawn on the device), token ids are seeded synthetic ids, and the cache of
 every request is filled with random keys and values up to the context length
 before the timed steps (their content does not change the work).  One JSON
@@ -99,17 +101,27 @@ def main() -> int:
             eng.cache.commit(r, start_ctx)
         toks = rng.integers(0, cfg["vocab_size"], batch).tolist()
         params, counters = [SamplingParams()] * batch, [0] * batch
+        state = {"pending": None, "n": 0}
 
         def one():
-            nonlocal toks
-            logits = eng.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
-            toks = sampler.sample(logits, params, counters)      # the copy to the host ends the step
+            # as the scheduler does with lookahead: the sampled ids stay on the device and the
+            # next step takes them from the engine's feedback buffer; the host reads them one
+            # step later, while the device is at work on the next step
+            first = state["n"] == 0
+            logits = eng.step([StepEntry(r, [t], [0], None if first else [i])
+                               for i, (r, t) in enumerate(zip(rids, toks))])
+            handle = sampler.sample_async(logits, params, counters, out=eng.feedback)
+            if state["pending"] is not None:
+                state["pending"].result()
+            state["pending"], state["n"] = handle, state["n"] + 1
         for _ in range(warmup):
             one()
+        state["pending"].result() if state["pending"] is not None else None
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(steps):
             one()
+        state["pending"].result()                    # the last step's tokens have reached the host
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         ctx_tokens = batch * (start_ctx + warmup + steps / 2.0)

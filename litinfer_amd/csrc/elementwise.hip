@@ -5,25 +5,32 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding
-// out[t, :] = float(table[ids[t], :])  (row copy, no scaling)
+// out[t, :] = float(table[id(t), :])  (row copy, no scaling), with id(t) = ids[t], or, where
+// id_src is given and id_src[t] >= 0, feedback[id_src[t]]: a token that an earlier kernel on the
+// stream chose and the host has not seen yet.
 template <typename T>
-__global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+__global__ void embedding_kernel(const int* __restrict__ ids, const int* __restrict__ id_src,
+                                 const int* __restrict__ feedback, const T* __restrict__ table,
                                  float* __restrict__ out, int H, int V) {
     const int t = blockIdx.x;
-    const int id = ids[t];
-    if (id < 0 || id >= V) return;                 // the host has checked; never read outside
+    int id = ids[t];
+    if (id_src) {
+        const int src = id_src[t];
+        if (src >= 0) id = feedback[src];
+    }
+    if (id < 0 || id >= V) return;                 // the host has checked what it knows; never read outside
     const T* row = table + (size_t)id * H;
     float* o = out + (size_t)t * H;
     for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = load_as_float(row + j);
 }
 
-extern "C" int li_embedding(const int* ids, const void* table, int table_dtype, float* out, int T,
-                            int H, int V, hipStream_t stream) {
-    if (T <= 0 || H <= 0) return LI_ERR_SIZE;
+extern "C" int li_embedding(const int* ids, const int* id_src, const int* feedback, const void* table,
+                            int table_dtype, float* out, int T, int H, int V, hipStream_t stream) {
+    if (T <= 0 || H <= 0 || (id_src && !feedback)) return LI_ERR_SIZE;
     if (table_dtype == LI_F32)
-        embedding_kernel<float><<<T, 256, 0, stream>>>(ids, (const float*)table, out, H, V);
+        embedding_kernel<float><<<T, 256, 0, stream>>>(ids, id_src, feedback, (const float*)table, out, H, V);
     else if (table_dtype == LI_BF16)
-        embedding_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, (const bf16_t*)table, out, H, V);
+        embedding_kernel<bf16_t><<<T, 256, 0, stream>>>(ids, id_src, feedback, (const bf16_t*)table, out, H, V);
     else return LI_ERR_DTYPE;
     return li_launch_status();
 }

@@ -22,6 +22,10 @@ class StepEntry:
     rid: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = ()          # places among `tokens` whose logits are asked for
+    # For each of `tokens`, -1 or a place in the engine's feedback buffer (`Engine.feedback`): the
+    # token's id is then read from there when the step runs, and the number in `tokens` is not
+    # used.  This is how a token sampled on the device enters the next step before the host knows it.
+    take: Optional[Sequence[int]] = None
 
 
 @dataclass
@@ -63,6 +67,8 @@ class StepContext:
         self.num_tokens = num_tokens
         self.num_segments = num_segments
         self.ids: torch.Tensor = None
+        self.id_src: torch.Tensor = None              # [T] int32: place in `feedback` or -1
+        self.feedback: torch.Tensor = None            # the engine's buffer of ids chosen on the device
         self.positions: torch.Tensor = None
         self.state_slots: torch.Tensor = None        # [segments] int32, device
         self.host_state_slots: np.ndarray = None
@@ -137,7 +143,7 @@ class BatchUploader:
 
 
 def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploader",
-                  pad_blocks: Optional[Sequence[int]] = None) -> StepContext:
+                  pad_blocks: Optional[Sequence[int]] = None, feedback: Optional[torch.Tensor] = None) -> StepContext:
     """Lay out the step's integers (see the module text) for the given entries
     against the cache's current tables, upload them, and return the context.
     Pages for the entries' tokens must have been reserved.  `pad_blocks` gives,
@@ -152,6 +158,10 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     cached = np.array([cache.cached_len(e.rid) for e in entries], dtype=np.int32)
     ctx_len = cached + q_len
     ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+    id_src = np.full(T, -1, dtype=np.int32)
+    for i, e in enumerate(entries):
+        if e.take is not None:
+            id_src[q_start[i]:q_start[i + 1]] = np.asarray(e.take, dtype=np.int32)
     seg_of_token = np.repeat(np.arange(nseg, dtype=np.int32), q_len)
     pos = (np.arange(T, dtype=np.int32) - q_start[seg_of_token] + cached[seg_of_token]).astype(np.int32)
     slots = np.array([cache.slot(e.rid) for e in entries], dtype=np.int32)
@@ -163,7 +173,8 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     tile_rows = [(i, int(q_start[i]) + a, min(32, int(q_len[i]) - a), 0)
                  for i in range(nseg) if q_len[i] > 1 for a in range(0, int(q_len[i]), 32)]
     tiles = np.asarray(tile_rows, dtype=np.int32).reshape(-1, 4)
-    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows, single, multi, tiles]
+    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows, single, multi, tiles,
+             id_src]
     tables, max_blocks = [], []
     for gi in range(len(cache.groups)):
         tabs = [cache.block_table(e.rid, gi) for e in entries]
@@ -183,12 +194,17 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     dev = uploader.upload(parts)
     ctx = StepContext(ws, T, nseg)
     (ctx.ids, ctx.positions, d_seg, d_qs, d_ql, d_cl, ctx.state_slots, ctx.want_rows,
-     d_single, d_multi, d_tiles) = dev[:11]
+     d_single, d_multi, d_tiles, ctx.id_src) = dev[:12]
+    ctx.feedback = feedback
+    if feedback is None:
+        if (id_src >= 0).any():
+            raise ValueError("step: an entry takes tokens from the feedback buffer, but there is none")
+        ctx.id_src = None
     ctx.num_want = len(want)
     ctx.host_state_slots = slots
     ctx.host_q_start, ctx.host_q_len, ctx.host_ctx_len = q_start[:-1], q_len, ctx_len
     for gi in range(len(cache.groups)):
-        d_tab, d_slot = dev[11 + 2 * gi], dev[12 + 2 * gi]
+        d_tab, d_slot = dev[12 + 2 * gi], dev[13 + 2 * gi]
         ctx._slot_maps.append(d_slot)
         ctx._attn.append(AttentionMeta(
             block_table=d_tab, max_blocks=max_blocks[gi], seg_of_token=d_seg, q_start=d_qs,

@@ -42,6 +42,9 @@ def parse_dtype(dtype) -> torch.dtype:
     return DTYPES[str(dtype)]
 
 
+FEEDBACK_SLOTS = 4096
+
+
 class StepError(ValueError):
     """The batch is not valid; nothing was changed."""
 
@@ -66,6 +69,9 @@ class Engine:
         self.cache: Optional[CacheManager] = None
         self.ws = Workspace(self.rt.device)
         self._uploader = BatchUploader(self.rt.device)
+        # ids of tokens chosen on the device (a sampler's output): an entry of the NEXT step may
+        # take its token from here (`StepEntry.take`), so the host need not wait for the number
+        self.feedback = torch.zeros(FEEDBACK_SLOTS, dtype=torch.int32, device=self.rt.device)
         self.steps_run = 0
         # decode steps (every request brings one token) are recorded as HIP graphs, one per batch
         # shape, and replayed: a step is some hundred small launches otherwise
@@ -143,6 +149,11 @@ class Engine:
             if toks.ndim != 1 or toks.dtype.kind not in "iu" or toks.min() < 0 or toks.max() >= vocab:
                 raise StepError(f"step: request {e.rid!r} brings a token id outside the vocabulary "
                                 f"of {vocab} (embedding: index out of range)")
+            if e.take is not None:
+                take = np.asarray(e.take)
+                if take.shape != (n,) or take.dtype.kind not in "iu" or take.min() < -1 or take.max() >= FEEDBACK_SLOTS:
+                    raise StepError(f"step: request {e.rid!r}: `take` must give, for each of its {n} "
+                                    f"tokens, -1 or a place below {FEEDBACK_SLOTS} in the feedback buffer")
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"step: request {e.rid!r} wants logits at place {w} of {n} tokens")
@@ -197,7 +208,7 @@ class Engine:
             self.cache.release(rid)
 
     def _build_context(self, entries: Sequence[StepEntry], pad_blocks=None) -> StepContext:
-        return build_context(self.cache, entries, self.ws, self._uploader, pad_blocks)
+        return build_context(self.cache, entries, self.ws, self._uploader, pad_blocks, self.feedback)
 
     # ---- recorded decode steps ----------------------------------------------
     def _graph_key(self, entries: Sequence[StepEntry]):

@@ -74,7 +74,7 @@ class Model:
         float32 logits [wanted, vocab] at the wanted rows (None if none)."""
         h = self.spec.hidden_size
         x = ctx.ws.buffer("model.residual", (ctx.num_tokens, h), torch.float32)
-        self.embedding.forward(ctx.ids, x)
+        self.embedding.forward(ctx.ids, x, ctx.id_src, ctx.feedback)
         stream = ResidualStream(x, ctx.ws)
         for i, e in enumerate(self.order):
             self.layers[e.layer].forward(stream, ctx, cache.view(i))

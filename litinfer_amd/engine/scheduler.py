@@ -22,6 +22,16 @@ and the caller spins (src/llaisys/models/qwen2.cpp:789-800, 832-845, 925-944;
 serving/engine_runtime.py:42-62).  Its finishing rules are kept: an end token
 is dropped and ends the request, the token that reaches max_new_tokens is kept
 (:1058-1073).
+
+With `lookahead` the scheduler does not wait for a step's sampled tokens before
+it plans and starts the next step: the sampler leaves them in the engine's
+feedback buffer on the device, the next step's entries take them from there,
+and the host reads them one step later, while the device is already at work.
+What can only be known from a token's value (an end token) is found out one
+step late: the request has then run one token too far, which is dropped.  What
+is counted (max_new_tokens, the model's length) is foreseen, and such a request
+is not run again until its last token has arrived.  The tokens are the same
+with and without it.
 """
 from __future__ import annotations
 
@@ -51,14 +61,23 @@ class Request:
     finish_reason: Optional[str] = None
     preemptions: int = 0
     arrival: int = 0
+    # lookahead: the request's newest token has been sampled but is not known here yet; it lies
+    # at this place of the engine's feedback buffer
+    pending_take: Optional[int] = None
+
+    @property
+    def num_generated(self) -> int:
+        return len(self.generated) + (self.pending_take is not None)
 
     @property
     def tokens(self) -> List[int]:
-        return self.prompt + self.generated
+        """Prompt and generated tokens; a pending token stands as 0 (its entry takes the id from
+        the feedback buffer)."""
+        return self.prompt + self.generated + ([0] if self.pending_take is not None else [])
 
     @property
     def remaining(self) -> int:
-        return len(self.prompt) + len(self.generated) - self.computed
+        return len(self.prompt) + self.num_generated - self.computed
 
 
 @dataclass
@@ -72,7 +91,7 @@ class Planned:
 class Scheduler:
     def __init__(self, engine, *, max_batch_tokens: int = 2048, chunk_size: int = 512,
                  max_running: Optional[int] = None, eos_token_ids: Optional[Sequence[int]] = None,
-                 sampler=None):
+                 sampler=None, lookahead: bool = False):
         if max_batch_tokens <= 0 or chunk_size <= 0:
             raise ValueError("scheduler: max_batch_tokens and chunk_size must be positive")
         self.engine = engine
@@ -90,6 +109,8 @@ class Scheduler:
         self.steps = 0
         self.preemptions = 0
         self.last_batch_tokens = 0
+        self.lookahead = bool(lookahead)
+        self._inflight = None            # (PendingTokens, [(request, params)]) of the step before
 
     # ---- submitting -----------------------------------------------------
     def add_request(self, prompt: Sequence[int], max_new_tokens: int = 128,
@@ -170,15 +191,23 @@ class Scheduler:
             n -= ((have - 1) % self.cache.page_size) + 1        # drop the last, partly used page
         return 0
 
+    def _end_lone(self, r: Request) -> None:
+        """A request that has the pool to itself and still cannot go on."""
+        self.running.remove(r)
+        self.engine.finish(r.rid)
+        r.state, r.finish_reason, r.pending_take = FINISHED, "error: kv capacity", None
+
     def plan(self) -> List[Planned]:
         """Decide the next batch.  Preempts if it must; changes nothing else."""
         while True:
             free = self.cache.free_pages()
             plan: List[Planned] = []
             budget = self.max_batch_tokens
-            decoding = [r for r in self.running if r.remaining == 1]
+            movable = [r for r in self.running if r.remaining > 0 and not self._ends_with_pending(r)]
             short = False
-            for r in decoding:
+            for r in movable:
+                if r.remaining != 1:
+                    continue
                 need = self._fits(free, r.rid, 1)
                 if need is None or budget <= 0:
                     short = need is None
@@ -190,72 +219,120 @@ class Scheduler:
                 self._preempt(self.running[-1])
                 continue
             if short:                                   # a lone request that outgrew the pool
-                r = self.running[0]
-                self.running.remove(r)
-                self.engine.finish(r.rid)
-                r.state, r.finish_reason = FINISHED, "error: kv capacity"
+                self._end_lone(self.running[0])
                 continue
-            break
-        for r in self.running:
-            if r.remaining <= 1 or budget <= 0:
-                continue
-            n = self._largest_fitting(free, r.rid, min(r.remaining, self.chunk_size, budget), None)
-            if n <= 0:
-                continue
-            free = [a - b for a, b in zip(free, self.cache.pages_needed(r.rid, n))]
-            budget -= n
-            plan.append(Planned(r, r.computed, n, n == r.remaining))
-        slots = self.cache.free_slots()
-        while self.waiting and budget > 0 and slots > 0 and len(self.running) < self.max_running:
-            r = self.waiting[0]
-            # admitted only when everything it has to compute fits the free pages now: a
-            # request let in on its first portion alone would soon be preempted again
-            if self._fits(free, None, r.remaining, 0) is None:
-                break                                   # first come first served: nobody overtakes
-            n = min(r.remaining, self.chunk_size, budget)
-            self.waiting.popleft()
-            r.state = RUNNING
-            self.running.append(r)
-            free = [a - b for a, b in zip(free, self.cache.pages_needed(None, n, cached=0))]
-            budget -= n
-            slots -= 1
-            plan.append(Planned(r, 0, n, n == r.remaining))
-        return plan
+            for r in movable:
+                if r.remaining <= 1 or budget <= 0:
+                    continue
+                n = self._largest_fitting(free, r.rid, min(r.remaining, self.chunk_size, budget), None)
+                if n <= 0:
+                    continue
+                free = [a - b for a, b in zip(free, self.cache.pages_needed(r.rid, n))]
+                budget -= n
+                plan.append(Planned(r, r.computed, n, n == r.remaining))
+            # Pages that the running requests' prompts will still take are spoken for: a waiting
+            # request is admitted only when everything it has to compute fits what is left after
+            # them (a request let in on its first portion alone would stall beside the others, each
+            # holding pages and none able to finish its prompt)
+            spare = self.cache.free_pages()
+            for r in self.running:
+                if r.remaining > 0:
+                    spare = [a - b for a, b in zip(spare, self.cache.pages_needed(r.rid, r.remaining))]
+            slots = self.cache.free_slots()
+            while self.waiting and budget > 0 and slots > 0 and len(self.running) < self.max_running:
+                r = self.waiting[0]
+                whole = self._fits(spare, None, r.remaining, 0)
+                if whole is None:
+                    break                               # first come first served: nobody overtakes
+                n = min(r.remaining, self.chunk_size, budget)
+                self.waiting.popleft()
+                r.state = RUNNING
+                self.running.append(r)
+                spare = [a - b for a, b in zip(spare, whole)]
+                budget -= n
+                slots -= 1
+                plan.append(Planned(r, 0, n, n == r.remaining))
+            if plan or not movable:
+                return plan
+            # requests are running, want to go on and none can (each holds pages, none is free):
+            # the most recently admitted gives way
+            if len(self.running) > 1:
+                self._preempt(self.running[-1])
+            else:
+                self._end_lone(self.running[0])
 
     # ---- one step ------------------------------------------------------------
+    def _ends_with_pending(self, r: Request) -> bool:
+        """The token that is still on its way is the request's last, whatever it is."""
+        return r.pending_take is not None and (
+            r.num_generated >= r.max_new_tokens
+            or len(r.prompt) + r.num_generated >= self.engine.spec.max_positions)
+
     def step(self, default_params: Optional[SamplingParams] = None) -> List[Tuple[Hashable, int]]:
         """Plan a batch, run it, sample, finish.  Returns (request id, token)
-        for every token appended in this step."""
+        for every token appended in this step (with lookahead: the tokens of the
+        step before, which have arrived by now)."""
         plan = self.plan()
         if not plan:
+            if self._inflight is not None:
+                return self._resolve()
             if self.has_unfinished() and not self.running:
                 # nothing runs and the head of the queue still does not fit: it never will
                 r = self.waiting.popleft()
                 r.state, r.finish_reason = FINISHED, "error: kv capacity"
             return []
-        entries = [StepEntry(p.request.rid, p.request.tokens[p.start:p.start + p.n],
-                             [p.n - 1] if p.wants_logits else []) for p in plan]
+        entries = []
+        for p in plan:
+            r = p.request
+            take = None
+            if r.pending_take is not None and p.start + p.n == len(r.prompt) + r.num_generated:
+                take = [-1] * (p.n - 1) + [r.pending_take]          # the portion ends with the pending token
+            entries.append(StepEntry(r.rid, r.tokens[p.start:p.start + p.n],
+                                     [p.n - 1] if p.wants_logits else [], take))
         self.last_batch_tokens = sum(p.n for p in plan)
         logits = self.engine.step(entries)
         self.steps += 1
         for p in plan:
             p.request.computed += p.n
         sampled = [p.request for p in plan if p.wants_logits]
-        produced: List[Tuple[Hashable, int]] = []
-        if sampled:
-            params, counters = [], []
-            for r in sampled:
-                sp = r.params or default_params or SamplingParams()
-                if r.first_token_greedy and not r.generated:
-                    sp = SamplingParams()
-                params.append(sp)
-                counters.append(r.samples_drawn)
-            tokens = self.sampler.sample(logits, params, counters)
-            for r, sp, tok in zip(sampled, params, tokens):
-                if not sp.greedy:
-                    r.samples_drawn += 1
-                if self._append(r, int(tok)):
-                    produced.append((r.rid, int(tok)))
+        params, counters = [], []
+        for r in sampled:
+            sp = r.params or default_params or SamplingParams()
+            if r.first_token_greedy and not r.num_generated:
+                sp = SamplingParams()
+            params.append(sp)
+            counters.append(r.samples_drawn)
+            if not sp.greedy:
+                r.samples_drawn += 1
+        if not self.lookahead:
+            produced: List[Tuple[Hashable, int]] = []
+            if sampled:
+                for r, tok in zip(sampled, self.sampler.sample(logits, params, counters)):
+                    if self._append(r, int(tok)):
+                        produced.append((r.rid, int(tok)))
+            return produced
+        handle = self.sampler.sample_async(logits, params, counters, out=self.engine.feedback) if sampled else None
+        produced = self._resolve()                   # the step before; the device is busy with this one
+        if handle is not None:
+            for i, r in enumerate(sampled):
+                if r.state != FINISHED:
+                    r.pending_take = i
+            self._inflight = (handle, sampled)
+        return produced
+
+    def _resolve(self) -> List[Tuple[Hashable, int]]:
+        """The tokens of the step in flight have to be known now: wait for them and apply them."""
+        if self._inflight is None:
+            return []
+        handle, sampled = self._inflight
+        self._inflight = None
+        produced = []
+        for r, tok in zip(sampled, handle.result()):
+            if r.state == FINISHED:                  # ended meanwhile (an end token one step back, an abort)
+                continue
+            r.pending_take = None
+            if self._append(r, int(tok)):
+                produced.append((r.rid, int(tok)))
         return produced
 
     def _append(self, r: Request, tok: int) -> bool:
@@ -272,8 +349,11 @@ class Scheduler:
 
     def _finish(self, r: Request, reason: str) -> None:
         r.state, r.finish_reason = FINISHED, reason
+        r.pending_take = None
         if r in self.running:
             self.running.remove(r)
+        elif r in self.waiting:                      # preempted while its last token was on its way
+            self.waiting.remove(r)
         self.engine.finish(r.rid)
 
     def run_to_completion(self, default_params: Optional[SamplingParams] = None, max_steps: int = 10 ** 9):

@@ -24,7 +24,7 @@ MAX_HEAD_DIM = 256
 P, I, F, L = c_void_p, c_int, c_float, c_long
 _SIGNATURES = {
     "elementwise": {
-        "li_embedding": [P, P, I, P, I, I, I],
+        "li_embedding": [P, P, P, P, I, P, I, I, I],
         "li_rmsnorm": [P, I, P, F, P, I, I, I],
         "li_gather_rows": [P, P, P, I, I],
         "li_cast": [P, I, P, I, L],
@@ -111,17 +111,25 @@ def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> N
 
 
 # ---------------------------------------------------------------- elementwise
-def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, :] = table[ids[t], :] as float32.  Ids must already be inside the
-    table (the step checks them on the host)."""
-    _gpu(ids, table, out)
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor,
+              id_src: Optional[torch.Tensor] = None, feedback: Optional[torch.Tensor] = None) -> None:
+    """out[t, :] = table[id(t), :] as float32 with id(t) = ids[t], or
+    feedback[id_src[t]] where id_src is given and id_src[t] >= 0 (a token chosen
+    on the device that the host has not seen yet).  Ids given by the host must
+    already be inside the table (the step checks them); an id outside it leaves
+    the row as it is."""
+    _gpu(ids, table, out, id_src, feedback)
     t, h = out.shape
     _chk(ids.dtype is torch.int32 and ids.numel() == t and ids.is_contiguous(), "embedding: ids")
     _chk(table.dim() == 2 and table.shape[1] == h and table.is_contiguous() and table.dtype in _DT,
          "embedding: table")
     _chk(out.dtype is torch.float32 and out.is_contiguous(), "embedding: out must be float32")
+    _chk(id_src is None or (feedback is not None and id_src.dtype is torch.int32 and id_src.numel() == t
+                            and id_src.is_contiguous() and feedback.dtype is torch.int32
+                            and feedback.is_contiguous()), "embedding: id_src / feedback")
     if t:
-        _run("elementwise", "li_embedding", ids.data_ptr(), table.data_ptr(), _DT[table.dtype],
+        _run("elementwise", "li_embedding", ids.data_ptr(), 0 if id_src is None else id_src.data_ptr(),
+             0 if id_src is None else feedback.data_ptr(), table.data_ptr(), _DT[table.dtype],
              out.data_ptr(), t, h, table.shape[0])
 
 

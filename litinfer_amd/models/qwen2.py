@@ -36,7 +36,7 @@ class Qwen2:
     def __init__(self, model_path, device: str = "cuda:0", quantize: Optional[str] = None, *,
                  dtype: str = "bfloat16", page_size: int = 16, num_pages: Optional[int] = None,
                  max_tokens: Optional[int] = None, max_seqs: int = 64, max_batch_tokens: int = 2048,
-                 chunk_size: int = 512, seed: int = 0):
+                 chunk_size: int = 512, seed: int = 0, lookahead: bool = True):
         if quantize is not None:
             raise NotImplementedError("quantized weights are not supported")
         self.model_path = Path(model_path)
@@ -45,7 +45,9 @@ class Qwen2:
                                       num_pages=num_pages, max_tokens=max_tokens, max_seqs=max_seqs)
         self.meta = self.engine.config
         self.seed = int(seed)
-        self._sched_args = dict(max_batch_tokens=max_batch_tokens, chunk_size=chunk_size)
+        # lookahead: a step is started before the tokens of the one before have reached the host
+        self._sched_args = dict(max_batch_tokens=max_batch_tokens, chunk_size=chunk_size,
+                                lookahead=bool(lookahead))
         self._scheduler: Optional[Scheduler] = None
         print(f"[litinfer_amd] ready: {self.engine.spec.architecture}, "
               f"{self.engine.model.weight_bytes() / 2**20:.1f} MiB of weights", flush=True)

@@ -32,8 +32,8 @@ class TokenEmbedding(Part):
     def load_params(self, get):
         self.table = self.rt.matrix(get(self.prefix + "weight"))
 
-    def forward(self, ids, out):
-        ops.embedding(ids, self.table, out)
+    def forward(self, ids, out, id_src=None, feedback=None):
+        ops.embedding(ids, self.table, out, id_src, feedback)
         return out
 
 

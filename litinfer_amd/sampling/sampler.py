@@ -11,7 +11,7 @@ on what else is in the batch or on how the steps were cut.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -43,25 +43,77 @@ def uniform(seed: int, counter: int) -> float:
     return (z >> 40) / float(1 << 24)
 
 
+class PendingTokens:
+    """Tokens that were chosen on the device and are on their way to the host."""
+
+    def __init__(self, sampler, host: torch.Tensor, n: int, event):
+        self._sampler, self._host, self._n, self._event = sampler, host, n, event
+        self._tokens: Optional[List[int]] = None
+
+    def result(self) -> List[int]:
+        """The tokens; waits for the device if they are not there yet."""
+        if self._tokens is None:
+            if self._event is not None:
+                self._event.synchronize()
+            self._tokens = self._host[:self._n].tolist()
+            self._sampler._give_back(self._host)
+            self._host = None
+        return self._tokens
+
+
 class Sampler:
     def __init__(self, device):
         self.device = torch.device(device)
+        self._free_host: List[torch.Tensor] = []
+        self._params_up = None
+
+    def _host_buffer(self, n: int) -> torch.Tensor:
+        for i, b in enumerate(self._free_host):
+            if b.numel() >= n:
+                return self._free_host.pop(i)
+        return torch.empty(max(n, 256), dtype=torch.int32, pin_memory=self.device.type == "cuda")
+
+    def _give_back(self, buf: torch.Tensor) -> None:
+        if len(self._free_host) < 8:
+            self._free_host.append(buf)
+
+    def sample_async(self, logits: torch.Tensor, params: Sequence[SamplingParams], counters: Sequence[int],
+                     out: Optional[torch.Tensor] = None) -> PendingTokens:
+        """One token for each row of logits [n, vocab] (float32, on the device),
+        written to out[:n] (int32, on the device; e.g. the engine's feedback
+        buffer, from which the next step can take them) and copied to the host
+        without waiting: `result()` of what is returned waits and gives the list."""
+        n = logits.shape[0]
+        assert n == len(params) == len(counters)
+        if out is None:
+            out = torch.empty(n, dtype=torch.int32, device=self.device)
+        assert out.dtype is torch.int32 and out.numel() >= n and out.device == logits.device
+        ids = out[:n]
+        if all(p.greedy for p in params):
+            ops.argmax_rows(logits, ids)
+        else:
+            host = np.empty((4, n), dtype=np.float32)
+            host[0] = [p.temperature if p.temperature > 0 else 0.0 for p in params]
+            host[1] = [p.top_p for p in params]
+            host[2] = [uniform(p.seed, c) for p, c in zip(params, counters)]
+            host[3] = np.array([p.top_k for p in params], dtype=np.int32).view(np.float32)
+            if self._params_up is None:
+                from ..engine.batch import BatchUploader
+                self._params_up = BatchUploader(self.device)       # pinned, so the copy does not wait for the stream
+            dev = self._params_up.upload([host.view(np.int32)])[0]
+            f = dev.view(torch.float32)
+            ops.sample_rows(logits, f[0], dev[3], f[1], f[2], ids)
+        hb = self._host_buffer(n)
+        if self.device.type == "cuda":
+            hb[:n].copy_(ids, non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+        else:
+            hb[:n].copy_(ids)
+            ev = None
+        return PendingTokens(self, hb, n, ev)
 
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams],
                counters: Sequence[int]) -> List[int]:
         """One token for each row of logits [n, vocab] (float32, on the device)."""
-        n = logits.shape[0]
-        assert n == len(params) == len(counters)
-        out = torch.empty(n, dtype=torch.int32, device=self.device)
-        if all(p.greedy for p in params):
-            ops.argmax_rows(logits, out)
-            return out.tolist()
-        host = np.empty((4, n), dtype=np.float32)
-        host[0] = [p.temperature if p.temperature > 0 else 0.0 for p in params]
-        host[1] = [p.top_p for p in params]
-        host[2] = [uniform(p.seed, c) for p, c in zip(params, counters)]
-        topk = np.array([p.top_k for p in params], dtype=np.int32)
-        host[3] = topk.view(np.float32)
-        dev = torch.from_numpy(host).to(self.device)
-        ops.sample_rows(logits, dev[0], dev[3].view(torch.int32), dev[1], dev[2], out)
-        return out.tolist()
+        return self.sample_async(logits, params, counters).result()

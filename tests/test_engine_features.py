@@ -512,3 +512,62 @@ def test_a_toy_routed_feed_forward_and_another_position_encoding(tmp_path, devic
     for kind in ("whole", "tail", "chunks", "mixed"):
         out = schedules.run(eng, reqs, getattr(schedules, kind)(reqs))
         assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind
+
+
+# ----------------------------- tokens fed back on the device, steps started ahead
+def test_an_entry_takes_its_token_from_the_feedback_buffer(tmp_path, device):
+    d = helpers.make_model(tmp_path, TINY_A, 0)
+    prompt = helpers.random_requests(256, [12], 5)["r0"]
+    eng = engine_for(d, device)
+    want = eng.step([StepEntry("a", prompt[:8], []), StepEntry("b", prompt, [11])]).clone()
+    eng.finish("a"), eng.finish("b")
+    # the same batch with three of the ids given through the buffer, beside wrong numbers in `tokens`
+    eng.feedback[5], eng.feedback[9], eng.feedback[2] = prompt[7], prompt[0], prompt[11]
+    a = StepEntry("a", prompt[:7] + [0], [], take=[-1] * 7 + [5])
+    b = StepEntry("b", [1] + prompt[1:11] + [3], [11], take=[9] + [-1] * 10 + [2])
+    got = eng.step([a, b])
+    assert torch.equal(got, want)
+    with pytest.raises(StepError):
+        eng.step([StepEntry("c", [1, 2], [], take=[0])])          # one place for two tokens
+
+
+@pytest.mark.parametrize("sampled", [False, True])
+def test_steps_started_ahead_give_the_same_tokens(tmp_path, device, sampled):
+    """The scheduler with lookahead against the one that waits for every token:
+    end tokens (found out one step late), length limits, portions, preemption."""
+    from litinfer_amd.engine import Scheduler
+    from litinfer_amd.sampling import SamplingParams
+    d = helpers.make_model(tmp_path, TINY_B, 1)
+    prompts = list(helpers.random_requests(320, [3, 30, 70, 9, 41, 18], 13).values())
+    limits = [40, 9, 25, 1, 33, 2]
+
+    def run(lookahead, eos, max_tokens):
+        eng = engine_for(d, device, page=8, max_tokens=max_tokens)
+        s = Scheduler(eng, eos_token_ids=eos, chunk_size=16, max_batch_tokens=40, lookahead=lookahead)
+        ids = [s.add_request(p, n, SamplingParams(temperature=0.9, top_k=50, seed=i) if sampled else None)
+               for i, (p, n) in enumerate(zip(prompts, limits))]
+        order = []
+        while s.has_unfinished():
+            order += s.step()
+            assert s.steps < 2000, "the scheduler does not come to an end"
+        eng.cache.check_invariants()
+        assert all(f == g.pool.capacity for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
+        by_request = {i: [t for r, t in order if r == i] for i in ids}
+        assert all(by_request[i] == s.output(i) for i in ids)        # every kept token was reported once
+        return [s.output(i) for i in ids], [s.requests[i].finish_reason for i in ids], s.preemptions, s.steps
+
+    free = run(False, (), 1024)
+    assert [len(t) for t in free[0]] == limits
+    # end tokens taken from what the requests do generate, so that some of them end early
+    eos = (free[0][0][10], free[0][2][5], free[0][4][20])
+    wait, ahead = run(False, eos, 1024), run(True, eos, 1024)
+    assert ahead[:2] == wait[:2]
+    assert "eos" in wait[1] and "length" in wait[1]
+    assert any(len(t) < n for t, n in zip(wait[0], limits))
+    # a pool so tight that running requests outgrow it and are preempted (and one of them with its
+    # newest token still on its way)
+    wait, ahead = run(False, (), 96), run(True, (), 96)
+    assert ahead[:2] == wait[:2] and ahead[0] == free[0]
+    assert wait[2] > 0 and ahead[2] > 0
+    wait, ahead = run(False, eos[1:], 96), run(True, eos[1:], 96)
+    assert ahead[:2] == wait[:2] and ahead[2] > 0

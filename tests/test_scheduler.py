@@ -144,6 +144,20 @@ def test_waiting_request_is_admitted_when_pages_come_back():
     assert s.output(b) == [5, 6] and s.requests[a].preemptions == 0
 
 
+def test_prompts_cut_into_portions_do_not_share_out_the_pool_and_stall():
+    # three prompts of 20 tokens in portions of 4, a pool of 8 pages of 4: each fits alone, two fit
+    # together, three do not.  Admitting each on its first portion would leave all three holding
+    # pages with none able to finish.
+    e = FakeEngine(num_pages=8, page=4, max_seqs=4)
+    s = sched(e, max_batch_tokens=12, chunk_size=4)
+    ids = [s.add_request([i] * 14, max_new_tokens=3) for i in range(3)]
+    s.step()
+    assert [r.state for r in s.requests.values()] == ["running", "running", "waiting"]
+    s.run_to_completion(max_steps=200)
+    assert not s.has_unfinished() and s.preemptions == 0
+    assert all(len(s.output(i)) == 3 for i in ids)
+
+
 def test_a_lone_request_that_outgrows_the_pool_ends_with_an_error():
     e = FakeEngine(num_pages=2, page=4)
     s = sched(e)

@@ -15,8 +15,11 @@ def require_gpu(device):
     return None
 
 
-def embedding(ids, table, out):
-    out.copy_(table[ids.long()].float())
+def embedding(ids, table, out, id_src=None, feedback=None):
+    ids = ids.long()
+    if id_src is not None:
+        ids = torch.where(id_src >= 0, feedback.long()[id_src.clamp(min=0).long()], ids)
+    out.copy_(table[ids].float())
 
 
 def rmsnorm(x, weight, eps, out):
