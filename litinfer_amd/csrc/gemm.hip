@@ -640,6 +640,12 @@ static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
 //
 // SWIGLU: W is [gate; up] with N rows each: tile 0 takes gate rows, tile 1 the
 // up rows of the same columns, and out[m, n] = up * gate / (1 + exp(-gate)).
+//
+// ROPE (one tile of rows and of columns): W is the packed [q; k; v] projection.  A block takes,
+// of one head, the 8 columns 8 i .. and their partners of the half-split rotation, dh / 2
+// further on, so that lane l and lane l ^ 32 hold the two members of a pair; the epilogue adds
+// the bias, rotates query and key heads by the row's angles (float32 tables), writes the
+// queries to out and keys and values straight into their page slots (and to out as well).
 #define SK_CHUNK 128
 
 struct SkinnyArgs {
@@ -648,10 +654,19 @@ struct SkinnyArgs {
     const float* bias;      // [N] or null
     void* out;              // [M, N]
     int M, N, K, accumulate;
+    // ROPE (the packed q/k/v projection of a decoding step): rotary tables [M, dh / 2], the page
+    // slot of each row, the cache layer's keys and values [pages, nkv, page_size, dh]
+    const float* cos;
+    const float* sin;
+    const int* slot_map;
+    bf16_t* kc;
+    bf16_t* vc;
+    int nh, nkv, dh, page_size, num_pages;
 };
 
-template <int MT, int NT, int WAVES, bool SWIGLU, typename TO>
+template <int MT, int NT, int WAVES, bool SWIGLU, typename TO, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs a) {
+    static_assert(!ROPE || (MT == 1 && NT == 1 && !SWIGLU), "the rotary epilogue takes one tile");
     __shared__ floatx4 red[WAVES][MT * NT][64];
     const int M = a.M, N = a.N, K = a.K;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -662,7 +677,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     for (int nt = 0; nt < NT; ++nt) {
         int row;
         if (SWIGLU) row = ((n0 + r16 < N) ? n0 + r16 : N - 1) + nt * N;      // gate row, up row
-        else row = (n0 + 16 * nt + r16 < N) ? n0 + 16 * nt + r16 : N - 1;    // rows past the end repeat the last
+        else if (ROPE) {
+            const int bph = a.dh / 16, head = blockIdx.x / bph, i = blockIdx.x % bph;
+            row = head * a.dh + 8 * i + (r16 < 8 ? r16 : a.dh / 2 + r16 - 8);
+        } else row = (n0 + 16 * nt + r16 < N) ? n0 + 16 * nt + r16 : N - 1;    // rows past the end repeat the last
         wrow[nt] = a.w + (size_t)row * K + 8 * g;
     }
     // x is read with whole rows of a chunk contiguous over 16 lanes (lane l: row l / 16 + 4 i,
@@ -764,7 +782,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     for (int t = threadIdx.x; t < MT * 64; t += WAVES * 64) {
         const int mt = t >> 6, l = t & 63;
         const int m = 16 * mt + (l & 15);
-        if (m >= M) continue;
+        if (m >= M) continue;                       // (with ROPE lanes l and l ^ 32 share m: both stay or both go)
         floatx4 s[NT];
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -775,7 +793,36 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 s[nt][0] += o[0]; s[nt][1] += o[1]; s[nt][2] += o[2]; s[nt][3] += o[3];
             }
         }
-        if constexpr (SWIGLU) {
+        if constexpr (ROPE) {
+            const int dh = a.dh, half = dh / 2, bph = dh / 16;
+            const int head = blockIdx.x / bph, i = blockIdx.x % bph;
+            const bool second = (l >> 4) >= 2;                       // this lane holds the pairs' second members
+            const int slot = a.slot_map[m];
+            const int page = slot / a.page_size, in_page = slot - page * a.page_size;
+            const bool page_ok = page >= 0 && page < a.num_pages;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = 8 * i + 4 * ((l >> 4) & 1) + r;        // the pair's number within the head
+                const int d = second ? half + j : j;
+                const int col = head * dh + d;
+                float own = s[0][r];
+                if (a.bias) own += a.bias[col];
+                const float other = __shfl_xor(own, 32, 64);
+                float v = own;
+                if (head < a.nh + a.nkv) {
+                    const float c = a.cos[(size_t)m * half + j], sn = a.sin[(size_t)m * half + j];
+                    v = second ? own * c + other * sn : own * c - other * sn;
+                }
+                const uint16_t bits = float_to_bf16(v);
+                reinterpret_cast<bf16_t*>(out)[(size_t)m * N + col].bits = bits;
+                if (head >= a.nh && page_ok) {
+                    const bool is_k = head < a.nh + a.nkv;
+                    const int kvh = is_k ? head - a.nh : head - a.nh - a.nkv;
+                    bf16_t* dst = (is_k ? a.kc : a.vc) + (((size_t)page * a.nkv + kvh) * a.page_size + in_page) * dh + d;
+                    dst->bits = bits;
+                }
+            }
+        } else if constexpr (SWIGLU) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int n = n0 + 4 * (l >> 4) + r;
@@ -816,7 +863,8 @@ extern "C" int li_linear_skinny(const void* x, const void* w, const float* bias,
     if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K % 8)) return LI_ERR_SIZE;
     if (accumulate && out_dtype != LI_F32) return LI_ERR_DTYPE;
     if (swiglu && (bias || accumulate || out_dtype != LI_BF16)) return LI_ERR_DTYPE;
-    SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, accumulate};
+    SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, accumulate,
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
     if (swiglu) launch_skinny<true, bf16_t>(a, stream);
     else if (out_dtype == LI_BF16) launch_skinny<false, bf16_t>(a, stream);
     else if (out_dtype == LI_F32) launch_skinny<false, float>(a, stream);
@@ -931,4 +979,21 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     if (c_mid <= c_small) return LI_DMA(256, 128, 64, 3);
     return LI_DMA(128, 128, 64, 4);
 #undef LI_DMA
+}
+
+// The packed q/k/v projection of up to 16 rows with the half-split rotary encoding of query and key
+// heads and the write of keys and values into their page slots as its epilogue (see ROPE above).
+// w [(nh + 2 nkv) dh, K] bfloat16, bias float32 or null, out [M, (nh + 2 nkv) dh] bfloat16 (rotated
+// q, rotated k, v), cos/sin float32 [M, dh / 2], slot_map int32 [M], kc/vc the cache layer.
+extern "C" int li_linear_rope_store(const void* x, const void* w, const float* bias, void* out, int M, int K,
+                                    const float* cos, const float* sin, const int* slot_map, void* kc, void* vc,
+                                    int nh, int nkv, int dh, int page_size, int num_pages, hipStream_t stream) {
+    if (M <= 0 || M > 16 || K <= 0 || K % 8 || nh <= 0 || nkv <= 0 || dh <= 0 || dh % 16 || page_size <= 0 ||
+        num_pages <= 0 || (long)(nh + 2 * nkv) * dh > 0x7fffffffL)
+        return LI_ERR_SIZE;
+    const int N = (nh + 2 * nkv) * dh;
+    SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, 0, cos, sin, slot_map,
+                 (bf16_t*)kc, (bf16_t*)vc, nh, nkv, dh, page_size, num_pages};
+    gemm_bf16_skinny_kernel<1, 1, 8, false, bf16_t, true><<<N / 16, 8 * 64, 0, stream>>>(a);
+    return li_launch_status();
 }

@@ -38,6 +38,7 @@ _SIGNATURES = {
         "li_linear": [P, P, P, P, I, I, I, I, I, I, P, L],
         "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
         "li_linear_swiglu": [P, P, P, I, I, I],
+        "li_linear_rope_store": [P, P, P, P, I, I, P, P, P, P, P, I, I, I, I, I],
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
@@ -327,6 +328,41 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_swiglu: contiguous operands")
     _chk(x.dtype is torch.bfloat16 and out.dtype is torch.bfloat16, "linear_swiglu: x and out must be bfloat16")
     _run("gemm", "li_linear_swiglu", x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k)
+
+
+ROPE_STORE_MAX_ROWS = 16
+
+
+def rope_store_takes(m: int, k: int, w_dtype: torch.dtype, dh: int, rotary_dim: int) -> bool:
+    """Whether `linear_rope_store` takes the packed projection of m rows over k."""
+    return (w_dtype is torch.bfloat16 and 0 < m <= ROPE_STORE_MAX_ROWS and k % 8 == 0
+            and dh % 16 == 0 and rotary_dim == dh)
+
+
+def linear_rope_store(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                      nh: int, nkv: int, dh: int, cos: torch.Tensor, sin: torch.Tensor,
+                      slot_map: torch.Tensor, k: torch.Tensor, v: torch.Tensor, page_size: int) -> None:
+    """Fused for a decoding step: out = x w^T + bias with w the packed [q; k; v]
+    projection, query and key heads rotated (half-split pairs, the whole head) by
+    the rows' angles, keys and values written into their page slots.  out holds
+    the rotated queries and keys and the values, as after the separate kernels."""
+    _gpu(x, w, bias, out, cos, sin, slot_map, k, v)
+    m, kk = x.shape
+    n = (nh + 2 * nkv) * dh
+    _chk(rope_store_takes(m, kk, w.dtype, dh, 2 * cos.shape[1]), "linear_rope_store: sizes or dtype not taken")
+    _chk(w.shape == (n, kk) and out.shape == (m, n), "linear_rope_store: shapes do not fit")
+    _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_rope_store: contiguous operands")
+    _chk(x.dtype is torch.bfloat16 and out.dtype is torch.bfloat16, "linear_rope_store: x and out must be bfloat16")
+    _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
+         "linear_rope_store: bias must be float32 [N]")
+    _check_cache(k, v, nkv, dh, page_size, out.dtype)
+    _chk(cos.shape == (m, dh // 2) and sin.shape == cos.shape and cos.dtype is torch.float32
+         and sin.dtype is torch.float32 and cos.is_contiguous() and sin.is_contiguous(), "linear_rope_store: tables")
+    _chk(slot_map.dtype is torch.int32 and slot_map.numel() == m and slot_map.is_contiguous(),
+         "linear_rope_store: slot_map")
+    _run("gemm", "li_linear_rope_store", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
+         out.data_ptr(), m, kk, cos.data_ptr(), sin.data_ptr(), slot_map.data_ptr(), k.data_ptr(), v.data_ptr(),
+         nh, nkv, dh, page_size, k.shape[0])
 
 
 # ----------------------------------------------------------------- attention

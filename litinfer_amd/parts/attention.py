@@ -83,12 +83,15 @@ class GQAttention(Mixer):
     def forward(self, xn, residual, ctx, cache):
         t = xn.shape[0]
         qkv = ctx.ws.buffer("attn.qkv", (t, self.n_q + 2 * self.n_kv), self.rt.dtype)
-        self.qkv(xn, qkv, ws=ctx.ws)
-        if self.position is not None:
-            self.position.encode_and_store(qkv, self.nh, self.nkv, self.dh, ctx, cache)
-        elif cache.owned:
-            ops.kv_store(qkv, self.nh, self.nkv, self.dh, ctx.slot_map(cache.group),
-                         cache.k, cache.v, cache.page_size)
+        fused = self.position is not None and self.position.project_encode_store(
+            self.qkv, xn, qkv, self.nh, self.nkv, self.dh, ctx, cache)
+        if not fused:                                # else projection, encoding and page write were one kernel
+            self.qkv(xn, qkv, ws=ctx.ws)
+            if self.position is not None:
+                self.position.encode_and_store(qkv, self.nh, self.nkv, self.dh, ctx, cache)
+            elif cache.owned:
+                ops.kv_store(qkv, self.nh, self.nkv, self.dh, ctx.slot_map(cache.group),
+                             cache.k, cache.v, cache.page_size)
         attn = ctx.ws.buffer("attn.out", (t, self.n_q), self.rt.dtype)
         ops.paged_attention(qkv, attn, cache.k, cache.v, ctx.attention_meta(cache.group),
                             self.nh, self.nkv, self.dh, cache.page_size, self.window, self.scale, ws=ctx.ws)

@@ -376,6 +376,46 @@ def test_rope_kv_store_and_plain_store(ops, dtype):
                            qkv[i, (nh + nkv) * dh:].reshape(nkv, dh))
 
 
+@pytest.mark.parametrize("t,nh,nkv,dh,k,bias", [
+    (8, 28, 4, 128, 3584, True),        # a decoding step at the 7B layer sizes
+    (1, 3, 1, 32, 96, True),
+    (16, 5, 5, 48, 120, False),         # a head size that is no power of two
+    (3, 6, 2, 64, 136, True),
+])
+def test_projection_with_rotary_encoding_and_page_write_as_its_epilogue(ops, t, nh, nkv, dh, k, bias):
+    g = torch.Generator().manual_seed(16)
+    n, page, pages = (nh + 2 * nkv) * dh, 8, 9
+    x = (torch.randn(t, k, generator=g) * 2).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    b = torch.randn(n, generator=g) if bias else None
+    pos = torch.randint(0, 3000, (t,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(pages * page, generator=g)[:t].to(torch.int32)
+    cos = torch.empty(t, dh // 2, device=DEV)
+    sin = torch.empty(t, dh // 2, device=DEV)
+    ops.rope_table(pos.to(DEV), 1e6, dh, cos, sin)
+    kc = torch.full((pages, nkv, page, dh), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full_like(kc, 7.0)
+    out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert ops.rope_store_takes(t, k, w.dtype, dh, dh)
+    ops.linear_rope_store(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, nh, nkv, dh, cos, sin,
+                          slots.to(DEV), kc, vc, page)
+    y = x.double().numpy() @ w.double().numpy().T
+    if b is not None:
+        y = y + b.double().numpy()
+    y = y.reshape(t, nh + 2 * nkv, dh)
+    ref = np.concatenate([plain_impl.rope_neox(y[:, :nh + nkv], pos.numpy(), 1e6), y[:, nh + nkv:]], axis=1)
+    assert rel(out, ref.reshape(t, n)) < 5e-3
+    o = out.cpu().view(t, nh + 2 * nkv, dh)
+    touched = torch.zeros(pages, page, dtype=torch.bool)
+    for i in range(t):                                   # the pages hold exactly what out holds
+        s = int(slots[i])
+        touched[s // page, s % page] = True
+        assert torch.equal(kc[s // page, :, s % page].cpu(), o[i, nh:nh + nkv])
+        assert torch.equal(vc[s // page, :, s % page].cpu(), o[i, nh + nkv:])
+    untouched = ~touched[:, None, :, None].expand(pages, nkv, page, dh)
+    assert (kc.cpu()[untouched] == 7.0).all() and (vc.cpu()[untouched] == 7.0).all()
+
+
 @pytest.mark.parametrize("shape", [(1, 4), (3, 4096), (5, 152064), (2, 301)])
 def test_argmax_rows_lowest_index_wins(ops, shape):
     g = torch.Generator().manual_seed(10)

@@ -135,12 +135,31 @@ def linear_swiglu(x, w, out):
     linear_skinny(x, w, None, out, False, swiglu=True)
 
 
+def rope_store_takes(m, k, w_dtype, dh, rotary_dim):
+    return w_dtype is torch.bfloat16 and 0 < m <= 16 and k % 8 == 0 and dh % 16 == 0 and rotary_dim == dh
+
+
+def linear_rope_store(x, w, bias, out, nh, nkv, dh, cos, sin, slot_map, k, v, page_size):
+    y = x.float() @ w.float().T
+    if bias is not None:
+        y = y + bias
+    # rotated from the 32-bit sums and rounded once, as the fused kernel does
+    t = y.shape[0]
+    heads = y.view(t, nh + 2 * nkv, dh)
+    rot = heads[:, :nh + nkv]
+    a, b = rot[..., :dh // 2].clone(), rot[..., dh // 2:].clone()
+    c, s = cos[:, None, :], sin[:, None, :]
+    rot[..., :dh // 2], rot[..., dh // 2:] = a * c - b * s, b * c + a * s
+    out.copy_(y.to(out.dtype))
+    kv_store(out, nh, nkv, dh, slot_map, k, v, page_size)
+
+
 def argmax_rows(logits, out):
     out.copy_(torch.argmax(logits, dim=-1).to(torch.int32))
 
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
-       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "check_attention_sizes",
+       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "rope_store_takes", "linear_rope_store", "check_attention_sizes",
        "paged_attention", "argmax_rows"]
 
 
