@@ -657,13 +657,17 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
         for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
     float m = -INFINITY, l = 0.f;
 
+    // Order of a turn: the block fetched during the LAST turn goes from the registers into the
+    // other stage of LDS, the block after it is fetched into the same registers, and then the
+    // block in this stage is worked on: a fetch has a whole turn to arrive.
     LI_PRE_FETCH(k_begin);
     LI_PRE_STASH(0);
+    if (k_begin + 32 < k_end) LI_PRE_FETCH(k_begin + 32);
     __syncthreads();
     int stage = 0;
     for (int kb = k_begin; kb < k_end; kb += 32, stage ^= 1) {
-        const bool more = kb + 32 < k_end;
-        if (more) LI_PRE_FETCH(kb + 32);              // in flight while this block is worked on
+        if (kb + 32 < k_end) LI_PRE_STASH(stage ^ 1);      // (its readers of the turn before are past the barrier)
+        if (kb + 64 < k_end) LI_PRE_FETCH(kb + 64);
         if (active) {
             // ---- S^T = K Q^T
             f32x16_t sv;
@@ -725,7 +729,6 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
                 }
             }
         }
-        if (more) LI_PRE_STASH(stage ^ 1);
         __syncthreads();
     }
     if (!active || ql >= nrows) return;
