@@ -13,6 +13,8 @@ its attention already derives each query's horizon as ctx - qlen + i
 """
 from __future__ import annotations
 
+import os
+import sys
 from pathlib import Path
 from typing import Any, Dict, Hashable, List, Optional, Sequence
 
@@ -23,6 +25,7 @@ from ..cache import CacheFull, CacheManager
 from ..config import load_config, lookup, architecture_name
 from ..config.spec import ModelSpec
 from ..parts.base import Runtime
+from ..utils.profiler import profiler, trace_enabled
 from ..weights import load_into, random_tensor
 from .batch import BatchUploader, StepContext, StepEntry, build_context
 from .model import Model
@@ -75,7 +78,8 @@ class Engine:
         self.steps_run = 0
         # decode steps (every request brings one token) are recorded as HIP graphs, one per batch
         # shape, and replayed: a step is some hundred small launches otherwise
-        self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda"
+        self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda" and not profiler.enabled
+        self._trace = trace_enabled()
         self._graphs: Dict[Any, Any] = {}
         self._graph_generation = (-1, -1)
         self.graph_replays = 0
@@ -119,6 +123,12 @@ class Engine:
     def _make_cache(self) -> None:
         needs, sources = self.model.cache_needs()
         pages = self._num_pages
+        env_pages = os.environ.get("LLAISYS_NUM_BLOCKS", "").strip()
+        if pages is None and self._max_tokens is None and env_pages:
+            # the reference's switch for its pool size (src/llaisys/models/qwen2.cpp:121)
+            if not env_pages.isdigit() or int(env_pages) <= 0:
+                raise ValueError(f"LLAISYS_NUM_BLOCKS must be a positive number of pages, found {env_pages!r}")
+            pages = int(env_pages)
         if pages is None and self._max_tokens is not None:
             pages = -(-int(self._max_tokens) // self.page_size)
         if pages is None:
@@ -193,6 +203,13 @@ class Engine:
                 cache.release(rid)
             raise
         key = self._graph_key(entries)
+        if profiler.enabled:
+            profiler.phase = "decode" if all(len(e.tokens) == 1 for e in entries) else "prefill"
+        if self._trace:
+            print(f"[litinfer_amd trace] step {self.steps_run}: {len(entries)} requests, "
+                  f"{sum(len(e.tokens) for e in entries)} tokens, {sum(len(e.want) for e in entries)} rows of logits, "
+                  f"{'recorded' if key is not None else 'eager'}, free pages {cache.free_pages()}",
+                  file=sys.stderr, flush=True)
         if key is None:
             logits = self.model.forward(self._build_context(entries), cache)
         else:

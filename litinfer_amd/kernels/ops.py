@@ -14,6 +14,7 @@ from typing import Optional
 import torch
 
 from . import build
+from ..utils.profiler import profiler
 
 float32 = torch.float32
 bfloat16 = torch.bfloat16
@@ -70,7 +71,12 @@ def _stream() -> int:
 
 
 def _run(module: str, name: str, *args) -> None:
-    rc = _fn(module, name)(*args, _stream())
+    if profiler.enabled:
+        rc = []
+        profiler.timed(name[3:], lambda: rc.append(_fn(module, name)(*args, _stream())), torch.cuda.synchronize)
+        rc = rc[0]
+    else:
+        rc = _fn(module, name)(*args, _stream())
     if rc != 0:
         raise RuntimeError(f"{name}: the kernel library refused the call (code {rc}): "
                            f"{_ERRORS.get(rc, 'unknown')}")

@@ -82,3 +82,34 @@ def test_order_must_read_an_earlier_owning_entry():
     for bad in ((ExecEntry(0, cache_from=0),), (ExecEntry(0), ExecEntry(1, 0), ExecEntry(1, 1)), (ExecEntry(5),)):
         with pytest.raises(ValueError):
             replace(spec, order=bad).validate()
+
+
+def test_the_references_environment_switches(tmp_path, monkeypatch, capsys, cpu_ops):
+    """LLAISYS_NUM_BLOCKS sizes the pool, LLAISYS_TRACE prints a line per step
+    (src/llaisys/models/qwen2.cpp:19, :121), LLAISYS_PROFILE's table lists the
+    operators by phase (src/utils/profiler.cpp:48-110)."""
+    import io
+    import helpers
+    from tiny_configs import TINY_A
+    from litinfer_amd.engine import Engine, StepEntry
+    from litinfer_amd.utils import OpProfiler
+    d = helpers.make_model(tmp_path, TINY_A, 0)
+    monkeypatch.setenv("LLAISYS_NUM_BLOCKS", "7")
+    monkeypatch.setenv("LLAISYS_TRACE", "1")
+    eng = Engine.from_dir(d, dtype="float32", device="cpu", page_size=16, max_seqs=2)
+    assert eng.cache.groups[0].pool.capacity == 7
+    eng.step([StepEntry("a", [1, 2, 3], [2])])
+    assert "step 0: 1 requests, 3 tokens, 1 rows of logits" in capsys.readouterr().err
+    monkeypatch.setenv("LLAISYS_NUM_BLOCKS", "many")
+    with pytest.raises(ValueError, match="LLAISYS_NUM_BLOCKS"):
+        Engine.from_dir(d, dtype="float32", device="cpu", page_size=16, max_seqs=2)
+    prof = OpProfiler(False)
+    prof.phase = "prefill"
+    prof.timed("linear", lambda: None, lambda: None)
+    prof.phase = "decode"
+    prof.timed("linear", lambda: None, lambda: None)
+    prof.timed("linear", lambda: None, lambda: None)
+    out = io.StringIO()
+    prof.report(out)
+    lines = out.getvalue().splitlines()
+    assert any(l.startswith("decode") and " 2 " in l for l in lines) and any(l.startswith("prefill") for l in lines)
