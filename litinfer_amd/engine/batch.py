@@ -16,6 +16,8 @@ from typing import Any, Callable, Dict, Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
+from ..utils.pinned import BatchUploader
+
 
 @dataclass
 class StepEntry:
@@ -95,51 +97,6 @@ class StepContext:
         if key not in self._shared:
             self._shared[key] = make()
         return self._shared[key]
-
-
-class BatchUploader:
-    """Packs the step's integers into pinned host memory and copies them to
-    the device once.  Two host buffers alternate, each guarded by an event, so
-    a buffer is not rewritten while its copy may still be in flight."""
-
-    def __init__(self, device):
-        self.device = torch.device(device)
-        self._host = [None, None]
-        self._events = [None, None]
-        self._dev = None
-        self._turn = 0
-        self.generation = 0          # goes up when the device buffer moves
-
-    def upload(self, parts: List[np.ndarray]) -> List[torch.Tensor]:
-        offs, total = [], 0
-        for p in parts:
-            offs.append(total)
-            total += (p.size + 3) // 4 * 4            # 16-byte alignment of every array
-        total = max(total, 4)
-        i = self._turn
-        self._turn ^= 1
-        cuda = self.device.type == "cuda"
-        if self._host[i] is None or self._host[i].numel() < total:
-            cap = total * 2
-            self._host[i] = torch.empty(cap, dtype=torch.int32, pin_memory=cuda)
-        elif self._events[i] is not None:
-            self._events[i].synchronize()
-        if self._dev is None or self._dev.numel() < total:
-            self._dev = torch.empty(max(total * 2, 1 << 16), dtype=torch.int32, device=self.device)
-            self.generation += 1
-        h = self._host[i].numpy()
-        for p, o in zip(parts, offs):
-            h[o:o + p.size] = p.reshape(-1)
-        if cuda:
-            # a fresh device buffer per step would be simpler; one buffer is enough because the
-            # copy is ordered on the stream after the kernels of the step before
-            self._dev[:total].copy_(self._host[i][:total], non_blocking=True)
-            ev = torch.cuda.Event()
-            ev.record()
-            self._events[i] = ev
-        else:
-            self._dev[:total].copy_(self._host[i][:total])
-        return [self._dev[o:o + p.size].view(p.shape) for p, o in zip(parts, offs)]
 
 
 def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploader",

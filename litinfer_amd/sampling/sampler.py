@@ -17,6 +17,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
+from ..utils.pinned import BatchUploader
 
 _MASK = (1 << 64) - 1
 
@@ -98,7 +99,6 @@ class Sampler:
             host[2] = [uniform(p.seed, c) for p, c in zip(params, counters)]
             host[3] = np.array([p.top_k for p in params], dtype=np.int32).view(np.float32)
             if self._params_up is None:
-                from ..engine.batch import BatchUploader
                 self._params_up = BatchUploader(self.device)       # pinned, so the copy does not wait for the stream
             dev = self._params_up.upload([host.view(np.int32)])[0]
             f = dev.view(torch.float32)
