@@ -13,6 +13,10 @@ Beside the pages there are `max_seqs` state slots.  A request holds one slot
 from admission to release; mixers with a `StateNeed` get a tensor
 [max_seqs, *shape] indexed by the slot, zeroed at admission.
 
+The bookkeeping itself (pools, tables, slots, the window's give-back) is done by
+the host library in C++ (csrc/host.cpp); this class owns the device tensors,
+maps request names to the library's handles and turns its codes into exceptions.
+
 The reference keeps one pool and one table per layer, all identical
 (src/llaisys/kv_cache/block_kv_cache.hpp:16-96, src/llaisys/models/qwen2.cpp:832-845)
 and frees only when a request ends (:1066-1070).
@@ -22,10 +26,13 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import ctypes
+
 import torch
 
 from ..parts.base import PagedKVNeed, StateNeed
-from .pool import PagePool
+from . import native
+from .pool import PagePool, PagePoolError
 
 
 class CacheFull(RuntimeError):
@@ -51,14 +58,6 @@ class _Group:
     data: torch.Tensor               # [n_entries, 2, pages, kv_heads, page_size, head_dim]
 
 
-@dataclass
-class _Request:
-    slot: int
-    cached: int = 0
-    tables: List[List[int]] = field(default_factory=list)    # per group: logical block -> page or -1
-    first_live: List[int] = field(default_factory=list)      # per group: first block not yet given back
-
-
 class CacheManager:
     def __init__(self, needs: Sequence[object], sources: Sequence[Optional[int]], *,
                  page_size: int, num_pages: int, max_seqs: int, dtype: torch.dtype,
@@ -68,6 +67,8 @@ class CacheManager:
         `num_pages` is the number of pages of EVERY group."""
         if page_size <= 0:
             raise ValueError("cache: page_size must be positive")
+        if int(num_pages) * int(page_size) >= 1 << 31:
+            raise ValueError("cache: more than 2^31 token slots in a group")
         self.page_size = int(page_size)
         self.max_seqs = int(max_seqs)
         self.device = torch.device(device)
@@ -91,16 +92,44 @@ class CacheManager:
                                                    device=self.device)
             else:
                 raise TypeError(f"cache: entry {i} has an unknown cache need {need!r}")
-        for gi, g in enumerate(self.groups):
-            order = None
-            if page_order_seed is not None:
+        orders = None
+        if page_order_seed is not None and self.groups:
+            orders = []
+            for gi in range(len(self.groups)):
                 gen = torch.Generator().manual_seed(page_order_seed + gi)
-                order = torch.randperm(num_pages, generator=gen).tolist()
-            g.pool = PagePool(num_pages, order)
+                orders += torch.randperm(num_pages, generator=gen).tolist()
+        self._lib = native.lib()
+        ng = len(self.groups)
+        self._book = self._lib.li_book_create(self.page_size, self.max_seqs, ng,
+                                              native.int_array([g.need.window for g in self.groups]),
+                                              int(num_pages), native.int_array(orders) if orders else None)
+        err = self._lib.li_book_error(self._book).decode()
+        if err:
+            self._lib.li_book_destroy(self._book)
+            self._book = None
+            raise ValueError(err)
+        self._ints = (ctypes.c_int * max(ng, 1))()
+        for gi, g in enumerate(self.groups):
+            g.pool = PagePool(num_pages, _borrowed=self._lib.li_book_pool(self._book, gi))
             g.data = torch.zeros((len(g.entries), 2, num_pages, g.need.num_kv_heads, self.page_size,
                                   g.need.head_dim), dtype=dtype, device=self.device)
-        self._free_slots = list(range(self.max_seqs))[::-1]
-        self._requests: Dict[Hashable, _Request] = {}
+        # requests are named by any hashable; the book knows them by number
+        self._handles: Dict[Hashable, int] = {}
+        self._next_handle = 0
+
+    def __del__(self):
+        if getattr(self, "_book", None):
+            self._lib.li_book_destroy(self._book)
+            self._book = None
+
+    def _error(self) -> str:
+        return self._lib.li_book_error(self._book).decode()
+
+    def _handle(self, rid) -> int:
+        h = self._handles.get(rid)
+        if h is None:
+            raise KeyError(rid)
+        return h
 
     # ---- views ---------------------------------------------------------
     def view(self, entry: int) -> CacheView:
@@ -116,108 +145,87 @@ class CacheManager:
 
     # ---- requests --------------------------------------------------------
     def has(self, rid) -> bool:
-        return rid in self._requests
+        return rid in self._handles
 
     def live(self) -> List[Hashable]:
-        return list(self._requests)
+        return list(self._handles)
+
+    def handle(self, rid) -> int:
+        """The number under which the host library knows a live request."""
+        return self._handle(rid)
+
+    @property
+    def book(self):
+        return self._book
 
     def free_slots(self) -> int:
-        return len(self._free_slots)
+        return self._lib.li_book_free_slots(self._book)
 
     def free_pages(self) -> List[int]:
-        return [g.pool.free for g in self.groups]
+        self._lib.li_book_free_pages(self._book, self._ints)
+        return list(self._ints[:len(self.groups)])
 
     def admit(self, rid) -> int:
-        if rid in self._requests:
+        if rid in self._handles:
             raise KeyError(f"cache: request {rid!r} is already live")
-        if not self._free_slots:
-            raise CacheFull(f"cache: all {self.max_seqs} state slots are taken")
-        slot = self._free_slots.pop()
-        self._requests[rid] = _Request(slot, 0, [[] for _ in self.groups], [0 for _ in self.groups])
+        h = self._next_handle
+        slot = self._lib.li_book_admit(self._book, h)
+        if slot == native.ERR_FULL:
+            raise CacheFull(self._error())
+        if slot < 0:
+            raise RuntimeError(self._error())
+        self._next_handle += 1
+        self._handles[rid] = h
         for st in self._entry_state.values():
             st[slot].zero_()
         return slot
 
     def slot(self, rid) -> int:
-        return self._requests[rid].slot
+        return self._lib.li_book_slot(self._book, self._handle(rid))
 
     def cached_len(self, rid) -> int:
-        return self._requests[rid].cached
+        return self._lib.li_book_cached(self._book, self._handle(rid))
 
     def block_table(self, rid, group: int) -> List[int]:
-        return self._requests[rid].tables[group]
+        h = self._handle(rid)
+        n = self._lib.li_book_table_len(self._book, h, group)
+        buf = (ctypes.c_int * max(n, 1))()
+        self._lib.li_book_table(self._book, h, group, buf, n)
+        return list(buf[:n])
 
-    def _first_needed_block(self, g: _Group, first_query_pos: int) -> int:
-        """First block that a query at `first_query_pos` or later can see."""
-        if g.need.window <= 0:
-            return 0
-        return max(0, first_query_pos - g.need.window + 1) // self.page_size
+    def table_len(self, rid, group: int) -> int:
+        return self._lib.li_book_table_len(self._book, self._handle(rid), group)
 
     def pages_needed(self, rid, n_new: int, cached: Optional[int] = None) -> List[int]:
         """Pages each group must take so that `n_new` more tokens of `rid` fit
         (rid may be unknown: then it is counted as a new request)."""
-        r = self._requests.get(rid)
-        have_cached = (r.cached if r is not None else 0) if cached is None else cached
-        out = []
-        for gi, g in enumerate(self.groups):
-            nblk = -(-(have_cached + n_new) // self.page_size)
-            have = len(r.tables[gi]) if r is not None else 0
-            out.append(max(0, nblk - have))
-        return out
+        h = self._handles.get(rid, -1)
+        self._lib.li_book_pages_needed(self._book, h, int(n_new), -1 if cached is None else int(cached), self._ints)
+        return list(self._ints[:len(self.groups)])
 
     def reserve(self, rid, n_new: int) -> None:
         """Take the pages that positions cached..cached+n_new-1 need, in every
         group, or none at all (CacheFull)."""
-        r = self._requests[rid]
-        need = self.pages_needed(rid, n_new)
-        for g, n in zip(self.groups, need):
-            if n > g.pool.free:
-                raise CacheFull(f"cache: request {rid!r} needs {n} more pages, "
-                                f"{g.pool.free} of {g.pool.capacity} are free")
-        for gi, (g, n) in enumerate(zip(self.groups, need)):
-            for _ in range(n):
-                r.tables[gi].append(g.pool.alloc())
+        rc = self._lib.li_book_reserve(self._book, self._handle(rid), int(n_new))
+        if rc == native.ERR_FULL:
+            raise CacheFull(f"{self._error()} (request {rid!r})")
+        if rc < 0:
+            raise PagePoolError(self._error())
 
     def commit(self, rid, n_new: int) -> None:
         """`n_new` tokens were written: advance, and give back the pages that
         the window has passed."""
-        r = self._requests[rid]
-        r.cached += n_new
-        for gi, g in enumerate(self.groups):
-            if g.need.window <= 0:
-                continue
-            keep_from = self._first_needed_block(g, r.cached)
-            for b in range(r.first_live[gi], min(keep_from, len(r.tables[gi]))):
-                if r.tables[gi][b] >= 0:
-                    g.pool.release(r.tables[gi][b])
-                    r.tables[gi][b] = -1
-            r.first_live[gi] = max(r.first_live[gi], min(keep_from, len(r.tables[gi])))
+        if self._lib.li_book_commit(self._book, self._handle(rid), int(n_new)) < 0:
+            raise PagePoolError(self._error())
 
     def release(self, rid) -> None:
-        r = self._requests.pop(rid)
-        for gi, g in enumerate(self.groups):
-            for p in r.tables[gi]:
-                if p >= 0:
-                    g.pool.release(p)
-        self._free_slots.append(r.slot)
+        h = self._handles.pop(rid)
+        if self._lib.li_book_release(self._book, h) < 0:
+            raise PagePoolError(self._error())
 
     def check_invariants(self) -> None:
         """No page lost, held twice or on the free list while in a table."""
-        for gi, g in enumerate(self.groups):
-            seen = {}
-            for rid, r in self._requests.items():
-                for p in r.tables[gi]:
-                    if p < 0:
-                        continue
-                    if p in seen:
-                        raise AssertionError(f"page {p} of group {gi} is held by {seen[p]!r} and {rid!r}")
-                    if not g.pool.is_held(p):
-                        raise AssertionError(f"page {p} of group {gi} is in a table but free")
-                    seen[p] = rid
-            if len(seen) != g.pool.used:
-                raise AssertionError(f"group {gi}: {g.pool.used} pages taken, {len(seen)} in tables")
-        slots = [r.slot for r in self._requests.values()]
-        if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):
-            raise AssertionError("state slots are held twice or free while held")
-        if len(slots) + len(self._free_slots) != self.max_seqs:
-            raise AssertionError("state slots lost")
+        if self._lib.li_book_check(self._book) < 0:
+            raise AssertionError(self._error())
+        if self._lib.li_book_num_live(self._book) != len(self._handles):
+            raise AssertionError("the book and the request names disagree")

@@ -1,4 +1,4 @@
-"""A pool of page ids with a free list.
+"""A pool of page ids with a free list (kept by the host library, csrc/host.cpp).
 
 The reference's pool (src/llaisys/kv_cache/block_kv_cache.hpp:16-63) is a LIFO
 list per layer without a guard; here one id is valid for every layer of a
@@ -6,7 +6,9 @@ group, and taking a page twice or giving one back twice is an error.
 """
 from __future__ import annotations
 
-from typing import Iterable, List, Optional
+from typing import Iterable, Optional
+
+from . import native
 
 
 class PagePoolError(RuntimeError):
@@ -14,42 +16,55 @@ class PagePoolError(RuntimeError):
 
 
 class PagePool:
-    def __init__(self, num_pages: int, order: Optional[Iterable[int]] = None):
-        if num_pages <= 0:
-            raise ValueError(f"page pool: needs at least one page, found {num_pages}")
-        self.capacity = int(num_pages)
-        ids = list(range(self.capacity)) if order is None else [int(i) for i in order]
-        if sorted(ids) != list(range(self.capacity)):
+    def __init__(self, num_pages: int, order: Optional[Iterable[int]] = None, _borrowed=None):
+        self._lib = native.lib()
+        self._owned = _borrowed is None
+        if _borrowed is not None:                      # a group's pool inside a cache manager's book
+            self._p = _borrowed
+            return
+        ids = None if order is None else [int(i) for i in order]
+        if ids is not None and len(ids) != int(num_pages):
             raise ValueError("page pool: the free-list order must be a permutation of all page ids")
-        self._free: List[int] = ids[::-1]          # alloc() pops from the end: first id of `order` first
-        self._held = [False] * self.capacity
-        self.total_allocations = 0
+        self._p = self._lib.li_pool_create(int(num_pages), native.int_array(ids) if ids is not None else None)
+        if self.capacity == 0:
+            msg = self._lib.li_pool_error(self._p).decode()
+            self._lib.li_pool_destroy(self._p)
+            self._p = None
+            raise ValueError(msg)
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and getattr(self, "_p", None):
+            self._lib.li_pool_destroy(self._p)
+            self._p = None
+
+    def _fail(self):
+        raise PagePoolError(self._lib.li_pool_error(self._p).decode())
+
+    @property
+    def capacity(self) -> int:
+        return self._lib.li_pool_capacity(self._p)
 
     @property
     def free(self) -> int:
-        return len(self._free)
+        return self._lib.li_pool_free(self._p)
 
     @property
     def used(self) -> int:
-        return self.capacity - len(self._free)
+        return self.capacity - self.free
+
+    @property
+    def total_allocations(self) -> int:
+        return self._lib.li_pool_total_allocations(self._p)
 
     def alloc(self) -> int:
-        if not self._free:
-            raise PagePoolError("page pool: no free page")
-        p = self._free.pop()
-        if self._held[p]:
-            raise PagePoolError(f"page pool: page {p} was on the free list while held")
-        self._held[p] = True
-        self.total_allocations += 1
+        p = self._lib.li_pool_alloc(self._p)
+        if p < 0:
+            self._fail()
         return p
 
     def release(self, page: int) -> None:
-        if not 0 <= page < self.capacity:
-            raise PagePoolError(f"page pool: page id {page} out of range")
-        if not self._held[page]:
-            raise PagePoolError(f"page pool: page {page} freed twice")
-        self._held[page] = False
-        self._free.append(page)
+        if self._lib.li_pool_release(self._p, int(page)) < 0:
+            self._fail()
 
     def is_held(self, page: int) -> bool:
-        return self._held[page]
+        return bool(self._lib.li_pool_is_held(self._p, int(page)))

@@ -16,7 +16,10 @@ from typing import Any, Callable, Dict, Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
+from ..cache import native
 from ..utils.pinned import BatchUploader
+
+TILE_ROWS = 32      # tokens of one segment that the attention kernel for portions takes as a tile
 
 
 @dataclass
@@ -105,73 +108,73 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     against the cache's current tables, upload them, and return the context.
     Pages for the entries' tokens must have been reserved.  `pad_blocks` gives,
     per page group, a width to pad the block tables to (for steps that are
-    replayed from a recorded graph, whose array shapes must not change)."""
-    P = cache.page_size
+    replayed from a recorded graph, whose array shapes must not change).
+    The arrays are filled by the host library straight into the pinned buffer
+    (csrc/host.cpp, li_book_build_batch)."""
+    lib = native.lib()
+    ng = len(cache.groups)
     nseg = len(entries)
-    q_len = np.array([len(e.tokens) for e in entries], dtype=np.int32)
-    q_start = np.zeros(nseg + 1, dtype=np.int32)
-    np.cumsum(q_len, out=q_start[1:])
-    T = int(q_start[-1])
-    cached = np.array([cache.cached_len(e.rid) for e in entries], dtype=np.int32)
-    ctx_len = cached + q_len
+    handles = np.fromiter((cache.handle(e.rid) for e in entries), dtype=np.int64, count=nseg)
+    q_len = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=nseg)
     ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
-    id_src = np.full(T, -1, dtype=np.int32)
-    for i, e in enumerate(entries):
-        if e.take is not None:
-            id_src[q_start[i]:q_start[i + 1]] = np.asarray(e.take, dtype=np.int32)
-    seg_of_token = np.repeat(np.arange(nseg, dtype=np.int32), q_len)
-    pos = (np.arange(T, dtype=np.int32) - q_start[seg_of_token] + cached[seg_of_token]).astype(np.int32)
-    slots = np.array([cache.slot(e.rid) for e in entries], dtype=np.int32)
-    want = [int(q_start[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
-    want_rows = np.asarray(want, dtype=np.int32)
-    single_mask = q_len[seg_of_token] == 1
-    single = np.nonzero(single_mask)[0].astype(np.int32)
-    multi = np.nonzero(~single_mask)[0].astype(np.int32)
-    tile_rows = [(i, int(q_start[i]) + a, min(32, int(q_len[i]) - a), 0)
-                 for i in range(nseg) if q_len[i] > 1 for a in range(0, int(q_len[i]), 32)]
-    tiles = np.asarray(tile_rows, dtype=np.int32).reshape(-1, 4)
-    parts = [ids, pos, seg_of_token, q_start[:-1].copy(), q_len, ctx_len, slots, want_rows, single, multi, tiles,
-             id_src]
-    tables, max_blocks = [], []
-    for gi in range(len(cache.groups)):
-        tabs = [cache.block_table(e.rid, gi) for e in entries]
-        mb = max(1, max(len(t) for t in tabs))
-        if pad_blocks is not None:
-            mb = max(mb, int(pad_blocks[gi]))
-        tab = np.full((nseg, mb), -1, dtype=np.int32)
-        for i, t in enumerate(tabs):
-            tab[i, :len(t)] = t
-        page = tab[seg_of_token, pos // P]
-        if (page < 0).any():
-            raise AssertionError("step: a token of the batch has no page")
-        slot_map = (page.astype(np.int64) * P + pos % P).astype(np.int32)
-        tables.append(tab)
-        max_blocks.append(mb)
-        parts += [tab, slot_map]
-    dev = uploader.upload(parts)
-    ctx = StepContext(ws, T, nseg)
-    (ctx.ids, ctx.positions, d_seg, d_qs, d_ql, d_cl, ctx.state_slots, ctx.want_rows,
-     d_single, d_multi, d_tiles, ctx.id_src) = dev[:12]
-    ctx.feedback = feedback
-    if feedback is None:
-        if (id_src >= 0).any():
+    id_src = None
+    if any(e.take is not None for e in entries):
+        if feedback is None:
             raise ValueError("step: an entry takes tokens from the feedback buffer, but there is none")
-        ctx.id_src = None
-    ctx.num_want = len(want)
-    ctx.host_state_slots = slots
-    ctx.host_q_start, ctx.host_q_len, ctx.host_ctx_len = q_start[:-1], q_len, ctx_len
-    for gi in range(len(cache.groups)):
-        d_tab, d_slot = dev[12 + 2 * gi], dev[13 + 2 * gi]
-        ctx._slot_maps.append(d_slot)
+        id_src = np.concatenate([np.full(len(e.tokens), -1, dtype=np.int32) if e.take is None
+                                 else np.asarray(e.take, dtype=np.int32) for e in entries])
+    want_off = np.zeros(nseg + 1, dtype=np.int32)
+    np.cumsum([len(e.want) for e in entries], out=want_off[1:])
+    want = np.fromiter((int(w) for e in entries for w in e.want), dtype=np.int32, count=int(want_off[-1]))
+    pad = None if pad_blocks is None else np.asarray(pad_blocks, dtype=np.int32)
+    offsets = np.zeros(12 + 2 * ng, dtype=np.int64)
+    info = np.zeros(8 + max(ng, 1), dtype=np.int32)
+
+    def ptr(a):
+        return None if a is None else a.ctypes.data
+
+    def call(out_ptr, cap):
+        n = lib.li_book_build_batch(cache.book, nseg, ptr(handles), ptr(q_len), ptr(ids), ptr(id_src),
+                                    ptr(want_off), ptr(want), ptr(pad), TILE_ROWS, out_ptr, cap,
+                                    ptr(offsets), ptr(info))
+        if n < 0:
+            raise AssertionError(cache._error())
+        return int(n)
+    total = call(None, 0)
+    host = uploader.stage(total)
+    call(host.data_ptr(), host.numel())
+    dev = uploader.push(total)
+    T, nwant, nsingle, nmulti, ntiles, max_q, max_ctx, max_single_ctx = (int(x) for x in info[:8])
+    hv = host.numpy()
+
+    def d(k, n, shape=None):
+        t = dev[int(offsets[k]):int(offsets[k]) + n]
+        return t if shape is None else t.view(shape)
+
+    def h(k, n):
+        return hv[int(offsets[k]):int(offsets[k]) + n].copy()
+    ctx = StepContext(ws, T, nseg)
+    ctx.ids, ctx.positions = d(0, T), d(1, T)
+    d_seg, d_qs, d_ql, d_cl = d(2, T), d(3, nseg), d(4, nseg), d(5, nseg)
+    ctx.state_slots, ctx.want_rows = d(6, nseg), d(7, nwant)
+    d_single, d_multi, d_tiles = d(8, nsingle), d(9, nmulti), d(10, ntiles * 4, (ntiles, 4))
+    ctx.id_src = d(11, T) if feedback is not None else None
+    ctx.feedback = feedback
+    ctx.num_want = nwant
+    ctx.host_state_slots = h(6, nseg)
+    ctx.host_q_start, ctx.host_q_len, ctx.host_ctx_len = h(3, nseg), h(4, nseg), h(5, nseg)
+    P = cache.page_size
+    for gi in range(ng):
+        mb = int(info[8 + gi])
+        ctx._slot_maps.append(d(13 + 2 * gi, T))
         ctx._attn.append(AttentionMeta(
-            block_table=d_tab, max_blocks=max_blocks[gi], seg_of_token=d_seg, q_start=d_qs,
+            block_table=d(12 + 2 * gi, nseg * mb, (nseg, mb)), max_blocks=mb, seg_of_token=d_seg, q_start=d_qs,
             q_len=d_ql, ctx_len=d_cl, num_segments=nseg, num_tokens=T,
-            max_q_len=int(q_len.max()), max_ctx_len=int(ctx_len.max()),
-            host_q_start=q_start[:-1], host_q_len=q_len, host_ctx_len=ctx_len,
-            single_tokens=d_single if len(multi) else None, num_single=len(single),
-            multi_tokens=d_multi if len(single) else None, num_multi=len(multi),
-            tiles=d_tiles, num_tiles=len(tile_rows),
+            max_q_len=max_q, max_ctx_len=max_ctx,
+            host_q_start=ctx.host_q_start, host_q_len=ctx.host_q_len, host_ctx_len=ctx.host_ctx_len,
+            single_tokens=d_single if nmulti else None, num_single=nsingle,
+            multi_tokens=d_multi if nsingle else None, num_multi=nmulti,
+            tiles=d_tiles, num_tiles=ntiles,
             # with padded tables the split count must not follow the context either
-            max_single_ctx=(max_blocks[gi] * P if pad_blocks is not None else
-                            int(ctx_len[q_len == 1].max()) if len(single) else 0)))
+            max_single_ctx=(mb * P if pad_blocks is not None else max_single_ctx)))
     return ctx

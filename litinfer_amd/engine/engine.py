@@ -238,7 +238,7 @@ class Engine:
             return None
         widths = []
         for gi in range(len(self.cache.groups)):
-            need = max(len(self.cache.block_table(e.rid, gi)) for e in entries)
+            need = max(self.cache.table_len(e.rid, gi) for e in entries)
             widths.append(max(16, 1 << (need - 1).bit_length()))
         return (len(entries), sum(len(e.want) for e in entries), tuple(widths))
 

@@ -33,7 +33,18 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
 # accumulation registers (and fewer registers in all).
 MODULE_FLAGS = {"attention": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 
-MODULES = ("elementwise", "gemm", "attention", "sampling")
+MODULES = ("elementwise", "gemm", "attention", "sampling", "host")
+# "host" is plain C++ (the cache's bookkeeping and the layout of a step's batch): no device code
+HOST_MODULES = ("host",)
+HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
+
+
+def _source(module: str) -> Path:
+    return CSRC / (f"{module}.cpp" if module in HOST_MODULES else f"{module}.hip")
+
+
+def _flags(module: str) -> List[str]:
+    return HOST_FLAGS if module in HOST_MODULES else FLAGS + MODULE_FLAGS.get(module, [])
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
@@ -57,10 +68,10 @@ def _headers() -> List[Path]:
 
 def _digest(module: str) -> str:
     h = hashlib.sha256()
-    for p in [CSRC / f"{module}.hip", *_headers()]:
+    for p in [_source(module), *([] if module in HOST_MODULES else _headers())]:
         h.update(p.name.encode())
         h.update(p.read_bytes())
-    h.update(" ".join(FLAGS + MODULE_FLAGS.get(module, [])).encode())
+    h.update(" ".join(_flags(module)).encode())
     return h.hexdigest()[:16]
 
 
@@ -107,14 +118,14 @@ def find_built(module: str) -> Optional[Path]:
 
 
 def compile_module(module: str, verbose: bool = True) -> Path:
-    """Compile csrc/<module>.hip now, whether or not a build exists."""
-    src = CSRC / f"{module}.hip"
+    """Compile the module's source under csrc/ now, whether or not a build exists."""
+    src = _source(module)
     if not src.exists():
         raise KernelBuildError(f"no source {src}")
     out_dir = _writable_dir()
     out = out_dir / lib_name(module)
     tmp = out_dir / f".{out.name}.{os.getpid()}.tmp"
-    cmd = [_hipcc(), *FLAGS, *MODULE_FLAGS.get(module, []), f"-I{CSRC}", str(src), "-o", str(tmp)]
+    cmd = [_hipcc(), *_flags(module), f"-I{CSRC}", str(src), "-o", str(tmp)]
     env = dict(os.environ)
     env.setdefault("HOME", tempfile.gettempdir())     # hipcc wants a HOME it can look into
     t0 = time.time()
