@@ -104,3 +104,31 @@ def test_recorded_decode_steps_equal_eager_ones_on_every_replay(models, dt):
     # and they are right, not only equal: request c was fed in order between the replays
     at, pos = last_c
     assert schedules.rel_err(outs[0][at].cpu().numpy()[0], ref["r5"][pos]) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt,name", [("bfloat16", "D"), ("bfloat16", "E"), ("float32", "B")])
+def test_a_long_prompt_in_portions_then_decoding(tmp_path, dt, name):
+    """Thousands of positions: many tiles of queries, block tables of hundreds of pages, many
+    key splits when decoding; a window far behind the head.  Portions of 2,048 and a ragged
+    rest, then tokens one by one, against the plain implementation."""
+    from litinfer_amd.engine import StepEntry
+    cfg = dict(CASES[name][0], max_position_embeddings=8192)
+    page = CASES[name][1]
+    stored = torch.float32 if dt == "float32" else torch.bfloat16
+    d = helpers.make_model(tmp_path, cfg, 31, stored)
+    n, tail = 4500, 6
+    toks = helpers.random_requests(cfg["vocab_size"], [n + tail], 32)["r0"]
+    ref = helpers.plain_logits(d, {"r0": toks})["r0"]
+    eng = _engine(d, dt, page, 4608 + 64)
+    got = {}
+    start = 0
+    for size in (2048, 2048, n - 4096):
+        want = [0, size // 2, size - 1]
+        out = eng.step([StepEntry("r0", toks[start:start + size], want)]).cpu().numpy()
+        for w, row in zip(want, out):
+            got[start + w] = row
+        start += size
+    for i in range(tail):
+        got[n + i] = eng.step([StepEntry("r0", [toks[n + i]], [0])]).cpu().numpy()[0]
+    worst = max(schedules.rel_err(v, ref[p]) for p, v in got.items())
+    assert worst < TOL[dt], f"{name} {dt}: {worst}"
