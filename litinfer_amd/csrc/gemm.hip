@@ -6,6 +6,7 @@
 // on M or on the element's place, so a row's result does not depend on which
 // other rows are in the batch.
 #include "common.h"
+#include <algorithm>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -510,8 +511,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     constexpr int ESTRIDE = EW + 4;
     float* band = reinterpret_cast<float*>(lds) + wave * 32 * ESTRIDE;
     const int ccol = lane & 31, crow = (lane >> 5) * 4;
-    constexpr int LPR = EW / 8, RPP = 64 / LPR;
-    const int erow = lane / LPR, ecol = (lane % LPR) * 8;
+    constexpr int LPR = EW / 8, RPP = 64 / LPR;     // lanes a row of the band takes; rows a pass of the wave covers
+    const int erow = lane / LPR, ecol = (lane % LPR) * 8;      // (where 64 is no multiple of LPR the last lanes idle)
     const int NO = SWIGLU ? N / 2 : N;             // columns of out
     const int col = (SWIGLU ? (n0 + wn) / 2 : n0 + wn) + ecol;
 #pragma unroll
@@ -534,9 +535,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
         }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int pass = 0; pass < 32 / RPP; ++pass) {
+        for (int pass = 0; pass < (32 + RPP - 1) / RPP; ++pass) {
             const int row = m0 + wm + 32 * i + RPP * pass + erow;
-            if (row >= M || col >= NO) continue;
+            if (erow >= RPP || RPP * pass + erow >= 32 || row >= M || col >= NO) continue;
             const float* src = &band[(RPP * pass + erow) * ESTRIDE + ecol];
             float v[8];
 #pragma unroll
@@ -928,7 +929,7 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
             if (out_dtype != LI_F32 && out_dtype != LI_BF16) return LI_ERR_DTYPE;
 #define LI_DMA(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, false, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                                : launch_dma<BM, BN, BK, NS, false, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
-            // Three tilings; the one with the least (rounds of blocks over the 256 compute units) x
+            // Four tilings; the one with the least (rounds of blocks over the 256 compute units) x
             // (area of a tile) / (its measured relative speed) is taken: large tiles are the fastest
             // per multiply-add but leave compute units idle when the matrix has few of them.
             if (K % 64 == 0) {
@@ -936,9 +937,12 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
                     const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
                     return (double)((tiles + 255) / 256) * bm * bn / speed;
                 };
-                const double c_large = cost(256, 256, 1.0), c_mid = cost(256, 128, 0.95), c_small = cost(128, 128, 0.8);
-                if (c_large <= c_mid && c_large <= c_small) return LI_DMA(256, 256, 64, 2);
-                if (c_mid <= c_small) return LI_DMA(256, 128, 64, 3);
+                const double c_large = cost(256, 256, 1.0), c_wide = cost(256, 192, 0.97), c_mid = cost(256, 128, 0.95),
+                             c_small = cost(128, 128, 0.8);
+                const double best = std::min(std::min(c_large, c_wide), std::min(c_mid, c_small));
+                if (c_large == best) return LI_DMA(256, 256, 64, 2);
+                if (c_wide == best) return LI_DMA(256, 192, 64, 2);
+                if (c_mid == best) return LI_DMA(256, 128, 64, 3);
                 return LI_DMA(128, 128, 64, 4);
             }
 #undef LI_DMA
