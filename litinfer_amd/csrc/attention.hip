@@ -549,6 +549,13 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
 #define PRE_WAVES 4
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
+// the largest of three in one instruction (no NaN can occur among scores and -inf)
+__device__ __forceinline__ float max3f(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 template <int DH>
 __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
@@ -584,38 +591,67 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
     const int* table = block_table + (size_t)s * max_blocks + first_block;
     for (int i = tid; i < nblocks; i += NT) pages[i] = table[i];
     __syncthreads();
-    // Element offset of a key's row in a cache layer; a key outside the tile's range gives the
-    // nearest key inside it (its scores are masked below).
-    const float inv_page = 1.0f / (float)page_size;
-    auto row_of = [&](int key) -> size_t {
-        key = key < lo0 ? lo0 : (key >= k_end ? k_end - 1 : key);
-        const int blk = (int)(((float)key + 0.5f) * inv_page);       // key / page_size, exact below 2^21 (checked by the host)
-        int page = pages[blk - first_block];
-        page = page < 0 ? 0 : (page >= num_pages ? num_pages - 1 : page);
-        return (((size_t)page * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
-    };
     // ---- fetching a block of 32 keys.  K: 16-byte chunks tid, tid + NT, ...  V: units of two
     // neighbouring key positions x 8 dimensions; position p of the key order holds the key
     // 16 (p / 16) + 4 ((p / 8) % 2) + (p % 8 < 4 ? p % 8 : p % 8 + 4).
+    // A thread fetches the same rows of every block, 32 keys further on each turn: it keeps each
+    // row's page block and place in the page and moves them on without a division.  Rows before
+    // the first or past the last key of the tile (their scores are masked) read whatever page the
+    // clamped table entry names: the cache holds finite numbers everywhere.
     constexpr int KCH = (32 * CPR + NT - 1) / NT;
     constexpr int VU = 16 * CPR, VCH = (VU + NT - 1) / NT;
+    constexpr int NROW = KCH + 2 * VCH;                 // rows this thread fetches: K rows, then pairs of V rows
     u32x4 kreg[KCH], vreg[VCH][2];
+    int row_blk[NROW], row_in[NROW], row_col[NROW];     // page block (relative to first_block), place in the page, column
+    {
+        int keys[NROW];
+#pragma unroll
+        for (int i = 0; i < KCH; ++i) {
+            int ch = tid + i * NT;
+            ch = ch < 32 * CPR ? ch : 32 * CPR - 1;
+            keys[i] = ch / CPR;
+            row_col[i] = 8 * (ch % CPR);
+        }
+#pragma unroll
+        for (int i = 0; i < VCH; ++i) {
+            int u = tid + i * NT;
+            u = u < VU ? u : VU - 1;
+            const int dg = (u & 3) + 4 * (u >> 6), pp = (u >> 2) & 15, pc = pp >> 2, ip = 2 * (pp & 3);
+            keys[KCH + 2 * i] = 16 * (pc >> 1) + 4 * (pc & 1) + (ip < 4 ? ip : ip + 4);
+            keys[KCH + 2 * i + 1] = keys[KCH + 2 * i] + 1;
+            row_col[KCH + 2 * i] = row_col[KCH + 2 * i + 1] = 8 * dg;
+        }
+#pragma unroll
+        for (int i = 0; i < NROW; ++i) {
+            const int key = k_begin + keys[i];
+            row_blk[i] = key / page_size - first_block;
+            row_in[i] = key % page_size;
+        }
+    }
+    const int step_blk = 32 / page_size, step_in = 32 % page_size;      // a turn moves every row 32 keys on
+    const size_t page_bytes = (size_t)nkv * page_size * DH * 2;
+    const char* kbase = reinterpret_cast<const char*>(kc) + (size_t)kvh * page_size * DH * 2;
+    const char* vbase = reinterpret_cast<const char*>(vc) + (size_t)kvh * page_size * DH * 2;
+    // the row's address in a cache layer, then on to the next block of keys
+#define LI_PRE_ROW(i, base)                                                                          \
+    ({                                                                                               \
+        int ix_ = row_blk[i] < 0 ? 0 : (row_blk[i] > PRE_TABLE_CAP - 1 ? PRE_TABLE_CAP - 1 : row_blk[i]); \
+        int page_ = pages[ix_];                                                                      \
+        page_ = page_ < 0 ? 0 : (page_ >= num_pages ? num_pages - 1 : page_);                        \
+        const char* p_ = (base) + (size_t)(unsigned)page_ * page_bytes + (unsigned)((row_in[i] * DH + row_col[i]) * 2); \
+        row_in[i] += step_in;                                                                        \
+        row_blk[i] += step_blk;                                                                      \
+        if (row_in[i] >= page_size) { row_in[i] -= page_size; row_blk[i] += 1; }                     \
+        p_;                                                                                          \
+    })
+    // (fetches are made for consecutive blocks: k_begin, k_begin + 32, ...)
 #define LI_PRE_FETCH(kb)                                                                             \
     {                                                                                                \
-        _Pragma("unroll") for (int i = 0; i < KCH; ++i) {                                            \
-            int ch = tid + i * NT;                                                                   \
-            ch = ch < 32 * CPR ? ch : 32 * CPR - 1;                                                  \
-            const size_t off = row_of((kb) + ch / CPR);                                               \
-            kreg[i] = *reinterpret_cast<const u32x4*>(kc + off + 8 * (ch % CPR));                    \
-        }                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < KCH; ++i)                                              \
+            kreg[i] = *reinterpret_cast<const u32x4*>(LI_PRE_ROW(i, kbase));                         \
         _Pragma("unroll") for (int i = 0; i < VCH; ++i) {                                            \
-            int u = tid + i * NT;                                                                    \
-            u = u < VU ? u : VU - 1;                                                                 \
-            const int dg = (u & 3) + 4 * (u >> 6), pp = (u >> 2) & 15, pc = pp >> 2, ip = 2 * (pp & 3); \
-            const int key = (kb) + 16 * (pc >> 1) + 4 * (pc & 1) + (ip < 4 ? ip : ip + 4);           \
-            const size_t o0 = row_of(key), o1 = row_of(key + 1);                                     \
-            vreg[i][0] = *reinterpret_cast<const u32x4*>(vc + o0 + 8 * dg);                          \
-            vreg[i][1] = *reinterpret_cast<const u32x4*>(vc + o1 + 8 * dg);                          \
+            vreg[i][0] = *reinterpret_cast<const u32x4*>(LI_PRE_ROW(KCH + 2 * i, vbase));            \
+            vreg[i][1] = *reinterpret_cast<const u32x4*>(LI_PRE_ROW(KCH + 2 * i + 1, vbase));        \
         }                                                                                            \
     }
 #define LI_PRE_STASH(stage)                                                                          \
@@ -664,8 +700,18 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
     LI_PRE_STASH(0);
     if (k_begin + 32 < k_end) LI_PRE_FETCH(k_begin + 32);
     __syncthreads();
-    int stage = 0;
-    for (int kb = k_begin; kb < k_end; kb += 32, stage ^= 1) {
+    // where this lane reads its fragments of K in a stage (the swizzle depends on the lane only)
+    int kaddr[KS];
+#pragma unroll
+    for (int st = 0; st < KS; ++st) kaddr[st] = ql * DH + ((((HD / 8) * h + st) ^ (ql & (CPR - 1))) << 3);
+    const int vaddr = ql * VS + 8 * h;
+    // two turns a trip, so that the stage is a constant of the code and the LDS addresses are
+    // a register plus an immediate
+    for (int kb2 = k_begin; kb2 < k_end; kb2 += 64) {
+#pragma unroll
+      for (int stage = 0; stage < 2; ++stage) {
+        const int kb = kb2 + 32 * stage;
+        if (kb >= k_end) break;
         if (kb + 32 < k_end) LI_PRE_STASH(stage ^ 1);      // (its readers of the turn before are past the barrier)
         if (kb + 64 < k_end) LI_PRE_FETCH(kb + 64);
         if (active) {
@@ -673,13 +719,11 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
             f32x16_t sv;
 #pragma unroll
             for (int r = 0; r < 16; ++r) sv[r] = 0.f;
+            frag8 kf[KS];
 #pragma unroll
-            for (int st = 0; st < KS; ++st) {
-                frag8 kf;
-                const int c = (HD / 8) * h + st;
-                kf.raw = *reinterpret_cast<const u32x4*>(&Ks[stage][ql * DH + ((c ^ (ql & (CPR - 1))) << 3)]);
-                sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qf[st].v, sv, 0, 0, 0);
-            }
+            for (int st = 0; st < KS; ++st) kf[st].raw = *reinterpret_cast<const u32x4*>(&Ks[stage][kaddr[st]]);
+#pragma unroll
+            for (int st = 0; st < KS; ++st) sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st].v, qf[st].v, sv, 0, 0, 0);
             // ---- softmax over the keys of this lane's query.  The running maximum m is only moved
             // (and the sums so far rescaled, for the whole wave) when some query's scores pass it by
             // more than 2^8: until then the exponentials are taken against the older maximum, which
@@ -693,10 +737,11 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
                     sv[r] = (key <= pq && key >= lq) ? sv[r] : -INFINITY;
                 }
             }
-            float mx = fmaxf(sv[0], sv[1]);
+            float mx = max3f(sv[0], sv[1], sv[2]);
 #pragma unroll
-            for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(sv[r], sv[r + 1]));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE)) * scale2;       // (scale2 > 0)
+            for (int r = 3; r < 15; r += 2) mx = max3f(mx, sv[r], sv[r + 1]);
+            mx = max3f(mx, sv[15], sv[15]);
+            mx = max3f(mx, __shfl_xor(mx, 32, LI_WAVE), mx) * scale2;   // (scale2 > 0)
             if (__any(mx > m + 8.0f)) {
                 const float mn = fmaxf(m, mx);
                 const float alpha = (mn == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - mn);   // (m = -inf: nothing summed yet)
@@ -720,16 +765,16 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
             // ---- O^T += V^T P^T
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                const int d = 32 * dt + ql;
 #pragma unroll
                 for (int st = 0; st < 2; ++st) {
                     frag8 vf;
-                    vf.raw = *reinterpret_cast<const u32x4*>(&Vt[stage][d * VS + ((2 * st + h) << 3)]);
+                    vf.raw = *reinterpret_cast<const u32x4*>(&Vt[stage][vaddr + 32 * dt * VS + 16 * st]);
                     acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
                 }
             }
         }
         __syncthreads();
+      }
     }
     if (!active || ql >= nrows) return;
     l += __shfl_xor(l, 32, LI_WAVE);               // (both halves of a query are past the return together)
@@ -766,6 +811,7 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
     if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
 #undef LI_PRE
 #undef LI_PRE_FETCH
+#undef LI_PRE_ROW
 #undef LI_PRE_STASH
     return li_launch_status();
 }
