@@ -188,6 +188,30 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 // step.  A row of a stage is 64 elements = 128 bytes = 8 chunks of 16 bytes;
 // chunk c of row r lies at position c ^ ((r >> 1) & 7), which spreads the 16
 // rows that one fragment read touches over all banks.
+// Blocks go to the 8 XCDs in turn (block b runs on XCD b % 8), and each XCD has an L2 of its
+// own.  The tiles are dealt so that the ~32 blocks an XCD runs at one time form a patch of up
+// to 8 row panels x 4 or more column panels: what the patch reads from beyond its L2 is then
+// (8 + 4) panels for 32 tiles.  Patches follow each other along the rows first, so a column
+// panel of W is read from HBM by one XCD only and stays in its L2 while the row panels go by.
+struct TileOrder {
+    int pm, gn, mgroups;                             // row panels and column panels of a patch; patches along the rows
+    __host__ __device__ TileOrder(int mtiles) {
+        pm = mtiles < 8 ? mtiles : 8;
+        gn = 32 / pm;
+        mgroups = (mtiles + pm - 1) / pm;
+    }
+    __host__ long blocks(long ntiles) const {        // grid size: whole patches on each of the 8 XCDs
+        return ((ntiles + 7) / 8 + gn - 1) / gn * (long)mgroups * pm * gn * 8;
+    }
+    __device__ bool tile(int block, int mtiles, int ntiles, int& mt, int& nt) const {
+        const int xcd = block & 7, idx = block >> 3;
+        const int patch = idx / (pm * gn), within = idx % (pm * gn);
+        mt = (patch % mgroups) * pm + within % pm;
+        nt = ((patch / mgroups) * gn + within / pm) * 8 + xcd;
+        return mt < mtiles && nt < ntiles;
+    }
+};
+
 template <int BM, int BN, int BK, typename TO>
 __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __restrict__ x,
                                                              const bf16_t* __restrict__ w,
@@ -203,16 +227,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
     uint16_t* Bs = lds + 2 * BM * BK;                             // [2][BN][BK]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
-    // Blocks go to the 8 XCDs in turn (block b runs on XCD b % 8), and each XCD has an L2 of its
-    // own.  The tiles are dealt so that the ~32 blocks an XCD runs at one time form a patch of
-    // all row panels x a few column panels: a column panel of W is then read from HBM by one
-    // XCD only, by blocks that run together, and x is read again per patch from the caches.
     const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    const int gn = mtiles >= 32 ? 1 : 32 / mtiles;                // column panels of a patch
-    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    const int patch = idx / (mtiles * gn), within = idx % (mtiles * gn);
-    const int mt = within % mtiles, nt = ((patch * gn) + within / mtiles) * 8 + xcd;
-    if (nt >= ntiles) return;
+    int mt, nt;
+    if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, mt, nt)) return;
     const int m0 = mt * BM, n0 = nt * BN;
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -391,11 +408,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
     const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    const int gn = mtiles >= 32 ? 1 : 32 / mtiles;               // see gemm_bf16_big_kernel: patches per XCD
-    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-    const int patch = idx / (mtiles * gn), within = idx % (mtiles * gn);
-    const int mt = within % mtiles, nt = ((patch * gn) + within / mtiles) * 8 + xcd;
-    if (nt >= ntiles) return;
+    int mt, nt;
+    if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, mt, nt)) return;
     const int m0 = mt * BM, n0 = nt * BN;
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -577,8 +591,7 @@ template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream, int nsplit = 1) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    const long gn = mtiles >= 32 ? 1 : 32 / mtiles;
-    const long per_xcd = ((ntiles + 7) / 8 + gn - 1) / gn * gn * mtiles;
+    const long per_xcd = TileOrder((int)mtiles).blocks(ntiles) / 8;
     if (per_xcd * 8 > 0x7fffffffL || nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
     constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool configured = false;
@@ -607,8 +620,7 @@ template <int BM, int BN, int BK, typename TO>
 static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    const long gn = mtiles >= 32 ? 1 : 32 / mtiles;
-    const long per_xcd = ((ntiles + 7) / 8 + gn - 1) / gn * gn * mtiles;     // whole patches
+    const long per_xcd = TileOrder((int)mtiles).blocks(ntiles) / 8;
     if (per_xcd * 8 > 0x7fffffffL) return LI_ERR_SIZE;
     dim3 grid((unsigned)(per_xcd * 8));
     constexpr int lds_bytes = 2 * (BM + BN) * BK * 2;
