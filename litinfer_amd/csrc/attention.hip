@@ -433,71 +433,75 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
                     kf[tt][j].raw = *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j);
             }
         };
-        if (k_begin < k_end) load_k(k_begin);
-        for (int kb = k_begin; kb < k_end; kb += 32) {
-            // ---- V rows of this lane: keys kb + 8g + i, dimensions 128 ns + 8c ..  (issued before
-            // K is waited for, so they stay in flight during Q K^T and the softmax)
-            u32x4 vraw[NS][8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                bool ok;
-                const size_t off = row_of(kb + 8 * g + i, ok);
-#pragma unroll
-                for (int ns = 0; ns < NS; ++ns) {
-                    const int d = 128 * ns + 8 * c;
-                    vraw[ns][i] = *reinterpret_cast<const u32x4*>(vc + off + (d < DH ? d : DH - 8));
-                }
-            }
-            // ---- S = Q K^T
-            f32x4_t sv[2];
-            bool sok[2] = {kok[0], kok[1]};
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int j = 0; j < KS; ++j)
-                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0);
-            }
-            // ---- the next block's K: in flight during the softmax and P V
-            if (kb + 32 < k_end) load_k(kb + 32);
-            // ---- online softmax; lanes whose key is past the end hold -inf
-            float alpha[4], pr[2][4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;
-                const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;
-                const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));     // the block has a key: mx is finite
-                alpha[r] = expf(m[r] - mx);
-                pr[0][r] = expf(s0 - mx);
-                pr[1][r] = expf(s1 - mx);
-                l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];
-                m[r] = mx;
-            }
-            __syncthreads();                                    // readers of the last block's P are done
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = float_to_bf16(pr[tt][r]);
-            __syncthreads();
-            frag8 pa;
-            pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);
-            // ---- O = alpha O + P V
-#pragma unroll
-            for (int ns = 0; ns < NS; ++ns) {
-#pragma unroll
-                for (int jj = 0; jj < 8; ++jj) {
-                    frag8 vf;
-#pragma unroll
-                    for (int ii = 0; ii < 4; ++ii)
-                        vf.raw.w[ii] = __builtin_amdgcn_perm(vraw[ns][2 * ii + 1].w[jj >> 1], vraw[ns][2 * ii].w[jj >> 1],
-                                                             (jj & 1) ? 0x07060302u : 0x05040100u);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[ns][jj][r] *= alpha[r];
-                    acc[ns][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vf.v, acc[ns][jj], 0, 0, 0);
-                }
-            }
+        // V rows of this lane: keys kb + 8g + i, dimensions 128 ns + 8c ..  Two sets of registers
+        // take turns, so that the values of the NEXT block are in flight while this one is worked on
+        u32x4 va[NS][8], vb[NS][8];
+#define LI_DEC_LOAD_V(kbv, dst)                                                                      \
+        _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                              \
+            bool ok_;                                                                                \
+            const size_t off_ = row_of((kbv) + 8 * g + i, ok_);                                      \
+            _Pragma("unroll") for (int ns = 0; ns < NS; ++ns) {                                      \
+                const int d_ = 128 * ns + 8 * c;                                                     \
+                dst[ns][i] = *reinterpret_cast<const u32x4*>(vc + off_ + (d_ < DH ? d_ : DH - 8));   \
+            }                                                                                        \
         }
+#define LI_DEC_STEP(kbv, vcur, vnext)                                                                \
+        {                                                                                            \
+            /* ---- S = Q K^T */                                                                     \
+            f32x4_t sv[2];                                                                           \
+            const bool sok[2] = {kok[0], kok[1]};                                                    \
+            _Pragma("unroll") for (int tt = 0; tt < 2; ++tt) {                                       \
+                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};                                                \
+                _Pragma("unroll") for (int j = 0; j < KS; ++j)                                       \
+                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0); \
+            }                                                                                        \
+            /* ---- the next block's K and V: in flight during the softmax and P V */                \
+            if ((kbv) + 32 < k_end) {                                                                \
+                load_k((kbv) + 32);                                                                  \
+                LI_DEC_LOAD_V((kbv) + 32, vnext)                                                     \
+            }                                                                                        \
+            /* ---- online softmax; lanes whose key is past the end hold -inf */                     \
+            float alpha[4], pr[2][4];                                                                \
+            _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                          \
+                const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;                              \
+                const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;                              \
+                const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));     /* the block has a key: mx is finite */ \
+                alpha[r] = expf(m[r] - mx);                                                          \
+                pr[0][r] = expf(s0 - mx);                                                            \
+                pr[1][r] = expf(s1 - mx);                                                            \
+                l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];                                        \
+                m[r] = mx;                                                                           \
+            }                                                                                        \
+            __syncthreads();                                    /* readers of the last block's P are done */ \
+            _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                         \
+                _Pragma("unroll") for (int r = 0; r < 4; ++r)                                        \
+                    p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = float_to_bf16(pr[tt][r]);           \
+            __syncthreads();                                                                         \
+            frag8 pa;                                                                                \
+            pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);                   \
+            /* ---- O = alpha O + P V */                                                             \
+            _Pragma("unroll") for (int ns = 0; ns < NS; ++ns) {                                      \
+                _Pragma("unroll") for (int jj = 0; jj < 8; ++jj) {                                   \
+                    frag8 vf;                                                                        \
+                    _Pragma("unroll") for (int ii = 0; ii < 4; ++ii)                                 \
+                        vf.raw.w[ii] = __builtin_amdgcn_perm(vcur[ns][2 * ii + 1].w[jj >> 1], vcur[ns][2 * ii].w[jj >> 1], \
+                                                             (jj & 1) ? 0x07060302u : 0x05040100u);  \
+                    _Pragma("unroll") for (int r = 0; r < 4; ++r) acc[ns][jj][r] *= alpha[r];        \
+                    acc[ns][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vf.v, acc[ns][jj], 0, 0, 0); \
+                }                                                                                    \
+            }                                                                                        \
+        }
+        if (k_begin < k_end) {
+            load_k(k_begin);
+            LI_DEC_LOAD_V(k_begin, va)
+        }
+        for (int kb = k_begin; kb < k_end; kb += 64) {
+            LI_DEC_STEP(kb, va, vb)
+            if (kb + 32 >= k_end) break;
+            LI_DEC_STEP(kb + 32, vb, va)
+        }
+#undef LI_DEC_STEP
+#undef LI_DEC_LOAD_V
 #pragma unroll
         for (int r = 0; r < 4; ++r) l[r] = row16_sum(l[r]);
 #pragma unroll
