@@ -7,6 +7,8 @@
 // other rows are in the batch.
 #include "common.h"
 #include <algorithm>
+#include <type_traits>
+#include <utility>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -390,6 +392,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),              \
                                      (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
+// f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>)
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// The same load with its address as (scalar base) + (32-bit offset of the lane): no address
+// arithmetic in vector registers.  M0 carries the LDS address, as in the compiler's own form.
+#define LI_LOAD_TO_LDS_AT(base, voff, lptr)                                                              \
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"                          \
+                 :: "s"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(lptr)), "v"(voff), "s"(base) : "memory", "m0")
+
 template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x,
                                                              const bf16_t* __restrict__ w,
@@ -422,50 +440,69 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     auto slot = [](int row, int c) { return row * BK + ((c ^ ((row / WRAP) & (CPR - 1))) << 3); };
     // this lane's part of a step: a wave takes BM / 4 rows of A and BN / 4 rows of B; one
     // instruction covers RPI rows, lane -> row lane / CPR, position lane % CPR
-    const bf16_t* ga[IA];
-    const bf16_t* gb[IB];
+    // Addresses: a base that is the same for the whole wave (scalar registers, moved on by a step's
+    // columns) plus this lane's 32-bit byte offset within the tile's rows, which never changes.
+    uint32_t ga[IA], gb[IB];
+    const bf16_t* abase = x + (size_t)m0 * K;
+    const bf16_t* bbase = w + (size_t)(SWIGLU ? n0 / 2 : n0) * K;
 #pragma unroll
     for (int i = 0; i < IA; ++i) {
         const int row = (BM / 4) * wave + RPI * i + lane / CPR, c = (lane % CPR) ^ ((row / WRAP) & (CPR - 1));
-        ga[i] = x + (size_t)((m0 + row < M) ? m0 + row : M - 1) * K + 8 * c;     // rows past the end: the last row
+        ga[i] = (uint32_t)(((size_t)((m0 + row < M) ? row : M - 1 - m0) * K + 8 * c) * 2);       // rows past the end: the last row
     }
 #pragma unroll
     for (int i = 0; i < IB; ++i) {
         const int row = (BN / 4) * wave + RPI * i + lane / CPR, c = (lane % CPR) ^ ((row / WRAP) & (CPR - 1));
-        int wrow = n0 + row;
+        size_t rel = (n0 + row < N) ? row : N - 1 - n0;            // row of w relative to the tile's first
         if constexpr (SWIGLU) {
             // w is [gate; up] with N / 2 rows each.  The tile's rows alternate in blocks of 32: 32
             // gate rows, the 32 up rows of the same outputs, the next 32 gate rows, ..., so that an
             // accumulator tile and its neighbour hold the two factors of one output tile.
             const int half = N / 2, blk = row / 32;
             const int o = n0 / 2 + (blk / 2) * 32 + row % 32;
-            wrow = (o < half ? o : half - 1) + (blk & 1) * half;
+            rel = (size_t)((o < half ? o : half - 1) - n0 / 2) + (size_t)(blk & 1) * half;
         }
-        gb[i] = w + (size_t)(wrow < N ? wrow : N - 1) * K + 8 * c;
+        gb[i] = (uint32_t)((rel * K + 8 * c) * 2);
     }
-    auto issue = [&](int kt) {
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    // load `idx` of a wave's LPW loads of step kt: first its rows of A, then its rows of B
+    auto issue_one = [&](int kt, int idx) {
         uint16_t* st = lds + (kt % NSTAGE) * STAGE;
+#ifdef LI_EXPT_NO_LOADS
+        return;
+#endif
+#ifdef LI_EXPT_SAME_COLUMNS
+        kt = 0;
+#endif
+        if (idx < IA) LI_LOAD_TO_LDS_AT(abase + (size_t)kt * BK, ga[idx], st + ((BM / 4) * uwave + RPI * idx) * BK);
+        else LI_LOAD_TO_LDS_AT(bbase + (size_t)kt * BK, gb[idx - IA], st + BM * BK + ((BN / 4) * uwave + RPI * (idx - IA)) * BK);
+    };
+    auto issue = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < IA; ++i) LI_LOAD_TO_LDS(ga[i] + (size_t)kt * BK, st + ((BM / 4) * wave + RPI * i) * BK);
-#pragma unroll
-        for (int i = 0; i < IB; ++i) LI_LOAD_TO_LDS(gb[i] + (size_t)kt * BK, st + BM * BK + ((BN / 4) * wave + RPI * i) * BK);
+        for (int i = 0; i < LPW; ++i) issue_one(kt, i);
     };
     const int frow = lane & 31, fh = lane >> 5;
     const int kt_first = (int)((long)(K / BK) * blockIdx.y / gridDim.y);
     const int nk = (int)((long)(K / BK) * (blockIdx.y + 1) / gridDim.y) - kt_first;
     out += (size_t)blockIdx.y * M * (SWIGLU ? N / 2 : N);
+    abase += (size_t)kt_first * BK;
+    bbase += (size_t)kt_first * BK;
+    constexpr int KS = BK / 16;                    // MFMA groups of a step: 16 columns each
+    constexpr int GM = TM * TN, GD = TM + TN;      // MFMAs and fragment reads of a group
+    // Order of a step.  A wave issues in order and is alone on its SIMD, and the CU's address unit
+    // takes a 16-byte-per-lane load of one wave every 16 cycles, i.e. one of each of the four waves
+    // every 64 = two MFMAs: loads issued back to back hold the wave, and with it the SIMD's
+    // MFMAs, until the unit has taken them.  So the loads of step kt + NSTAGE - 1 (into the stage
+    // that the barrier of step kt - 1 freed) are issued one by one between the MFMAs of the first
+    // groups of step kt, at most one per two MFMAs.  Each group's MFMAs run while the fragments
+    // of the next 16 columns are read; in the middle of the LAST group the wave waits for the
+    // loads of step kt + 1, meets the others at the barrier (stage kt + 1 is there for all, stage kt
+    // is read by all) and reads the first fragments of step kt + 1, so that the barrier and the
+    // latency of LDS fall under the remaining MFMAs.
+    constexpr int PER0 = GM / 2 > 0 ? GM / 2 : 1, PER1 = (LPW + KS - 2) / (KS - 1);
+    constexpr int PER = PER0 > PER1 ? PER0 : PER1;                     // loads of one group
 #pragma unroll
-    for (int i = 0; i < IA; ++i) ga[i] += (size_t)kt_first * BK;
-#pragma unroll
-    for (int i = 0; i < IB; ++i) gb[i] += (size_t)kt_first * BK;
-    constexpr int KS = BK / 16;                    // MFMA steps of a stage (even)
-    // Order of a step: the MFMAs of stage kt run while the fragments of its next 16 columns are
-    // read; in the middle of the stage's LAST 16 columns the wave waits for stage kt + 1 (loaded
-    // long before), meets the others at the barrier, starts the load of stage kt + NSTAGE into
-    // the stage all waves have just finished reading, and reads the first fragments of stage
-    // kt + 1, so that the barrier and the latency of LDS fall under the remaining MFMAs.
-#pragma unroll
-    for (int p = 0; p < NSTAGE; ++p)
+    for (int p = 0; p < NSTAGE - 1; ++p)
         if (p < nk) issue(p);
     bf16x8 af[2][TM], bfr[2][TN];
 #define LI_FREAD(stage_, ks, buf)                                                                          \
@@ -481,35 +518,51 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #define LI_WAIT_YOUNGER(y)                                                                                 \
     { if ((y) >= 3) LI_VMCNT(3 * LPW); else if ((y) == 2) LI_VMCNT(2 * LPW); else if ((y) == 1) LI_VMCNT(LPW); else LI_VMCNT(0); }
     {
-        const int younger = nk - 1 < NSTAGE - 1 ? nk - 1 : NSTAGE - 1;     // loads of later stages in flight
-        LI_WAIT_YOUNGER(younger)
+        const int inflight = nk < NSTAGE - 1 ? nk : NSTAGE - 1;
+        LI_WAIT_YOUNGER(inflight - 1)
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         LI_FREAD(0, 0, 0)
     }
-    for (int kt = 0; kt < nk; ++kt) {
+    // one step; LOADS: the loads of step kt + NSTAGE - 1 are issued in it
+    auto step = [&](int kt, auto loads_tag) {
+        constexpr bool LOADS = decltype(loads_tag)::value;
         const int stage = kt % NSTAGE;
+        static_for<KS - 1>([&](auto ks_tag) {
+            constexpr int ks = decltype(ks_tag)::value;
+            constexpr int l0 = ks * PER < LPW ? ks * PER : LPW, l1 = (ks + 1) * PER < LPW ? (ks + 1) * PER : LPW;
+            constexpr int NL = LOADS ? l1 - l0 : 0;
+            const uint16_t* As_ = lds + stage * STAGE;
+            const uint16_t* Bs_ = As_ + BM * BK;
+            const int c_ = 2 * (ks + 1) + fh;
+            // written in the order it is to run, and kept so: after MFMA m the m-th fragment read
+            // of the next 16 columns and the loads that fall to it
+            static_for<GM>([&](auto m_tag) {
+                constexpr int m = decltype(m_tag)::value;
+                constexpr int r0 = GD > GM ? (m * GD) / GM : (m < GD ? m : GD), r1 = GD > GM ? ((m + 1) * GD) / GM : (m < GD ? m + 1 : GD);
+                acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][m / TN], bfr[ks & 1][m % TN], acc[m / TN][m % TN], 0, 0, 0);
 #pragma unroll
-        for (int ks = 0; ks < KS - 1; ++ks) {
-            LI_FREAD(stage, ks + 1, (ks + 1) & 1)
+                for (int r = r0; r < r1; ++r) {
+                    if (r < TM) af[(ks + 1) & 1][r] = *reinterpret_cast<const bf16x8*>(&As_[slot(wm + 32 * r + frow, c_)]);
+                    else bfr[(ks + 1) & 1][r - TM] = *reinterpret_cast<const bf16x8*>(&Bs_[slot(wn + 32 * (r - TM) + frow, c_)]);
+                }
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bfr[ks & 1][j], acc[i][j], 0, 0, 0);
-        }
-        constexpr int BL = (KS - 1) & 1;           // = 1: the fragments of the last 16 columns
+                for (int l = l0 + (m * NL) / GM; l < l0 + ((m + 1) * NL) / GM; ++l) issue_one(kt + NSTAGE - 1, l);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
+        constexpr int BL = (KS - 1) & 1;           // the buffer with the fragments of the last 16 columns
 #pragma unroll
         for (int i = 0; i < TM / 2; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][i], bfr[BL][j], acc[i][j], 0, 0, 0);
         if (kt + 1 < nk) {
-            const int younger = nk - 2 - kt < NSTAGE - 2 ? nk - 2 - kt : NSTAGE - 2;
+            // loads of later steps that may stay in flight: steps kt + 2 .. kt + NSTAGE - 1, where they exist
+            const int younger = LOADS ? NSTAGE - 2 : (nk - 2 - kt < NSTAGE - 2 ? nk - 2 - kt : NSTAGE - 2);
             LI_WAIT_YOUNGER(younger)
-            __builtin_amdgcn_s_barrier();          // stage kt + 1 is in LDS for all waves; stage kt is read by all
+            __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (kt + NSTAGE < nk) issue(kt + NSTAGE);          // into the stage of step kt
             LI_FREAD((kt + 1) % NSTAGE, 0, 0)
         }
 #pragma unroll
@@ -517,7 +570,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][i], bfr[BL][j], acc[i][j], 0, 0, 0);
-    }
+    };
+    int kt = 0;
+    for (; kt + NSTAGE - 1 < nk; ++kt) step(kt, std::true_type{});
+    for (; kt < nk; ++kt) step(kt, std::false_type{});
 #undef LI_FREAD
 #undef LI_WAIT_YOUNGER
     __syncthreads();                               // the main loop's LDS is free now
