@@ -499,10 +499,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     // loads of step kt + 1, meets the others at the barrier (stage kt + 1 is there for all, stage kt
     // is read by all) and reads the first fragments of step kt + 1, so that the barrier and the
     // latency of LDS fall under the remaining MFMAs.
+    // With 64 rows of x a step has few MFMAs and the product waits for w from memory: there the
+    // loads of step kt + NSTAGE are issued all at once, right after the barrier of step kt, so that as
+    // many bytes as possible are on their way.
+    constexpr bool SPREAD = BM >= 128;
+    constexpr int AHEAD = SPREAD ? NSTAGE - 1 : NSTAGE;                // steps loaded before the first is multiplied
     constexpr int PER0 = GM / 2 > 0 ? GM / 2 : 1, PER1 = (LPW + KS - 2) / (KS - 1);
     constexpr int PER = PER0 > PER1 ? PER0 : PER1;                     // loads of one group
 #pragma unroll
-    for (int p = 0; p < NSTAGE - 1; ++p)
+    for (int p = 0; p < AHEAD; ++p)
         if (p < nk) issue(p);
     bf16x8 af[2][TM], bfr[2][TN];
 #define LI_FREAD(stage_, ks, buf)                                                                          \
@@ -518,34 +523,37 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #define LI_WAIT_YOUNGER(y)                                                                                 \
     { if ((y) >= 3) LI_VMCNT(3 * LPW); else if ((y) == 2) LI_VMCNT(2 * LPW); else if ((y) == 1) LI_VMCNT(LPW); else LI_VMCNT(0); }
     {
-        const int inflight = nk < NSTAGE - 1 ? nk : NSTAGE - 1;
+        const int inflight = nk < AHEAD ? nk : AHEAD;
         LI_WAIT_YOUNGER(inflight - 1)
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         LI_FREAD(0, 0, 0)
     }
-    // one step; LOADS: the loads of step kt + NSTAGE - 1 are issued in it
+    // one step; LOADS: the loads of step kt + NSTAGE - 1 are issued between its MFMAs
     auto step = [&](int kt, auto loads_tag) {
         constexpr bool LOADS = decltype(loads_tag)::value;
         const int stage = kt % NSTAGE;
         static_for<KS - 1>([&](auto ks_tag) {
             constexpr int ks = decltype(ks_tag)::value;
             constexpr int l0 = ks * PER < LPW ? ks * PER : LPW, l1 = (ks + 1) * PER < LPW ? (ks + 1) * PER : LPW;
-            constexpr int NL = LOADS ? l1 - l0 : 0;
+            constexpr int NL = LOADS && SPREAD ? l1 - l0 : 0;
             const uint16_t* As_ = lds + stage * STAGE;
             const uint16_t* Bs_ = As_ + BM * BK;
             const int c_ = 2 * (ks + 1) + fh;
-            // written in the order it is to run, and kept so: after MFMA m the m-th fragment read
-            // of the next 16 columns and the loads that fall to it
+            // written in the order it is to run, and kept so: before MFMA m the m-th fragment read of
+            // the next 16 columns (the earlier MFMAs the more, where there are more reads than MFMAs:
+            // the group's remaining MFMAs are what covers the latency of LDS), after it the loads that
+            // fall to it
             static_for<GM>([&](auto m_tag) {
                 constexpr int m = decltype(m_tag)::value;
-                constexpr int r0 = GD > GM ? (m * GD) / GM : (m < GD ? m : GD), r1 = GD > GM ? ((m + 1) * GD) / GM : (m < GD ? m + 1 : GD);
-                acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][m / TN], bfr[ks & 1][m % TN], acc[m / TN][m % TN], 0, 0, 0);
+                constexpr int r0 = GD > GM ? GD - ((GM - m) * GD) / GM : (m < GD ? m : GD);
+                constexpr int r1 = GD > GM ? GD - ((GM - m - 1) * GD) / GM : (m < GD ? m + 1 : GD);
 #pragma unroll
                 for (int r = r0; r < r1; ++r) {
                     if (r < TM) af[(ks + 1) & 1][r] = *reinterpret_cast<const bf16x8*>(&As_[slot(wm + 32 * r + frow, c_)]);
                     else bfr[(ks + 1) & 1][r - TM] = *reinterpret_cast<const bf16x8*>(&Bs_[slot(wn + 32 * (r - TM) + frow, c_)]);
                 }
+                acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][m / TN], bfr[ks & 1][m % TN], acc[m / TN][m % TN], 0, 0, 0);
 #pragma unroll
                 for (int l = l0 + (m * NL) / GM; l < l0 + ((m + 1) * NL) / GM; ++l) issue_one(kt + NSTAGE - 1, l);
                 __builtin_amdgcn_sched_barrier(0);
@@ -563,6 +571,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
             LI_WAIT_YOUNGER(younger)
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            if constexpr (!SPREAD) {
+                if (kt + NSTAGE < nk) issue(kt + NSTAGE);              // into the stage of step kt
+            }
             LI_FREAD((kt + 1) % NSTAGE, 0, 0)
         }
 #pragma unroll
@@ -572,7 +583,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][i], bfr[BL][j], acc[i][j], 0, 0, 0);
     };
     int kt = 0;
-    for (; kt + NSTAGE - 1 < nk; ++kt) step(kt, std::true_type{});
+    if constexpr (SPREAD)
+        for (; kt + NSTAGE - 1 < nk; ++kt) step(kt, std::true_type{});
     for (; kt < nk; ++kt) step(kt, std::false_type{});
 #undef LI_FREAD
 #undef LI_WAIT_YOUNGER
@@ -970,6 +982,36 @@ static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, 
     return li_launch_status();
 }
 
+// More than 64 rows but so few 128 x 128 tiles that half of the compute units would idle (a narrow
+// matrix with a long K, like the feed-forward's way back at 128 to 512 rows): K is cut into parts
+// here too.  Returns the number of parts, 1 for none.
+static int split_parts_many_rows(int M, int N, int K) {
+    if (M <= 64 || K % 64) return 1;
+    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles >= 128) return 1;
+    int nsplit = (int)(256 / tiles);
+    if (nsplit > 8) nsplit = 8;
+    if (nsplit > K / 64 / 8) nsplit = K / 64 / 8;              // at least 8 steps a part
+    return nsplit < 2 ? 1 : nsplit;
+}
+
+// Bytes of workspace with which li_linear cuts this product along K (0: it would not).
+extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
+    if (in_dtype != LI_BF16 || M <= 32 || N <= 0 || K <= 0 || K % 64) return 0;
+    int nsplit = 1;
+    if (M <= 64) {
+        const int tiles = (N + 127) / 128;
+        if (tiles < 128) {
+            nsplit = 256 / tiles;
+            if (nsplit > 8) nsplit = 8;
+            if (nsplit > K / 64 / 8) nsplit = K / 64 / 8;
+        }
+    } else {
+        nsplit = split_parts_many_rows(M, N, K);
+    }
+    return nsplit < 2 ? 0 : (long)nsplit * M * N * (long)sizeof(float);
+}
+
 // `work` (may be null): device memory of work_bytes for the partial sums of a product cut along K.
 extern "C" int li_linear(const void* x, const void* w, const float* bias, void* out, int M, int N,
                          int K, int in_dtype, int out_dtype, int accumulate, void* work, long work_bytes,
@@ -1001,6 +1043,17 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
             // (area of a tile) / (its measured relative speed) is taken: large tiles are the fastest
             // per multiply-add but leave compute units idle when the matrix has few of them.
             if (K % 64 == 0) {
+                const int nsplit = split_parts_many_rows(M, N, K);
+                const size_t mn = (size_t)M * N;
+                if (nsplit > 1 && work && (size_t)work_bytes >= (size_t)nsplit * mn * sizeof(float)) {
+                    const int rc = launch_dma<128, 128, 64, 4, false, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)work,
+                                                                              M, N, K, 0, stream, nsplit);
+                    if (rc != LI_OK) return rc;
+                    const unsigned blocks = (unsigned)((mn + 255) / 256);
+                    if (out_dtype == LI_F32) splitk_reduce_kernel<float><<<blocks, 256, 0, stream>>>((const float*)work, nsplit, mn, N, bias, (float*)out, accumulate);
+                    else splitk_reduce_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const float*)work, nsplit, mn, N, bias, (bf16_t*)out, accumulate);
+                    return li_launch_status();
+                }
                 auto cost = [&](int bm, int bn, double speed) {
                     const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
                     return (double)((tiles + 255) / 256) * bm * bn / speed;

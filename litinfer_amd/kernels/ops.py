@@ -66,6 +66,15 @@ def _fn(module: str, name: str):
     return f
 
 
+def _work_bytes(m: int, n: int, k: int, dtype: int) -> int:
+    f = _fn_cache.get(("gemm", "li_linear_work_bytes"))
+    if f is None:
+        f = build.load("gemm").li_linear_work_bytes
+        f.argtypes, f.restype = [c_int, c_int, c_int, c_int], c_long
+        _fn_cache[("gemm", "li_linear_work_bytes")] = f
+    return int(f(m, n, k, dtype))
+
+
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
@@ -283,9 +292,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
          "linear: bias must be float32 [N]")
     if m:
         work, work_bytes = 0, 0
-        if ws is not None and x.dtype is torch.bfloat16 and SKINNY_MAX_ROWS // 2 < m <= SKINNY_MAX_ROWS:
-            buf = ws.buffer("gemm.parts", (SPLITK_MAX_PARTS * SKINNY_MAX_ROWS * n,), torch.float32)
-            work, work_bytes = buf.data_ptr(), buf.numel() * 4
+        if ws is not None and x.dtype is torch.bfloat16 and m > SKINNY_MAX_ROWS // 2:
+            # few rows over a long k and few columns: the library cuts k into parts if it is lent room for their sums
+            need = _work_bytes(m, n, k, _DT[x.dtype])
+            if need:
+                if m <= SKINNY_MAX_ROWS:            # one size for all row counts of a decode batch: the buffer does not move
+                    need = max(need, SPLITK_MAX_PARTS * SKINNY_MAX_ROWS * n * 4)
+                buf = ws.buffer("gemm.parts", (need // 4,), torch.float32)
+                work, work_bytes = buf.data_ptr(), buf.numel() * 4
         _run("gemm", "li_linear", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
              out.data_ptr(), m, n, k, _DT[x.dtype], _DT[out.dtype], int(bool(accumulate)), work, work_bytes)
 

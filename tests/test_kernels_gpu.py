@@ -136,8 +136,11 @@ class _Lender:
     (64, 136, 512, torch.bfloat16, False, False),        # too short a K for parts
     (40, 20000, 128, torch.float32, True, False),        # many tiles of 128 columns
     (64, 37000, 64, torch.bfloat16, False, False),       # many tiles of 256 columns
+    (128, 3584, 18944, torch.float32, False, True),      # more rows, but few tiles over a long K: parts again
+    (200, 300, 4096, torch.bfloat16, True, False),
+    (500, 1000, 1024, torch.float32, True, False),       # 32 tiles, two parts
 ])
-def test_linear_between_33_and_64_rows(ops, m, n, k, out_dtype, bias, acc):
+def test_linear_with_k_in_parts(ops, m, n, k, out_dtype, bias, acc):
     g = torch.Generator().manual_seed(15)
     x = (torch.randn(m, k, generator=g) * 2).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
