@@ -743,12 +743,25 @@ struct SkinnyArgs {
     bf16_t* kc;
     bf16_t* vc;
     int nh, nkv, dh, page_size, num_pages;
+    // An RMS norm between two products of up to 16 rows, without a pass of its own.  The product
+    // BEFORE it (float out with accumulate: the residual sum) also writes xg[m, n] = bf16(gamma[n] *
+    // out[m, n]) and, per block, the sums of squares of its columns of out to sq_parts[block * 16 + m].
+    const float* gamma;
+    bf16_t* xg;
+    float* sq_parts;
+    // The product AFTER it takes such an xg as its x and scales row m's sums by
+    // 1 / sqrt(sum_p row_parts[p * 16 + m] / K + eps): the factor of a row does not depend on k.
+    const float* row_parts;
+    int nparts;
+    float eps;
 };
+#define SK_MAX_PARTS 512            // blocks of a producing product whose sums one consumer adds up
 
 template <int MT, int NT, int WAVES, bool SWIGLU, typename TO, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs a) {
     static_assert(!ROPE || (MT == 1 && NT == 1 && !SWIGLU), "the rotary epilogue takes one tile");
     __shared__ floatx4 red[WAVES][MT * NT][64];
+    __shared__ float part_sums[WAVES * 4][16];
     const int M = a.M, N = a.N, K = a.K;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
@@ -841,6 +854,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     };
     if constexpr (AHEAD) {
         if (wave < nchunks) load_chunk(wave, wbuf[0], xbuf[0]);
+        if (a.row_parts) {
+            // the rows' sums of squares: thread t adds the parts t / 16, t / 16 + G, ... of row t % 16 in
+            // that order; the epilogue adds the G sums in theirs.  The loads are issued together, behind
+            // those of the first chunk, only as many rounds as there are parts, and never conditional
+            // within a round (a part past the end reads the last one).
+            constexpr int G = WAVES * 4, PER = SK_MAX_PARTS / G;
+            const int m = threadIdx.x & 15, q = threadIdx.x >> 4;
+            float part[PER];
+#pragma unroll
+            for (int i = 0; i < PER; ++i) {
+                part[i] = 0.f;
+                if (i * G < a.nparts) {
+                    const int p = q + i * G;
+                    part[i] = a.row_parts[(size_t)(p < a.nparts ? p : a.nparts - 1) * 16 + m];
+                }
+            }
+            float mine = 0.f;
+#pragma unroll
+            for (int i = 0; i < PER; ++i) mine += (q + i * G < a.nparts) ? part[i] : 0.f;
+            part_sums[q][m] = mine;
+        }
         for (int c = wave; c < nchunks; c += 2 * WAVES) {          // two chunks a turn: buffer numbers are constants
             if (c + WAVES < nchunks) load_chunk(c + WAVES, wbuf[1], xbuf[1]);
             multiply(wbuf[0], xbuf[0]);
@@ -873,6 +907,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 const floatx4 o = red[wv][mt * NT + nt][l];
                 s[nt][0] += o[0]; s[nt][1] += o[1]; s[nt][2] += o[2]; s[nt][3] += o[3];
             }
+        }
+        if (AHEAD && a.row_parts) {
+            float sq = part_sums[0][m & 15];
+#pragma unroll
+            for (int q = 1; q < WAVES * 4; ++q) sq += part_sums[q][m & 15];
+            const float inv = 1.0f / sqrtf(sq / (float)K + a.eps);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) { s[nt][0] *= inv; s[nt][1] *= inv; s[nt][2] *= inv; s[nt][3] *= inv; }
         }
         if constexpr (ROPE) {
             const int dh = a.dh, half = dh / 2, bph = dh / 16;
@@ -913,6 +955,31 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 }
             }
         } else {
+            if constexpr (sizeof(TO) == 4 && MT == 1) {
+                if (a.xg) {                          // the sum goes out three ways (see SkinnyArgs)
+                    float sq = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int n = n0 + 16 * nt + 4 * (l >> 4) + r;
+                            if (n < N) {
+                                const size_t idx = (size_t)m * N + n;
+                                float v = s[nt][r];
+                                if (a.bias) v += a.bias[n];
+                                if (a.accumulate) v += reinterpret_cast<const float*>(out)[idx];
+                                reinterpret_cast<float*>(out)[idx] = v;
+                                a.xg[idx].bits = float_to_bf16(a.gamma[n] * v);
+                                sq += v * v;
+                            }
+                        }
+                    // the four lanes of a row (l, l ^ 16, l ^ 32, l ^ 48: all of them are here, or none)
+                    sq += __shfl_xor(sq, 16, 64);
+                    sq += __shfl_xor(sq, 32, 64);
+                    if ((l >> 4) == 0) a.sq_parts[(size_t)blockIdx.x * 16 + m] = sq;
+                    continue;
+                }
+            }
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -945,11 +1012,29 @@ extern "C" int li_linear_skinny(const void* x, const void* w, const float* bias,
     if (accumulate && out_dtype != LI_F32) return LI_ERR_DTYPE;
     if (swiglu && (bias || accumulate || out_dtype != LI_BF16)) return LI_ERR_DTYPE;
     SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, accumulate,
-                 nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, nullptr, 0, 0.f};
     if (swiglu) launch_skinny<true, bf16_t>(a, stream);
     else if (out_dtype == LI_BF16) launch_skinny<false, bf16_t>(a, stream);
     else if (out_dtype == LI_F32) launch_skinny<false, float>(a, stream);
     else return LI_ERR_DTYPE;
+    return li_launch_status();
+}
+
+// The product before an RMS norm that is fused into its neighbours (see SkinnyArgs): out += x w^T + bias
+// in float32, xg = bf16(gamma * out), sq_parts[block * 16 + m] = the block's share of row m's sum of
+// squares.  Up to 16 rows.  li_residual_norm_parts(N) is the number of blocks, i.e. of parts.
+extern "C" int li_residual_norm_parts(int N) {
+    const int per = N >= 8192 ? 32 : 16;               // as launch_skinny tiles the columns of few rows
+    return (N + per - 1) / per;
+}
+
+extern "C" int li_linear_residual_norm(const void* x, const void* w, const float* bias, float* out, int M, int N,
+                                       int K, const float* gamma, void* xg, float* sq_parts, hipStream_t stream) {
+    if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K % 8) || !gamma || !xg || !sq_parts) return LI_ERR_SIZE;
+    if (li_residual_norm_parts(N) > SK_MAX_PARTS) return LI_ERR_SIZE;
+    SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, 1,
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, gamma, (bf16_t*)xg, sq_parts, nullptr, 0, 0.f};
+    launch_skinny<false, float>(a, stream);
     return li_launch_status();
 }
 
@@ -1082,10 +1167,19 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
 // out[m, n] = up * gate / (1 + exp(-gate)) with [gate, up] = x w^T, w = [gate; up] of I rows each:
 // the activation as the product's epilogue, so the 2 I columns never go to memory.  bfloat16;
 // K a multiple of 8 for up to 64 rows, a multiple of 64 above.
+// row_parts (may be null): x is the xg of li_linear_residual_norm and these are its sq_parts, nparts of
+// them; every row's result is that of the RMS norm with eps (up to 16 rows).
 extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, int I, int K,
-                                hipStream_t stream) {
+                                const float* row_parts, int nparts, float eps, hipStream_t stream) {
     if (M <= 0 || I <= 0 || K <= 0 || I > 0x3fffffff) return LI_ERR_SIZE;
     const int N = 2 * I;
+    if (row_parts) {
+        if (M > 16 || (K % 8) || nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f) return LI_ERR_SIZE;
+        SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, nullptr, out, M, I, K, 0,
+                     nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, row_parts, nparts, eps};
+        launch_skinny<true, bf16_t>(a, stream);
+        return li_launch_status();
+    }
     if (M > 32 && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
         if ((N + 255) / 256 >= 128)
             return launch_dma<64, 256, 64, 3, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
@@ -1110,15 +1204,19 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
 // heads and the write of keys and values into their page slots as its epilogue (see ROPE above).
 // w [(nh + 2 nkv) dh, K] bfloat16, bias float32 or null, out [M, (nh + 2 nkv) dh] bfloat16 (rotated
 // q, rotated k, v), cos/sin float32 [M, dh / 2], slot_map int32 [M], kc/vc the cache layer.
+// row_parts, nparts, eps: as for li_linear_swiglu.
 extern "C" int li_linear_rope_store(const void* x, const void* w, const float* bias, void* out, int M, int K,
                                     const float* cos, const float* sin, const int* slot_map, void* kc, void* vc,
-                                    int nh, int nkv, int dh, int page_size, int num_pages, hipStream_t stream) {
+                                    int nh, int nkv, int dh, int page_size, int num_pages,
+                                    const float* row_parts, int nparts, float eps, hipStream_t stream) {
     if (M <= 0 || M > 16 || K <= 0 || K % 8 || nh <= 0 || nkv <= 0 || dh <= 0 || dh % 16 || page_size <= 0 ||
         num_pages <= 0 || (long)(nh + 2 * nkv) * dh > 0x7fffffffL)
         return LI_ERR_SIZE;
     const int N = (nh + 2 * nkv) * dh;
     SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, 0, cos, sin, slot_map,
-                 (bf16_t*)kc, (bf16_t*)vc, nh, nkv, dh, page_size, num_pages};
+                 (bf16_t*)kc, (bf16_t*)vc, nh, nkv, dh, page_size, num_pages,
+                 nullptr, nullptr, nullptr, row_parts, row_parts ? nparts : 0, eps};
+    if (row_parts && (nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f)) return LI_ERR_SIZE;
     gemm_bf16_skinny_kernel<1, 1, 8, false, bf16_t, true><<<N / 16, 8 * 64, 0, stream>>>(a);
     return li_launch_status();
 }

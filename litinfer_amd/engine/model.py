@@ -77,6 +77,9 @@ class Model:
         self.embedding.forward(ctx.ids, x, ctx.id_src, ctx.feedback)
         stream = ResidualStream(x, ctx.ws)
         for i, e in enumerate(self.order):
+            # the block is told through which norm the next one reads what it leaves
+            follower = self.layers[self.order[i + 1].layer] if i + 1 < len(self.order) else None
+            stream.next_norm = follower.first_norm() if follower is not None else None
             self.layers[e.layer].forward(stream, ctx, cache.view(i))
         x = stream.tensor()
         if ctx.num_want == 0:

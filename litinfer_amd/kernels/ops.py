@@ -38,8 +38,9 @@ _SIGNATURES = {
     "gemm": {
         "li_linear": [P, P, P, P, I, I, I, I, I, I, P, L],
         "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
-        "li_linear_swiglu": [P, P, P, I, I, I],
-        "li_linear_rope_store": [P, P, P, P, I, I, P, P, P, P, P, I, I, I, I, I],
+        "li_linear_swiglu": [P, P, P, I, I, I, P, I, F],
+        "li_linear_residual_norm": [P, P, P, P, I, I, I, P, P, P],
+        "li_linear_rope_store": [P, P, P, P, I, I, P, P, P, P, P, I, I, I, I, I, P, I, F],
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
@@ -336,9 +337,71 @@ def swiglu_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
     return w_dtype is torch.bfloat16 and m > 0 and (k % 8 == 0 if m <= SKINNY_MAX_ROWS else k % 64 == 0)
 
 
-def linear_swiglu(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+# An RMS norm between two products of few rows (a decoding step), without a pass of its own: the
+# product before it, which adds to the float32 sum, also writes the sum times the norm's weights in
+# bfloat16 and each block's share of the rows' sums of squares (`linear_residual_norm`); the product
+# after it multiplies those rows and scales each row's result by the norm's factor (`row_scale` of
+# `linear_swiglu` and `linear_rope_store`).
+RESIDUAL_NORM_MAX_ROWS = 16
+RESIDUAL_NORM_MAX_PARTS = 512
+
+
+class RowScale:
+    """What the product after a fused RMS norm needs beside its rows: the shares of the rows' sums
+    of squares [nparts * 16] float32 and the norm's eps."""
+    def __init__(self, sq_parts: torch.Tensor, nparts: int, eps: float):
+        self.sq_parts, self.nparts, self.eps = sq_parts, int(nparts), float(eps)
+
+
+def residual_norm_parts(n: int) -> int:
+    """Blocks of `linear_residual_norm` over n columns, i.e. shares of a row's sum of squares."""
+    per = 32 if n >= 8192 else 16
+    return -(-n // per)
+
+
+def residual_norm_takes(m: int, n: int, k: int, w_dtype: torch.dtype) -> bool:
+    return (w_dtype is torch.bfloat16 and 0 < m <= RESIDUAL_NORM_MAX_ROWS and k % 8 == 0
+            and residual_norm_parts(n) <= RESIDUAL_NORM_MAX_PARTS)
+
+
+def linear_residual_norm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                         gamma: torch.Tensor, xg: torch.Tensor, sq_parts: torch.Tensor) -> int:
+    """out += x w^T + bias (float32); xg = bfloat16(gamma * out); sq_parts[p * 16 + m] = block p's
+    share of sum_n out[m, n]^2.  Returns the number of blocks p."""
+    _gpu(x, w, bias, out, gamma, xg, sq_parts)
+    m, k = x.shape
+    n = w.shape[0]
+    _chk(residual_norm_takes(m, n, k, w.dtype), "linear_residual_norm: sizes or dtype not taken")
+    _chk(x.dtype is torch.bfloat16 and w.shape == (n, k) and x.is_contiguous() and w.is_contiguous(),
+         "linear_residual_norm: x and w must be contiguous bfloat16 [M, K] and [N, K]")
+    _chk(out.dtype is torch.float32 and out.shape == (m, n) and out.is_contiguous(), "linear_residual_norm: out must be float32 [M, N]")
+    _chk(xg.dtype is torch.bfloat16 and xg.shape == (m, n) and xg.is_contiguous(), "linear_residual_norm: xg must be bfloat16 [M, N]")
+    _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
+         "linear_residual_norm: bias must be float32 [N]")
+    _chk(gamma.dtype is torch.float32 and gamma.shape == (n,) and gamma.is_contiguous(), "linear_residual_norm: gamma must be float32 [N]")
+    parts = residual_norm_parts(n)
+    _chk(sq_parts.dtype is torch.float32 and sq_parts.is_contiguous() and sq_parts.numel() >= parts * 16,
+         "linear_residual_norm: sq_parts must be float32 with 16 places a block")
+    _run("gemm", "li_linear_residual_norm", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
+         out.data_ptr(), m, n, k, gamma.data_ptr(), xg.data_ptr(), sq_parts.data_ptr())
+    return parts
+
+
+def _check_row_scale(what: str, m: int, row_scale: Optional[RowScale]):
+    if row_scale is None:
+        return 0, 0, 0.0
+    _gpu(row_scale.sq_parts)
+    _chk(0 < m <= RESIDUAL_NORM_MAX_ROWS, f"{what}: a row scale goes with up to {RESIDUAL_NORM_MAX_ROWS} rows")
+    _chk(0 < row_scale.nparts <= RESIDUAL_NORM_MAX_PARTS and row_scale.eps >= 0, f"{what}: row scale out of range")
+    _chk(row_scale.sq_parts.dtype is torch.float32 and row_scale.sq_parts.is_contiguous()
+         and row_scale.sq_parts.numel() >= row_scale.nparts * 16, f"{what}: the row scale's parts must be float32 [nparts * 16]")
+    return row_scale.sq_parts.data_ptr(), row_scale.nparts, row_scale.eps
+
+
+def linear_swiglu(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_scale: Optional[RowScale] = None) -> None:
     """out[m, n] = up * gate / (1 + exp(-gate)) with [gate, up] = x w^T, w = [gate; up]
-    (2 N rows): the activation in the product's epilogue, from the product's float32 sums."""
+    (2 N rows): the activation in the product's epilogue, from the product's float32 sums.
+    With `row_scale`, x is the xg of `linear_residual_norm` and the result is that of the norm."""
     _gpu(x, w, out)
     _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear_swiglu: needs matrices")
     m, k = x.shape
@@ -347,7 +410,8 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     _chk(w.shape == (2 * n, k) and out.shape[0] == m, "linear_swiglu: shapes do not fit")
     _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_swiglu: contiguous operands")
     _chk(x.dtype is torch.bfloat16 and out.dtype is torch.bfloat16, "linear_swiglu: x and out must be bfloat16")
-    _run("gemm", "li_linear_swiglu", x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k)
+    _run("gemm", "li_linear_swiglu", x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
+         *_check_row_scale("linear_swiglu", m, row_scale))
 
 
 ROPE_STORE_MAX_ROWS = 16
@@ -361,11 +425,13 @@ def rope_store_takes(m: int, k: int, w_dtype: torch.dtype, dh: int, rotary_dim: 
 
 def linear_rope_store(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                       nh: int, nkv: int, dh: int, cos: torch.Tensor, sin: torch.Tensor,
-                      slot_map: torch.Tensor, k: torch.Tensor, v: torch.Tensor, page_size: int) -> None:
+                      slot_map: torch.Tensor, k: torch.Tensor, v: torch.Tensor, page_size: int,
+                      row_scale: Optional[RowScale] = None) -> None:
     """Fused for a decoding step: out = x w^T + bias with w the packed [q; k; v]
     projection, query and key heads rotated (half-split pairs, the whole head) by
     the rows' angles, keys and values written into their page slots.  out holds
-    the rotated queries and keys and the values, as after the separate kernels."""
+    the rotated queries and keys and the values, as after the separate kernels.
+    With `row_scale`, x is the xg of `linear_residual_norm` and the result is that of the norm."""
     _gpu(x, w, bias, out, cos, sin, slot_map, k, v)
     m, kk = x.shape
     n = (nh + 2 * nkv) * dh
@@ -382,7 +448,7 @@ def linear_rope_store(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Ten
          "linear_rope_store: slot_map")
     _run("gemm", "li_linear_rope_store", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
          out.data_ptr(), m, kk, cos.data_ptr(), sin.data_ptr(), slot_map.data_ptr(), k.data_ptr(), v.data_ptr(),
-         nh, nkv, dh, page_size, k.shape[0])
+         nh, nkv, dh, page_size, k.shape[0], *_check_row_scale("linear_rope_store", m, row_scale))
 
 
 # ----------------------------------------------------------------- attention

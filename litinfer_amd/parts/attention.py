@@ -80,6 +80,18 @@ class GQAttention(Mixer):
         self.out = Linear(self.rt, get(p + "o_proj.weight"),
                           get(p + "o_proj.bias") if self.out_bias else None)
 
+    def forward_prenorm(self, norm, residual, xn, ctx, cache):
+        # few rows (decoding): the product before the norm may have left its rows scaled by the
+        # norm's weights; then projection, rows' factors, encoding and page write are one kernel
+        sc = residual.scaled_rows(norm)
+        if sc is not None and self.position is not None:
+            qkv = ctx.ws.buffer("attn.qkv", (sc.rows.shape[0], self.n_q + 2 * self.n_kv), self.rt.dtype)
+            if self.position.project_encode_store(self.qkv, sc.rows, qkv, self.nh, self.nkv, self.dh, ctx, cache,
+                                                  row_scale=sc.scale):
+                return self._attend(qkv, residual, ctx, cache)
+        residual.normed(norm, xn)
+        self.forward(xn, residual, ctx, cache)
+
     def forward(self, xn, residual, ctx, cache):
         t = xn.shape[0]
         qkv = ctx.ws.buffer("attn.qkv", (t, self.n_q + 2 * self.n_kv), self.rt.dtype)
@@ -92,7 +104,10 @@ class GQAttention(Mixer):
             elif cache.owned:
                 ops.kv_store(qkv, self.nh, self.nkv, self.dh, ctx.slot_map(cache.group),
                              cache.k, cache.v, cache.page_size)
-        attn = ctx.ws.buffer("attn.out", (t, self.n_q), self.rt.dtype)
+        self._attend(qkv, residual, ctx, cache)
+
+    def _attend(self, qkv, residual, ctx, cache):
+        attn = ctx.ws.buffer("attn.out", (qkv.shape[0], self.n_q), self.rt.dtype)
         ops.paged_attention(qkv, attn, cache.k, cache.v, ctx.attention_meta(cache.group),
                             self.nh, self.nkv, self.dh, cache.page_size, self.window, self.scale, ws=ctx.ws)
         residual.add_linear(self.out, attn)

@@ -92,11 +92,34 @@ class Part:
         optional tensor is absent."""
 
 
+@dataclass(frozen=True)
+class RmsScaling:
+    """An RMS norm, y = weight * x / sqrt(mean(x^2) + eps), in the form in which the
+    products on its two sides can take it over: the one before writes weight * x, the
+    one after scales its rows by 1 / sqrt(mean(x^2) + eps)."""
+    weight: torch.Tensor          # float32 [size]
+    eps: float
+
+
+@dataclass
+class ScaledRows:
+    """The input of a norm as the product before it left it: `rows` = weight * x
+    in the engine's dtype, `scale` what the product after it needs for the rows'
+    factors (an `ops.RowScale`)."""
+    rows: torch.Tensor
+    scale: Any
+
+
 class Norm(Part):
     category = "norm"
 
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
+
+    def as_scaling(self) -> Optional[RmsScaling]:
+        """How the products on the two sides of this norm can share it between them
+        (an RmsScaling), or None: then the norm is always a pass of its own."""
+        return None
 
 
 class Mixer(Part):
@@ -108,6 +131,14 @@ class Mixer(Part):
     def forward(self, xn, residual, ctx, cache) -> None:
         raise NotImplementedError
 
+    def forward_prenorm(self, norm: Norm, residual, xn, ctx, cache) -> None:
+        """x += mixer(norm(x)) for the residual stream x; `xn` is room for the
+        normed rows.  The default norms in a pass of its own.  A mixer whose first
+        product can scale its rows overrides this and asks the stream for
+        `scaled_rows(norm)`, which the product before the norm may have left."""
+        residual.normed(norm, xn)
+        self.forward(xn, residual, ctx, cache)
+
 
 class FeedForward(Part):
     category = "feed_forward"
@@ -115,11 +146,22 @@ class FeedForward(Part):
     def forward(self, xn, residual, ctx) -> None:
         raise NotImplementedError
 
+    def forward_prenorm(self, norm: Norm, residual, xn, ctx) -> None:
+        """x += feed_forward(norm(x)); see Mixer.forward_prenorm."""
+        residual.normed(norm, xn)
+        self.forward(xn, residual, ctx)
+
 
 class Block(Part):
     category = "block"
 
     def cache_need(self):
+        return None
+
+    def first_norm(self) -> Optional[Norm]:
+        """The norm through which this block first reads the residual stream, if
+        that is how it begins: the block before it is told, so that its last
+        product can prepare the rows."""
         return None
 
     def forward(self, x, ctx, cache) -> None:

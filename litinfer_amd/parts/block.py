@@ -33,12 +33,17 @@ class PreNormBlock(Block):
         for p in self._all:
             p.load_params(get)
 
+    def first_norm(self):
+        return self.norm1
+
     def forward(self, stream, ctx, cache):
         xn = ctx.ws.buffer("block.xn", stream.shape, self.rt.dtype)
-        stream.normed(self.norm1, xn)
-        self.mixer.forward(xn, stream, ctx, cache)
-        stream.normed(self.norm2, xn)
-        self.ffn.forward(xn, stream, ctx)
+        after = stream.next_norm                   # the norm that reads the stream after this block
+        stream.next_norm = self.norm2
+        self.mixer.forward_prenorm(self.norm1, stream, xn, ctx, cache)
+        stream.next_norm = after
+        self.ffn.forward_prenorm(self.norm2, stream, xn, ctx)
+        stream.next_norm = None
 
 
 register_part("block", "prenorm", PreNormBlock)

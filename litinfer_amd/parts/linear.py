@@ -23,15 +23,28 @@ class Linear:
         return (x.dtype is torch.bfloat16 and self.bias is None
                 and ops.swiglu_takes(x.shape[0], self.in_features, self.weight.dtype))
 
+    def takes_scaling(self, x: torch.Tensor, out: torch.Tensor) -> bool:
+        """Whether out += x W^T + b can also leave out times a norm's weights and the
+        shares of the rows' sums of squares (few rows, bfloat16 operands)."""
+        return (x.dtype is torch.bfloat16 and out.dtype is torch.float32
+                and ops.residual_norm_takes(x.shape[0], self.out_features, self.in_features, self.weight.dtype))
+
+    def add_with_scaling(self, x: torch.Tensor, out: torch.Tensor, scaling, rows: torch.Tensor, ws):
+        """out += x W^T + b; rows = scaling.weight * out.  Returns what the product
+        behind the norm needs for the rows' factors."""
+        parts = ws.buffer("linear.sq_parts", (ops.RESIDUAL_NORM_MAX_PARTS * 16,), torch.float32)
+        n = ops.linear_residual_norm(x, self.weight, self.bias, out, scaling.weight, rows, parts)
+        return ops.RowScale(parts, n, scaling.eps)
+
     def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ws=None,
-                 swiglu: bool = False):
+                 swiglu: bool = False, row_scale=None):
         """out = x W^T + b, or out += ... when `accumulate` (out is float32 then).
         With `swiglu` (only where `takes_swiglu`) W is [gate; up] and out gets
-        up * silu(gate).  A matrix that is stored in 32-bit is multiplied in
+        up * silu(gate); `row_scale` then says that x came out of `add_with_scaling`.  A matrix that is stored in 32-bit is multiplied in
         32-bit also when the activations are bfloat16: they are widened for it,
         exactly."""
         if swiglu:
-            ops.linear_swiglu(x, self.weight, out)
+            ops.linear_swiglu(x, self.weight, out, row_scale=row_scale)
         elif self.weight.dtype is torch.float32 and x.dtype is not torch.float32:
             x32 = ws.buffer("linear.x32", x.shape, torch.float32)
             ops.cast(x, x32)

@@ -35,6 +35,17 @@ class SwiGLUMLP(FeedForward):
         self.gate_up = Linear(self.rt, torch.cat([g.to(dt), u.to(dt)], dim=0))
         self.down = Linear(self.rt, get(p + "down_proj.weight"))
 
+    def forward_prenorm(self, norm, residual, xn, ctx):
+        # few rows (decoding): the product before the norm may have left its rows scaled by the
+        # norm's weights; the gate/up product then applies the rows' factors with its activation
+        sc = residual.scaled_rows(norm)
+        if sc is not None and self.gate_up.takes_swiglu(sc.rows):
+            h = ctx.ws.buffer("mlp.h", (sc.rows.shape[0], self.inter), self.rt.dtype)
+            self.gate_up(sc.rows, h, ws=ctx.ws, swiglu=True, row_scale=sc.scale)
+            return residual.add_linear(self.down, h)
+        residual.normed(norm, xn)
+        self.forward(xn, residual, ctx)
+
     def forward(self, xn, residual, ctx):
         t = xn.shape[0]
         h = ctx.ws.buffer("mlp.h", (t, self.inter), self.rt.dtype)

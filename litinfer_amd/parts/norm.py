@@ -5,7 +5,7 @@ from __future__ import annotations
 
 from ..kernels import ops
 from ..weights.loader import ParamSpec
-from .base import Norm, register_part
+from .base import Norm, RmsScaling, register_part
 
 
 class RMSNorm(Norm):
@@ -28,6 +28,9 @@ class RMSNorm(Norm):
     def forward(self, x, out):
         ops.rmsnorm(x, self.weight, self.eps, out)
         return out
+
+    def as_scaling(self):
+        return RmsScaling(self.weight, self.eps)
 
 
 register_part("norm", "rmsnorm", RMSNorm)

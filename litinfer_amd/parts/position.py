@@ -27,10 +27,13 @@ class Position(Part):
         h*head_dim..) in place."""
         raise NotImplementedError
 
-    def project_encode_store(self, proj, xn, qkv, num_heads, num_kv_heads, head_dim, ctx, cache) -> bool:
+    def project_encode_store(self, proj, xn, qkv, num_heads, num_kv_heads, head_dim, ctx, cache,
+                             row_scale=None) -> bool:
         """An encoding that has the packed projection, the encoding and the page
         write in ONE kernel for this batch does all three and returns True; the
-        default has none, and the mixer then projects and calls `encode_and_store`."""
+        default has none, and the mixer then projects and calls `encode_and_store`.
+        With `row_scale`, `xn` is a norm's input times its weights and the kernel
+        would have to apply the rows' factors as well."""
         return False
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache) -> None:
@@ -78,7 +81,7 @@ class RopeNeox(Position):
         cos, sin = self.tables(ctx)
         ops.rope_apply(qkv, n_heads_total, head_dim, self.rotary_dim, cos, sin)
 
-    def project_encode_store(self, proj, xn, qkv, num_heads, num_kv_heads, head_dim, ctx, cache):
+    def project_encode_store(self, proj, xn, qkv, num_heads, num_kv_heads, head_dim, ctx, cache, row_scale=None):
         # few rows (decoding): the rotation and the page write are the projection's epilogue
         if not (cache.owned and xn.dtype is ops.bfloat16 and proj.weight.dtype is ops.bfloat16
                 and ops.rope_store_takes(xn.shape[0], proj.in_features, proj.weight.dtype, head_dim,
@@ -86,7 +89,7 @@ class RopeNeox(Position):
             return False
         cos, sin = self.tables(ctx)
         ops.linear_rope_store(xn, proj.weight, proj.bias, qkv, num_heads, num_kv_heads, head_dim, cos, sin,
-                              ctx.slot_map(cache.group), cache.k, cache.v, cache.page_size)
+                              ctx.slot_map(cache.group), cache.k, cache.v, cache.page_size, row_scale=row_scale)
         return True
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, cache):

@@ -196,6 +196,87 @@ def test_linear_with_swiglu_epilogue(ops, m, n, k):
     assert torch.count_nonzero(o).item() <= 2 * m + 1
 
 
+@pytest.mark.parametrize("m,n,kprev,inter,eps", [
+    (8, 3584, 512, 1024, 1e-6),      # a decoding step at the 7B width
+    (1, 40, 8, 24, 1e-5),
+    (16, 8200, 64, 48, 1e-5),        # a width from which the product before takes 32 columns a block; ragged
+    (5, 200, 136, 301, 0.1),         # a ragged last block of 16 columns; an eps that counts
+])
+def test_rms_norm_shared_between_the_products_on_its_two_sides(ops, m, n, kprev, inter, eps):
+    """x += h Wo^T leaves gamma * x and the shares of the rows' sums of squares; the gate/up product
+    with SwiGLU (and the packed projection with rotary encoding and page write) scales its rows."""
+    g = torch.Generator().manual_seed(18)
+    h = torch.randn(m, kprev, generator=g).to(torch.bfloat16)
+    wo = (torch.randn(n, kprev, generator=g) / math.sqrt(kprev)).to(torch.bfloat16)
+    bias = torch.randn(n, generator=g) * 0.1
+    base = torch.randn(m, n, generator=g) * torch.logspace(-2, 2, m)[:, None]       # rows of very different size
+    gamma = torch.rand(n, generator=g) + 0.5
+    x = base.double().numpy() + h.double().numpy() @ wo.double().numpy().T + bias.double().numpy()
+    assert ops.residual_norm_takes(m, n, kprev, wo.dtype)
+    out = base.to(DEV)
+    xg = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    parts = torch.full((ops.RESIDUAL_NORM_MAX_PARTS * 16,), float("nan"), device=DEV)
+    nparts = ops.linear_residual_norm(h.to(DEV), wo.to(DEV), bias.to(DEV), out, gamma.to(DEV), xg, parts)
+    assert nparts == ops.residual_norm_parts(n) == -(-n // (32 if n >= 8192 else 16))
+    for i in range(m):
+        assert rel(out[i], x[i]) < 1e-5, i
+        assert rel(xg[i], gamma.double().numpy() * x[i]) < 2.0 ** -8, i
+    sq = parts[:nparts * 16].view(nparts, 16)[:, :m].double().sum(dim=0).cpu().numpy()
+    assert np.allclose(sq, (x * x).sum(axis=1), rtol=1e-5)
+    # the same sum as the product alone leaves it
+    alone = base.to(DEV)
+    ops.linear(h.to(DEV), wo.to(DEV), bias.to(DEV), alone, True)
+    assert torch.equal(alone, out)
+    scale = ops.RowScale(parts, nparts, eps)
+    xn = plain_impl.rms_norm(x, gamma.double().numpy(), eps)
+    xb = xg.double().cpu().numpy()                       # what the product after the norm multiplies
+    inv = 1.0 / np.sqrt((x * x).mean(axis=1, keepdims=True) + eps)
+    # -- gate/up with SwiGLU
+    w = (torch.randn(2 * inter, n, generator=g) / math.sqrt(n)).to(torch.bfloat16)
+    y = xn @ w.double().numpy().T
+    ref = plain_impl.swiglu(y[:, :inter], y[:, inter:])
+    got = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear_swiglu(xg, w.to(DEV), got, row_scale=scale)
+    yb = (xb @ w.double().numpy().T) * inv
+    refb = plain_impl.swiglu(yb[:, :inter], yb[:, inter:])
+    for i in range(m):                                   # the kernel's own arithmetic, row by row
+        assert rel(got[i], refb[i]) < 5e-3, i
+    # against the plain norm and product, element by element within what rounding the rows to
+    # bfloat16 (each term by at most 2^-9 of itself) and the output can do:
+    # |d out| <= |silu(g)| |d u| + |u| |silu'(g)| |d g| + 2^-9 |out|, |silu'| <= 1.1
+    ya = np.abs(xn) @ np.abs(w.double().numpy()).T
+    g_, u_ = y[:, :inter], y[:, inter:]
+    bound = 2.0 ** -9 * (np.abs(g_ / (1 + np.exp(-g_))) * ya[:, inter:] + 1.1 * np.abs(u_) * ya[:, :inter] + np.abs(ref))
+    err = np.abs(got.double().cpu().numpy() - ref)
+    assert (err <= 1.01 * bound + 1e-30).all(), float((err / (bound + 1e-30)).max())
+    # -- the packed projection with rotary encoding and page write
+    nh, nkv, dh, page, pages = 3, 1, 32, 8, 5
+    nq = (nh + 2 * nkv) * dh
+    wq = (torch.randn(nq, n, generator=g) / math.sqrt(n)).to(torch.bfloat16)
+    bq = torch.randn(nq, generator=g)
+    pos = torch.randint(0, 3000, (m,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(pages * page, generator=g)[:m].to(torch.int32)
+    cos = torch.empty(m, dh // 2, device=DEV)
+    sin = torch.empty(m, dh // 2, device=DEV)
+    ops.rope_table(pos.to(DEV), 1e6, dh, cos, sin)
+    kc = torch.zeros((pages, nkv, page, dh), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    q = torch.full((m, nq), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.linear_rope_store(xg, wq.to(DEV), bq.to(DEV), q, nh, nkv, dh, cos, sin, slots.to(DEV), kc, vc, page,
+                          row_scale=scale)
+    yq = ((xb @ wq.double().numpy().T) * inv + bq.double().numpy()).reshape(m, nh + 2 * nkv, dh)
+    refq = np.concatenate([plain_impl.rope_neox(yq[:, :nh + nkv], pos.numpy(), 1e6), yq[:, nh + nkv:]], axis=1)
+    assert rel(q, refq.reshape(m, nq)) < 5e-3
+    qv = q.cpu().view(m, nh + 2 * nkv, dh)
+    for i in range(m):
+        sl = int(slots[i])
+        assert torch.equal(kc[sl // page, :, sl % page].cpu(), qv[i, nh:nh + nkv])
+        assert torch.equal(vc[sl // page, :, sl % page].cpu(), qv[i, nh + nkv:])
+    with pytest.raises(ValueError):                      # more rows than the kernels scale
+        ops.linear_swiglu(torch.zeros(17, n, dtype=torch.bfloat16, device=DEV), w.to(DEV),
+                          torch.empty(17, inter, dtype=torch.bfloat16, device=DEV), row_scale=scale)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_linear_rows_do_not_depend_on_the_batch(ops, dtype):
     g = torch.Generator().manual_seed(3)

@@ -131,16 +131,54 @@ def swiglu_takes(m, k, w_dtype):
     return w_dtype is torch.bfloat16 and m > 0 and (k % 8 == 0 if m <= 64 else k % 64 == 0)
 
 
-def linear_swiglu(x, w, out):
-    linear_skinny(x, w, None, out, False, swiglu=True)
+RESIDUAL_NORM_MAX_PARTS = 512
+
+
+class RowScale:
+    def __init__(self, sq_parts, nparts, eps):
+        self.sq_parts, self.nparts, self.eps = sq_parts, int(nparts), float(eps)
+
+
+def residual_norm_parts(n):
+    return -(-n // (32 if n >= 8192 else 16))
+
+
+def residual_norm_takes(m, n, k, w_dtype):
+    return w_dtype is torch.bfloat16 and 0 < m <= 16 and k % 8 == 0 and residual_norm_parts(n) <= RESIDUAL_NORM_MAX_PARTS
+
+
+def linear_residual_norm(x, w, bias, out, gamma, xg, sq_parts):
+    linear(x, w, bias, out, True)
+    xg.copy_((gamma * out).to(xg.dtype))
+    per = 32 if out.shape[1] >= 8192 else 16
+    parts = residual_norm_parts(out.shape[1])
+    for p in range(parts):                               # one share a block of columns, 16 places each
+        sq_parts[p * 16:p * 16 + out.shape[0]] = (out[:, p * per:(p + 1) * per] ** 2).sum(dim=1)
+    return parts
+
+
+def _row_factors(row_scale, m, k):
+    sq = row_scale.sq_parts[:row_scale.nparts * 16].view(row_scale.nparts, 16)[:, :m].sum(dim=0)
+    return (1.0 / torch.sqrt(sq / k + row_scale.eps))[:, None]
+
+
+def linear_swiglu(x, w, out, row_scale=None):
+    if row_scale is None:
+        return linear_skinny(x, w, None, out, False, swiglu=True)
+    y = (x.float() @ w.float().T) * _row_factors(row_scale, x.shape[0], x.shape[1])
+    n = out.shape[1]
+    g, u = y[:, :n], y[:, n:]
+    out.copy_((u * (g / (1 + torch.exp(-g)))).to(out.dtype))
 
 
 def rope_store_takes(m, k, w_dtype, dh, rotary_dim):
     return w_dtype is torch.bfloat16 and 0 < m <= 16 and k % 8 == 0 and dh % 16 == 0 and rotary_dim == dh
 
 
-def linear_rope_store(x, w, bias, out, nh, nkv, dh, cos, sin, slot_map, k, v, page_size):
+def linear_rope_store(x, w, bias, out, nh, nkv, dh, cos, sin, slot_map, k, v, page_size, row_scale=None):
     y = x.float() @ w.float().T
+    if row_scale is not None:
+        y = y * _row_factors(row_scale, x.shape[0], x.shape[1])
     if bias is not None:
         y = y + bias
     # rotated from the 32-bit sums and rounded once, as the fused kernel does
