@@ -134,7 +134,7 @@ def main() -> int:
     value = a.batch * a.steps / dt
     nbytes = decode_bytes(cfg, a.layers, ctx_tokens, es)
     out = {
-        "metric": "decode tok/s (Qwen2-7B shape, batch 8, context 4096)", "value": round(value, 2),
+        "metric": f"decode tok/s (Qwen2-7B shape, batch {a.batch}, context {CONTEXT})", "value": round(value, 2),
         "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype,
         "data": "synthetic: seeded random token ids, random weights N(0, 0.02), random cache content",

@@ -661,6 +661,10 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
     const long per_xcd = TileOrder((int)mtiles).blocks(ntiles) / 8;
     if (per_xcd * 8 > 0x7fffffffL || nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
+    // a lane's byte offset from its tile's first row is kept in 32 bits (the gate and up rows of a
+    // SwiGLU tile lie N / 2 rows apart)
+    const unsigned long long span_rows = SWIGLU ? (unsigned long long)N / 2 + BN : (unsigned long long)(BM > BN ? BM : BN);
+    if (span_rows * (unsigned long long)K * 2ull >= (1ull << 32)) return LI_ERR_SIZE;
     constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool configured = false;
     if (!configured) {
