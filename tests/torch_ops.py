@@ -198,6 +198,7 @@ def argmax_rows(logits, out):
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
        "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "rope_store_takes", "linear_rope_store", "check_attention_sizes",
+       "RowScale", "RESIDUAL_NORM_MAX_PARTS", "residual_norm_parts", "residual_norm_takes", "linear_residual_norm",
        "paged_attention", "argmax_rows"]
 
 
