@@ -164,11 +164,20 @@ extern "C" int li_rope_table(const int* pos, float theta, int rotary_dim, float*
 }
 
 // y[j] = a cos - b sin; y[j + half] = b cos + a sin with a = x[j], b = x[j + half]
+// One rotation, with its roundings spelled out (one product rounded, the other fused into the sum),
+// so that every kernel here gives the same bits whatever the compiler would contract.
+__device__ __forceinline__ void rotate_values(float a, float b, float c, float s, float& ra, float& rb) {
+    ra = __builtin_fmaf(a, c, -__fmul_rn(b, s));
+    rb = __builtin_fmaf(b, c, __fmul_rn(a, s));
+}
+
 template <typename T>
 __device__ __forceinline__ void rotate_pair(T* head, int j, int half, float c, float s, T* dst) {
     const float a = load_as_float(head + j), b = load_as_float(head + j + half);
-    store_from_float(dst + j, a * c - b * s);
-    store_from_float(dst + j + half, b * c + a * s);
+    float ra, rb;
+    rotate_values(a, b, c, s, ra, rb);
+    store_from_float(dst + j, ra);
+    store_from_float(dst + j + half, rb);
 }
 
 template <typename T>
@@ -233,11 +242,72 @@ __global__ void kv_store_kernel(T* __restrict__ qkv, int row_stride, int nh, int
     }
 }
 
+// The same with 16 bytes a lane, for whole-head rotation (rotary_dim == dh) or none, where a half
+// head is a whole number of 16-byte pieces and rows start on 16 bytes: thread (t, head, c) takes
+// the pieces c of the head's two halves, i.e. E pairs when it rotates.
+template <typename T, bool ROTATE>
+__global__ __launch_bounds__(256) void kv_store_vec_kernel(T* __restrict__ qkv, int row_stride, int nh, int nkv, int dh,
+                                                            const float* __restrict__ cosv, const float* __restrict__ sinv,
+                                                            const int* __restrict__ slot_map, T* __restrict__ kc,
+                                                            T* __restrict__ vc, int page_size, int num_pages, long total) {
+    constexpr int E = 16 / (int)sizeof(T);
+    struct __attribute__((aligned(16))) piece { T e[E]; };
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int half = dh / 2, cph = half / E;                     // pieces in half a head
+    const int nheads = ROTATE ? nh + 2 * nkv : 2 * nkv;
+    const int c = (int)(i % cph);
+    const int hh = (int)((i / cph) % nheads) + (ROTATE ? 0 : nh);
+    const int t = (int)(i / ((long)cph * nheads));
+    T* head = qkv + (size_t)t * row_stride + (size_t)hh * dh;
+    T* dst = head;                                               // query heads: rotated in place
+    if (hh >= nh) {
+        const int slot = slot_map[t];
+        if (slot < 0 || slot >= num_pages * page_size) return;   // never write outside the pool
+        dst = hh < nh + nkv ? cache_row(kc, slot, page_size, nkv, hh - nh, dh)
+                            : cache_row(vc, slot, page_size, nkv, hh - nh - nkv, dh);
+    }
+    piece a = *reinterpret_cast<const piece*>(head + E * c), b = *reinterpret_cast<const piece*>(head + half + E * c);
+    if (ROTATE && hh < nh + nkv) {
+        const float* cs = cosv + (size_t)t * half + E * c;
+        const float* sn = sinv + (size_t)t * half + E * c;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float ra, rb;
+            rotate_values(load_as_float(&a.e[e]), load_as_float(&b.e[e]), cs[e], sn[e], ra, rb);
+            store_from_float(&a.e[e], ra);
+            store_from_float(&b.e[e], rb);
+        }
+    } else if (dst == head) {
+        return;                                                  // (cannot happen: an unrotated head is a cache head)
+    }
+    *reinterpret_cast<piece*>(dst + E * c) = a;
+    *reinterpret_cast<piece*>(dst + half + E * c) = b;
+}
+
+template <typename T, bool ROTATE>
+static bool kv_store_vec(T* qkv, int row_stride, int nh, int nkv, int dh, int rotary_dim, const float* cosv,
+                         const float* sinv, const int* slot_map, T* kc, T* vc, int page_size, int num_pages, int Tn,
+                         hipStream_t stream) {
+    constexpr int E = 16 / (int)sizeof(T);
+    if ((ROTATE && rotary_dim != dh) || dh % (2 * E) || row_stride % E || ((uintptr_t)qkv | (uintptr_t)kc | (uintptr_t)vc) % 16 ||
+        (ROTATE && (((uintptr_t)cosv | (uintptr_t)sinv) % 16)))
+        return false;
+    const long total = (long)Tn * (ROTATE ? nh + 2 * nkv : 2 * nkv) * (dh / 2 / E);
+    const long blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffL) return false;
+    kv_store_vec_kernel<T, ROTATE><<<(unsigned)blocks, 256, 0, stream>>>(qkv, row_stride, nh, nkv, dh, cosv, sinv, slot_map, kc, vc,
+                                                                        page_size, num_pages, total);
+    return true;
+}
+
 extern "C" int li_kv_store(void* qkv, int dtype, int row_stride, int nh, int nkv, int dh,
                            const int* slot_map, void* kc, void* vc, int page_size, int num_pages,
                            int T, hipStream_t stream) {
     if (T <= 0 || nkv <= 0 || 2 * nkv > 65535 || page_size <= 0) return LI_ERR_SIZE;
     dim3 grid(T, 2 * nkv);
+    if (dtype == LI_F32 && kv_store_vec<float, false>((float*)qkv, row_stride, nh, nkv, dh, 0, nullptr, nullptr, slot_map, (float*)kc, (float*)vc, page_size, num_pages, T, stream)) return li_launch_status();
+    if (dtype == LI_BF16 && kv_store_vec<bf16_t, false>((bf16_t*)qkv, row_stride, nh, nkv, dh, 0, nullptr, nullptr, slot_map, (bf16_t*)kc, (bf16_t*)vc, page_size, num_pages, T, stream)) return li_launch_status();
     if (dtype == LI_F32) kv_store_kernel<float, false><<<grid, 64, 0, stream>>>((float*)qkv, row_stride, nh, nkv, dh, 0, nullptr, nullptr, slot_map, (float*)kc, (float*)vc, page_size, num_pages);
     else if (dtype == LI_BF16) kv_store_kernel<bf16_t, false><<<grid, 64, 0, stream>>>((bf16_t*)qkv, row_stride, nh, nkv, dh, 0, nullptr, nullptr, slot_map, (bf16_t*)kc, (bf16_t*)vc, page_size, num_pages);
     else return LI_ERR_DTYPE;
@@ -250,6 +320,8 @@ extern "C" int li_rope_kv_store(void* qkv, int dtype, int row_stride, int nh, in
                                 int num_pages, int T, hipStream_t stream) {
     if (T <= 0 || nh + 2 * nkv > 65535 || page_size <= 0 || rotary_dim > dh || (rotary_dim & 1)) return LI_ERR_SIZE;
     dim3 grid(T, nh + 2 * nkv);
+    if (dtype == LI_F32 && kv_store_vec<float, true>((float*)qkv, row_stride, nh, nkv, dh, rotary_dim, cosv, sinv, slot_map, (float*)kc, (float*)vc, page_size, num_pages, T, stream)) return li_launch_status();
+    if (dtype == LI_BF16 && kv_store_vec<bf16_t, true>((bf16_t*)qkv, row_stride, nh, nkv, dh, rotary_dim, cosv, sinv, slot_map, (bf16_t*)kc, (bf16_t*)vc, page_size, num_pages, T, stream)) return li_launch_status();
     if (dtype == LI_F32) kv_store_kernel<float, true><<<grid, 64, 0, stream>>>((float*)qkv, row_stride, nh, nkv, dh, rotary_dim, cosv, sinv, slot_map, (float*)kc, (float*)vc, page_size, num_pages);
     else if (dtype == LI_BF16) kv_store_kernel<bf16_t, true><<<grid, 64, 0, stream>>>((bf16_t*)qkv, row_stride, nh, nkv, dh, rotary_dim, cosv, sinv, slot_map, (bf16_t*)kc, (bf16_t*)vc, page_size, num_pages);
     else return LI_ERR_DTYPE;

@@ -427,10 +427,11 @@ def test_window_edge(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_rope_kv_store_and_plain_store(ops, dtype):
+@pytest.mark.parametrize("dh,pad", [(48, 5), (48, 16), (128, 0), (20, 0)])      # rows that do and do not start on 16 bytes
+def test_rope_kv_store_and_plain_store(ops, dtype, dh, pad):
     g = torch.Generator().manual_seed(9)
-    t, nh, nkv, dh, page, pages = 37, 3, 2, 48, 8, 11
-    qkv = torch.randn(t, (nh + 2 * nkv) * dh + 5, generator=g).to(dtype)[:, :(nh + 2 * nkv) * dh]
+    t, nh, nkv, page, pages = 37, 3, 2, 8, 11
+    qkv = torch.randn(t, (nh + 2 * nkv) * dh + pad, generator=g).to(dtype)[:, :(nh + 2 * nkv) * dh]
     pos = torch.randint(0, 200, (t,), generator=g, dtype=torch.int32)
     slots = torch.randperm(pages * page, generator=g)[:t].to(torch.int32)
     cos = torch.empty(t, dh // 2, device=DEV)
