@@ -38,43 +38,46 @@ extern "C" int li_embedding(const int* ids, const int* id_src, const int* feedba
 // ------------------------------------------------------------------ rmsnorm
 // y = w * x * rsqrt(mean(x^2) + eps), eps inside the root; one block per row.  The row is
 // read once and kept in registers (up to RN_PER elements a thread); longer rows are read again.
-#define RN_NT 1024
-#define RN_PER 8
-
-template <typename TI, typename TO>
-__global__ __launch_bounds__(RN_NT) void rmsnorm_kernel(const TI* __restrict__ x, const float* __restrict__ w,
-                                                         float eps, TO* __restrict__ out, int H) {
-    __shared__ float red[RN_NT / LI_WAVE];
+// Few rows (a decoding step): 1024 threads a row, so that the one row is read with the least
+// latency; many rows (a prompt): 256 threads a row, less of a block's time goes into meeting.
+template <typename TI, typename TO, int NT, int PER>
+__global__ __launch_bounds__(NT) void rmsnorm_kernel(const TI* __restrict__ x, const float* __restrict__ w,
+                                                      float eps, TO* __restrict__ out, int H) {
+    __shared__ float red[NT / LI_WAVE];
     const TI* row = x + (size_t)blockIdx.x * H;
     TO* o = out + (size_t)blockIdx.x * H;
-    float v[RN_PER];
+    float v[PER];
     float ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < RN_PER; ++i) {
-        const int j = threadIdx.x + i * RN_NT;
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * NT;
         v[i] = (j < H) ? load_as_float(row + j) : 0.f;
         ss += v[i] * v[i];
     }
-    for (int j = threadIdx.x + RN_PER * RN_NT; j < H; j += RN_NT) { const float t = load_as_float(row + j); ss += t * t; }
-    ss = block_sum<RN_NT>(ss, red);
+    for (int j = threadIdx.x + PER * NT; j < H; j += NT) { const float t = load_as_float(row + j); ss += t * t; }
+    ss = block_sum<NT>(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float)H + eps);
 #pragma unroll
-    for (int i = 0; i < RN_PER; ++i) {
-        const int j = threadIdx.x + i * RN_NT;
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * NT;
         if (j < H) store_from_float(o + j, w[j] * v[i] * inv);
     }
-    for (int j = threadIdx.x + RN_PER * RN_NT; j < H; j += RN_NT)
+    for (int j = threadIdx.x + PER * NT; j < H; j += NT)
         store_from_float(o + j, w[j] * load_as_float(row + j) * inv);
 }
 
 extern "C" int li_rmsnorm(const void* x, int x_dtype, const float* w, float eps, void* out,
                           int out_dtype, int T, int H, hipStream_t stream) {
     if (T <= 0 || H <= 0) return LI_ERR_SIZE;
-#define LI_NORM(TI, TO) rmsnorm_kernel<TI, TO><<<T, RN_NT, 0, stream>>>((const TI*)x, w, eps, (TO*)out, H)
-    if (x_dtype == LI_F32 && out_dtype == LI_F32) LI_NORM(float, float);
-    else if (x_dtype == LI_F32 && out_dtype == LI_BF16) LI_NORM(float, bf16_t);
-    else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) LI_NORM(bf16_t, bf16_t);
-    else if (x_dtype == LI_BF16 && out_dtype == LI_F32) LI_NORM(bf16_t, float);
+#define LI_NORM(TI, TO)                                                                                        \
+    {                                                                                                          \
+        if (T >= 256) rmsnorm_kernel<TI, TO, 256, 16><<<T, 256, 0, stream>>>((const TI*)x, w, eps, (TO*)out, H); \
+        else rmsnorm_kernel<TI, TO, 1024, 8><<<T, 1024, 0, stream>>>((const TI*)x, w, eps, (TO*)out, H);        \
+    }
+    if (x_dtype == LI_F32 && out_dtype == LI_F32) LI_NORM(float, float)
+    else if (x_dtype == LI_F32 && out_dtype == LI_BF16) LI_NORM(float, bf16_t)
+    else if (x_dtype == LI_BF16 && out_dtype == LI_BF16) LI_NORM(bf16_t, bf16_t)
+    else if (x_dtype == LI_BF16 && out_dtype == LI_F32) LI_NORM(bf16_t, float)
     else return LI_ERR_DTYPE;
 #undef LI_NORM
     return li_launch_status();
