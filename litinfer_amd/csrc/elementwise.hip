@@ -66,6 +66,40 @@ __global__ __launch_bounds__(NT) void rmsnorm_kernel(const TI* __restrict__ x, c
         store_from_float(o + j, w[j] * load_as_float(row + j) * inv);
 }
 
+// Many rows of float32 whose length is a multiple of 4 (a prompt's residual rows): 16 bytes a lane.
+template <typename TO, int NT, int PER>
+__global__ __launch_bounds__(NT) void rmsnorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                          float eps, TO* __restrict__ out, int H) {
+    __shared__ float red[NT / LI_WAVE];
+    const float4* row = reinterpret_cast<const float4*>(x + (size_t)blockIdx.x * H);
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    TO* o = out + (size_t)blockIdx.x * H;
+    const int n4 = H / 4;
+    float4 v[PER];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * NT;
+        v[i] = (j < n4) ? row[j] : float4{0.f, 0.f, 0.f, 0.f};
+        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+    ss = block_sum<NT>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = threadIdx.x + i * NT;
+        if (j < n4) {
+            const float4 g = w4[j];
+            const float y0 = g.x * v[i].x * inv, y1 = g.y * v[i].y * inv, y2 = g.z * v[i].z * inv, y3 = g.w * v[i].w * inv;
+            if constexpr (sizeof(TO) == 2) {
+                *reinterpret_cast<uint2*>(o + 4 * j) = uint2{pack2_bf16(y0, y1), pack2_bf16(y2, y3)};
+            } else {
+                *reinterpret_cast<float4*>(o + 4 * j) = float4{y0, y1, y2, y3};
+            }
+        }
+    }
+}
+
 extern "C" int li_rmsnorm(const void* x, int x_dtype, const float* w, float eps, void* out,
                           int out_dtype, int T, int H, hipStream_t stream) {
     if (T <= 0 || H <= 0) return LI_ERR_SIZE;
@@ -73,6 +107,12 @@ extern "C" int li_rmsnorm(const void* x, int x_dtype, const float* w, float eps,
     {                                                                                                          \
         if (T >= 256) rmsnorm_kernel<TI, TO, 256, 16><<<T, 256, 0, stream>>>((const TI*)x, w, eps, (TO*)out, H); \
         else rmsnorm_kernel<TI, TO, 1024, 8><<<T, 1024, 0, stream>>>((const TI*)x, w, eps, (TO*)out, H);        \
+    }
+    if (x_dtype == LI_F32 && T >= 256 && H % 4 == 0 && H <= 4 * 256 * 8 && ((uintptr_t)x | (uintptr_t)w | (uintptr_t)out) % 16 == 0) {
+        if (out_dtype == LI_F32) rmsnorm_vec_kernel<float, 256, 8><<<T, 256, 0, stream>>>((const float*)x, w, eps, (float*)out, H);
+        else if (out_dtype == LI_BF16) rmsnorm_vec_kernel<bf16_t, 256, 8><<<T, 256, 0, stream>>>((const float*)x, w, eps, (bf16_t*)out, H);
+        else return LI_ERR_DTYPE;
+        return li_launch_status();
     }
     if (x_dtype == LI_F32 && out_dtype == LI_F32) LI_NORM(float, float)
     else if (x_dtype == LI_F32 && out_dtype == LI_BF16) LI_NORM(float, bf16_t)

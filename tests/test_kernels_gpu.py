@@ -45,7 +45,8 @@ def test_embedding(ops, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape,eps", [((1, 4), 1e-5), ((33, 120), 1e-6), ((512, 4096), 1e-5), ((3, 3584), 1e-6)])
+@pytest.mark.parametrize("shape,eps", [((1, 4), 1e-5), ((33, 120), 1e-6), ((512, 4096), 1e-5), ((3, 3584), 1e-6),
+                                        ((300, 1002), 1e-6), ((257, 8196), 1e-5), ((256, 20), 0.1)])      # many rows: of any length, too long for registers, short
 def test_rmsnorm(ops, dtype, shape, eps):
     g = torch.Generator().manual_seed(1)
     x = torch.randn(*shape, generator=g) * 3
