@@ -153,7 +153,7 @@ def main() -> int:
     if not a.no_prefill:
         prompt = rng.integers(0, cfg["vocab_size"], PREFILL_TOKENS).tolist()
         times = []
-        for i in range(3):
+        for i in range(5):                           # one to warm up, the best of four
             torch.cuda.synchronize()
             t = time.perf_counter()
             logits = eng.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
