@@ -196,6 +196,57 @@ def test_feed_forward_part_alone(device):
     assert schedules.rel_err(out.cpu().numpy(), ref) < 2e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_norm_shared_through_the_stream(device, dtype):
+    """The product before a norm may leave the rows that the part behind the norm
+    multiplies; any other write to the stream forgets them; a part that knows nothing
+    of this gets the norm as a pass of its own.  The result is the same either way."""
+    from litinfer_amd.parts.linear import Linear
+    g = torch.Generator().manual_seed(3)
+    h, i, k, t = 72, 200, 40, 5
+    rt = _rt(device, dtype)
+    stored = lambda x: x.to(dtype)
+    ws = {f"f.{n}_proj.weight": stored(torch.randn(*s, generator=g) * 0.1) for n, s in
+          (("gate", (i, h)), ("up", (i, h)), ("down", (h, i)))}
+    gamma = 1 + 0.1 * torch.randn(h, generator=g)
+    ffn = _load(build_part("feed_forward", PartSpec("swiglu_mlp", "f.", {"hidden_size": h, "intermediate_size": i}), rt), ws)
+    norm = _load(build_part("norm", PartSpec("rmsnorm", "n.", {"size": h, "eps": 1e-5}), rt), {"n.weight": gamma})
+    other = _load(build_part("norm", PartSpec("rmsnorm", "o.", {"size": h, "eps": 1e-5}), rt), {"o.weight": gamma})
+    wprev = stored(torch.randn(h, k, generator=g) * 0.2)
+    prev = Linear(rt, wprev)
+    hp = stored(torch.randn(t, k, generator=g))
+    res = torch.randn(t, h, generator=g) * torch.logspace(-1, 1, t)[:, None]
+    x1 = res.double().numpy() + hp.double().numpy() @ wprev.double().numpy().T
+    d = {n: v.double().numpy() for n, v in ws.items()}
+    xn = P.rms_norm(x1, gamma.double().numpy(), 1e-5)
+    ref = x1 + P.swiglu(xn @ d["f.gate_proj.weight"].T, xn @ d["f.up_proj.weight"].T) @ d["f.down_proj.weight"].T
+    outs = []
+    for announce in (True, False):
+        ctx = type("Ctx", (), {"ws": Workspace(device)})()
+        stream = ResidualStream(res.clone().to(device), ctx.ws)
+        stream.next_norm = norm if announce else None
+        stream.add_linear(prev, hp.to(device))
+        left = stream.scaled_rows(norm)
+        assert (left is not None) == (announce and dtype is torch.bfloat16)       # few bfloat16 rows: the kernels take it
+        assert stream.scaled_rows(other) is None                                     # another norm's reader finds nothing
+        buf = torch.empty(t, h, dtype=dtype, device=device)
+        ffn.forward_prenorm(norm, stream, buf, ctx)
+        outs.append(stream.tensor().cpu().numpy())
+        assert schedules.rel_err(outs[-1], ref) < (F32_TOL if dtype is torch.float32 else BF16_TOL)
+    # whoever takes the sum itself may write to it: what was left for the norm is forgotten
+    ctx = type("Ctx", (), {"ws": Workspace(device)})()
+    stream = ResidualStream(res.clone().to(device), ctx.ws)
+    stream.next_norm = norm
+    stream.add_linear(prev, hp.to(device))
+    stream.tensor()
+    assert stream.scaled_rows(norm) is None
+    stream.next_norm = norm
+    stream.add_linear(prev, hp.to(device))
+    stream.next_norm = None
+    stream.add_linear(prev, hp.to(device))                       # a second addition, with no reader announced
+    assert stream.scaled_rows(norm) is None
+
+
 def _mixer_case(device, window, cache_steps):
     """Run the attention mixer alone over two requests in several steps and
     return (its additions to a zero residual, the plain result)."""
