@@ -688,6 +688,50 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ part, int nsplit,
     epilogue_store(out, i, v, bias, (int)(i % N), accumulate);
 }
 
+// The same for the residual sum, one block a row, with the RMS norm of the new sum as a second
+// result: out[m, :] += sum of the parts + bias (float32), xn[m, :] = gamma * out[m, :] /
+// sqrt(mean(out[m, :]^2) + eps).  A row is kept in registers (N <= NT * PER).
+template <typename TN, int NT, int PER>
+__global__ __launch_bounds__(NT) void splitk_reduce_norm_kernel(const float* __restrict__ part, int nsplit, size_t mn, int N,
+                                                                 const float* __restrict__ bias, float* __restrict__ out,
+                                                                 const float* __restrict__ gamma, float eps,
+                                                                 TN* __restrict__ xn) {
+    __shared__ float red[NT / LI_WAVE];
+    const size_t row = (size_t)blockIdx.x * N;
+    float v[PER];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int n = threadIdx.x + i * NT;
+        v[i] = 0.f;
+        if (n < N) {
+            // all loads at once (a part past the last reads the first and is not added): the block is
+            // one of few and must not wait for memory part after part
+            float a[8];
+#pragma unroll
+            for (int sp = 0; sp < 8; ++sp) a[sp] = part[(size_t)(sp < nsplit ? sp : 0) * mn + row + n];
+            const float o = out[row + n];
+            float t = a[0];
+#pragma unroll
+            for (int sp = 1; sp < 8; ++sp) t += sp < nsplit ? a[sp] : 0.f;
+            if (bias) t += bias[n];
+            t += o;
+            out[row + n] = t;
+            v[i] = t;
+        }
+        ss += v[i] * v[i];
+    }
+    ss = block_sum<NT>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)N + eps);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int n = threadIdx.x + i * NT;
+        if (n < N) store_from_float(xn + row + n, gamma[n] * v[i] * inv);
+    }
+}
+#define REDUCE_NORM_NT 1024
+#define REDUCE_NORM_PER 8
+
 template <int BM, int BN, int BK, typename TO>
 static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream) {
@@ -1099,6 +1143,33 @@ extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
         nsplit = split_parts_many_rows(M, N, K);
     }
     return nsplit < 2 ? 0 : (long)nsplit * M * N * (long)sizeof(float);
+}
+
+// out += x w^T + bias (float32 out: the residual sum) and xn = the RMS norm of the new out with weights
+// gamma, where li_linear would cut K into parts anyway: the kernel that adds the parts up then has
+// whole rows in its hands.  xn is bfloat16 (xn_dtype LI_BF16) or float32.  Returns -1, having done
+// nothing, where the product is not cut (the caller then multiplies and norms in two calls).
+extern "C" int li_linear_then_norm(const void* x, const void* w, const float* bias, float* out, int M, int N, int K,
+                                   void* work, long work_bytes, const float* gamma, float eps, void* xn,
+                                   int xn_dtype, hipStream_t stream) {
+    if (M <= 32 || N <= 0 || K <= 0 || (K % 64) || !gamma || !xn || eps < 0.f) return -1;
+    if (N > REDUCE_NORM_NT * REDUCE_NORM_PER || (xn_dtype != LI_BF16 && xn_dtype != LI_F32)) return -1;
+    const long need = li_linear_work_bytes(M, N, K, LI_BF16);
+    if (need <= 0 || !work || work_bytes < need) return -1;
+    const size_t mn = (size_t)M * N;
+    const int nsplit = (int)(need / (long)(mn * sizeof(float)));
+    if (nsplit > 8) return -1;                      // (the adding-up kernel takes up to 8 parts)
+    const int rc = M <= 64
+        ? launch_dma<64, 128, 64, 4, false, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)work, M, N, K, 0, stream, nsplit)
+        : launch_dma<128, 128, 64, 4, false, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)work, M, N, K, 0, stream, nsplit);
+    if (rc != LI_OK) return rc;
+    if (xn_dtype == LI_BF16)
+        splitk_reduce_norm_kernel<bf16_t, REDUCE_NORM_NT, REDUCE_NORM_PER><<<M, REDUCE_NORM_NT, 0, stream>>>(
+            (const float*)work, nsplit, mn, N, bias, out, gamma, eps, (bf16_t*)xn);
+    else
+        splitk_reduce_norm_kernel<float, REDUCE_NORM_NT, REDUCE_NORM_PER><<<M, REDUCE_NORM_NT, 0, stream>>>(
+            (const float*)work, nsplit, mn, N, bias, out, gamma, eps, (float*)xn);
+    return li_launch_status();
 }
 
 // `work` (may be null): device memory of work_bytes for the partial sums of a product cut along K.

@@ -40,6 +40,7 @@ _SIGNATURES = {
         "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
         "li_linear_swiglu": [P, P, P, I, I, I, P, I, F],
         "li_linear_residual_norm": [P, P, P, P, I, I, I, P, P, P],
+        "li_linear_then_norm": [P, P, P, P, I, I, I, P, L, P, F, P, I],
         "li_linear_rope_store": [P, P, P, P, I, I, P, P, P, P, P, I, I, I, I, I, P, I, F],
     },
     "attention": {
@@ -385,6 +386,40 @@ def linear_residual_norm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.
     _run("gemm", "li_linear_residual_norm", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
          out.data_ptr(), m, n, k, gamma.data_ptr(), xg.data_ptr(), sq_parts.data_ptr())
     return parts
+
+
+def linear_then_norm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                     gamma: torch.Tensor, eps: float, xn: torch.Tensor, ws) -> bool:
+    """out += x w^T + bias (float32) and xn = gamma * out / sqrt(mean(out^2) + eps), in the kernel
+    that adds up the parts of a product cut along K.  Returns False, having done nothing, where
+    `linear` would not cut this product (then multiply and norm in two calls)."""
+    _gpu(x, w, bias, out, gamma, xn)
+    if ws is None or x.dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16:
+        return False
+    _chk(x.dim() == 2 and w.dim() == 2, "linear_then_norm: needs matrices")
+    m, k = x.shape
+    n = w.shape[0]
+    need = _work_bytes(m, n, k, _DT[x.dtype])
+    if not need:
+        return False
+    _chk(w.shape == (n, k) and x.is_contiguous() and w.is_contiguous(), "linear_then_norm: contiguous [M, K] and [N, K]")
+    _chk(out.dtype is torch.float32 and out.shape == (m, n) and out.is_contiguous(), "linear_then_norm: out must be float32 [M, N]")
+    _chk(xn.dtype in _DT and xn.shape == (m, n) and xn.is_contiguous(), "linear_then_norm: xn must be [M, N]")
+    _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
+         "linear_then_norm: bias must be float32 [N]")
+    _chk(gamma.dtype is torch.float32 and gamma.shape == (n,) and gamma.is_contiguous() and eps >= 0,
+         "linear_then_norm: gamma must be float32 [N], eps not negative")
+    if m <= SKINNY_MAX_ROWS:                # one size for all row counts of a decode batch: the buffer does not move
+        need = max(need, SPLITK_MAX_PARTS * SKINNY_MAX_ROWS * n * 4)
+    buf = ws.buffer("gemm.parts", (need // 4,), torch.float32)
+    rc = _fn("gemm", "li_linear_then_norm")(x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
+                                             out.data_ptr(), m, n, k, buf.data_ptr(), buf.numel() * 4, gamma.data_ptr(),
+                                             float(eps), xn.data_ptr(), _DT[xn.dtype], _stream())
+    if rc == -1:
+        return False
+    if rc != 0:
+        raise RuntimeError(f"li_linear_then_norm: the kernel library refused the call (code {rc}): {_ERRORS.get(rc, 'unknown')}")
+    return True
 
 
 def _check_row_scale(what: str, m: int, row_scale: Optional[RowScale]):

@@ -89,8 +89,7 @@ class GQAttention(Mixer):
             if self.position.project_encode_store(self.qkv, sc.rows, qkv, self.nh, self.nkv, self.dh, ctx, cache,
                                                   row_scale=sc.scale):
                 return self._attend(qkv, residual, ctx, cache)
-        residual.normed(norm, xn)
-        self.forward(xn, residual, ctx, cache)
+        self.forward(residual.normed(norm, xn), residual, ctx, cache)
 
     def forward(self, xn, residual, ctx, cache):
         t = xn.shape[0]

@@ -136,8 +136,7 @@ class Mixer(Part):
         normed rows.  The default norms in a pass of its own.  A mixer whose first
         product can scale its rows overrides this and asks the stream for
         `scaled_rows(norm)`, which the product before the norm may have left."""
-        residual.normed(norm, xn)
-        self.forward(xn, residual, ctx, cache)
+        self.forward(residual.normed(norm, xn), residual, ctx, cache)
 
 
 class FeedForward(Part):
@@ -148,8 +147,7 @@ class FeedForward(Part):
 
     def forward_prenorm(self, norm: Norm, residual, xn, ctx) -> None:
         """x += feed_forward(norm(x)); see Mixer.forward_prenorm."""
-        residual.normed(norm, xn)
-        self.forward(xn, residual, ctx)
+        self.forward(residual.normed(norm, xn), residual, ctx)
 
 
 class Block(Part):

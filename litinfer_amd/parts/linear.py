@@ -36,6 +36,13 @@ class Linear:
         n = ops.linear_residual_norm(x, self.weight, self.bias, out, scaling.weight, rows, parts)
         return ops.RowScale(parts, n, scaling.eps)
 
+    def add_then_norm(self, x: torch.Tensor, out: torch.Tensor, scaling, xn: torch.Tensor, ws) -> bool:
+        """out += x W^T + b and xn = the RMS norm of the new out, in one go where the
+        kernels have that (a product cut along K); False, with nothing done, where not."""
+        if self.weight.dtype is not torch.bfloat16 or x.dtype is not torch.bfloat16 or out.dtype is not torch.float32:
+            return False
+        return ops.linear_then_norm(x, self.weight, self.bias, out, scaling.weight, scaling.eps, xn, ws)
+
     def __call__(self, x: torch.Tensor, out: torch.Tensor, accumulate: bool = False, ws=None,
                  swiglu: bool = False, row_scale=None):
         """out = x W^T + b, or out += ... when `accumulate` (out is float32 then).

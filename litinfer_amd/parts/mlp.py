@@ -43,8 +43,7 @@ class SwiGLUMLP(FeedForward):
             h = ctx.ws.buffer("mlp.h", (sc.rows.shape[0], self.inter), self.rt.dtype)
             self.gate_up(sc.rows, h, ws=ctx.ws, swiglu=True, row_scale=sc.scale)
             return residual.add_linear(self.down, h)
-        residual.normed(norm, xn)
-        self.forward(xn, residual, ctx)
+        self.forward(residual.normed(norm, xn), residual, ctx)
 
     def forward(self, xn, residual, ctx):
         t = xn.shape[0]

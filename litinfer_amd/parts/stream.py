@@ -28,6 +28,7 @@ class ResidualStream:
         self.ws = ws
         self.next_norm = None                 # the norm through which the stream is read next, if known
         self._scaled = None                   # (norm, ScaledRows) left by the last add_linear
+        self._normed = None                   # (norm, its result) left by the last add_linear
 
     @property
     def shape(self):
@@ -35,18 +36,24 @@ class ResidualStream:
 
     def tensor(self) -> torch.Tensor:
         """The sum so far (whoever takes it may write to it)."""
-        self._scaled = None
+        self._scaled = self._normed = None
         return self.x
 
     def add_linear(self, linear, h: torch.Tensor) -> None:
         """x += h W^T + b."""
-        norm, self._scaled = self.next_norm, None
+        norm, self._scaled, self._normed = self.next_norm, None, None
         scaling = norm.as_scaling() if norm is not None else None
         if scaling is not None and linear.takes_scaling(h, self.x):
             rows = self.ws.buffer("stream.scaled_rows", self.x.shape, h.dtype)
             self._scaled = (norm, ScaledRows(rows, linear.add_with_scaling(h, self.x, scaling, rows, self.ws)))
-        else:
-            linear(h, self.x, accumulate=True, ws=self.ws)
+            return
+        if scaling is not None:
+            # some more rows: where the product is cut along K, the kernel that adds the parts up norms as well
+            rows = self.ws.buffer("stream.normed_rows", self.x.shape, h.dtype)
+            if linear.add_then_norm(h, self.x, scaling, rows, self.ws):
+                self._normed = (norm, rows)
+                return
+        linear(h, self.x, accumulate=True, ws=self.ws)
 
     def scaled_rows(self, norm) -> Optional[ScaledRows]:
         """What the last addition left for this norm's reader, if it did."""
@@ -55,6 +62,8 @@ class ResidualStream:
         return None
 
     def normed(self, norm, out: torch.Tensor) -> torch.Tensor:
-        """out = norm(x)."""
+        """norm(x): in `out`, or in the tensor that the last addition already left."""
+        if self._normed is not None and self._normed[0] is norm:
+            return self._normed[1]
         norm.forward(self.x, out)
         return out

@@ -163,6 +163,42 @@ def test_linear_with_k_in_parts(ops, m, n, k, out_dtype, bias, acc):
     assert torch.equal(again, outs[0])                   # the parts are added in a fixed order
 
 
+@pytest.mark.parametrize("m,n,k,bias,taken", [
+    (64, 3584, 18944, False, True),      # a decoding batch of 64 at the 7B sizes
+    (40, 200, 1024, True, True),
+    (200, 300, 4096, True, True),        # more than 64 rows, few tiles
+    (64, 37000, 64, False, False),       # no cut along K: nothing is done
+    (8, 200, 1024, False, False),        # few rows: another kernel's business
+])
+def test_linear_into_the_residual_sum_with_its_norm(ops, m, n, k, bias, taken):
+    g = torch.Generator().manual_seed(19)
+    x = torch.randn(m, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    b = torch.randn(n, generator=g) * 0.1 if bias else None
+    base = torch.randn(m, n, generator=g) * torch.logspace(-2, 2, m)[:, None]       # rows of very different size
+    gamma, eps = torch.rand(n, generator=g) + 0.5, 1e-5
+    out = base.to(DEV)
+    xn = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    did = ops.linear_then_norm(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, gamma.to(DEV), eps, xn, _Lender())
+    assert did == taken
+    if not taken:
+        assert torch.equal(out.cpu(), base) and torch.isnan(xn.float()).all()        # nothing was touched
+        return
+    y = base.double().numpy() + x.double().numpy() @ w.double().numpy().T + (0 if b is None else b.double().numpy())
+    ref = plain_impl.rms_norm(y, gamma.double().numpy(), eps)
+    for i in range(m):
+        assert rel(out[i], y[i]) < 4 * math.sqrt(k) * 2.0 ** -24, i
+        assert rel(xn[i], ref[i]) < 8e-3, i
+    # the sum is the one that the product alone leaves, bit for bit
+    alone = base.to(DEV)
+    ops.linear(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), alone, True, ws=_Lender())
+    assert torch.equal(alone, out)
+    # and the norm is the one that the norm's own kernel makes of that sum, up to the order of its additions
+    own = torch.empty_like(xn)
+    ops.rmsnorm(out, gamma.to(DEV), eps, own)
+    assert (own.float() - xn.float()).abs().max().item() <= 2.0 ** -7 * own.float().abs().max().item()
+
+
 @pytest.mark.parametrize("m,n,k", [
     (8, 200, 96),                # few rows: the decode kernel
     (40, 20000, 128),            # 33 to 64 rows: tiles of 64 rows

@@ -157,6 +157,10 @@ def linear_residual_norm(x, w, bias, out, gamma, xg, sq_parts):
     return parts
 
 
+def linear_then_norm(x, w, bias, out, gamma, eps, xn, ws):
+    return False                                         # the stand-ins cut no product along K
+
+
 def _row_factors(row_scale, m, k):
     sq = row_scale.sq_parts[:row_scale.nparts * 16].view(row_scale.nparts, 16)[:, :m].sum(dim=0)
     return (1.0 / torch.sqrt(sq / k + row_scale.eps))[:, None]
@@ -198,7 +202,7 @@ def argmax_rows(logits, out):
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
        "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "rope_store_takes", "linear_rope_store", "check_attention_sizes",
-       "RowScale", "RESIDUAL_NORM_MAX_PARTS", "residual_norm_parts", "residual_norm_takes", "linear_residual_norm",
+       "RowScale", "RESIDUAL_NORM_MAX_PARTS", "residual_norm_parts", "residual_norm_takes", "linear_residual_norm", "linear_then_norm",
        "paged_attention", "argmax_rows"]
 
 
