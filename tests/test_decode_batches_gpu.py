@@ -1,0 +1,223 @@
+"""Decoding with many live requests, as serving and the benchmark do it: 8, 16, 17, 32,
+33 and 64 requests are first prefilled in portions that share steps, then decode together
+for a dozen steps (recorded as graphs and replayed, and once eagerly), one of them ends on
+the way and another takes its slot and pages.  Every logit of every token is compared with
+the plain implementation, in 32-bit and in bfloat16.  The row counts are the edges of the
+kernels' choices for few rows (16 | 17 and 32 | 33 and 64), and some requests are long enough
+for several key splits and for a block table that grows past a recorded width.
+
+The reference's engine step runs all unfinished sequences as one batch in the same way
+(src/llaisys/models/qwen2.cpp:922-1080)."""
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import schedules
+from tiny_configs import TINY_D, TINY_D_PAGE, TINY_E, TINY_E_PAGE
+
+pytestmark = pytest.mark.gpu
+
+CASES = {"D": (dict(TINY_D, max_position_embeddings=1024), TINY_D_PAGE, 3),
+         "E": (dict(TINY_E, max_position_embeddings=1024), TINY_E_PAGE, 4)}
+SHAPE_7B = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "num_hidden_layers": 2, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
+    "head_dim": 128, "intermediate_size": 18944, "vocab_size": 1000, "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "use_sliding_window": False,
+    "max_position_embeddings": 4096,
+}
+N_DECODE = 12
+# float32: the rounding of another order of summation.  bfloat16: three times what the GPU
+# shows (4.1e-3 to 5.8e-3 at the tiny sizes; `pytest -s` prints the observed values):
+# activations are rounded to bfloat16 between kernels, the plain side computes in float64 from
+# the same stored weights.
+TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}
+TOL_7B = 4e-2          # observed 1.4e-2: sums over 3,584 and 18,944 terms of bfloat16 activations
+
+
+def many_requests(vocab: int, n: int, seed: int, long_every: int = 8, longest: int = 600):
+    """n requests: prompts of 1 to 40 tokens, every `long_every`-th one of some hundred (several
+    key splits when decoding; one of them crosses 256 positions while it decodes), each followed
+    by N_DECODE tokens that are fed one by one.  Request 0 decodes four tokens only, and a late
+    request takes its place."""
+    rng = np.random.default_rng(seed)
+    prompts = {}
+    for i in range(n):
+        p = int(rng.integers(1, 41))
+        if i % long_every == 3:
+            p = int(rng.integers(150, longest))
+        if i == 5:
+            p = 250                                       # crosses a width of 256 positions while decoding
+        prompts[f"q{i}"] = p
+    prompts["late"] = 23
+    toks = {rid: rng.integers(0, vocab, p + (4 if rid == "q0" else N_DECODE)).tolist()
+            for rid, p in prompts.items()}
+    return toks, prompts
+
+
+def batch_schedule(toks, prompts, budget: int):
+    """Steps in the form of schedules.py: the prompts of all requests but the late one in
+    portions under a token budget, several requests a step, cut wherever the budget ends;
+    then decode steps of all live requests; after the fourth, request q0 ends and the late
+    request's whole prompt stands beside the others' single tokens."""
+    steps = []
+    first = [r for r in toks if r != "late"]
+    at = {r: 0 for r in toks}
+    pending = list(first)
+    while pending:
+        room, entries = budget, []
+        while pending and room > 0:
+            r = pending[0]
+            n = min(room, prompts[r] - at[r])
+            entries.append((r, at[r], n))
+            at[r] += n
+            room -= n
+            if at[r] == prompts[r]:
+                pending.pop(0)
+        steps.append((entries, []))
+    live = list(first)
+    for k in range(N_DECODE + 1):
+        entries, end = [], []
+        if k == 4:
+            entries.append(("late", 0, prompts["late"]))
+            at["late"] = prompts["late"]
+        for r in live:
+            if at[r] < len(toks[r]):
+                entries.append((r, at[r], 1))
+                at[r] += 1
+                if at[r] == len(toks[r]):
+                    end.append(r)
+        if k == 4:
+            live.append("late")
+        live = [r for r in live if r not in end]
+        if entries:
+            steps.append((entries, end))
+    while any(at[r] < len(toks[r]) for r in live):      # the late request's last tokens
+        entries = [(r, at[r], 1) for r in live if at[r] < len(toks[r])]
+        end = []
+        for r, i, _ in entries:
+            at[r] = i + 1
+            if at[r] == len(toks[r]):
+                end.append(r)
+        live = [r for r in live if r not in end]
+        steps.append((entries, end))
+    assert all(at[r] == len(toks[r]) for r in toks)
+    return steps
+
+
+def _check(d, dt, page, toks, prompts, ref, n_live, graphs, budget, label, tol=None):
+    from litinfer_amd.engine import Engine
+    steps = batch_schedule(toks, prompts, budget)
+    assert max(len(e) for e, _ in steps) >= n_live
+    eng = Engine.from_dir(d, dtype=dt, device="cuda:0", page_size=page, max_seqs=n_live, page_order_seed=7,
+                          max_tokens=schedules.max_live_tokens(toks, steps, page), use_graphs=graphs)
+    out = schedules.run(eng, toks, steps)
+    eng.cache.check_invariants()
+    assert all(f == g.pool.capacity for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
+    if graphs:
+        assert eng.graph_replays >= N_DECODE - 6, "the decode steps were not replayed from graphs"
+    else:
+        assert eng.graph_replays == 0
+    worst = max(schedules.rel_err(out[r], ref[r]) for r in toks)
+    worst_decode = max(schedules.rel_err(out[r][prompts[r]:], ref[r][prompts[r]:]) for r in toks)
+    print(f"[observed] {label} {dt} live={n_live} graphs={graphs}: all {worst:.3e}, decoded rows {worst_decode:.3e}")
+    assert worst < (tol or TOL[dt]), f"{label} {dt} live={n_live} graphs={graphs}: {worst}"
+    del eng
+    torch.cuda.empty_cache()
+
+
+@pytest.fixture(scope="module")
+def tiny_models(tmp_path_factory):
+    out = {}
+    for name, (cfg, page, seed) in CASES.items():
+        for dt in ("float32", "bfloat16"):
+            stored = torch.float32 if dt == "float32" else torch.bfloat16
+            out[(name, dt)] = helpers.make_model(tmp_path_factory.mktemp(f"db{name}{dt}"), cfg, seed, stored)
+    return out
+
+
+@pytest.fixture(scope="module")
+def plain_cache():
+    return {}
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CASES))
+@pytest.mark.parametrize("n_live", [8, 16, 17, 32, 33, 64])
+def test_decode_batches_match_the_plain_implementation(tiny_models, plain_cache, name, dt, n_live):
+    cfg, page, seed = CASES[name]
+    d = tiny_models[(name, dt)]
+    toks, prompts = many_requests(cfg["vocab_size"], n_live, seed * 100 + n_live)
+    key = (name, dt, n_live)
+    if key not in plain_cache:
+        plain_cache[key] = helpers.plain_logits(d, toks)
+    _check(d, dt, page, toks, prompts, plain_cache[key], n_live, True, 96, name)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_live", [17, 64])
+def test_decode_batches_without_recorded_steps(tiny_models, plain_cache, dt, n_live):
+    cfg, page, seed = CASES["E"]
+    d = tiny_models[("E", dt)]
+    toks, prompts = many_requests(cfg["vocab_size"], n_live, seed * 100 + n_live)
+    key = ("E", dt, n_live)
+    if key not in plain_cache:
+        plain_cache[key] = helpers.plain_logits(d, toks)
+    _check(d, dt, page, toks, prompts, plain_cache[key], n_live, False, 50, "E")
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_forty_decoding_requests_beside_a_portion_of_a_hundred_tokens(tiny_models, dt):
+    """One step holds 40 single tokens and a 100-token portion of another request's prompt,
+    twice over (the portion's second half follows), then all 41 decode."""
+    from litinfer_amd.engine import Engine, StepEntry
+    cfg, page, seed = CASES["D"]
+    d = tiny_models[("D", dt)]
+    rng = np.random.default_rng(77)
+    toks = {f"q{i}": rng.integers(0, cfg["vocab_size"], int(rng.integers(2, 30)) + 8).tolist() for i in range(40)}
+    toks["big"] = rng.integers(0, cfg["vocab_size"], 206).tolist()
+    ref = helpers.plain_logits(d, toks)
+    eng = Engine.from_dir(d, dtype=dt, device="cuda:0", page_size=page, max_seqs=41, page_order_seed=3,
+                          max_tokens=sum(-(-len(t) // page) * page for t in toks.values()))
+    got = {r: [] for r in toks}
+    small = [r for r in toks if r != "big"]
+
+    def step(entries):
+        out = eng.step([StepEntry(r, toks[r][i:i + n], list(range(n))) for r, i, n in entries]).cpu().numpy()
+        o = 0
+        for r, i, n in entries:
+            got[r].append(out[o:o + n])
+            o += n
+    step([(r, 0, len(toks[r]) - 8) for r in small[:20]])
+    step([(r, 0, len(toks[r]) - 8) for r in small[20:]])
+    at = {r: len(toks[r]) - 8 for r in small}
+    at["big"] = 0
+    for k in range(8):
+        entries = [(r, at[r], 1) for r in small]
+        if k in (1, 2):
+            entries.insert(17, ("big", at["big"], 100))          # in the middle of the batch
+            at["big"] += 100
+        elif k > 2:
+            entries.append(("big", at["big"], 1))
+            at["big"] += 1
+        for r in small:
+            at[r] += 1
+        step(entries)
+    step([("big", at["big"], 1)])
+    worst = max(schedules.rel_err(np.concatenate(got[r]), ref[r][:sum(len(x) for x in got[r])]) for r in toks)
+    print(f"[observed] 40 + portion {dt}: {worst:.3e}")
+    assert worst < TOL[dt]
+
+
+@pytest.fixture(scope="module")
+def model_7b(tmp_path_factory):
+    return helpers.make_model(tmp_path_factory.mktemp("db7b"), SHAPE_7B, 21, torch.bfloat16)
+
+
+@pytest.mark.parametrize("n_live", [8, 64])
+def test_decode_batches_at_the_7b_layer_sizes(model_7b, n_live):
+    """The sizes the benchmark times (two layers of them, a small vocabulary), in bfloat16."""
+    toks, prompts = many_requests(SHAPE_7B["vocab_size"], n_live, 900 + n_live, long_every=16, longest=260)
+    ref = helpers.plain_logits(model_7b, toks)
+    _check(model_7b, "bfloat16", 16, toks, prompts, ref, n_live, True, 128, "7B sizes", tol=TOL_7B)

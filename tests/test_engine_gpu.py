@@ -18,7 +18,7 @@ LENGTHS = [5, 17, 33, 70, 100, 41, 64, 2, 1]
 # float32: rounding of a different summation order only.  bfloat16: weights are
 # bfloat16 on both sides (the plain side computes in float64 from the stored
 # values); what differs is the rounding of activations to bfloat16 between kernels.
-TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}
 
 
 @pytest.fixture(scope="module")
@@ -55,6 +55,7 @@ def test_schedules_match_the_plain_implementation(models, name, dt, kind):
     if kind == "mixed":
         assert all(g.pool.total_allocations > g.pool.capacity for g in eng.cache.groups), "no page was used again"
     worst = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
+    print(f"[observed] {name} {dt} {kind}: {worst:.3e}")
     assert worst < TOL[dt], f"{name} {dt} {kind}: {worst}"
 
 
@@ -131,4 +132,5 @@ def test_a_long_prompt_in_portions_then_decoding(tmp_path, dt, name):
     for i in range(tail):
         got[n + i] = eng.step([StepEntry("r0", [toks[n + i]], [0])]).cpu().numpy()[0]
     worst = max(schedules.rel_err(v, ref[p]) for p, v in got.items())
+    print(f"[observed] long prompt {name} {dt}: {worst:.3e}")
     assert worst < TOL[dt], f"{name} {dt}: {worst}"

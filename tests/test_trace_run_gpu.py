@@ -15,7 +15,7 @@ from tiny_configs import TINY_A, TINY_B
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent
-TOL = {"float32": 2e-5, "bfloat16": 4e-2}
+TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}
 
 
 def replay(model_dir, dtype, requests, steps, out_dir, max_tokens):
@@ -54,6 +54,7 @@ def test_trace_run_schedules(tmp_path, cfg, seed, dtype):
         steps = getattr(schedules, kind)(reqs)
         out = replay(d, dtype, reqs, steps, tmp_path / f"out_{kind}", schedules.max_live_tokens(reqs, steps))
         worst = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
+        print(f"[observed] trace_run {dtype} {kind}: {worst:.3e}")
         assert worst < TOL[dtype], f"{kind}: {worst}"
 
 
