@@ -129,6 +129,15 @@ class Qwen2Config:
         return 0
 
 
+# other names under which the reference takes three of the tensors
+# (python/llaisys/models/qwen2.py:139-149): stored name -> the model's name
+QWEN2_WEIGHT_ALIASES = {
+    "transformer.wte.weight": "model.embed_tokens.weight",
+    "model.lm_head.weight": "lm_head.weight",
+    "transformer.ln_f.weight": "model.norm.weight",
+}
+
+
 def qwen2_model_spec(c: Qwen2Config) -> ModelSpec:
     """The Qwen2 decoder as data: per layer RMSNorm -> grouped-query attention
     with biased q/k/v and half-split rotary positions -> residual -> RMSNorm ->
@@ -163,5 +172,6 @@ def qwen2_model_spec(c: Qwen2Config) -> ModelSpec:
         final_norm=PartSpec("rmsnorm", "model.norm.", {"size": c.hidden_size, "eps": c.rms_norm_eps}),
         head=PartSpec("linear_head", "lm_head.", {
             "vocab_size": c.vocab_size, "hidden_size": c.hidden_size,
-            "tied_to": "model.embed_tokens.weight" if c.tie_word_embeddings else None}),
+            "tied_to": "model.embed_tokens.weight" if c.tie_word_embeddings else None,
+            "tie_if_absent": True}),
         eos_token_ids=c.eos_token_ids)

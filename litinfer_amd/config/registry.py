@@ -1,15 +1,20 @@
 """One registry from the architecture's name to its model definition.
 
-An architecture is a pair: a typed configuration class with `from_dict`, and a
-function from that configuration to a `ModelSpec`.  The name comes from
-config.json (`architectures[0]`, else `model_type`).
+An architecture is a typed configuration class with `from_dict` and a function
+from that configuration to a `ModelSpec`; beside them it may name other names
+under which checkpoints store its tensors (`weight_aliases`: stored name ->
+the model's name) and an entry class of its own for `models.load` (the generic
+one otherwise).  The name comes from config.json (`architectures[0]`, else
+`model_type`).  This is the only table from names to models: loading, the
+command line, replay and the benchmark all look here.
 """
 from __future__ import annotations
 
 import json
 from dataclasses import dataclass
 from pathlib import Path
-from typing import Any, Callable, Dict, Tuple
+from dataclasses import field
+from typing import Any, Callable, Dict, Mapping, Optional, Tuple
 
 from .spec import ModelSpec
 
@@ -19,13 +24,19 @@ class Architecture:
     name: str
     config_from_dict: Callable[[Dict[str, Any]], Any]
     model_spec: Callable[[Any], ModelSpec]
+    weight_aliases: Mapping[str, str] = field(default_factory=dict)
+    entry: Optional[type] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, config_from_dict, model_spec, aliases=()) -> None:
-    arch = Architecture(name, config_from_dict, model_spec)
+def register_architecture(name: str, config_from_dict, model_spec, aliases=(), weight_aliases=None,
+                          entry=None) -> None:
+    """`aliases`: further names of the architecture.  `weight_aliases`: stored tensor
+    name -> the name the model's parts use.  `entry`: the class that `models.load`
+    builds for a model folder of this architecture (default: the generic one)."""
+    arch = Architecture(name, config_from_dict, model_spec, dict(weight_aliases or {}), entry)
     for n in (name, *aliases):
         _ARCHITECTURES[n] = arch
 

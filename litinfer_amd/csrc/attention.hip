@@ -363,6 +363,15 @@ union frag8 { u32x4 raw; bf16x8_t v; };
 
 #define DEC_TABLE_CAP 1024      // pages of one split that fit the kernel's copy of the block table
 
+// The most pages one of `nsplit` splits can touch, for block tables of max_blocks pages.
+extern "C" long li_decode_split_blocks(int max_blocks, int page_size, int window, int nsplit) {
+    if (max_blocks <= 0 || page_size <= 0 || nsplit <= 0) return -1;
+    long keys = (long)max_blocks * page_size;
+    if (window > 0 && window < keys) keys = window;
+    const long per = (((keys + nsplit - 1) / nsplit) + 31) & ~31L;
+    return (per + page_size - 2) / page_size + 1;
+}
+
 template <int DH>
 __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
@@ -864,14 +873,17 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dh <= 0 || dh > ATT_MAX_DH || page_size <= 0 ||
         max_blocks <= 0)
         return LI_ERR_SIZE;
+    if (nsplit < 1 || nsplit > MERGE_MAX_SPLITS) return LI_ERR_SIZE;      // the merge kernel keeps a weight per split in LDS
     if (dtype == LI_F32)
         return launch_decode<float>((const float*)q, q_row_stride, (float*)out, (const float*)kc, (const float*)vc,
                                     block_table, max_blocks, token_list, n_tokens, seg_of_token, q_start, q_len,
                                     ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages, window, scale,
                                     nsplit, stream);
-    if (nsplit > MERGE_MAX_SPLITS) return LI_ERR_SIZE;
     if (dtype == LI_BF16 && use_mfma) {
-        if (nkv > 65535 || nsplit < 1) return LI_ERR_SIZE;
+        if (nkv > 65535) return LI_ERR_SIZE;
+        // a split's pages must fit the kernel's copy of the block table: `per` keys that begin
+        // anywhere in a page touch at most (per + page_size - 2) / page_size + 1 pages
+        if (li_decode_split_blocks(max_blocks, page_size, window, nsplit) > DEC_TABLE_CAP) return LI_ERR_SIZE;
         dim3 grid(n_tokens, nkv, nsplit);
 #define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV><<<grid, 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \

@@ -18,9 +18,12 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const int* __restr
         const int src = id_src[t];
         if (src >= 0) id = feedback[src];
     }
-    if (id < 0 || id >= V) return;                 // the host has checked what it knows; never read outside
-    const T* row = table + (size_t)id * H;
     float* o = out + (size_t)t * H;
+    if (id < 0 || id >= V) {                       // the host has checked what it knows; never read outside:
+        for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = 0.f;      // a row of zeros, not what an earlier step left
+        return;
+    }
+    const T* row = table + (size_t)id * H;
     for (int j = threadIdx.x; j < H; j += blockDim.x) o[j] = load_as_float(row + j);
 }
 

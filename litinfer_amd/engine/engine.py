@@ -76,6 +76,7 @@ class Engine:
         # take its token from here (`StepEntry.take`), so the host need not wait for the number
         self.feedback = torch.zeros(FEEDBACK_SLOTS, dtype=torch.int32, device=self.rt.device)
         self.steps_run = 0
+        self.unused_weights: List[str] = []
         # decode steps (every request brings one token) are recorded as HIP graphs, one per batch
         # shape, and replayed: a step is some hundred small launches otherwise
         self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda" and not profiler.enabled
@@ -86,12 +87,13 @@ class Engine:
 
     # ---- construction -----------------------------------------------------
     @classmethod
-    def from_dir(cls, model_dir, **kw) -> "Engine":
+    def from_dir(cls, model_dir, strict_weights: bool = False, **kw) -> "Engine":
         """Model class, sizes and constants come from config.json; weights from
-        the folder's safetensors files."""
+        the folder's safetensors files.  Stored tensors that the model does not
+        use are reported in one line, or refused when `strict_weights`."""
         arch, cfg, spec = load_config(model_dir)
         eng = cls(spec, config=cfg, **kw)
-        load_into(eng.model, model_dir)
+        eng.unused_weights = load_into(eng.model, model_dir, aliases=arch.weight_aliases, strict=strict_weights)
         eng._make_cache()
         return eng
 
@@ -178,7 +180,11 @@ class Engine:
         The tensor may be the output buffer of a recorded step: it is valid until
         the next step (copy it to keep it).
         Raises StepError for a bad batch and CacheFull when pages or slots do
-        not suffice; in both cases the cache is as before."""
+        not suffice; in both cases the cache is as before.  If the model's
+        forward itself raises (a size that a kernel refuses), no cached length
+        moves, requests that this step admitted are released again, and pages
+        reserved for requests that were live already stay with them: the next
+        step uses them, or they go back when the request ends."""
         self._validate(entries)
         cache = self.cache
         admitted, reserved = [], []
@@ -210,10 +216,15 @@ class Engine:
                   f"{sum(len(e.tokens) for e in entries)} tokens, {sum(len(e.want) for e in entries)} rows of logits, "
                   f"{'recorded' if key is not None else 'eager'}, free pages {cache.free_pages()}",
                   file=sys.stderr, flush=True)
-        if key is None:
-            logits = self.model.forward(self._build_context(entries), cache)
-        else:
-            logits = self._forward_graphed(key, self._build_context(entries, pad_blocks=key[2]))
+        try:
+            if key is None:
+                logits = self.model.forward(self._build_context(entries), cache)
+            else:
+                logits = self._forward_graphed(key, self._build_context(entries, pad_blocks=key[2]))
+        except BaseException:
+            for rid in admitted:
+                cache.release(rid)
+            raise
         for e in entries:
             cache.commit(e.rid, len(e.tokens))
         self.steps_run += 1

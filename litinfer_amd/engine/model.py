@@ -36,11 +36,7 @@ class Model:
         for layer in self.layers:
             layer.load_params(get)
         self.final_norm.load_params(get)
-        tied = getattr(self.head, "tied_to", None)
-        if tied:
-            self.head.load_params(get, tied_table=self.embedding.table)
-        else:
-            self.head.load_params(get)
+        self.head.load_params(get, tied_table=getattr(self.embedding, "table", None))
 
     def weight_bytes(self) -> int:
         seen, total = set(), 0

@@ -34,7 +34,13 @@ def main(argv=None) -> int:
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--max-seqs", type=int, default=16, help="requests that may be live at a time")
     ap.add_argument("--device", default="cuda:0")
+    ap.add_argument("--page-order-seed", "--shuffle-pages", dest="page_order_seed", type=int, default=None,
+                    help="shuffle the order in which free pages are handed out, so that block tables are not contiguous")
+    ap.add_argument("--plugin", action="append", default=[],
+                    help="a module to import first (one that registers further parts or architectures)")
     args = ap.parse_args(argv)
+    for mod in args.plugin:
+        __import__(mod)
 
     out_dir = Path(args.out)
     out_dir.mkdir(parents=True, exist_ok=True)
@@ -50,7 +56,7 @@ def main(argv=None) -> int:
     _log(f"loading {args.model} as {args.dtype} ...")
     pages = -(-max(1, args.max_tokens) // args.page_size)
     engine = Engine.from_dir(args.model, dtype=args.dtype, device=args.device, page_size=args.page_size,
-                             num_pages=pages, max_seqs=args.max_seqs)
+                             num_pages=pages, max_seqs=args.max_seqs, page_order_seed=args.page_order_seed)
     _log(f"ready: {engine.spec.architecture}, {pages} pages of {args.page_size} tokens in each of "
          f"{len(engine.cache.groups)} cache group(s)")
     while True:

@@ -487,6 +487,22 @@ def linear_rope_store(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Ten
 
 
 # ----------------------------------------------------------------- attention
+DECODE_MAX_SPLITS = 64       # the merge kernel keeps a weight per split
+DECODE_TABLE_CAP = 1024      # pages of one split that the matrix-core decode kernel copies into LDS
+
+
+def decode_split_blocks(max_blocks: int, page_size: int, window: int, nsplit: int) -> int:
+    """The most pages one of `nsplit` splits of the keys can touch, for block tables of
+    `max_blocks` pages: the keys (at most the table's, or the window's) are cut into runs
+    of a multiple of 32, and a run that begins anywhere in a page touches one page more
+    than its length fills.  The kernel library computes the same bound and refuses a call
+    beyond its table."""
+    keys = max_blocks * page_size
+    if 0 < window < keys:
+        keys = window
+    per = (-(-keys // nsplit) + 31) & ~31
+    return (per + page_size - 2) // page_size + 1
+
 def _decode_kernel_takes(dtype: torch.dtype, dh: int) -> bool:
     """The single-query kernel spreads a key's row over dh / (16 bytes) lanes, a power of two."""
     per = 8 if dtype is torch.bfloat16 else 4
@@ -526,13 +542,14 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         # block of four waves per split on the vector ALU
         mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
         if mfma:
-            nsplit = max(1, min(-(-2048 // (n_single * nkv)), -(-keys // 128), 64))
-            # a split's pages must fit the kernel's copy of the block table (1024 entries)
-            nsplit = max(nsplit, -(-(keys + 64) // (1000 * page_size)))
-            _chk(nsplit <= 64, f"attention: a context of {keys} keys in pages of {page_size} is too "
-                               f"long for the decode kernel")
+            nsplit = max(1, min(-(-2048 // (n_single * nkv)), -(-keys // 128), DECODE_MAX_SPLITS))
+            # a split's pages must fit the kernel's copy of the block table
+            while nsplit <= DECODE_MAX_SPLITS and decode_split_blocks(meta.max_blocks, page_size, window, nsplit) > DECODE_TABLE_CAP:
+                nsplit += 1
+            _chk(nsplit <= DECODE_MAX_SPLITS, f"attention: block tables of {meta.max_blocks} pages of {page_size} "
+                                              f"are too long for the decode kernel")
         else:
-            nsplit = max(1, min(-(-512 // (n_single * nkv)), -(-keys // 256), 64))
+            nsplit = max(1, min(-(-512 // (n_single * nkv)), -(-keys // 256), DECODE_MAX_SPLITS))
         acc = ml = None
         if nsplit > 1:
             shape_a, shape_m = (n_single, nh, nsplit, dh), (n_single, nh, nsplit, 2)

@@ -20,7 +20,7 @@ class RMSNorm(Norm):
         self.weight = None
 
     def expected_params(self):
-        return {self.prefix + "weight": ParamSpec((self.size,))}
+        return {self.prefix + "weight": ParamSpec((self.size,), init="one_plus_normal")}
 
     def load_params(self, get):
         self.weight = self.rt.vector(get(self.prefix + "weight"))

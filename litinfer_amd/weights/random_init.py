@@ -2,10 +2,9 @@
 
 Each tensor has a generator of its own, seeded from (seed, tensor name), so a
 tensor's values do not depend on which other tensors exist or on the order of
-generation.  Matrices and biases are N(0, 0.02); norm weights (one-dimensional
-tensors whose name ends in 'norm.weight' or 'layernorm.weight') are
-1 + N(0, 0.02).  Values are drawn in float32 and rounded once to the stored
-dtype.
+generation.  How a tensor is drawn is what its part says (`ParamSpec.init`):
+matrices and biases N(0, 0.02), the weights of a norm 1 + N(0, 0.02), zeros or
+ones.  Values are drawn in float32 and rounded once to the stored dtype.
 """
 from __future__ import annotations
 
@@ -28,18 +27,16 @@ def _tensor_seed(seed: int, name: str) -> int:
     return int.from_bytes(h[:8], "little") & 0x7FFFFFFFFFFFFFFF
 
 
-def is_norm_weight(name: str, shape) -> bool:
-    return len(shape) == 1 and (name.endswith("norm.weight") or name.endswith("layernorm.weight"))
-
-
 def random_tensor(seed: int, name: str, spec: ParamSpec, dtype: torch.dtype,
                   device="cpu") -> torch.Tensor:
     g = torch.Generator(device=device)
     g.manual_seed(_tensor_seed(seed, name))
     if spec.integer:
         return torch.randint(0, 2 ** 15, spec.shape, generator=g, device=device, dtype=torch.int32)
+    if spec.init in ("zeros", "ones"):
+        return torch.full(spec.shape, float(spec.init == "ones"), device=device, dtype=dtype)
     t = torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32) * STD
-    if is_norm_weight(name, spec.shape):
+    if spec.init == "one_plus_normal":
         t += 1.0
     return t.to(dtype)
 

@@ -36,3 +36,28 @@ def test_no_gpu_means_an_error_not_a_fallback(tmp_path):
     from litinfer_amd.kernels import ops
     with pytest.raises(RuntimeError, match="not on the GPU"):
         ops.rmsnorm(torch.zeros(2, 4), torch.ones(4), 1e-6, torch.zeros(2, 4))
+
+
+def test_a_forward_that_raises_leaves_no_request_behind(tmp_path, cpu_ops, monkeypatch):
+    from litinfer_amd.engine import StepEntry
+    d = helpers.make_model(tmp_path, TINY_A, 0)
+    eng = Engine.from_dir(d, dtype="float32", device="cpu", page_size=16, max_seqs=2, max_tokens=128)
+    eng.step([StepEntry("old", [1, 2, 3], [])])
+    free = eng.cache.free_pages()
+    real = eng.model.forward
+
+    def broken(ctx, cache):
+        raise ValueError("a kernel refused the size")
+    monkeypatch.setattr(eng.model, "forward", broken)
+    with pytest.raises(ValueError, match="refused"):
+        eng.step([StepEntry("old", [4] * 20, []), StepEntry("new", [5, 6], [1])])
+    assert not eng.cache.has("new") and eng.cache.cached_len("old") == 3
+    assert eng.cache.free_slots() == 1
+    eng.cache.check_invariants()
+    monkeypatch.setattr(eng.model, "forward", real)
+    # the request that was live goes on as if nothing had happened; its reserved pages are used now
+    ref = helpers.plain_logits(d, {"r": [1, 2, 3] + [4] * 20})["r"]
+    got = eng.step([StepEntry("old", [4] * 20, [19])]).numpy()
+    assert schedules.rel_err(got[0], ref[22]) < 2e-5
+    eng.finish("old")
+    assert eng.cache.free_pages() == [f + 1 for f in free]

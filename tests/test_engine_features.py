@@ -19,6 +19,7 @@ from litinfer_amd.engine.workspace import Workspace
 from litinfer_amd.parts import FeedForward, Mixer, Position, ResidualStream, Runtime, StateNeed, build_part, register_part
 from litinfer_amd.weights import ParamSpec
 from tiny_configs import TINY_A, TINY_B, TINY_C
+from toy_parts import ToyConfig
 
 
 @pytest.fixture(params=[pytest.param("cpu"), pytest.param("gpu", marks=pytest.mark.gpu)])
@@ -172,7 +173,7 @@ def test_norm_part_alone(device):
     g = torch.Generator().manual_seed(0)
     x, w = torch.randn(9, 120, generator=g), 1 + 0.1 * torch.randn(120, generator=g)
     part = _load(build_part("norm", PartSpec("rmsnorm", "n.", {"size": 120, "eps": 1e-4}), _rt(device)), {"n.weight": w})
-    assert part.expected_params() == {"n.weight": ParamSpec((120,))}
+    assert part.expected_params() == {"n.weight": ParamSpec((120,), init="one_plus_normal")}
     out = torch.empty(9, 120, device=device)
     part.forward(x.to(device), out)
     assert schedules.rel_err(out.cpu().numpy(), P.rms_norm(x.double().numpy(), w.double().numpy(), 1e-4)) < 2e-6
@@ -361,82 +362,16 @@ def test_a_layer_named_twice_and_a_layer_reading_anothers_cache(tmp_path, device
         assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind
 
 
-# ------------------------------ a toy mixer with state of its own, defined here
-class ToyStateMixer(Mixer):
-    """s_t = decay * s_{t-1} + xn_t, y_t = s_t W^T: a recurrent mixer whose state
-    lives in the request's state slot.  Written with torch: it is a toy."""
-
-    def __init__(self, spec, rt):
-        super().__init__(spec, rt)
-        self.h = spec.args["hidden_size"]
-        self.decay = spec.args["decay"]
-        self.w = None
-
-    def cache_need(self):
-        return StateNeed((self.h,), torch.float32)
-
-    def expected_params(self):
-        return {self.prefix + "w": ParamSpec((self.h, self.h))}
-
-    def load_params(self, get):
-        self.w = get(self.prefix + "w").to(torch.float32).to(self.rt.device)
-
-    def forward(self, xn, residual, ctx, cache):
-        residual = residual.tensor()
-        for s in range(ctx.num_segments):
-            q0, n, slot = int(ctx.host_q_start[s]), int(ctx.host_q_len[s]), int(ctx.host_state_slots[s])
-            state = cache.state[slot]
-            for t in range(q0, q0 + n):
-                state.mul_(self.decay).add_(xn[t].float())
-                residual[t] += state @ self.w.T
-
-
-@dataclass(frozen=True)
-class ToyConfig:
-    hidden_size: int
-    vocab_size: int
-    decay: float
-    inner: Qwen2Config
-
-    @classmethod
-    def from_dict(cls, raw):
-        return cls(raw["hidden_size"], raw["vocab_size"], raw["toy_decay"], Qwen2Config.from_dict(raw))
-
-
-def _toy_spec(c: ToyConfig) -> ModelSpec:
-    base = qwen2_model_spec(c.inner)
-    l0 = base.layers[0]
-    toy = LayerSpec("prenorm", dict(l0.parts, mixer=PartSpec("toy_state", "model.layers.0.toy.",
-                                                             {"hidden_size": c.hidden_size, "decay": c.decay})))
-    return replace(base, architecture="ToyStateLM", layers=(toy,) + base.layers[1:])
-
-
+# ------------------------------ a toy mixer with state of its own, defined in tests/toy_parts.py
 def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, device):
-    register_part("mixer", "toy_state", ToyStateMixer)
-    register_architecture("ToyStateLM", ToyConfig.from_dict, _toy_spec)
+    import toy_parts                                       # registers the part and the architecture
     cfg = dict(TINY_A, architectures=["ToyStateLM"], toy_decay=0.9)
     d = helpers.make_model(tmp_path, cfg, 6)
     pcfg, w = P.load_folder(d)
     assert "model.layers.0.toy.w" in w and "model.layers.0.self_attn.q_proj.weight" not in w
-
-    def plain(ids):
-        pos = np.arange(len(ids))
-        x = P.embedding(ids, w["model.embed_tokens.weight"])
-        xn = P.rms_norm(x, w["model.layers.0.input_layernorm.weight"], 1e-6)
-        s = np.zeros(64)
-        y = np.zeros_like(x)
-        for t in range(len(ids)):
-            s = 0.9 * s + xn[t]
-            y[t] = s @ w["model.layers.0.toy.w"].T
-        x = x + y
-        xn = P.rms_norm(x, w["model.layers.0.post_attention_layernorm.weight"], 1e-6)
-        p = "model.layers.0.mlp."
-        x = x + P.swiglu(xn @ w[p + "gate_proj.weight"].T, xn @ w[p + "up_proj.weight"].T) @ w[p + "down_proj.weight"].T
-        x, _ = P.decoder_layer(x, pos, w, "model.layers.1.", pcfg, 0)
-        return P.rms_norm(x, w["model.norm.weight"], 1e-6) @ w["model.embed_tokens.weight"].T
-
+    assert not w["model.layers.0.toy.b"].any()             # the part said "zeros" of its bias
     reqs = helpers.random_requests(256, [21, 40, 3, 30, 12], 7)
-    ref = {r: plain(np.asarray(t)) for r, t in reqs.items()}
+    ref = {r: toy_parts.plain_toy_state_logits(pcfg, w, t, 0.9) for r, t in reqs.items()}
     eng = engine_for(d, device)
     assert len(eng.cache.groups) == 1 and eng.cache.groups[0].entries == [1]
     assert eng.cache.view(0).state.shape == (4, 64)

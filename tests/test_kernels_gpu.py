@@ -357,10 +357,12 @@ def test_rope(ops, dtype, t, heads, dh, theta, start):
     assert rel(xd, ref) < tol(dtype, 2e-4 if start else 2e-6, 8e-3)
 
 
-def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_one=None):
+def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_one=None, row=None):
     """seg_specs: list of (ctx_len, q_len).  Builds random K/V for every
     segment, scatters them into shuffled pages, and compares the kernel with
-    the plain attention on the logical sequences."""
+    the plain attention on the logical sequences.  `scale_one` is the index of a
+    key that is made to stand out for query `row` of its segment (the last one
+    when `row` is None)."""
     g = torch.Generator().manual_seed(seed)
     nseg = len(seg_specs)
     blocks = [-(-c // page) for c, _ in seg_specs]
@@ -378,10 +380,12 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
         v = torch.randn(c, nkv, dh, generator=g).to(dtype)
         if scale_one is not None:             # make one far key stand out for the last query
             far = scale_one
+            big = math.sqrt(12.0 * math.sqrt(dh))      # its score is 12 after scaling: e^12 against some hundred keys near 1
             k[far] = 0
-            k[far, :, 0] = 6.0
-            q[o + ql - 1].view(nh, dh)[:, :] = 0
-            q[o + ql - 1].view(nh, dh)[:, 0] = 6.0
+            k[far, :, 0] = big
+            r = ql - 1 if row is None else row
+            q[o + r].view(nh, dh)[:, :] = 0
+            q[o + r].view(nh, dh)[:, 0] = big
         for b in range(blocks[s]):
             tab[s, b] = perm.pop()
             n = min(page, c - b * page)
@@ -447,20 +451,56 @@ def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_paged_attention_finds_one_far_key(ops, dtype):
+@pytest.mark.parametrize("dh", [32, 64, 128])          # 64 and 128 take the matrix-core kernels in bfloat16
+def test_paged_attention_finds_one_far_key(ops, dtype, dh):
     # one key among hundreds carries almost all the weight: a kernel that skips
     # or misplaces a page gives a visibly different output
     for far in (0, 15, 16, 333, 511):
-        out, ref = _paged_case(ops, dtype, [(512, 1)], 4, 2, 64, 16, 0, seed=7, scale_one=far)
+        out, ref = _paged_case(ops, dtype, [(512, 1)], 4, 2, dh, 16, 0, seed=7, scale_one=far)
         assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_window_edge(ops, dtype):
+@pytest.mark.parametrize("dh", [32, 64, 128])
+@pytest.mark.parametrize("ctx,ql", [(512, 70), (300, 33)])
+def test_portions_find_one_far_key_for_any_row_of_a_tile(ops, dtype, dh, ctx, ql):
+    # portions: the standout key for the first row of a 32-row tile, its last row, the first
+    # row of the next tile and the portion's last row; at the start of the sequence, in the
+    # middle, just before the portion and at the row's own position
+    for row in (0, 31, 32, ql - 1):
+        p = ctx - ql + row
+        for far in (0, 97, ctx - ql - 1, p):
+            out, ref = _paged_case(ops, dtype, [(ctx, ql)], 6, 2, dh, 16, 0, seed=7, scale_one=far, row=row)
+            assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2), (row, far)
+        if p + 1 < ctx:                                # the key after the row's own is not seen
+            out, ref = _paged_case(ops, dtype, [(ctx, ql)], 6, 2, dh, 16, 0, seed=7, scale_one=p + 1, row=row)
+            assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2), (row, "next")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dh", [32, 64, 128])
+def test_window_edge(ops, dtype, dh):
     # the key just outside the window must not count, the one just inside must
     for window, far, visible in ((32, 512 - 32, True), (32, 512 - 33, False)):
-        out, ref = _paged_case(ops, dtype, [(512, 1)], 2, 1, 32, 8, window, seed=8, scale_one=far)
+        out, ref = _paged_case(ops, dtype, [(512, 1)], 2, 1, dh, 8, window, seed=8, scale_one=far)
         assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("dh", [32, 64, 128])
+@pytest.mark.parametrize("ctx,ql,window", [(512, 70, 48), (300, 33, 100), (512, 70, 37)])
+def test_window_edge_for_any_row_of_a_tile(ops, dtype, dh, ctx, ql, window):
+    # the first and last row of a 32-row tile, the first row of the next tile, a row whose
+    # window begins on a block of 32 keys, and the last row: the key at the window's first
+    # position counts, the one before it does not
+    rows = {0, 31, 32, ql - 1}
+    rows.add(next(r for r in range(ql) if (ctx - ql + r - window + 1) % 32 == 0))
+    for row in sorted(rows):
+        first = ctx - ql + row - window + 1            # the first key that the row sees
+        for far in (first, first - 1):
+            assert far >= 0
+            out, ref = _paged_case(ops, dtype, [(ctx, ql)], 4, 2, dh, 16, window, seed=8, scale_one=far, row=row)
+            assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2), (row, far - first)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -64,6 +64,7 @@ def test_expected_tensor_names_are_the_checkpoints():
     names = expected_params_of_spec(qwen2_model_spec(Qwen2Config.from_dict(TINY_B)))
     assert names["model.embed_tokens.weight"].shape == (320, 96)
     assert names["lm_head.weight"].shape == (320, 96) and names["model.norm.weight"].shape == (96,)
+    assert not names["lm_head.weight"].required          # absent: tied to the table, as in the reference
     p = "model.layers.2."
     assert names[p + "self_attn.q_proj.weight"].shape == (96, 96)
     assert names[p + "self_attn.k_proj.weight"].shape == (32, 96)
@@ -94,9 +95,18 @@ def test_random_model_folder_is_seeded_and_distributed_as_said(tmp_path):
                            "model.safetensors").entries[name][0] == "BF16"
 
 
-def _load(folder, cpu_ops):
+def _load(folder, cpu_ops, **kw):
     from litinfer_amd.engine import Engine
-    return Engine.from_dir(folder, dtype="float32", device="cpu", max_tokens=64, max_seqs=2)
+    return Engine.from_dir(folder, dtype="float32", device="cpu", max_tokens=64, max_seqs=2, **kw)
+
+
+def _rewrite(folder, change):
+    f = SafetensorsFile(folder / "model.safetensors")
+    tensors = {n: f.tensor(n).clone() for n in f.entries}
+    f.close()
+    change(tensors)
+    write_safetensors(folder / "model.safetensors", tensors.items())
+    return tensors
 
 
 def test_loader_raises_one_error_for_a_broken_folder(tmp_path, cpu_ops):
@@ -110,10 +120,75 @@ def test_loader_raises_one_error_for_a_broken_folder(tmp_path, cpu_ops):
     tensors["model.layers.9.mlp.up_proj.weight"] = torch.zeros(2, 2)
     write_safetensors(d / "model.safetensors", tensors.items())
     with pytest.raises(WeightError) as e:
-        _load(d, cpu_ops)
+        _load(d, cpu_ops, strict_weights=True)
     assert e.value.missing == ["model.layers.1.mlp.down_proj.weight", "model.norm.weight"]
     assert e.value.unexpected == ["model.layers.9.mlp.up_proj.weight"]
     assert e.value.wrong_shape == [("model.layers.0.self_attn.k_proj.weight", (32, 64), (16, 64))]
+    # without the strict switch an unknown tensor is no fault (python/llaisys/models/qwen2.py:152-194
+    # lets unknown names fall through); what is missing or misshapen still is, in the same one error
+    with pytest.raises(WeightError) as e:
+        _load(d, cpu_ops)
+    assert e.value.missing == ["model.layers.1.mlp.down_proj.weight", "model.norm.weight"]
+    assert e.value.unexpected == []
+    assert e.value.wrong_shape == [("model.layers.0.self_attn.k_proj.weight", (32, 64), (16, 64))]
+
+
+def test_unknown_tensors_are_counted_and_reported_in_one_line(tmp_path, cpu_ops, capsys):
+    d = write_random_model(tmp_path / "m", TINY_B, seed=1, dtype=torch.float32)
+
+    def change(t):
+        t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)      # holds no weights: not even counted
+        t["model.layers.7.mlp.up_proj.weight"] = torch.zeros(2, 2)
+        t["some.other.tensor"] = torch.zeros(3)
+    _rewrite(d, change)
+    eng = _load(d, cpu_ops)
+    assert eng.unused_weights == ["model.layers.7.mlp.up_proj.weight", "some.other.tensor"]
+    err = capsys.readouterr().err
+    lines = [l for l in err.splitlines() if "not used" in l]
+    assert len(lines) == 1 and "2 stored tensor(s)" in lines[0] and "some.other.tensor" in lines[0]
+
+
+def test_the_references_other_names_for_three_tensors_are_taken(tmp_path, cpu_ops):
+    """transformer.wte.weight, model.lm_head.weight and transformer.ln_f.weight
+    (python/llaisys/models/qwen2.py:139-149)."""
+    d = write_random_model(tmp_path / "m", TINY_B, seed=1, dtype=torch.float32)
+    want_norm = _load(d, cpu_ops).model.final_norm.weight.clone()      # (on the CPU a tensor may be the file's mapping)
+
+    def change(t):
+        t["transformer.wte.weight"] = t.pop("model.embed_tokens.weight")
+        t["model.lm_head.weight"] = t.pop("lm_head.weight")
+        t["transformer.ln_f.weight"] = t.pop("model.norm.weight")
+    stored = _rewrite(d, change)
+    eng = _load(d, cpu_ops, strict_weights=True)
+    assert eng.unused_weights == []
+    assert torch.equal(eng.model.embedding.table, stored["transformer.wte.weight"])
+    assert torch.equal(eng.model.head.proj.weight, stored["model.lm_head.weight"])
+    assert torch.equal(eng.model.final_norm.weight, want_norm)
+    # a tensor stored under its own name wins; the alias beside it is one tensor too many
+    _rewrite(d, lambda t: t.__setitem__("model.norm.weight", torch.ones(96)))
+    eng = _load(d, cpu_ops)
+    assert torch.equal(eng.model.final_norm.weight, torch.ones(96))
+    assert eng.unused_weights == ["transformer.ln_f.weight"]
+
+
+def test_head_matrix_stray_when_tied_and_absent_when_untied(tmp_path, cpu_ops, capsys):
+    # tie_word_embeddings = true: a stored lm_head.weight is not used
+    d = write_random_model(tmp_path / "a", TINY_A, seed=0, dtype=torch.float32)
+    _rewrite(d, lambda t: t.__setitem__("lm_head.weight", torch.zeros(256, 64)))
+    eng = _load(d, cpu_ops)
+    assert eng.unused_weights == ["lm_head.weight"]
+    assert eng.model.head.proj.weight.data_ptr() == eng.model.embedding.table.data_ptr()
+    with pytest.raises(WeightError) as e:
+        _load(d, cpu_ops, strict_weights=True)
+    assert e.value.unexpected == ["lm_head.weight"]
+    # untied, but no lm_head.weight stored: the table is used, with a note
+    # (python/llaisys/models/qwen2.py:196-199)
+    d = write_random_model(tmp_path / "b", TINY_B, seed=1, dtype=torch.float32)
+    _rewrite(d, lambda t: t.pop("lm_head.weight"))
+    capsys.readouterr()
+    eng = _load(d, cpu_ops)
+    assert eng.model.head.proj.weight.data_ptr() == eng.model.embedding.table.data_ptr()
+    assert "lm_head.weight is not stored" in capsys.readouterr().err
 
 
 def test_biases_are_optional_and_tied_head_shares_the_table(tmp_path, cpu_ops):
