@@ -2,7 +2,10 @@
 // and temperature / top-k / top-p sampling by inverse CDF with a uniform
 // number that the host derives from the request's own counter-based stream.
 #include "common.h"
+#include "li_noalloc.h"
 #include <math.h>
+#include <mutex>
+#include <stdio.h>
 
 #define SMP_NT 1024
 
@@ -72,6 +75,76 @@ extern "C" int li_argmax_rows(const float* logits, int* out, float* scratch_v, i
     argmax_partial_kernel<<<dim3(n, nchunks), SMP_NT, 0, stream>>>(logits, scratch_v, scratch_i, V, chunk);
     argmax_final_kernel<<<n, 64, 0, stream>>>(scratch_v, scratch_i, out, nchunks);
     return li_launch_status();
+}
+
+// ------------------------------------------------- argmax that allocates nothing
+// The same two kernels with their partial results in a file-scope device array instead of
+// buffers that the caller brings: for callers that cannot allocate (li_noalloc.h).  Every
+// GPU holds its own copy of the array at its own address; host code must use the address
+// that hipGetSymbolAddress gives for the current device, never the array's name.
+static __device__ __align__(256) unsigned char scratch[LI_ARGMAX_NOALLOC_MAX_ROWS * ARGMAX_CHUNKS * 8];
+
+#define LI_NOALLOC_MAX_DEVICES 64
+static void* g_scratch_ptr[LI_NOALLOC_MAX_DEVICES];       // the array's address on each device, once asked for
+static std::mutex g_scratch_mutex;
+static thread_local char g_noalloc_error[200];
+
+static int noalloc_fail(int code, const char* what, hipError_t e) {
+    if (e != hipSuccess) snprintf(g_noalloc_error, sizeof g_noalloc_error, "%s: %s", what, hipGetErrorString(e));
+    else snprintf(g_noalloc_error, sizeof g_noalloc_error, "%s", what);
+    return code;
+}
+
+// The scratch array's address on the current device (asked for once per device).
+static int noalloc_scratch(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return noalloc_fail(LI_ERR_LAUNCH, "li_argmax_rows_noalloc: hipGetDevice", e);
+    if (dev < 0 || dev >= LI_NOALLOC_MAX_DEVICES)
+        return noalloc_fail(LI_ERR_SIZE, "li_argmax_rows_noalloc: device number beyond the table of scratch addresses", hipSuccess);
+    std::lock_guard<std::mutex> hold(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) return noalloc_fail(LI_ERR_LAUNCH, "li_argmax_rows_noalloc: hipGetSymbolAddress(scratch)", e);
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return LI_OK;
+}
+
+extern "C" int li_argmax_rows_noalloc_init(void) {
+    void* p;
+    return noalloc_scratch(&p);
+}
+
+extern "C" int li_argmax_rows_noalloc_max_rows(void) { return LI_ARGMAX_NOALLOC_MAX_ROWS; }
+
+extern "C" const char* li_argmax_rows_noalloc_error(void) { return g_noalloc_error; }
+
+extern "C" int li_argmax_rows_noalloc(const float* logits, int* out, int n, int V, hipStream_t stream) {
+    g_noalloc_error[0] = 0;
+    if (n <= 0 || V <= 0) return noalloc_fail(LI_ERR_SIZE, "li_argmax_rows_noalloc: rows and vocabulary must be positive", hipSuccess);
+    if (n > LI_ARGMAX_NOALLOC_MAX_ROWS) {
+        snprintf(g_noalloc_error, sizeof g_noalloc_error,
+                 "li_argmax_rows_noalloc: %d rows are more than the %d that the scratch array holds; "
+                 "use li_argmax_rows with buffers of the caller", n, LI_ARGMAX_NOALLOC_MAX_ROWS);
+        return LI_ERR_SIZE;
+    }
+    void* base = nullptr;
+    const int rc = noalloc_scratch(&base);
+    if (rc != LI_OK) return rc;
+    // partial maxima first, their indices behind them; stage 1 writes every place that stage 2
+    // reads, so nothing of an earlier call's contents has to be cleared
+    float* pv = reinterpret_cast<float*>(base);
+    int* pi = reinterpret_cast<int*>(static_cast<unsigned char*>(base) + (size_t)LI_ARGMAX_NOALLOC_MAX_ROWS * ARGMAX_CHUNKS * 4);
+    int nchunks = (V + 4095) / 4096;
+    if (nchunks > ARGMAX_CHUNKS) nchunks = ARGMAX_CHUNKS;
+    const int chunk = (V + nchunks - 1) / nchunks;
+    argmax_partial_kernel<<<dim3(n, nchunks), SMP_NT, 0, stream>>>(logits, pv, pi, V, chunk);
+    argmax_final_kernel<<<n, 64, 0, stream>>>(pv, pi, out, nchunks);
+    if (li_launch_status() != LI_OK) return noalloc_fail(LI_ERR_LAUNCH, "li_argmax_rows_noalloc: launch failed", hipSuccess);
+    return LI_OK;
 }
 
 // ---------------------------------------------------------------- sampling
