@@ -218,6 +218,13 @@ class CacheManager:
         if self._lib.li_book_commit(self._book, self._handle(rid), int(n_new)) < 0:
             raise PagePoolError(self._error())
 
+    def rewind(self, rid, n: int) -> None:
+        """Forget the last `n` tokens of `rid`: their positions will be computed and written
+        again.  The pages stay with the request.  Refused (ValueError) where a windowed group has
+        already given back a page that the earlier position still sees."""
+        if self._lib.li_book_rewind(self._book, self._handle(rid), int(n)) < 0:
+            raise ValueError(self._error())
+
     def release(self, rid) -> None:
         h = self._handles.pop(rid)
         if self._lib.li_book_release(self._book, h) < 0:

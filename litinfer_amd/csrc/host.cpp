@@ -248,6 +248,21 @@ int li_book_commit(void* vb, int64_t h, int n_new) {
     }
     return 0;
 }
+// the last n tokens are forgotten (their places will be written again); the pages stay with the
+// request.  Refused where a windowed group has already given back a page that a query at the new
+// position would see.
+int li_book_rewind(void* vb, int64_t h, int n) {
+    Book* b = (Book*)vb;
+    Request* r = b->find(h);
+    if (!r) return b->fail(ERR_UNKNOWN, "cache: unknown request");
+    if (n < 0 || n > r->cached) return b->fail(ERR_ARG, "cache: cannot forget " + std::to_string(n) + " of " +
+                                                            std::to_string(r->cached) + " cached tokens");
+    for (size_t g = 0; g < b->pools.size(); ++g)
+        if (b->first_needed_block((int)g, r->cached - n) < r->first_live[g])
+            return b->fail(ERR_ARG, "cache: a windowed group has given back pages that the earlier position still sees");
+    r->cached -= n;
+    return 0;
+}
 int li_book_release(void* vb, int64_t h) {
     Book* b = (Book*)vb;
     auto it = b->requests.find(h);

@@ -36,7 +36,10 @@ MODULE_FLAGS = {"attention": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
                 # list, which the compiler remarks upon for every instance
                 "gemm": ["-Wno-inline-asm"]}
 
-MODULES = ("elementwise", "gemm", "attention", "sampling", "host")
+MODULES = ("elementwise", "gemm", "attention", "sampling", "host")     # what a model needs
+# measuring kernels of the benchmark (a streaming read, a copy, a matrix-core loop): built with the
+# rest by `build_all(everything=True)`, otherwise when the benchmark first asks for them
+EXTRA_MODULES = ("probe",)
 # "host" is plain C++ (the cache's bookkeeping and the layout of a step's batch): no device code
 HOST_MODULES = ("host",)
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
@@ -155,8 +158,10 @@ def compile_module(module: str, verbose: bool = True) -> Path:
     return out
 
 
-def build_all(verbose: bool = True, force: bool = True) -> List[Path]:
-    """Compile every module (in parallel)."""
+def build_all(verbose: bool = True, force: bool = True, everything: bool = False) -> List[Path]:
+    """Compile every module that a model needs (in parallel); with `everything`, the
+    benchmark's measuring kernels too."""
+    modules = MODULES + (EXTRA_MODULES if everything else ())
     outs: Dict[str, Path] = {}
     errs: List[BaseException] = []
 
@@ -166,14 +171,14 @@ def build_all(verbose: bool = True, force: bool = True) -> List[Path]:
         except BaseException as e:           # noqa: BLE001 - reported below
             errs.append(e)
 
-    threads = [threading.Thread(target=work, args=(m,)) for m in MODULES]
+    threads = [threading.Thread(target=work, args=(m,)) for m in modules]
     for t in threads:
         t.start()
     for t in threads:
         t.join()
     if errs:
         raise errs[0]
-    return [outs[m] for m in MODULES]
+    return [outs[m] for m in modules]
 
 
 def load(module: str) -> ctypes.CDLL:

@@ -96,6 +96,31 @@ def test_window_gives_pages_back_and_never_the_visible_ones():
     assert m.free_pages() == [12, 12]
 
 
+def test_rewind_forgets_tokens_keeps_pages_and_respects_the_window():
+    m = _manager(num_pages=6, page=4)
+    m.admit("a")
+    m.reserve("a", 9)
+    m.commit("a", 9)
+    table = m.block_table("a", 0)
+    m.rewind("a", 2)
+    assert m.cached_len("a") == 7 and m.block_table("a", 0) == table and m.free_pages() == [3]
+    m.reserve("a", 2)                                  # the same places again: no new page
+    m.commit("a", 2)
+    assert m.cached_len("a") == 9 and m.block_table("a", 0) == table
+    with pytest.raises(ValueError):
+        m.rewind("a", 10)
+    m.check_invariants()
+    w = _manager(num_pages=12, page=4, window=6)
+    w.admit("a")
+    w.reserve("a", 20)
+    w.commit("a", 20)                                  # the windowed group has given back blocks 0..2
+    w.rewind("a", 1)                                   # position 19 sees keys from 14 on: block 3, still held
+    with pytest.raises(ValueError, match="given back"):
+        w.rewind("a", 4)                               # position 15 would see key 10 in block 2, which is gone
+    assert w.cached_len("a") == 19
+    w.check_invariants()
+
+
 def test_slots_and_state_are_zeroed_at_admission():
     m = CacheManager([StateNeed((3,), torch.float32), PagedKVNeed(1, 4, 0)], [None, None], page_size=4,
                      num_pages=4, max_seqs=2, dtype=torch.float32, device="cpu")
