@@ -303,9 +303,10 @@ def headline(a) -> Dict[str, object]:
     eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
                              num_pages=max_b * CONTEXT // PAGE + PREFILL_TOKENS // PAGE, max_seqs=max_b + 1)
     for g in eng.cache.groups:                       # synthetic cache content
-        flat = g.data.view(-1)
-        for i in range(0, flat.numel(), 1 << 28):
-            flat[i:i + (1 << 28)].normal_(0, 0.5)
+        for data in g.data.values():
+            flat = data.view(-1)
+            for i in range(0, flat.numel(), 1 << 28):
+                flat[i:i + (1 << 28)].normal_(0, 0.5)
     torch.cuda.synchronize()
     log(f"model and cache ready in {time.time() - t0:.1f} s ({eng.model.weight_bytes() / 1e9:.2f} GB of weights)")
     sampler = Sampler(dev)

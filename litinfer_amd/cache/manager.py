@@ -2,10 +2,12 @@
 and slots for per-request state of fixed size.
 
 Entries of the model's execution order that need a cache are put into GROUPS
-by what they need (kv heads, head size, window).  A group has one page pool
-and one device tensor [entries, 2 (K|V), pages, kv_heads, page_size, head_dim];
-a page id is valid in every entry of its group, and each request has one block
-table per group.  A windowed group gives a page back as soon as no later query
+by what they need: the named tensors they keep per token (keys and values of
+some head layout, a compressed latent, keys alone ...) and the window.  A
+group has one page pool and, for each of its tensors, one device tensor
+[entries, pages, *leading sizes, page_size, last size]; a page id is valid in
+every entry and every tensor of its group, and each request has one block table
+per group.  A windowed group gives a page back as soon as no later query
 can see any of its positions; its table entry becomes -1 and is never
 addressed again.  All pages of a request go back when it is released.
 
@@ -30,7 +32,7 @@ import ctypes
 
 import torch
 
-from ..parts.base import PagedKVNeed, StateNeed
+from ..parts.base import PagedNeed, StateNeed
 from . import native
 from .pool import PagePool, PagePoolError
 
@@ -44,18 +46,29 @@ class CacheView:
     """What a mixer sees of the cache for one entry of the execution order."""
     owned: bool                      # False: reads another entry's cache, writes nothing
     group: Optional[int] = None      # index of the page group (paged needs)
-    k: Optional[torch.Tensor] = None     # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None
+    tensors: Optional[Dict[str, torch.Tensor]] = None    # name -> [pages, *leading sizes, page_size, last size]
     page_size: int = 0
     state: Optional[torch.Tensor] = None  # [max_seqs, *shape] (state needs)
+
+    @property
+    def k(self) -> Optional[torch.Tensor]:
+        """The tensor named "k" (keys [pages, kv_heads, page_size, head_dim] of a PagedKVNeed)."""
+        return self.tensors["k"] if self.tensors else None
+
+    @property
+    def v(self) -> Optional[torch.Tensor]:
+        return self.tensors["v"] if self.tensors else None
 
 
 @dataclass
 class _Group:
-    need: PagedKVNeed
+    need: PagedNeed
     entries: List[int]
     pool: PagePool
-    data: torch.Tensor               # [n_entries, 2, pages, kv_heads, page_size, head_dim]
+    data: Dict[str, torch.Tensor]    # name -> [n_entries, pages, *leading sizes, page_size, last size]
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for t in self.data.values())
 
 
 class CacheManager:
@@ -76,11 +89,15 @@ class CacheManager:
         self._entry_group: Dict[int, Tuple[int, int]] = {}     # entry -> (group, index in group)
         self._entry_state: Dict[int, torch.Tensor] = {}
         self._sources = list(sources)
-        by_need: Dict[PagedKVNeed, int] = {}
+        by_need: Dict[PagedNeed, int] = {}
         for i, need in enumerate(needs):
             if sources[i] is not None or need is None:
                 continue
-            if isinstance(need, PagedKVNeed):
+            if isinstance(need, PagedNeed):
+                names = [t.name for t in need.tensors]
+                if not names or len(set(names)) != len(names) or any(not t.shape or min(t.shape) <= 0 for t in need.tensors):
+                    raise ValueError(f"cache: entry {i} asks for paged tensors {need.tensors!r}: they need "
+                                     f"distinct names and positive sizes")
                 if need not in by_need:
                     by_need[need] = len(self.groups)
                     self.groups.append(_Group(need, [], None, None))
@@ -111,8 +128,8 @@ class CacheManager:
         self._ints = (ctypes.c_int * max(ng, 1))()
         for gi, g in enumerate(self.groups):
             g.pool = PagePool(num_pages, _borrowed=self._lib.li_book_pool(self._book, gi))
-            g.data = torch.zeros((len(g.entries), 2, num_pages, g.need.num_kv_heads, self.page_size,
-                                  g.need.head_dim), dtype=dtype, device=self.device)
+            g.data = {t.name: torch.zeros((len(g.entries), num_pages, *t.page_shape(self.page_size)),
+                                          dtype=t.dtype or dtype, device=self.device) for t in g.need.tensors}
         # requests are named by any hashable; the book knows them by number
         self._handles: Dict[Hashable, int] = {}
         self._next_handle = 0
@@ -137,8 +154,8 @@ class CacheManager:
         owner = entry if src is None else src
         if owner in self._entry_group:
             g, j = self._entry_group[owner]
-            d = self.groups[g].data
-            return CacheView(owned=src is None, group=g, k=d[j, 0], v=d[j, 1], page_size=self.page_size)
+            return CacheView(owned=src is None, group=g, page_size=self.page_size,
+                             tensors={name: d[j] for name, d in self.groups[g].data.items()})
         if owner in self._entry_state:
             return CacheView(owned=src is None, state=self._entry_state[owner])
         return CacheView(owned=src is None)

@@ -36,7 +36,7 @@ def lib() -> ctypes.CDLL:
             "li_book_rewind": ([c_void_p, c_int64, c_int], c_int),
             "li_book_release": ([c_void_p, c_int64], c_int), "li_book_check": ([c_void_p], c_int),
             "li_book_build_batch": ([c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                     c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p], c_long),
+                                     c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p], c_long),
         }
         for name, (args, res) in sig.items():
             f = getattr(l, name)

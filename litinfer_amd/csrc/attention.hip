@@ -305,6 +305,14 @@ __global__ __launch_bounds__(128) void attention_merge_kernel(
     const int ti = blockIdx.x, head = blockIdx.y;
     const int t = token_list ? token_list[ti] : ti;
     const size_t base = ((size_t)ti * nh + head) * nsplit;
+    // The partial results of this thread's first dimension are asked for before the weights
+    // are known (up to 32 splits, all loads at once and never conditional): their way from
+    // memory then runs beside the weights' way and arithmetic, not behind them.
+    constexpr int AHEAD = 32;
+    float pa[AHEAD];
+    const int d0 = threadIdx.x < dh ? threadIdx.x : 0;
+#pragma unroll
+    for (int sp = 0; sp < AHEAD; ++sp) pa[sp] = part_acc[(base + (sp < nsplit ? sp : nsplit - 1)) * dh + d0];
     if (threadIdx.x < 64) {
         const int sp = threadIdx.x;
         const float ms = sp < nsplit ? part_ml[(base + sp) * 2] : -INFINITY;
@@ -320,8 +328,15 @@ __global__ __launch_bounds__(128) void attention_merge_kernel(
     __syncthreads();
     for (int d = threadIdx.x; d < dh; d += 128) {
         float at = 0.f;
+        if (d == d0) {                               // (the same order of additions as below)
+#pragma unroll
+            for (int sp = 0; sp < AHEAD; ++sp) at += sp < nsplit ? pa[sp] * wgt[sp] : 0.f;
 #pragma unroll 8
-        for (int sp = 0; sp < nsplit; ++sp) at += part_acc[(base + sp) * dh + d] * wgt[sp];
+            for (int sp = AHEAD; sp < nsplit; ++sp) at += part_acc[(base + sp) * dh + d] * wgt[sp];
+        } else {
+#pragma unroll 8
+            for (int sp = 0; sp < nsplit; ++sp) at += part_acc[(base + sp) * dh + d] * wgt[sp];
+        }
         store_from_float(out + (size_t)t * nh * dh + (size_t)head * dh + d, at * inv_l);
     }
 }

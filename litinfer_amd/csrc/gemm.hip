@@ -75,6 +75,92 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
     }
 }
 
+// ------------------------------------------------------ float32, few rows (decode)
+// The product streams W once: a wave owns F32R_NT consecutive columns of the output and
+// walks K with 16 bytes a lane; the MT rows of x come from the caches (every wave of the
+// grid reads the same few rows).  More than MT rows run as passes of MT; the passes of one
+// group of columns are neighbouring blocks, so that the second finds the matrix's rows in L2.
+// Each output element is the butterfly sum of its 64 lanes' strided partial sums: an order
+// that depends on K alone.
+#define F32R_NT 4
+#define F32R_WAVES 4
+
+template <int MT>
+__global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const float* __restrict__ x,
+                                                                        const float* __restrict__ w,
+                                                                        const float* __restrict__ bias,
+                                                                        float* __restrict__ out, int M, int N, int K,
+                                                                        int accumulate, int npass) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pass = blockIdx.x % npass, group = blockIdx.x / npass;
+    const int n0 = (group * F32R_WAVES + wave) * F32R_NT;
+    const int m0 = pass * MT;
+    if (n0 >= N) return;
+    float acc[MT][F32R_NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < F32R_NT; ++j) acc[i][j] = 0.f;
+    const float* wrow[F32R_NT];
+#pragma unroll
+    for (int j = 0; j < F32R_NT; ++j) wrow[j] = w + (size_t)(n0 + j < N ? n0 + j : N - 1) * K;
+    const float* xrow[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) xrow[i] = x + (size_t)(m0 + i < M ? m0 + i : M - 1) * K;
+    for (int k = 4 * lane; k < K; k += 256) {
+        floatx4 wv[F32R_NT], xv[MT];
+#pragma unroll
+        for (int j = 0; j < F32R_NT; ++j) wv[j] = *reinterpret_cast<const floatx4*>(wrow[j] + k);
+#pragma unroll
+        for (int i = 0; i < MT; ++i) xv[i] = *reinterpret_cast<const floatx4*>(xrow[i] + k);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < F32R_NT; ++j) acc[i][j] = fmaf(xv[i][e], wv[j][e], acc[i][j]);
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < F32R_NT; ++j) {
+            float v = acc[i][j];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+            acc[i][j] = v;
+        }
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            if (m0 + i >= M) continue;
+#pragma unroll
+            for (int j = 0; j < F32R_NT; ++j)
+                if (n0 + j < N) epilogue_store(out, (size_t)(m0 + i) * N + n0 + j, acc[i][j], bias, n0 + j, accumulate != 0);
+        }
+    }
+}
+
+#define F32_ROWS_MAX 64          // up to this many rows the row kernel is taken (K a multiple of 4)
+
+static int launch_f32_rows(const float* x, const float* w, const float* bias, float* out, int M, int N, int K,
+                           int accumulate, hipStream_t stream) {
+    const int mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    const int npass = (M + mt - 1) / mt;
+    const long groups = (N + F32R_WAVES * F32R_NT - 1) / (F32R_WAVES * F32R_NT);
+    if (groups * npass > 0x7fffffffL) return LI_ERR_SIZE;
+    const unsigned grid = (unsigned)(groups * npass);
+#define LI_F32R(MT) gemm_f32_rows_kernel<MT><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass)
+    switch (mt) {
+        case 1: LI_F32R(1); break;
+        case 2: LI_F32R(2); break;
+        case 4: LI_F32R(4); break;
+        case 8: LI_F32R(8); break;
+        default: LI_F32R(16); break;
+    }
+#undef LI_F32R
+    return li_launch_status();
+}
+
 // ----------------------------------------------------------- bfloat16 MFMA
 // Block tile 128 x 128, K in steps of 32, 4 waves in a 2 x 2 grid, each wave a
 // 64 x 64 tile made of 2 x 2 MFMA 32x32x16 tiles.  Operand layout of
@@ -845,6 +931,45 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
 
+    // What the epilogue adds to or multiplies with the sums (bias, the residual sum, a norm's
+    // weights, the rotation's cosines and sines, the page slot) is asked for now, by the wave
+    // that will write the results: the answers arrive with the first chunk, and the epilogue
+    // waits for no memory.  Never conditional per lane: a place past the end reads the last one.
+    constexpr bool PRE = MT == 1 && !SWIGLU;
+    float pre_bias[NT][4], pre_res[NT][4], pre_gamma[NT][4], pre_cos[4], pre_sin[4];
+    int pre_slot = 0;
+    if constexpr (PRE) {
+        if (wave == 0) {
+            const int m = (lane & 15) < M ? (lane & 15) : M - 1;
+            if constexpr (ROPE) {
+                const int dh = a.dh, half = dh / 2, bph = dh / 16;
+                const int head = blockIdx.x / bph, i = blockIdx.x % bph;
+                const bool second = (lane >> 4) >= 2;
+                pre_slot = a.slot_map[m];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = 8 * i + 4 * ((lane >> 4) & 1) + r;
+                    pre_bias[0][r] = a.bias ? a.bias[head * dh + (second ? half + j : j)] : 0.f;
+                    pre_cos[r] = a.cos[(size_t)m * half + j];
+                    pre_sin[r] = a.sin[(size_t)m * half + j];
+                }
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int n = n0 + 16 * nt + 4 * (lane >> 4) + r;
+                        const int nc = n < N ? n : N - 1;
+                        pre_bias[nt][r] = a.bias ? a.bias[nc] : 0.f;
+                        pre_gamma[nt][r] = a.gamma ? a.gamma[nc] : 0.f;
+                        if constexpr (sizeof(TO) == 4)
+                            pre_res[nt][r] = a.accumulate ? reinterpret_cast<const float*>(a.out)[(size_t)m * N + nc] : 0.f;
+                        else pre_res[nt][r] = 0.f;
+                    }
+            }
+        }
+    }
+
     // The memory counter of a wave retires loads in the order they were issued, so waiting for
     // a chunk's x pieces also waits for every load issued before them.  All loads of a chunk (W
     // and x) are therefore issued together, one chunk ahead of their use: when chunk c is
@@ -968,7 +1093,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
             const int dh = a.dh, half = dh / 2, bph = dh / 16;
             const int head = blockIdx.x / bph, i = blockIdx.x % bph;
             const bool second = (l >> 4) >= 2;                       // this lane holds the pairs' second members
-            const int slot = a.slot_map[m];
+            const int slot = pre_slot;                               // (MT is 1: thread t is lane l of wave 0, which asked for these)
             const int page = slot / a.page_size, in_page = slot - page * a.page_size;
             const bool page_ok = page >= 0 && page < a.num_pages;
 #pragma unroll
@@ -976,12 +1101,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 const int j = 8 * i + 4 * ((l >> 4) & 1) + r;        // the pair's number within the head
                 const int d = second ? half + j : j;
                 const int col = head * dh + d;
-                float own = s[0][r];
-                if (a.bias) own += a.bias[col];
+                float own = s[0][r] + pre_bias[0][r];
                 const float other = __shfl_xor(own, 32, 64);
                 float v = own;
                 if (head < a.nh + a.nkv) {
-                    const float c = a.cos[(size_t)m * half + j], sn = a.sin[(size_t)m * half + j];
+                    const float c = pre_cos[r], sn = pre_sin[r];
                     v = second ? own * c + other * sn : own * c - other * sn;
                 }
                 const uint16_t bits = float_to_bf16(v);
@@ -1013,11 +1137,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                             const int n = n0 + 16 * nt + 4 * (l >> 4) + r;
                             if (n < N) {
                                 const size_t idx = (size_t)m * N + n;
-                                float v = s[nt][r];
-                                if (a.bias) v += a.bias[n];
-                                if (a.accumulate) v += reinterpret_cast<const float*>(out)[idx];
+                                const float v = (s[nt][r] + pre_bias[nt][r]) + pre_res[nt][r];
                                 reinterpret_cast<float*>(out)[idx] = v;
-                                a.xg[idx].bits = float_to_bf16(a.gamma[n] * v);
+                                a.xg[idx].bits = float_to_bf16(pre_gamma[nt][r] * v);
                                 sq += v * v;
                             }
                         }
@@ -1033,7 +1155,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int n = n0 + 16 * nt + 4 * (l >> 4) + r;
-                    if (n < N) epilogue_store(out, (size_t)m * N + n, s[nt][r], a.bias, n, a.accumulate);
+                    if (n >= N) continue;
+                    if constexpr (PRE) store_from_float(out + (size_t)m * N + n, (s[nt][r] + pre_bias[nt][r]) + pre_res[nt][r]);
+                    else epilogue_store(out, (size_t)m * N + n, s[nt][r], a.bias, n, a.accumulate);
                 }
         }
     }
@@ -1180,6 +1304,8 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
     if (accumulate && out_dtype != LI_F32) return LI_ERR_DTYPE;
     if (in_dtype == LI_F32) {
         if (out_dtype != LI_F32) return LI_ERR_DTYPE;
+        if (M <= F32_ROWS_MAX && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0)
+            return launch_f32_rows((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate, stream);
         dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
         if (grid.y > 65535) return LI_ERR_SIZE;
         gemm_f32_kernel<<<grid, 256, 0, stream>>>((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate);

@@ -321,13 +321,15 @@ int li_book_check(void* vb) {
 // want_off[i + 1] index `want`.  pad_blocks (null or [ngroups]) widens the tables.
 // offsets [12 + 2 * ngroups] receives where each array starts; info receives
 //   {T, nwant, num_single, num_multi, num_tiles, max_q_len, max_ctx_len, max_single_ctx, widths...}.
+// tile_rows > 0: the tiles array is laid out, with tiles of that many tokens (0: none; the model's
+// parts say whether their kernels want it).  token_kinds != 0: the single and multi lists are.
 // With out == null nothing is written but offsets, info and the return value (the words needed).
 long li_book_build_batch(void* vb, int nseg, const int64_t* handles, const int* q_len, const int* ids, const int* id_src,
-                         const int* want_off, const int* want, const int* pad_blocks, int tile_rows,
+                         const int* want_off, const int* want, const int* pad_blocks, int tile_rows, int token_kinds,
                          int32_t* out, long out_cap, long* offsets, int* info) {
     Book* b = (Book*)vb;
     const int G = (int)b->pools.size(), P = b->page_size;
-    if (nseg <= 0 || tile_rows <= 0) return b->fail(ERR_ARG, "step: empty batch");
+    if (nseg <= 0 || tile_rows < 0) return b->fail(ERR_ARG, "step: empty batch");
     std::vector<Request*> reqs(nseg);
     long T = 0;
     int ntiles = 0, max_q = 0, max_ctx = 0, max_single_ctx = 0, nsingle = 0;
@@ -340,7 +342,7 @@ long li_book_build_batch(void* vb, int nseg, const int64_t* handles, const int* 
         max_q = std::max(max_q, q_len[i]);
         max_ctx = std::max(max_ctx, ctx);
         if (q_len[i] == 1) { ++nsingle; max_single_ctx = std::max(max_single_ctx, ctx); }
-        else ntiles += (q_len[i] + tile_rows - 1) / tile_rows;
+        else if (tile_rows > 0) ntiles += (q_len[i] + tile_rows - 1) / tile_rows;
     }
     const int nwant = want_off[nseg];
     std::vector<int> widths(G);
@@ -351,7 +353,8 @@ long li_book_build_batch(void* vb, int nseg, const int64_t* handles, const int* 
         widths[g] = w;
     }
     long o = 0;
-    const long sizes[12] = {T, T, T, nseg, nseg, nseg, nseg, nwant, T, T, (long)ntiles * 4, T};
+    const long kinds = token_kinds ? T : 0;
+    const long sizes[12] = {T, T, T, nseg, nseg, nseg, nseg, nwant, kinds, kinds, (long)ntiles * 4, T};
     for (int k = 0; k < 12; ++k) { offsets[k] = o; o += align4(sizes[k]); }
     for (int g = 0; g < G; ++g) {
         offsets[12 + 2 * g] = o; o += align4((long)nseg * widths[g]);
@@ -385,7 +388,7 @@ long li_book_build_batch(void* vb, int nseg, const int64_t* handles, const int* 
             if (want[w] < 0 || want[w] >= q_len[i]) return b->fail(ERR_ARG, "step: a wanted place is outside the entry's tokens");
             d_want[nw++] = t + want[w];
         }
-        if (q_len[i] > 1)
+        if (q_len[i] > 1 && tile_rows > 0)
             for (int a = 0; a < q_len[i]; a += tile_rows) {
                 d_tiles[4 * nt] = i; d_tiles[4 * nt + 1] = t + a;
                 d_tiles[4 * nt + 2] = std::min(tile_rows, q_len[i] - a); d_tiles[4 * nt + 3] = 0;
@@ -394,7 +397,8 @@ long li_book_build_batch(void* vb, int nseg, const int64_t* handles, const int* 
         for (int j = 0; j < q_len[i]; ++j, ++t) {
             d_pos[t] = r->cached + j;
             d_seg[t] = i;
-            if (q_len[i] == 1) d_single[ns++] = t; else d_multi[nm++] = t;
+            if (q_len[i] == 1) { if (token_kinds) d_single[ns] = t; ++ns; }
+            else { if (token_kinds) d_multi[nm] = t; ++nm; }
         }
     }
     info[2] = ns; info[3] = nm;

@@ -19,8 +19,6 @@ import torch
 from ..cache import native
 from ..utils.pinned import BatchUploader
 
-TILE_ROWS = 32      # tokens of one segment that the attention kernel for portions takes as a tile
-
 
 @dataclass
 class StepEntry:
@@ -50,16 +48,18 @@ class AttentionMeta:
     host_q_start: np.ndarray
     host_q_len: np.ndarray
     host_ctx_len: np.ndarray
+    # What follows is laid out only when a part of the model asks for it (`Part.batch_needs`).
     # tokens of segments that bring ONE token (decoding) and the other tokens, as lists of token
     # numbers; None when all tokens of the batch are of that kind (then no list is needed)
     single_tokens: Optional[torch.Tensor] = None
     num_single: int = 0
     multi_tokens: Optional[torch.Tensor] = None
     num_multi: int = 0
-    # the tokens of segments with several tokens, cut into tiles of up to 32 consecutive tokens
-    # of one segment: int32 [tiles, 4] = (segment, first token, tokens, 0)
+    # the tokens of segments with several tokens, cut into tiles of up to `tile_rows` consecutive
+    # tokens of one segment: int32 [tiles, 4] = (segment, first token, tokens, 0)
     tiles: Optional[torch.Tensor] = None
     num_tiles: int = 0
+    tile_rows: int = 0
     max_single_ctx: int = 0
     extra: Dict[Any, Any] = field(default_factory=dict)    # what kernels derive and keep for the step
 
@@ -103,12 +103,15 @@ class StepContext:
 
 
 def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploader",
-                  pad_blocks: Optional[Sequence[int]] = None, feedback: Optional[torch.Tensor] = None) -> StepContext:
+                  pad_blocks: Optional[Sequence[int]] = None, feedback: Optional[torch.Tensor] = None,
+                  needs=None) -> StepContext:
     """Lay out the step's integers (see the module text) for the given entries
     against the cache's current tables, upload them, and return the context.
     Pages for the entries' tokens must have been reserved.  `pad_blocks` gives,
     per page group, a width to pad the block tables to (for steps that are
     replayed from a recorded graph, whose array shapes must not change).
+    `needs` (a `parts.BatchNeeds`) says which further index arrays the model's parts
+    want: tiles of some number of tokens, the lists of single and multi tokens.
     The arrays are filled by the host library straight into the pinned buffer
     (csrc/host.cpp, li_book_build_batch)."""
     lib = native.lib()
@@ -127,6 +130,8 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     np.cumsum([len(e.want) for e in entries], out=want_off[1:])
     want = np.fromiter((int(w) for e in entries for w in e.want), dtype=np.int32, count=int(want_off[-1]))
     pad = None if pad_blocks is None else np.asarray(pad_blocks, dtype=np.int32)
+    tile_rows = int(needs.tile_rows) if needs is not None else 0
+    token_kinds = bool(needs.token_kinds) if needs is not None else False
     offsets = np.zeros(12 + 2 * ng, dtype=np.int64)
     info = np.zeros(8 + max(ng, 1), dtype=np.int32)
 
@@ -135,7 +140,7 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
 
     def call(out_ptr, cap):
         n = lib.li_book_build_batch(cache.book, nseg, ptr(handles), ptr(q_len), ptr(ids), ptr(id_src),
-                                    ptr(want_off), ptr(want), ptr(pad), TILE_ROWS, out_ptr, cap,
+                                    ptr(want_off), ptr(want), ptr(pad), tile_rows, int(token_kinds), out_ptr, cap,
                                     ptr(offsets), ptr(info))
         if n < 0:
             raise AssertionError(cache._error())
@@ -157,7 +162,9 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     ctx.ids, ctx.positions = d(0, T), d(1, T)
     d_seg, d_qs, d_ql, d_cl = d(2, T), d(3, nseg), d(4, nseg), d(5, nseg)
     ctx.state_slots, ctx.want_rows = d(6, nseg), d(7, nwant)
-    d_single, d_multi, d_tiles = d(8, nsingle), d(9, nmulti), d(10, ntiles * 4, (ntiles, 4))
+    d_single = d(8, nsingle) if token_kinds else None
+    d_multi = d(9, nmulti) if token_kinds else None
+    d_tiles = d(10, ntiles * 4, (ntiles, 4)) if tile_rows else None
     ctx.id_src = d(11, T) if feedback is not None else None
     ctx.feedback = feedback
     ctx.num_want = nwant
@@ -174,7 +181,7 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
             host_q_start=ctx.host_q_start, host_q_len=ctx.host_q_len, host_ctx_len=ctx.host_ctx_len,
             single_tokens=d_single if nmulti else None, num_single=nsingle,
             multi_tokens=d_multi if nsingle else None, num_multi=nmulti,
-            tiles=d_tiles, num_tiles=ntiles,
+            tiles=d_tiles, num_tiles=ntiles, tile_rows=tile_rows,
             # with padded tables the split count must not follow the context either
             max_single_ctx=(mb * P if pad_blocks is not None else max_single_ctx)))
     return ctx

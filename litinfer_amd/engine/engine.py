@@ -117,10 +117,9 @@ class Engine:
 
     def _bytes_per_page(self) -> int:
         needs, sources = self.model.cache_needs()
-        from ..parts.base import PagedKVNeed
-        es = 4 if self.rt.dtype is torch.float32 else 2
-        return sum(2 * n.num_kv_heads * n.head_dim * self.page_size * es
-                   for n, s in zip(needs, sources) if s is None and isinstance(n, PagedKVNeed))
+        from ..parts.base import PagedNeed
+        return sum(n.bytes_per_token(self.rt.dtype) * self.page_size
+                   for n, s in zip(needs, sources) if s is None and isinstance(n, PagedNeed))
 
     def _make_cache(self) -> None:
         needs, sources = self.model.cache_needs()
@@ -236,7 +235,8 @@ class Engine:
             self.cache.release(rid)
 
     def _build_context(self, entries: Sequence[StepEntry], pad_blocks=None) -> StepContext:
-        return build_context(self.cache, entries, self.ws, self._uploader, pad_blocks, self.feedback)
+        return build_context(self.cache, entries, self.ws, self._uploader, pad_blocks, self.feedback,
+                             needs=self.model.batch_needs())
 
     # ---- recorded decode steps ----------------------------------------------
     def _graph_key(self, entries: Sequence[StepEntry]):

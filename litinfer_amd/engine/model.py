@@ -23,6 +23,7 @@ class Model:
         self.final_norm = build_part("norm", spec.final_norm, rt)
         self.head = build_part("head", spec.head, rt)
         self.order = list(spec.order)
+        self._batch_needs = None
 
     # ---- weights ----------------------------------------------------------
     def expected_params(self) -> Dict[str, ParamSpec]:
@@ -53,6 +54,16 @@ class Model:
                 elif hasattr(v, "__dict__") and not isinstance(v, (Runtime, ModelSpec, PartSpec, type)):
                     stack.append(v)
         return total
+
+    def batch_needs(self):
+        """The index arrays that the parts' kernels want laid out with every step's batch."""
+        if self._batch_needs is None:
+            from ..parts.base import BatchNeeds
+            needs = BatchNeeds()
+            for p in (self.embedding, *self.layers, self.final_norm, self.head):
+                needs = needs.merged(p.batch_needs())
+            self._batch_needs = needs
+        return self._batch_needs
 
     @property
     def graph_safe(self) -> bool:

@@ -487,6 +487,7 @@ def linear_rope_store(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Ten
 
 
 # ----------------------------------------------------------------- attention
+PREFILL_TILE_ROWS = 32       # queries of one segment that a block of the matrix-core kernel for portions takes
 DECODE_MAX_SPLITS = 64       # the merge kernel keeps a weight per split
 DECODE_TABLE_CAP = 1024      # pages of one split that the matrix-core decode kernel copies into LDS
 
@@ -531,6 +532,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
          and bt.is_contiguous(), "attention: block table")
     _chk(meta.max_blocks * page_size >= meta.max_ctx_len, "attention: block table too short")
     _chk(meta.num_single + meta.num_multi == t, "attention: token lists do not cover the batch")
+    _chk(meta.num_single in (0, t) or (meta.single_tokens is not None and meta.multi_tokens is not None),
+         "attention: a batch of single-token and longer segments needs their token lists (BatchNeeds.token_kinds)")
     if not t:
         return
     n_single, n_multi = meta.num_single, meta.num_multi
@@ -569,7 +572,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
     # the matrix-core kernel for portions keeps a tile's pages in LDS (8192 entries) and divides
     # positions by the page size in float, exact below 2^21 keys; longer tables take the general kernel
     if (n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles
-            and n_multi == meta.num_multi and meta.max_blocks <= 8192 and meta.max_blocks * page_size <= 1 << 21):
+            and meta.tile_rows == PREFILL_TILE_ROWS and n_multi == meta.num_multi and meta.max_blocks <= 8192 and meta.max_blocks * page_size <= 1 << 21):
         _run("attention", "li_paged_attention_prefill", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), bt.data_ptr(), meta.max_blocks, meta.tiles.data_ptr(),
              meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),

@@ -1,5 +1,5 @@
-from .base import (Block, FeedForward, Mixer, Norm, PagedKVNeed, Part, Runtime, StateNeed,
-                   build_part, register_part)
+from .base import (BatchNeeds, Block, FeedForward, Mixer, Norm, PagedKVNeed, PagedNeed, PagedTensor, Part,
+                   Runtime, StateNeed, build_part, register_part)
 from .position import Position, RopeNeox
 from .linear import Linear
 from .stream import ResidualStream
@@ -9,6 +9,7 @@ from .mlp import SwiGLUMLP
 from .block import PreNormBlock
 from .embedding import LinearHead, TokenEmbedding
 
-__all__ = ["Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "Part", "Runtime", "StateNeed",
+__all__ = ["BatchNeeds", "Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "PagedNeed", "PagedTensor",
+           "Part", "Runtime", "StateNeed",
            "build_part", "register_part", "Position", "RopeNeox", "Linear", "ResidualStream", "RMSNorm",
            "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding"]

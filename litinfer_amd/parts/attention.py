@@ -17,7 +17,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import ParamSpec
-from .base import Mixer, PagedKVNeed, build_part, register_part
+from .base import BatchNeeds, Mixer, PagedKVNeed, build_part, register_part
 from .linear import Linear
 
 
@@ -49,6 +49,10 @@ class GQAttention(Mixer):
 
     def cache_need(self):
         return PagedKVNeed(self.nkv, self.dh, self.window)
+
+    def batch_needs(self):
+        # the kernels take single-token segments (split keys) and the others (tiles of queries) apart
+        return BatchNeeds(tile_rows=ops.PREFILL_TILE_ROWS, token_kinds=True)
 
     def expected_params(self):
         p = self.prefix

@@ -9,7 +9,8 @@ here.
 Interfaces (T = tokens of the step, H = hidden size):
 
 * Norm.forward(x [T, H] float32, out) -> out [T, H] in the activation dtype.
-* Mixer.cache_need() -> PagedKVNeed | StateNeed | None;
+* Mixer.cache_need() -> PagedNeed (named tensors per token, in pages; PagedKVNeed(...)
+  builds the usual keys and values) | StateNeed | None;
   Mixer.forward(xn [T, H], residual, ctx, cache): ADDS its output to the
   residual stream in 32-bit.  `residual` is a `ResidualStream`
   (parts/stream.py): `residual.add_linear(linear, h)` adds h W^T + b, and
@@ -56,12 +57,59 @@ class Runtime:
 
 
 @dataclass(frozen=True)
-class PagedKVNeed:
-    """Keys and values of every token in pages; `window` > 0 keeps only the
-    last `window` positions visible (older pages are given back)."""
-    num_kv_heads: int
-    head_dim: int
+class PagedTensor:
+    """One tensor that a mixer keeps for every token of a request, in pages: `shape` is
+    what one token holds, e.g. (kv_heads, head_dim) for keys or (latent,) for a compressed
+    cache; `dtype` None means the engine's activation dtype.  A page of it is laid out as
+    [*shape[:-1], page_size, shape[-1]]: the rows of one head lie together."""
+    name: str
+    shape: Tuple[int, ...]
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        return (*self.shape[:-1], page_size, self.shape[-1])
+
+
+@dataclass(frozen=True)
+class PagedNeed:
+    """What a mixer keeps per token in pages: any number of named tensors of any shapes;
+    `window` > 0 keeps only the last `window` positions visible (older pages are given
+    back).  Entries of the execution order with equal needs share a page group: one page
+    id and one block table per request serve all of them."""
+    tensors: Tuple[PagedTensor, ...]
     window: int = 0
+
+    def bytes_per_token(self, default_dtype: torch.dtype) -> int:
+        total = 0
+        for t in self.tensors:
+            n = 1
+            for s in t.shape:
+                n *= int(s)
+            total += n * torch.empty((), dtype=t.dtype or default_dtype).element_size()
+        return total
+
+
+def PagedKVNeed(num_kv_heads: int, head_dim: int, window: int = 0) -> PagedNeed:
+    """Keys and values of equal shape (kv_heads, head_dim), named "k" and "v": what the
+    attention of the reference keeps (src/llaisys/kv_cache/block_kv_cache.hpp:16-63)."""
+    shape = (int(num_kv_heads), int(head_dim))
+    return PagedNeed((PagedTensor("k", shape), PagedTensor("v", shape)), int(window))
+
+
+@dataclass(frozen=True)
+class BatchNeeds:
+    """Index arrays, beyond the basic ones, that a part's kernels want laid out with a
+    step's batch (they travel in the step's one upload).  `tile_rows` > 0: the tokens of
+    segments with several tokens cut into tiles of up to that many consecutive tokens of one
+    segment; `token_kinds`: the lists of tokens of single-token segments and of the others."""
+    tile_rows: int = 0
+    token_kinds: bool = False
+
+    def merged(self, other: "BatchNeeds") -> "BatchNeeds":
+        if self.tile_rows and other.tile_rows and self.tile_rows != other.tile_rows:
+            raise ValueError(f"parts ask for tiles of {self.tile_rows} and of {other.tile_rows} tokens; "
+                             f"a step's batch is laid out with one tile size")
+        return BatchNeeds(self.tile_rows or other.tile_rows, self.token_kinds or other.token_kinds)
 
 
 @dataclass(frozen=True)
@@ -86,6 +134,11 @@ class Part:
     def expected_params(self) -> Dict[str, ParamSpec]:
         """Full tensor name -> ParamSpec."""
         return {}
+
+    def batch_needs(self) -> BatchNeeds:
+        """What this part's kernels want laid out with a step's batch beyond ids, positions,
+        segments, block tables and page slots (nothing, for most parts)."""
+        return BatchNeeds()
 
     def load_params(self, get: Callable[[str], Optional[torch.Tensor]]) -> None:
         """`get(name)` returns the stored tensor on the CPU, or None when an

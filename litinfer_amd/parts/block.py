@@ -23,6 +23,12 @@ class PreNormBlock(Block):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    def batch_needs(self):
+        needs = super().batch_needs()
+        for p in self._all:
+            needs = needs.merged(p.batch_needs())
+        return needs
+
     def expected_params(self):
         e = {}
         for p in self._all:

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from litinfer_amd.cache import CacheFull, CacheManager, PagePool, PagePoolError
-from litinfer_amd.parts import PagedKVNeed, StateNeed
+from litinfer_amd.parts import PagedKVNeed, PagedNeed, PagedTensor, StateNeed
 
 
 def test_pool_guards():
@@ -35,13 +35,39 @@ def _manager(num_pages=12, page=4, window=0, max_seqs=3, seed=None):
 def test_groups_by_need_and_views():
     m = _manager(window=6)
     assert len(m.groups) == 2 and m.groups[0].entries == [0] and m.groups[1].entries == [1, 2]
-    assert m.groups[1].data.shape == (2, 2, 12, 2, 4, 8)
+    assert set(m.groups[1].data) == {"k", "v"} and m.groups[1].data["k"].shape == (2, 12, 2, 4, 8)
     v = m.view(2)
     assert v.owned and v.group == 1 and v.k.shape == (12, 2, 4, 8)
-    assert v.k.data_ptr() == m.groups[1].data[1, 0].data_ptr()
+    assert v.k.data_ptr() == m.groups[1].data["k"][1].data_ptr()
     assert m.view(3).group is None
     one = _manager(window=0)
     assert len(one.groups) == 1 and one.groups[0].entries == [0, 1, 2]
+
+
+def test_pages_of_any_named_tensors_group_by_their_need():
+    """A need is a list of named tensors per token: keys alone, a latent of another dtype
+    beside a small vector, keys and values of unequal head sizes."""
+    latent = PagedNeed((PagedTensor("c", (24,), torch.float32), PagedTensor("pe", (2, 6))), window=0)
+    uneven = PagedNeed((PagedTensor("k", (2, 16)), PagedTensor("v", (2, 8))), window=5)
+    needs = [latent, PagedKVNeed(2, 8, 0), uneven, latent, PagedKVNeed(2, 8, 0)]
+    m = CacheManager(needs, [None] * 5, page_size=4, num_pages=6, max_seqs=2, dtype=torch.bfloat16, device="cpu")
+    assert [g.entries for g in m.groups] == [[0, 3], [1, 4], [2]]
+    assert m.groups[0].data["c"].shape == (2, 6, 4, 24) and m.groups[0].data["c"].dtype is torch.float32
+    assert m.groups[0].data["pe"].shape == (2, 6, 2, 4, 6) and m.groups[0].data["pe"].dtype is torch.bfloat16
+    assert m.groups[2].data["k"].shape == (1, 6, 2, 4, 16) and m.groups[2].data["v"].shape == (1, 6, 2, 4, 8)
+    v = m.view(3)
+    assert set(v.tensors) == {"c", "pe"} and v.tensors["c"].shape == (6, 4, 24)
+    assert latent.bytes_per_token(torch.bfloat16) == 24 * 4 + 12 * 2
+    m.admit("a")
+    m.reserve("a", 9)
+    m.commit("a", 9)
+    assert m.free_pages() == [3, 3, 4]                 # the windowed group has given its first page back
+    m.check_invariants()
+    with pytest.raises(ValueError, match="distinct names"):
+        CacheManager([PagedNeed((PagedTensor("k", (2,)), PagedTensor("k", (2,))))], [None], page_size=4,
+                     num_pages=2, max_seqs=1, dtype=torch.float32, device="cpu")
+    with pytest.raises(TypeError):
+        CacheManager(["pages please"], [None], page_size=4, num_pages=2, max_seqs=1, dtype=torch.float32, device="cpu")
 
 
 def test_shared_cache_view_is_the_owners():

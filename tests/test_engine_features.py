@@ -16,7 +16,8 @@ from litinfer_amd.config import ExecEntry, LayerSpec, ModelSpec, PartSpec, Qwen2
 from litinfer_amd.engine import Engine, StepEntry, StepError
 from litinfer_amd.engine.batch import BatchUploader, build_context
 from litinfer_amd.engine.workspace import Workspace
-from litinfer_amd.parts import FeedForward, Mixer, Position, ResidualStream, Runtime, StateNeed, build_part, register_part
+from litinfer_amd.parts import (BatchNeeds, FeedForward, Mixer, PagedNeed, PagedTensor, Position, ResidualStream, Runtime,
+                                StateNeed, build_part, register_part)
 from litinfer_amd.weights import ParamSpec
 from tiny_configs import TINY_A, TINY_B, TINY_C
 from toy_parts import ToyConfig
@@ -379,6 +380,92 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, device
         out = schedules.run(eng, reqs, getattr(schedules, kind)(reqs))
         assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind   # slots reused, state zeroed
     eng.cache.check_invariants()
+
+
+# ------------- a toy mixer with a cache of its own shape: one latent vector per token, in pages
+class ToyLatentAttention(Mixer):
+    """One head over a compressed cache: c_t = xn_t Wc (a latent of `rank` numbers, kept in
+    pages as float32 under the name "c"), score(t, s) = (xn_t Wq) . c_s / sqrt(rank) for
+    s <= t, y_t = softmax(score) c, output y_t Wo.  Neither keys nor values are stored.
+    Written with torch: it is a toy that shows the interface, not a kernel."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.h, self.rank = spec.args["hidden_size"], spec.args["rank"]
+
+    def cache_need(self):
+        return PagedNeed((PagedTensor("c", (self.rank,), torch.float32),))
+
+    def expected_params(self):
+        p = self.prefix
+        return {p + "wc": ParamSpec((self.rank, self.h)), p + "wq": ParamSpec((self.rank, self.h)),
+                p + "wo": ParamSpec((self.h, self.rank))}
+
+    def load_params(self, get):
+        self.wc, self.wq, self.wo = (get(self.prefix + n).to(torch.float32).to(self.rt.device) for n in ("wc", "wq", "wo"))
+
+    def forward(self, xn, residual, ctx, cache):
+        x = xn.float()
+        pages = cache.tensors["c"]                                     # [pages, page_size, rank]
+        flat = pages.view(-1, self.rank)
+        flat[ctx.slot_map(cache.group).long()] = x @ self.wc.T         # written before it is read, like keys
+        q = x @ self.wq.T
+        table = ctx.attention_meta(cache.group).block_table.cpu()
+        out = residual.tensor()
+        for s in range(ctx.num_segments):
+            q0, n, have = int(ctx.host_q_start[s]), int(ctx.host_q_len[s]), int(ctx.host_ctx_len[s])
+            blocks = table[s, :-(-have // cache.page_size)].long().to(pages.device)
+            c = pages[blocks].reshape(-1, self.rank)[:have]            # the request's latents in order
+            score = q[q0:q0 + n] @ c.T / math.sqrt(self.rank)
+            pos = torch.arange(have - n, have, device=score.device)[:, None]
+            score = score.masked_fill(torch.arange(have, device=score.device)[None, :] > pos, float("-inf"))
+            out[q0:q0 + n] += torch.softmax(score, dim=-1) @ c @ self.wo.T
+
+
+def _latent_spec(c: ToyConfig) -> ModelSpec:
+    base = qwen2_model_spec(c.inner)
+    layers = tuple(LayerSpec("prenorm", dict(l.parts, mixer=PartSpec("toy_latent", f"model.layers.{i}.lat.",
+                                                                     {"hidden_size": c.hidden_size, "rank": 12})))
+                   for i, l in enumerate(base.layers))
+    return replace(base, architecture="ToyLatentLM", layers=layers)
+
+
+def test_a_toy_mixer_keeps_one_latent_vector_per_token_in_pages(tmp_path, device):
+    register_part("mixer", "toy_latent", ToyLatentAttention)
+    register_architecture("ToyLatentLM", ToyConfig.from_dict, _latent_spec)
+    cfg = dict(TINY_A, architectures=["ToyLatentLM"], toy_decay=0.0)
+    d = helpers.make_model(tmp_path, cfg, 12)
+    pcfg, w = P.load_folder(d)
+
+    def plain(ids):
+        x = P.embedding(ids, w["model.embed_tokens.weight"])
+        for l in range(2):
+            p = f"model.layers.{l}."
+            xn = P.rms_norm(x, w[p + "input_layernorm.weight"], 1e-6)
+            c, q = xn @ w[p + "lat.wc"].T, xn @ w[p + "lat.wq"].T
+            score = q @ c.T / math.sqrt(12)
+            score[np.triu_indices(len(ids), 1)] = -np.inf
+            e = np.exp(score - score.max(-1, keepdims=True))
+            x = x + (e / e.sum(-1, keepdims=True)) @ c @ w[p + "lat.wo"].T
+            xn = P.rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-6)
+            x = x + P.swiglu(xn @ w[p + "mlp.gate_proj.weight"].T, xn @ w[p + "mlp.up_proj.weight"].T) @ w[p + "mlp.down_proj.weight"].T
+        return P.rms_norm(x, w["model.norm.weight"], 1e-6) @ w["model.embed_tokens.weight"].T
+
+    reqs = helpers.random_requests(256, [33, 18, 5, 26, 47], 9)
+    ref = {r: plain(np.asarray(t)) for r, t in reqs.items()}
+    for kind in ("whole", "tail", "chunks", "mixed"):
+        steps = getattr(schedules, kind)(reqs)
+        eng = engine_for(d, device, page=8, max_tokens=schedules.max_live_tokens(reqs, steps, 8 if kind == "mixed" else 64),
+                         page_order_seed=4)
+        g = eng.cache.groups
+        assert len(g) == 1 and set(g[0].data) == {"c"} and g[0].data["c"].shape[2:] == (8, 12)
+        assert g[0].data["c"].dtype is torch.float32 and g[0].entries == [0, 1]
+        assert eng.model.batch_needs() == BatchNeeds()         # nobody here wants tiles or token lists laid out
+        out = schedules.run(eng, reqs, steps)
+        assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind
+        eng.cache.check_invariants()
+    # the architecture's own model does ask for them, through its attention
+    assert engine_for(helpers.make_model(tmp_path / "a", TINY_A, 0), device).model.batch_needs() == BatchNeeds(32, True)
 
 
 # --------- a toy feed-forward with routing and a toy position encoding, defined here

@@ -70,7 +70,9 @@ def test_rmsnorm_zero_row_is_zero_not_nan(ops):
     ((70, 200, 96), False, True), ((130, 129, 264), True, True), ((512, 512, 1024), True, False),
     ((64, 3584, 3584), False, False), ((3, 37, 90), True, False), ((257, 64, 36), False, False),
     ((17, 37, 264), True, True), ((33, 130, 1160), False, False), ((48, 16, 8), True, False),
-    ((8, 4608, 3584), True, False), ((65, 50, 128), False, True)])
+    ((8, 4608, 3584), True, False), ((65, 50, 128), False, True),
+    ((1, 1000, 3584), True, False), ((16, 70, 260), True, True), ((40, 19, 100), False, True),      # few rows in 32-bit
+    ((9, 18, 4), True, False)])
 def test_linear(ops, dtype, mnk, bias, acc):
     m, n, k = mnk
     g = torch.Generator().manual_seed(2)
@@ -410,7 +412,7 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
                          tiles=dev(np.asarray([(i, int(q_start[i]) + a, min(32, int(q_len[i]) - a), 0)
                                                for i in range(nseg) if q_len[i] > 1
                                                for a in range(0, int(q_len[i]), 32)], dtype=np.int32).reshape(-1, 4)),
-                         num_tiles=sum(-(-int(n) // 32) for n in q_len if n > 1),
+                         num_tiles=sum(-(-int(n) // 32) for n in q_len if n > 1), tile_rows=32,
                          max_single_ctx=int(ctx_len[q_len == 1].max()) if len(single) else 0)
     out = torch.empty(T, nh * dh, dtype=dtype, device=DEV)
     scale = 1.0 / math.sqrt(dh)
