@@ -124,12 +124,27 @@ def test_argmax_takes_the_first_maximum():
 
 
 def _tiny_weights(cfg, seed, dtype=np.float64):
-    from litinfer_amd.config import Qwen2Config, qwen2_model_spec
-    from litinfer_amd.engine import expected_params_of_spec
+    """Random tensors under the names of the reference's checkpoint table
+    (python/llaisys/models/qwen2.py:139-194), written out here: the tests of the plain
+    implementation take nothing from the product package."""
     rng = np.random.default_rng(seed)
+    h, nh, inter, voc = cfg["hidden_size"], cfg["num_attention_heads"], cfg["intermediate_size"], cfg["vocab_size"]
+    nkv = cfg.get("num_key_value_heads", nh)
+    dh = cfg.get("head_dim") or h // nh
+    shapes = {"model.embed_tokens.weight": (voc, h), "model.norm.weight": (h,)}
+    if not cfg.get("tie_word_embeddings", False):
+        shapes["lm_head.weight"] = (voc, h)
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        shapes.update({p + "input_layernorm.weight": (h,), p + "post_attention_layernorm.weight": (h,),
+                       p + "self_attn.q_proj.weight": (nh * dh, h), p + "self_attn.q_proj.bias": (nh * dh,),
+                       p + "self_attn.k_proj.weight": (nkv * dh, h), p + "self_attn.k_proj.bias": (nkv * dh,),
+                       p + "self_attn.v_proj.weight": (nkv * dh, h), p + "self_attn.v_proj.bias": (nkv * dh,),
+                       p + "self_attn.o_proj.weight": (h, nh * dh), p + "mlp.gate_proj.weight": (inter, h),
+                       p + "mlp.up_proj.weight": (inter, h), p + "mlp.down_proj.weight": (h, inter)})
     out = {}
-    for name, ps in expected_params_of_spec(qwen2_model_spec(Qwen2Config.from_dict(cfg))).items():
-        a = rng.standard_normal(ps.shape) * 0.05
+    for name, shape in shapes.items():
+        a = rng.standard_normal(shape) * 0.05
         out[name] = (a + 1 if name.endswith("norm.weight") else a).astype(dtype)
     return out
 
@@ -158,6 +173,57 @@ def test_model_closed_forms():
             g, u = xn @ w[p + "mlp.gate_proj.weight"].T, xn @ w[p + "mlp.up_proj.weight"].T
             x = x + P.swiglu(g, u) @ w[p + "mlp.down_proj.weight"].T
         assert np.allclose(P.forward(cfg, w, [7]), P.rms_norm(x, w["model.norm.weight"], eps) @ head.T)
+
+
+def test_attention_layer_in_closed_form_with_complex_rotations():
+    """A layer whose query and key matrices are zero, so that q and k are their BIASES at every
+    token, and whose feed-forward adds nothing: the scores then follow from the biases and the
+    distance alone.  Written out independently of this file's functions, the pair (j, j + dh/2) of a
+    head as one complex number z_j that the position p turns by exp(i p theta^(-2j/dh)):
+    score(p, t) = Re sum_j q_j conj(k_j) exp(i (p - t) angle_j) / sqrt(dh).  It fails if the biases
+    are left out or added after the rotation, if the rotation's sign or pairing is another, if the
+    scale is 1 / sqrt(hidden / heads) (the sizes differ here), if query head h reads kv head h % 2
+    instead of h // 2, or if the blocks' norms stand elsewhere (src/llaisys/models/qwen2.cpp:613-629,
+    :690; src/ops/rope/op.cpp:13-20; src/ops/paged_attention/op.cpp:20-42)."""
+    cfg = {"num_hidden_layers": 1, "hidden_size": 20, "num_attention_heads": 4, "num_key_value_heads": 2,
+           "head_dim": 6, "intermediate_size": 8, "vocab_size": 11, "rope_theta": 100.0, "rms_norm_eps": 1e-5,
+           "tie_word_embeddings": True, "max_position_embeddings": 64}
+    w = _tiny_weights(cfg, 5)
+    pre = "model.layers.0."
+    for n in ("q_proj.weight", "k_proj.weight"):
+        w[pre + "self_attn." + n][:] = 0
+    for n in ("q_proj.bias", "k_proj.bias", "v_proj.bias"):
+        w[pre + "self_attn." + n] = RNG.standard_normal(w[pre + "self_attn." + n].shape)
+    w[pre + "mlp.down_proj.weight"][:] = 0
+    ids = [3, 9, 4, 4, 1]
+    nh, nkv, dh, half = 4, 2, 6, 3
+    E, eps = w["model.embed_tokens.weight"], cfg["rms_norm_eps"]
+    x = E[ids]
+    xn = w[pre + "input_layernorm.weight"] * x / np.sqrt((x * x).mean(-1, keepdims=True) + eps)
+    v = (xn @ w[pre + "self_attn.v_proj.weight"].T + w[pre + "self_attn.v_proj.bias"]).reshape(len(ids), nkv, dh)
+    bq = w[pre + "self_attn.q_proj.bias"].reshape(nh, dh)
+    bk = w[pre + "self_attn.k_proj.bias"].reshape(nkv, dh)
+    zq, zk = bq[:, :half] + 1j * bq[:, half:], bk[:, :half] + 1j * bk[:, half:]
+    angle = 100.0 ** (-2.0 * np.arange(half) / dh)
+
+    def logits(kv_of_head):
+        attn = np.zeros((len(ids), nh, dh))
+        for h in range(nh):
+            kh = kv_of_head(h)
+            for p in range(len(ids)):
+                s = np.array([(zq[h] * np.conj(zk[kh]) * np.exp(1j * (p - t) * angle)).real.sum() / math.sqrt(dh)
+                              for t in range(p + 1)])
+                pr = np.exp(s - s.max())
+                attn[p, h] = (pr / pr.sum()) @ v[:p + 1, kh]
+        y = x + attn.reshape(len(ids), nh * dh) @ w[pre + "self_attn.o_proj.weight"].T
+        return w["model.norm.weight"] * y / np.sqrt((y * y).mean(-1, keepdims=True) + eps) @ E.T
+
+    got = P.forward(cfg, w, ids)
+    assert np.allclose(got, logits(lambda h: h // 2), atol=1e-12)
+    assert not np.allclose(got, logits(lambda h: h % 2), atol=1e-6)          # interleaved heads would show
+    no_bias = dict(w)
+    no_bias[pre + "self_attn.q_proj.bias"] = np.zeros(nh * dh)
+    assert not np.allclose(P.forward(cfg, no_bias, ids), got, atol=1e-6)      # the biases do act
 
 
 def test_model_depends_on_distances_only():
