@@ -30,6 +30,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import ctypes
 
+import numpy as np
 import torch
 
 from ..parts.base import PagedNeed, StateNeed
@@ -218,6 +219,47 @@ class CacheManager:
         (rid may be unknown: then it is counted as a new request)."""
         h = self._handles.get(rid, -1)
         self._lib.li_book_pages_needed(self._book, h, int(n_new), -1 if cached is None else int(cached), self._ints)
+        return list(self._ints[:len(self.groups)])
+
+    # ---- whole batches in one call (the step function and the scheduler go through these) ----
+    def handles_of(self, rids, unknown: int = -1) -> "np.ndarray":
+        """int64 handles of the requests; `unknown` for one that is not live."""
+        get = self._handles.get
+        return np.fromiter((get(r, unknown) for r in rids), dtype=np.int64, count=len(rids))
+
+    def pages_needed_many(self, handles, n_new) -> "np.ndarray":
+        """[n, groups]: pages each request must take for its n_new[i] more tokens (a handle < 0
+        is counted as a new request)."""
+        n = len(handles)
+        out = np.zeros((n, max(len(self.groups), 1)), dtype=np.int32)
+        n_new = np.ascontiguousarray(n_new, dtype=np.int32)
+        self._lib.li_book_pages_needed_many(self._book, n, handles.ctypes.data, n_new.ctypes.data, out.ctypes.data)
+        return out[:, :len(self.groups)]
+
+    def reserve_many(self, handles, n_new) -> None:
+        """Pages for every request of the batch, or none at all (CacheFull)."""
+        n_new = np.ascontiguousarray(n_new, dtype=np.int32)
+        rc = self._lib.li_book_reserve_many(self._book, len(handles), handles.ctypes.data, n_new.ctypes.data)
+        if rc == native.ERR_FULL:
+            raise CacheFull(self._error())
+        if rc < 0:
+            raise PagePoolError(self._error())
+
+    def commit_many(self, handles, n_new) -> None:
+        n_new = np.ascontiguousarray(n_new, dtype=np.int32)
+        if self._lib.li_book_commit_many(self._book, len(handles), handles.ctypes.data, n_new.ctypes.data) < 0:
+            raise PagePoolError(self._error())
+
+    def cached_many(self, handles) -> "np.ndarray":
+        """Cached lengths (0 for a handle < 0, a request that is not live yet)."""
+        out = np.zeros(len(handles), dtype=np.int32)
+        self._lib.li_book_cached_many(self._book, len(handles), handles.ctypes.data, out.ctypes.data)
+        return np.maximum(out, 0)
+
+    def max_table_len(self, handles) -> List[int]:
+        """The longest block table among the requests, per group."""
+        if self._lib.li_book_max_table_len(self._book, len(handles), handles.ctypes.data, self._ints) < 0:
+            raise KeyError(self._error())
         return list(self._ints[:len(self.groups)])
 
     def reserve(self, rid, n_new: int) -> None:

@@ -34,6 +34,11 @@ def lib() -> ctypes.CDLL:
             "li_book_reserve": ([c_void_p, c_int64, c_int], c_int),
             "li_book_commit": ([c_void_p, c_int64, c_int], c_int),
             "li_book_rewind": ([c_void_p, c_int64, c_int], c_int),
+            "li_book_pages_needed_many": ([c_void_p, c_int, c_void_p, c_void_p, c_void_p], c_int),
+            "li_book_reserve_many": ([c_void_p, c_int, c_void_p, c_void_p], c_int),
+            "li_book_max_table_len": ([c_void_p, c_int, c_void_p, c_void_p], c_int),
+            "li_book_cached_many": ([c_void_p, c_int, c_void_p, c_void_p], c_int),
+            "li_book_commit_many": ([c_void_p, c_int, c_void_p, c_void_p], c_int),
             "li_book_release": ([c_void_p, c_int64], c_int), "li_book_check": ([c_void_p], c_int),
             "li_book_build_batch": ([c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p], c_long),

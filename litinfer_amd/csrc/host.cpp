@@ -229,6 +229,71 @@ int li_book_reserve(void* vb, int64_t h, int n_new) {
         }
     return 0;
 }
+// The same for a whole batch in one call (a step's entries): pages each of the n requests must take
+// for its n_new[i] more tokens, out [n * ngroups]; a handle < 0 counts as a new request.
+int li_book_pages_needed_many(void* vb, int n, const int64_t* handles, const int* n_new, int* out) {
+    Book* b = (Book*)vb;
+    const size_t G = b->pools.size();
+    for (int i = 0; i < n; ++i)
+        b->pages_needed(handles[i] >= 0 ? b->find(handles[i]) : nullptr, n_new[i], -1, out + (size_t)i * G);
+    return 0;
+}
+// All the pages that the batch needs, in every group, or none at all (ERR_FULL, nothing changed).
+int li_book_reserve_many(void* vb, int n, const int64_t* handles, const int* n_new) {
+    Book* b = (Book*)vb;
+    const size_t G = b->pools.size();
+    std::vector<int> need((size_t)n * G), total(G, 0);
+    for (int i = 0; i < n; ++i) {
+        Request* r = b->find(handles[i]);
+        if (!r) return b->fail(ERR_UNKNOWN, "cache: unknown request");
+        b->pages_needed(r, n_new[i], -1, need.data() + (size_t)i * G);
+        for (size_t g = 0; g < G; ++g) total[g] += need[(size_t)i * G + g];
+    }
+    for (size_t g = 0; g < G; ++g)
+        if (total[g] > b->pools[g].free_count())
+            return b->fail(ERR_FULL, "step: the batch needs " + std::to_string(total[g]) + " more pages, " +
+                                         std::to_string(b->pools[g].free_count()) + " of " +
+                                         std::to_string(b->pools[g].capacity) + " are free");
+    for (int i = 0; i < n; ++i) {
+        Request* r = b->find(handles[i]);
+        for (size_t g = 0; g < G; ++g)
+            for (int k = 0; k < need[(size_t)i * G + g]; ++k) {
+                const int p = b->pools[g].alloc();
+                if (p < 0) return b->fail(p, b->pools[g].error);
+                r->tables[g].push_back(p);
+            }
+    }
+    return 0;
+}
+// The longest block table of the batch in every group, out [ngroups].
+int li_book_max_table_len(void* vb, int n, const int64_t* handles, int* out) {
+    Book* b = (Book*)vb;
+    const size_t G = b->pools.size();
+    for (size_t g = 0; g < G; ++g) out[g] = 0;
+    for (int i = 0; i < n; ++i) {
+        Request* r = b->find(handles[i]);
+        if (!r) return b->fail(ERR_UNKNOWN, "cache: unknown request");
+        for (size_t g = 0; g < G; ++g) out[g] = std::max(out[g], (int)r->tables[g].size());
+    }
+    return 0;
+}
+// Cached lengths of the batch's requests, out [n] (-1 for a request that is not live).
+int li_book_cached_many(void* vb, int n, const int64_t* handles, int* out) {
+    Book* b = (Book*)vb;
+    for (int i = 0; i < n; ++i) {
+        Request* r = handles[i] >= 0 ? b->find(handles[i]) : nullptr;
+        out[i] = r ? r->cached : -1;
+    }
+    return 0;
+}
+int li_book_commit(void* vb, int64_t h, int n_new);
+int li_book_commit_many(void* vb, int n, const int64_t* handles, const int* n_new) {
+    for (int i = 0; i < n; ++i) {
+        const int rc = li_book_commit(vb, handles[i], n_new[i]);
+        if (rc < 0) return rc;
+    }
+    return 0;
+}
 // n_new tokens were written: advance, and give back the pages the window has passed
 int li_book_commit(void* vb, int64_t h, int n_new) {
     Book* b = (Book*)vb;

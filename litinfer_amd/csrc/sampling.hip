@@ -211,6 +211,80 @@ __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
         if (tid == 0) out[r] = i;
         return;
     }
+    {
+        // Temperature alone (no top-k, no top-p: every id survives), the common case: no thresholds
+        // to search for and no ties to count, so the row is read three times in whole lines.
+        // Ids are taken in tiles of SMP_NT * 8: thread t holds the 8 consecutive ids t * 8 .. of a
+        // tile.  The inverse CDF runs over ascending ids: tile by tile (sums of whole tiles, each a
+        // block sum in its fixed order), then thread by thread within the tile that holds the
+        // target, then id by id within that thread.
+        const int kk = top_k[r];
+        const float pp = top_p[r];
+        constexpr int TILE = SMP_NT * 8;
+        const int ntiles = (V + TILE - 1) / TILE;
+        if (!(kk > 0 && kk < V) && !(pp > 0.f && pp < 1.f) && ntiles <= SMP_NT) {
+            float m = -INFINITY;
+            for (int j = tid; j < V; j += SMP_NT) m = fmaxf(m, row[j] / T);
+            m = block_max_f(m, sf);
+            auto mine_of = [&](int tile) {               // this thread's 8 ids of a tile, in id order
+                const int j0 = tile * TILE + tid * 8;
+                float s = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s += (j0 + e < V) ? expf(row[j0 + e] / T - m) : 0.f;
+                return s;
+            };
+            for (int tile = 0; tile < ntiles; ++tile) {
+                const float ts = block_sum<SMP_NT>(mine_of(tile), sf);
+                if (tid == 0) part_f[tile] = ts;         // (ntiles <= SMP_NT places)
+            }
+            __syncthreads();
+            if (tid == 0) {
+                float total = 0.f;
+                for (int t = 0; t < ntiles; ++t) total += part_f[t];
+                const float target = uniform[r] * total;
+                float run = 0.f;
+                int pick = ntiles - 1;                   // rounding may leave the target just above the total
+                for (int t = 0; t < ntiles; ++t) {
+                    if (run + part_f[t] >= target) { pick = t; break; }
+                    run += part_f[t];
+                }
+                si[0] = pick;
+                sf[0] = run;
+                sf[1] = target;
+            }
+            __syncthreads();
+            const int tile = si[0];
+            const float before_tile = sf[0], target = sf[1];
+            __syncthreads();
+            part_f[tid] = mine_of(tile);
+            __syncthreads();
+            if (tid == 0) {
+                float run = before_tile;
+                int pick = -1, last = 0;
+                for (int t = 0; t < SMP_NT; ++t) {
+                    if (tile * TILE + t * 8 < V) last = t;
+                    if (pick < 0 && tile * TILE + t * 8 < V && run + part_f[t] >= target) pick = t;
+                    if (pick < 0) run += part_f[t];
+                }
+                if (pick < 0) { pick = last; run -= part_f[last]; }
+                chosen_thread = pick;
+                sf[0] = run;
+            }
+            __syncthreads();
+            if (tid == chosen_thread) {
+                float run = sf[0];
+                const int j0 = tile * TILE + tid * 8;
+                int pick = j0;
+                for (int e = 0; e < 8 && j0 + e < V; ++e) {
+                    pick = j0 + e;
+                    run += expf(row[j0 + e] / T - m);
+                    if (run >= target) break;
+                }
+                out[r] = pick;
+            }
+            return;
+        }
+    }
     // contiguous chunk of ids per thread, so that block scans run in id order
     const int chunk = (V + SMP_NT - 1) / SMP_NT;
     const int c0 = min(tid * chunk, V), c1 = min(c0 + chunk, V);

@@ -104,7 +104,7 @@ class StepContext:
 
 def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploader",
                   pad_blocks: Optional[Sequence[int]] = None, feedback: Optional[torch.Tensor] = None,
-                  needs=None) -> StepContext:
+                  needs=None, handles=None) -> StepContext:
     """Lay out the step's integers (see the module text) for the given entries
     against the cache's current tables, upload them, and return the context.
     Pages for the entries' tokens must have been reserved.  `pad_blocks` gives,
@@ -117,15 +117,22 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
     lib = native.lib()
     ng = len(cache.groups)
     nseg = len(entries)
-    handles = np.fromiter((cache.handle(e.rid) for e in entries), dtype=np.int64, count=nseg)
+    if handles is None:
+        handles = np.fromiter((cache.handle(e.rid) for e in entries), dtype=np.int64, count=nseg)
     q_len = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=nseg)
-    ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+    if int(q_len.max()) == 1:                        # single tokens all: no array per entry
+        ids = np.fromiter((e.tokens[0] for e in entries), dtype=np.int32, count=nseg)
+    else:
+        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
     id_src = None
     if any(e.take is not None for e in entries):
         if feedback is None:
             raise ValueError("step: an entry takes tokens from the feedback buffer, but there is none")
-        id_src = np.concatenate([np.full(len(e.tokens), -1, dtype=np.int32) if e.take is None
-                                 else np.asarray(e.take, dtype=np.int32) for e in entries])
+        if int(q_len.max()) == 1:
+            id_src = np.fromiter((-1 if e.take is None else e.take[0] for e in entries), dtype=np.int32, count=nseg)
+        else:
+            id_src = np.concatenate([np.full(len(e.tokens), -1, dtype=np.int32) if e.take is None
+                                     else np.asarray(e.take, dtype=np.int32) for e in entries])
     want_off = np.zeros(nseg + 1, dtype=np.int32)
     np.cumsum([len(e.want) for e in entries], out=want_off[1:])
     want = np.fromiter((int(w) for e in entries for w in e.want), dtype=np.int32, count=int(want_off[-1]))

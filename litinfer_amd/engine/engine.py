@@ -144,16 +144,34 @@ class Engine:
                                   page_order_seed=self._page_order_seed)
 
     # ---- the step ---------------------------------------------------------
-    def _validate(self, entries: Sequence[StepEntry]) -> None:
+    def _validate(self, entries: Sequence[StepEntry]):
+        """Checks the batch; returns (handles, token counts) of the entries, a handle of -1
+        standing for a request that is not live yet.  Nothing is changed."""
         if not entries:
             raise StepError("step: empty batch")
-        seen = set()
         vocab = self.spec.vocab_size
-        for e in entries:
-            if e.rid in seen:
-                raise StepError(f"step: request {e.rid!r} appears twice in one batch")
-            seen.add(e.rid)
-            n = len(e.tokens)
+        if len({e.rid for e in entries}) != len(entries):
+            seen = set()
+            for e in entries:
+                if e.rid in seen:
+                    raise StepError(f"step: request {e.rid!r} appears twice in one batch")
+                seen.add(e.rid)
+        counts = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=len(entries))
+        for e, n in zip(entries, counts):
+            if n == 1:                               # a decoded token: the common case, checked without arrays
+                t = e.tokens[0]
+                ok = isinstance(t, (int, np.integer)) and not isinstance(t, bool) and 0 <= t < vocab
+                if e.take is not None:
+                    k = e.take[0] if len(e.take) == 1 else None
+                    if not (isinstance(k, (int, np.integer)) and not isinstance(k, bool) and -1 <= k < FEEDBACK_SLOTS):
+                        raise StepError(f"step: request {e.rid!r}: `take` must give, for each of its 1 "
+                                        f"tokens, -1 or a place below {FEEDBACK_SLOTS} in the feedback buffer")
+                if not ok:
+                    raise StepError(f"step: request {e.rid!r} brings a token id outside the vocabulary "
+                                    f"of {vocab} (embedding: index out of range)")
+                if e.want and (len(e.want) != 1 or int(e.want[0]) != 0):
+                    raise StepError(f"step: request {e.rid!r} wants logits at places {list(e.want)} of 1 token")
+                continue
             if n == 0:
                 raise StepError(f"step: request {e.rid!r} brings no tokens")
             toks = np.asarray(e.tokens)
@@ -168,10 +186,13 @@ class Engine:
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"step: request {e.rid!r} wants logits at place {w} of {n} tokens")
-            have = self.cache.cached_len(e.rid) if self.cache.has(e.rid) else 0
-            if have + n > self.spec.max_positions:
-                raise StepError(f"step: request {e.rid!r} would reach {have + n} positions, the "
-                                f"model max sequence length is {self.spec.max_positions}")
+        handles = self.cache.handles_of([e.rid for e in entries])
+        reach = self.cache.cached_many(handles) + counts
+        if int(reach.max()) > self.spec.max_positions:
+            i = int(np.argmax(reach))
+            raise StepError(f"step: request {entries[i].rid!r} would reach {int(reach[i])} positions, the "
+                            f"model max sequence length is {self.spec.max_positions}")
+        return handles, counts
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of
@@ -184,48 +205,40 @@ class Engine:
         moves, requests that this step admitted are released again, and pages
         reserved for requests that were live already stay with them: the next
         step uses them, or they go back when the request ends."""
-        self._validate(entries)
+        handles, counts = self._validate(entries)
         cache = self.cache
-        admitted, reserved = [], []
+        admitted = []
         try:
-            for e in entries:
-                if not cache.has(e.rid):
-                    cache.admit(e.rid)
-                    admitted.append(e.rid)
-            # all-or-nothing over the batch: check the sum first
-            total = [0] * len(cache.groups)
-            for e in entries:
-                for gi, n in enumerate(cache.pages_needed(e.rid, len(e.tokens))):
-                    total[gi] += n
-            for gi, g in enumerate(cache.groups):
-                if total[gi] > g.pool.free:
-                    raise CacheFull(f"step: the batch needs {total[gi]} more pages, "
-                                    f"{g.pool.free} of {g.pool.capacity} are free")
-            for e in entries:
-                cache.reserve(e.rid, len(e.tokens))
+            if (handles < 0).any():
+                for i, e in enumerate(entries):
+                    if handles[i] < 0:
+                        cache.admit(e.rid)
+                        admitted.append(e.rid)
+                        handles[i] = cache.handle(e.rid)
+            cache.reserve_many(handles, counts)      # all-or-nothing over the batch
         except CacheFull:
             for rid in admitted:
                 cache.release(rid)
             raise
-        key = self._graph_key(entries)
+        decode_only = int(counts.max()) == 1
+        key = self._graph_key(entries, handles) if decode_only else None
         if profiler.enabled:
-            profiler.phase = "decode" if all(len(e.tokens) == 1 for e in entries) else "prefill"
+            profiler.phase = "decode" if decode_only else "prefill"
         if self._trace:
             print(f"[litinfer_amd trace] step {self.steps_run}: {len(entries)} requests, "
-                  f"{sum(len(e.tokens) for e in entries)} tokens, {sum(len(e.want) for e in entries)} rows of logits, "
+                  f"{int(counts.sum())} tokens, {sum(len(e.want) for e in entries)} rows of logits, "
                   f"{'recorded' if key is not None else 'eager'}, free pages {cache.free_pages()}",
                   file=sys.stderr, flush=True)
         try:
             if key is None:
-                logits = self.model.forward(self._build_context(entries), cache)
+                logits = self.model.forward(self._build_context(entries, handles=handles), cache)
             else:
-                logits = self._forward_graphed(key, self._build_context(entries, pad_blocks=key[2]))
+                logits = self._forward_graphed(key, self._build_context(entries, pad_blocks=key[2], handles=handles))
         except BaseException:
             for rid in admitted:
                 cache.release(rid)
             raise
-        for e in entries:
-            cache.commit(e.rid, len(e.tokens))
+        cache.commit_many(handles, counts)
         self.steps_run += 1
         return logits
 
@@ -234,24 +247,19 @@ class Engine:
         if self.cache.has(rid):
             self.cache.release(rid)
 
-    def _build_context(self, entries: Sequence[StepEntry], pad_blocks=None) -> StepContext:
+    def _build_context(self, entries: Sequence[StepEntry], pad_blocks=None, handles=None) -> StepContext:
         return build_context(self.cache, entries, self.ws, self._uploader, pad_blocks, self.feedback,
-                             needs=self.model.batch_needs())
+                             needs=self.model.batch_needs(), handles=handles)
 
     # ---- recorded decode steps ----------------------------------------------
-    def _graph_key(self, entries: Sequence[StepEntry]):
-        """(segments, wanted rows, table width per group) of a batch that may be
-        replayed from a graph, else None.  Table widths are rounded up to powers
-        of two so that a graph serves a range of context lengths."""
+    def _graph_key(self, entries: Sequence[StepEntry], handles):
+        """(segments, wanted rows, table width per group) of a batch of single tokens
+        that may be replayed from a graph, else None.  Table widths are rounded up
+        to powers of two so that a graph serves a range of context lengths."""
         if not self.use_graphs or not self.model.graph_safe:
             return None
-        if any(len(e.tokens) != 1 for e in entries):
-            return None
-        widths = []
-        for gi in range(len(self.cache.groups)):
-            need = max(self.cache.table_len(e.rid, gi) for e in entries)
-            widths.append(max(16, 1 << (need - 1).bit_length()))
-        return (len(entries), sum(len(e.want) for e in entries), tuple(widths))
+        widths = tuple(max(16, 1 << (max(need, 1) - 1).bit_length()) for need in self.cache.max_table_len(handles))
+        return (len(entries), sum(len(e.want) for e in entries), widths)
 
     def _forward_graphed(self, key, ctx: StepContext):
         gen = (self.ws.generation, self._uploader.generation)

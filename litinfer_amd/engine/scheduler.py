@@ -40,6 +40,8 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 from ..cache import CacheFull
 from ..sampling import Sampler, SamplingParams
 from .batch import StepEntry
@@ -78,6 +80,17 @@ class Request:
     @property
     def remaining(self) -> int:
         return len(self.prompt) + self.num_generated - self.computed
+
+    def slice_tokens(self, start: int, n: int) -> List[int]:
+        """tokens[start:start + n] without putting the whole list together."""
+        lp = len(self.prompt)
+        if start + n <= lp:
+            return self.prompt[start:start + n]
+        out = self.prompt[start:] if start < lp else []
+        out = out + self.generated[max(start - lp, 0):start + n - lp]
+        if len(out) < n:
+            out.append(0)                              # the pending token's place
+        return out
 
 
 @dataclass
@@ -203,18 +216,24 @@ class Scheduler:
             free = self.cache.free_pages()
             plan: List[Planned] = []
             budget = self.max_batch_tokens
-            movable = [r for r in self.running if r.remaining > 0 and not self._ends_with_pending(r)]
+            left = {id(r): r.remaining for r in self.running}
+            movable = [r for r in self.running if left[id(r)] > 0 and not self._ends_with_pending(r)]
             short = False
-            for r in movable:
-                if r.remaining != 1:
-                    continue
-                need = self._fits(free, r.rid, 1)
-                if need is None or budget <= 0:
-                    short = need is None
-                    break
-                free = [a - b for a, b in zip(free, need)]
-                budget -= 1
-                plan.append(Planned(r, r.computed, 1, True))
+            decoding = [r for r in movable if left[id(r)] == 1]
+            if decoding:
+                # what each of them must take for its one token, asked for in one call; in order of
+                # admission, each must fit beside those before it
+                need = self.cache.pages_needed_many(self.cache.handles_of([r.rid for r in decoding]),
+                                                    np.ones(len(decoding), dtype=np.int32))
+                fits = (np.cumsum(need, axis=0) <= np.asarray(free, dtype=np.int64)).all(axis=1)
+                for i, r in enumerate(decoding):
+                    if not fits[i] or budget <= 0:
+                        short = not fits[i]
+                        break
+                    budget -= 1
+                    plan.append(Planned(r, r.computed, 1, True))
+                taken = need[:len(plan)].sum(axis=0) if plan else np.zeros(len(free), dtype=np.int64)
+                free = [int(a - b) for a, b in zip(free, taken)]
             if short and len(self.running) > 1:
                 self._preempt(self.running[-1])
                 continue
@@ -222,23 +241,26 @@ class Scheduler:
                 self._end_lone(self.running[0])
                 continue
             for r in movable:
-                if r.remaining <= 1 or budget <= 0:
+                if left[id(r)] <= 1 or budget <= 0:
                     continue
-                n = self._largest_fitting(free, r.rid, min(r.remaining, self.chunk_size, budget), None)
+                n = self._largest_fitting(free, r.rid, min(left[id(r)], self.chunk_size, budget), None)
                 if n <= 0:
                     continue
                 free = [a - b for a, b in zip(free, self.cache.pages_needed(r.rid, n))]
                 budget -= n
-                plan.append(Planned(r, r.computed, n, n == r.remaining))
+                plan.append(Planned(r, r.computed, n, n == left[id(r)]))
             # Pages that the running requests' prompts will still take are spoken for: a waiting
             # request is admitted only when everything it has to compute fits what is left after
             # them (a request let in on its first portion alone would stall beside the others, each
             # holding pages and none able to finish its prompt)
             spare = self.cache.free_pages()
-            for r in self.running:
-                if r.remaining > 0:
-                    spare = [a - b for a, b in zip(spare, self.cache.pages_needed(r.rid, r.remaining))]
             slots = self.cache.free_slots()
+            if self.waiting and budget > 0 and slots > 0 and len(self.running) < self.max_running:
+                going = [r for r in self.running if left[id(r)] > 0]
+                if going:
+                    need = self.cache.pages_needed_many(self.cache.handles_of([r.rid for r in going]),
+                                                        np.asarray([left[id(r)] for r in going], dtype=np.int32))
+                    spare = [int(a - b) for a, b in zip(spare, need.sum(axis=0))]
             while self.waiting and budget > 0 and slots > 0 and len(self.running) < self.max_running:
                 r = self.waiting[0]
                 whole = self._fits(spare, None, r.remaining, 0)
@@ -287,7 +309,7 @@ class Scheduler:
             take = None
             if r.pending_take is not None and p.start + p.n == len(r.prompt) + r.num_generated:
                 take = [-1] * (p.n - 1) + [r.pending_take]          # the portion ends with the pending token
-            entries.append(StepEntry(r.rid, r.tokens[p.start:p.start + p.n],
+            entries.append(StepEntry(r.rid, r.slice_tokens(p.start, p.n),
                                      [p.n - 1] if p.wants_logits else [], take))
         self.last_batch_tokens = sum(p.n for p in plan)
         logits = self.engine.step(entries)

@@ -650,6 +650,26 @@ def test_sample_rows_against_the_plain_sampler(ops, vocab):
     assert same >= n - 1
 
 
+@pytest.mark.parametrize("vocab", [8, 301, 8192, 8193, 152064])
+def test_sample_rows_with_temperature_alone(ops, vocab):
+    # no top-k and no top-p: the kernel's short way; uniform numbers at both ends among them
+    g = torch.Generator().manual_seed(15)
+    n = 24
+    logits = torch.randn(n, vocab, generator=g) * 4
+    temperature = [0.3 + 0.1 * i for i in range(n)]
+    u = torch.rand(n, generator=g).tolist()
+    u[0], u[1], u[2] = 0.0, 0.99999994, 0.5
+    picks = _sample(ops, logits, temperature, [0] * n, [1.0] * n, u)
+    rows = logits.double().numpy()
+    for r in range(n):
+        assert 0 <= picks[r] < vocab
+        assert _pick_is_right(rows[r], temperature[r], 0, 1.0, u[r], picks[r]), r
+    # and mostly the very id of the float64 sampler (among 152,064 ids a float32 sum's rounding moves an
+    # interval's edge past the uniform number now and then; each such pick was checked above)
+    same = sum(picks[r] == plain_impl.sample_with_uniform(rows[r], temperature[r], 0, 1.0, u[r]) for r in range(n))
+    assert same >= n - 4
+
+
 def test_sample_rows_frequencies_and_ties(ops):
     lg = torch.tensor([[2.0, 1.0, 3.0, 3.0, -1.0, 0.5, 2.5, 0.0]])
     n = 4000
