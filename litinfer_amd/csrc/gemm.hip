@@ -75,17 +75,101 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
     }
 }
 
+// The same product in tiles of 128 x 128 with 8 x 8 outputs a thread, for many rows and columns:
+// a step reads 16 floats from LDS for 64 multiply-adds (the small tile reads 8 for 16), so the
+// FMA units and not LDS bound it.  Every output element still adds its products up in ascending
+// k, one fused multiply-add after the other: the results are those of the small tile bit for bit.
+#define F32B_BM 128
+#define F32B_BN 128
+#define F32B_BK 8
+
+__global__ __launch_bounds__(256) void gemm_f32_big_kernel(const float* __restrict__ x,
+                                                            const float* __restrict__ w,
+                                                            const float* __restrict__ bias,
+                                                            float* __restrict__ out, int M, int N, int K,
+                                                            int accumulate) {
+    __shared__ __attribute__((aligned(16))) float As[2][F32B_BK][F32B_BM + 4];
+    __shared__ __attribute__((aligned(16))) float Bs[2][F32B_BK][F32B_BN + 4];
+    const int tid = threadIdx.x;
+    const int m0 = blockIdx.y * F32B_BM, n0 = blockIdx.x * F32B_BN;
+    const int ty = tid / 16, tx = tid % 16;                  // outputs rows 4 ty .. +3 and 64 + 4 ty .., columns likewise
+    const int lrow = tid / 2, lk = (tid % 2) * 4;            // this thread's 4 consecutive k of one row of each operand
+    const bool vec = (K % 4) == 0;
+    const float* arow = x + (size_t)(m0 + lrow < M ? m0 + lrow : M - 1) * K;
+    const float* brow = w + (size_t)(n0 + lrow < N ? n0 + lrow : N - 1) * K;
+    float acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+    float a[4], b[4];
+    auto fetch = [&](int k0) {
+        if (vec && k0 + lk + 4 <= K) {
+            const floatx4 av = *reinterpret_cast<const floatx4*>(arow + k0 + lk);
+            const floatx4 bv = *reinterpret_cast<const floatx4*>(brow + k0 + lk);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { a[i] = av[i]; b[i] = bv[i]; }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int k = k0 + lk + i;
+                a[i] = k < K ? arow[k] : 0.f;
+                b[i] = k < K ? brow[k] : 0.f;
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { As[buf][lk + i][lrow] = a[i]; Bs[buf][lk + i][lrow] = b[i]; }
+    };
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += F32B_BK) {
+        const bool more = k0 + F32B_BK < K;
+        if (more) fetch(k0 + F32B_BK);                       // on its way while this step is multiplied
+#pragma unroll
+        for (int k = 0; k < F32B_BK; ++k) {
+            const floatx4 a0 = *reinterpret_cast<const floatx4*>(&As[buf][k][4 * ty]);
+            const floatx4 a1 = *reinterpret_cast<const floatx4*>(&As[buf][k][64 + 4 * ty]);
+            const floatx4 b0 = *reinterpret_cast<const floatx4*>(&Bs[buf][k][4 * tx]);
+            const floatx4 b1 = *reinterpret_cast<const floatx4*>(&Bs[buf][k][64 + 4 * tx]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float av = i < 4 ? a0[i] : a1[i - 4];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(av, j < 4 ? b0[j] : b1[j - 4], acc[i][j]);
+            }
+        }
+        if (more) {
+            stash(buf ^ 1);
+            __syncthreads();
+            buf ^= 1;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = m0 + (i < 4 ? 4 * ty + i : 64 + 4 * ty + i - 4);
+        if (row >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int col = n0 + (j < 4 ? 4 * tx + j : 64 + 4 * tx + j - 4);
+            if (col < N) epilogue_store(out, (size_t)row * N + col, acc[i][j], bias, col, accumulate);
+        }
+    }
+}
+
 // ------------------------------------------------------ float32, few rows (decode)
-// The product streams W once: a wave owns F32R_NT consecutive columns of the output and
+// The product streams W once: a wave owns NT consecutive columns of the output and
 // walks K with 16 bytes a lane; the MT rows of x come from the caches (every wave of the
 // grid reads the same few rows).  More than MT rows run as passes of MT; the passes of one
 // group of columns are neighbouring blocks, so that the second finds the matrix's rows in L2.
 // Each output element is the butterfly sum of its 64 lanes' strided partial sums: an order
 // that depends on K alone.
-#define F32R_NT 4
 #define F32R_WAVES 4
 
-template <int MT>
+template <int MT, int NT>
 __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const float* __restrict__ x,
                                                                         const float* __restrict__ w,
                                                                         const float* __restrict__ bias,
@@ -93,24 +177,24 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
                                                                         int accumulate, int npass) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pass = blockIdx.x % npass, group = blockIdx.x / npass;
-    const int n0 = (group * F32R_WAVES + wave) * F32R_NT;
+    const int n0 = (group * F32R_WAVES + wave) * NT;
     const int m0 = pass * MT;
     if (n0 >= N) return;
-    float acc[MT][F32R_NT];
+    float acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < F32R_NT; ++j) acc[i][j] = 0.f;
-    const float* wrow[F32R_NT];
+        for (int j = 0; j < NT; ++j) acc[i][j] = 0.f;
+    const float* wrow[NT];
 #pragma unroll
-    for (int j = 0; j < F32R_NT; ++j) wrow[j] = w + (size_t)(n0 + j < N ? n0 + j : N - 1) * K;
+    for (int j = 0; j < NT; ++j) wrow[j] = w + (size_t)(n0 + j < N ? n0 + j : N - 1) * K;
     const float* xrow[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) xrow[i] = x + (size_t)(m0 + i < M ? m0 + i : M - 1) * K;
     for (int k = 4 * lane; k < K; k += 256) {
-        floatx4 wv[F32R_NT], xv[MT];
+        floatx4 wv[NT], xv[MT];
 #pragma unroll
-        for (int j = 0; j < F32R_NT; ++j) wv[j] = *reinterpret_cast<const floatx4*>(wrow[j] + k);
+        for (int j = 0; j < NT; ++j) wv[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(wrow[j] + k));
 #pragma unroll
         for (int i = 0; i < MT; ++i) xv[i] = *reinterpret_cast<const floatx4*>(xrow[i] + k);
 #pragma unroll
@@ -118,12 +202,12 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
 #pragma unroll
             for (int i = 0; i < MT; ++i)
 #pragma unroll
-                for (int j = 0; j < F32R_NT; ++j) acc[i][j] = fmaf(xv[i][e], wv[j][e], acc[i][j]);
+                for (int j = 0; j < NT; ++j) acc[i][j] = fmaf(xv[i][e], wv[j][e], acc[i][j]);
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < F32R_NT; ++j) {
+        for (int j = 0; j < NT; ++j) {
             float v = acc[i][j];
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -134,7 +218,7 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
         for (int i = 0; i < MT; ++i) {
             if (m0 + i >= M) continue;
 #pragma unroll
-            for (int j = 0; j < F32R_NT; ++j)
+            for (int j = 0; j < NT; ++j)
                 if (n0 + j < N) epilogue_store(out, (size_t)(m0 + i) * N + n0 + j, acc[i][j], bias, n0 + j, accumulate != 0);
         }
     }
@@ -145,17 +229,27 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
 static int launch_f32_rows(const float* x, const float* w, const float* bias, float* out, int M, int N, int K,
                            int accumulate, hipStream_t stream) {
     const int mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    const int nt = (mt <= 8 && N >= 8192) ? 8 : 4;            // columns a wave owns: more where the matrix has many
     const int npass = (M + mt - 1) / mt;
-    const long groups = (N + F32R_WAVES * F32R_NT - 1) / (F32R_WAVES * F32R_NT);
+    const long groups = (N + F32R_WAVES * nt - 1) / (F32R_WAVES * nt);
     if (groups * npass > 0x7fffffffL) return LI_ERR_SIZE;
     const unsigned grid = (unsigned)(groups * npass);
-#define LI_F32R(MT) gemm_f32_rows_kernel<MT><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass)
-    switch (mt) {
-        case 1: LI_F32R(1); break;
-        case 2: LI_F32R(2); break;
-        case 4: LI_F32R(4); break;
-        case 8: LI_F32R(8); break;
-        default: LI_F32R(16); break;
+#define LI_F32R(MT, NT) gemm_f32_rows_kernel<MT, NT><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass)
+    if (nt == 8) {
+        switch (mt) {
+            case 1: LI_F32R(1, 8); break;
+            case 2: LI_F32R(2, 8); break;
+            case 4: LI_F32R(4, 8); break;
+            default: LI_F32R(8, 8); break;
+        }
+    } else {
+        switch (mt) {
+            case 1: LI_F32R(1, 4); break;
+            case 2: LI_F32R(2, 4); break;
+            case 4: LI_F32R(4, 4); break;
+            case 8: LI_F32R(8, 4); break;
+            default: LI_F32R(16, 4); break;
+        }
     }
 #undef LI_F32R
     return li_launch_status();
@@ -1306,6 +1400,12 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         if (out_dtype != LI_F32) return LI_ERR_DTYPE;
         if (M <= F32_ROWS_MAX && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0)
             return launch_f32_rows((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate, stream);
+        if (M >= 2 * F32B_BM && N >= F32B_BN) {              // enough of both for the large tile to fill the chip
+            dim3 big((N + F32B_BN - 1) / F32B_BN, (M + F32B_BM - 1) / F32B_BM);
+            if (big.y > 65535) return LI_ERR_SIZE;
+            gemm_f32_big_kernel<<<big, 256, 0, stream>>>((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate);
+            return li_launch_status();
+        }
         dim3 grid((N + F32_BN - 1) / F32_BN, (M + F32_BM - 1) / F32_BM);
         if (grid.y > 65535) return LI_ERR_SIZE;
         gemm_f32_kernel<<<grid, 256, 0, stream>>>((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate);

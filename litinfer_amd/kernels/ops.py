@@ -487,6 +487,9 @@ def linear_rope_store(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Ten
 
 
 # ----------------------------------------------------------------- attention
+# waves that the split-key decode kernel on the matrix cores is cut into at least (where the keys allow):
+# four a compute unit; more splits cost more in the merge than they gain (measured at 8 and 64 requests)
+_DEC_WAVES = 1024
 PREFILL_TILE_ROWS = 32       # queries of one segment that a block of the matrix-core kernel for portions takes
 DECODE_MAX_SPLITS = 64       # the merge kernel keeps a weight per split
 DECODE_TABLE_CAP = 1024      # pages of one split that the matrix-core decode kernel copies into LDS
@@ -545,7 +548,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         # block of four waves per split on the vector ALU
         mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
         if mfma:
-            nsplit = max(1, min(-(-2048 // (n_single * nkv)), -(-keys // 128), DECODE_MAX_SPLITS))
+            nsplit = max(1, min(-(-_DEC_WAVES // (n_single * nkv)), -(-keys // 128), DECODE_MAX_SPLITS))
             # a split's pages must fit the kernel's copy of the block table
             while nsplit <= DECODE_MAX_SPLITS and decode_split_blocks(meta.max_blocks, page_size, window, nsplit) > DECODE_TABLE_CAP:
                 nsplit += 1
