@@ -209,13 +209,23 @@ class StepLoop:
             b = eng.step(entries).clone()
         finally:
             eng.use_graphs = was
+        # The two runs may cut the keys of the decode attention differently (a recorded step is laid
+        # out for the block table's padded width), so they agree to rounding, not to the bit: the
+        # logits must be close, and where the greedy tokens differ the two candidates must be that close.
         params = [SamplingParams()] * batch
         ta = self.sampler.sample(a, params, [0] * batch)
         tb = self.sampler.sample(b, params, [0] * batch)
-        if ta != tb:
-            worst = float((a - b).abs().max())
-            raise RuntimeError(f"bench: a recorded decode step and an eager one of the same batch of {batch} "
-                               f"chose different tokens (largest logit difference {worst:.3e})")
+        worst = float((a - b).abs().max())
+        scale = float(a.abs().max())
+        tol = (3e-2 if self.eng.rt.dtype is torch.bfloat16 else 1e-4) * scale
+        if not worst <= tol:
+            raise RuntimeError(f"bench: a recorded decode step and an eager one of the same batch of {batch} differ by "
+                               f"{worst:.3e} in a logit (largest logit {scale:.3e})")
+        for i, (x, y) in enumerate(zip(ta, tb)):
+            if x != y and float(a[i, x] - a[i, y]) > 2 * worst:
+                raise RuntimeError(f"bench: a recorded decode step and an eager one of the same batch of {batch} "
+                                   f"chose different tokens for row {i} (logits {float(a[i, x]):.4f} and {float(a[i, y]):.4f}, "
+                                   f"largest logit difference {worst:.3e})")
 
 
 # ------------------------------------------------------ through the scheduler

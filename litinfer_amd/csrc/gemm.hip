@@ -982,27 +982,35 @@ struct SkinnyArgs {
     const float* row_parts;
     int nparts;
     float eps;
+    // Columns a block takes (with ROPE: rotation pairs a block takes); 0: as many as its tiles hold.
+    // Fewer than the tiles hold where that spreads a matrix of few columns evenly over the compute units.
+    int cols;
 };
 #define SK_MAX_PARTS 512            // blocks of a producing product whose sums one consumer adds up
 
 template <int MT, int NT, int WAVES, bool SWIGLU, typename TO, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs a) {
-    static_assert(!ROPE || (MT == 1 && NT == 1 && !SWIGLU), "the rotary epilogue takes one tile");
+    static_assert(!ROPE || (MT == 1 && !SWIGLU), "the rotary epilogue takes one tile of rows");
     __shared__ floatx4 red[WAVES][MT * NT][64];
     __shared__ float part_sums[WAVES * 4][16];
     const int M = a.M, N = a.N, K = a.K;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
-    const int n0 = blockIdx.x * 16 * (SWIGLU ? 1 : NT);
+    const int per_block = a.cols > 0 ? a.cols : (ROPE ? 8 : 16) * (SWIGLU ? 1 : NT);
+    const int n0 = blockIdx.x * per_block;                  // first column (with ROPE: first pair) of this block
+    const int half = a.dh / 2;
+    const int total = ROPE ? (a.nh + 2 * a.nkv) * half : N;
+    const int nend = n0 + per_block < total ? n0 + per_block : total;     // one past its last
     const bf16_t* wrow[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         int row;
         if (SWIGLU) row = ((n0 + r16 < N) ? n0 + r16 : N - 1) + nt * N;      // gate row, up row
-        else if (ROPE) {
-            const int bph = a.dh / 16, head = blockIdx.x / bph, i = blockIdx.x % bph;
-            row = head * a.dh + 8 * i + (r16 < 8 ? r16 : a.dh / 2 + r16 - 8);
-        } else row = (n0 + 16 * nt + r16 < N) ? n0 + 16 * nt + r16 : N - 1;    // rows past the end repeat the last
+        else if (ROPE) {                                    // rows 0..7 of a tile: first members of 8 pairs, 8..15: their partners
+            int p = n0 + 8 * nt + (r16 & 7);
+            p = p < nend ? p : nend - 1;
+            row = (p / half) * a.dh + p % half + (r16 < 8 ? 0 : half);
+        } else row = (n0 + 16 * nt + r16 < nend) ? n0 + 16 * nt + r16 : nend - 1;    // rows past the end repeat the last
         wrow[nt] = a.w + (size_t)row * K + 8 * g;
     }
     // x is read with whole rows of a chunk contiguous over 16 lanes (lane l: row l / 16 + 4 i,
@@ -1030,30 +1038,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     // that will write the results: the answers arrive with the first chunk, and the epilogue
     // waits for no memory.  Never conditional per lane: a place past the end reads the last one.
     constexpr bool PRE = MT == 1 && !SWIGLU;
-    float pre_bias[NT][4], pre_res[NT][4], pre_gamma[NT][4], pre_cos[4], pre_sin[4];
+    float pre_bias[NT][4], pre_res[NT][4], pre_gamma[NT][4], pre_cos[NT][4], pre_sin[NT][4];
     int pre_slot = 0;
     if constexpr (PRE) {
         if (wave == 0) {
             const int m = (lane & 15) < M ? (lane & 15) : M - 1;
             if constexpr (ROPE) {
-                const int dh = a.dh, half = dh / 2, bph = dh / 16;
-                const int head = blockIdx.x / bph, i = blockIdx.x % bph;
                 const bool second = (lane >> 4) >= 2;
                 pre_slot = a.slot_map[m];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int j = 8 * i + 4 * ((lane >> 4) & 1) + r;
-                    pre_bias[0][r] = a.bias ? a.bias[head * dh + (second ? half + j : j)] : 0.f;
-                    pre_cos[r] = a.cos[(size_t)m * half + j];
-                    pre_sin[r] = a.sin[(size_t)m * half + j];
-                }
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        int p = n0 + 8 * nt + 4 * ((lane >> 4) & 1) + r;
+                        p = p < nend ? p : nend - 1;
+                        const int head = p / half, j = p % half;
+                        pre_bias[nt][r] = a.bias ? a.bias[head * a.dh + (second ? half + j : j)] : 0.f;
+                        pre_cos[nt][r] = a.cos[(size_t)m * half + j];
+                        pre_sin[nt][r] = a.sin[(size_t)m * half + j];
+                    }
             } else {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         const int n = n0 + 16 * nt + 4 * (lane >> 4) + r;
-                        const int nc = n < N ? n : N - 1;
+                        const int nc = n < nend ? n : nend - 1;
                         pre_bias[nt][r] = a.bias ? a.bias[nc] : 0.f;
                         pre_gamma[nt][r] = a.gamma ? a.gamma[nc] : 0.f;
                         if constexpr (sizeof(TO) == 4)
@@ -1184,33 +1194,36 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
             for (int nt = 0; nt < NT; ++nt) { s[nt][0] *= inv; s[nt][1] *= inv; s[nt][2] *= inv; s[nt][3] *= inv; }
         }
         if constexpr (ROPE) {
-            const int dh = a.dh, half = dh / 2, bph = dh / 16;
-            const int head = blockIdx.x / bph, i = blockIdx.x % bph;
+            const int dh = a.dh;
             const bool second = (l >> 4) >= 2;                       // this lane holds the pairs' second members
             const int slot = pre_slot;                               // (MT is 1: thread t is lane l of wave 0, which asked for these)
             const int page = slot / a.page_size, in_page = slot - page * a.page_size;
             const bool page_ok = page >= 0 && page < a.num_pages;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int j = 8 * i + 4 * ((l >> 4) & 1) + r;        // the pair's number within the head
-                const int d = second ? half + j : j;
-                const int col = head * dh + d;
-                float own = s[0][r] + pre_bias[0][r];
-                const float other = __shfl_xor(own, 32, 64);
-                float v = own;
-                if (head < a.nh + a.nkv) {
-                    const float c = pre_cos[r], sn = pre_sin[r];
-                    v = second ? own * c + other * sn : own * c - other * sn;
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int p = n0 + 8 * nt + 4 * ((l >> 4) & 1) + r;  // the pair's number among all heads' pairs
+                    float own = s[nt][r] + pre_bias[nt][r];
+                    const float other = __shfl_xor(own, 32, 64);
+                    if (p >= nend) continue;                         // (lanes l and l ^ 32 share p: the exchange above is done by both)
+                    const int head = p / half, j = p - head * half;
+                    const int d = second ? half + j : j;
+                    const int col = head * dh + d;
+                    float v = own;
+                    if (head < a.nh + a.nkv) {
+                        const float c = pre_cos[nt][r], sn = pre_sin[nt][r];
+                        v = second ? own * c + other * sn : own * c - other * sn;
+                    }
+                    const uint16_t bits = float_to_bf16(v);
+                    reinterpret_cast<bf16_t*>(out)[(size_t)m * N + col].bits = bits;
+                    if (head >= a.nh && page_ok) {
+                        const bool is_k = head < a.nh + a.nkv;
+                        const int kvh = is_k ? head - a.nh : head - a.nh - a.nkv;
+                        bf16_t* dst = (is_k ? a.kc : a.vc) + (((size_t)page * a.nkv + kvh) * a.page_size + in_page) * dh + d;
+                        dst->bits = bits;
+                    }
                 }
-                const uint16_t bits = float_to_bf16(v);
-                reinterpret_cast<bf16_t*>(out)[(size_t)m * N + col].bits = bits;
-                if (head >= a.nh && page_ok) {
-                    const bool is_k = head < a.nh + a.nkv;
-                    const int kvh = is_k ? head - a.nh : head - a.nh - a.nkv;
-                    bf16_t* dst = (is_k ? a.kc : a.vc) + (((size_t)page * a.nkv + kvh) * a.page_size + in_page) * dh + d;
-                    dst->bits = bits;
-                }
-            }
         } else if constexpr (SWIGLU) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -1229,7 +1242,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
 #pragma unroll
                         for (int r = 0; r < 4; ++r) {
                             const int n = n0 + 16 * nt + 4 * (l >> 4) + r;
-                            if (n < N) {
+                            if (n < nend) {
                                 const size_t idx = (size_t)m * N + n;
                                 const float v = (s[nt][r] + pre_bias[nt][r]) + pre_res[nt][r];
                                 reinterpret_cast<float*>(out)[idx] = v;
@@ -1249,7 +1262,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int n = n0 + 16 * nt + 4 * (l >> 4) + r;
-                    if (n >= N) continue;
+                    if (n >= nend) continue;
                     if constexpr (PRE) store_from_float(out + (size_t)m * N + n, (s[nt][r] + pre_bias[nt][r]) + pre_res[nt][r]);
                     else epilogue_store(out, (size_t)m * N + n, s[nt][r], a.bias, n, a.accumulate);
                 }
@@ -1257,16 +1270,46 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     }
 }
 
+// Compute units of the current device (256 where it cannot be asked).
+static int compute_units() {
+    static int units[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void)hipGetLastError(); return 256; }
+    if (!units[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) { (void)hipGetLastError(); n = 256; }
+        units[dev] = n;
+    }
+    return units[dev];
+}
+
+// Up to 16 rows against a matrix of few columns (or rotation pairs: `unit` is 16 columns or 8 pairs a
+// tile): a compute unit takes in what its blocks ask for at a rate of its own, far below its share of
+// the memory's rate times the number of units, so the time of such a product is that of the unit with the
+// most blocks.  Every unit therefore gets one block and every block the same number of columns (at
+// most two tiles' worth, at least half a tile's), not whole tiles.
+static int balanced_per_block(int total, int unit) {
+    const int cu = compute_units();
+    int per = (total + cu - 1) / cu;
+    per = per < unit / 2 ? unit / 2 : per;
+    return per > 2 * unit ? 0 : per;
+}
+
 template <bool SWIGLU, typename TO>
-static void launch_skinny(const SkinnyArgs& a, hipStream_t stream) {
+static void launch_skinny(SkinnyArgs a, hipStream_t stream) {
     const int M = a.M, N = a.N;
 #define LI_SK(MT, NT, WV) gemm_bf16_skinny_kernel<MT, NT, WV, SWIGLU, TO><<<(N + 16 * (SWIGLU ? 1 : NT) - 1) / (16 * (SWIGLU ? 1 : NT)), WV * 64, 0, stream>>>(a)
     if constexpr (SWIGLU) {
         if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
     } else if (N >= 8192) {                                 // many columns: many blocks, two tiles share each piece of x
         if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
-    } else {                                                // few columns: few blocks, so more waves split K
-        if (M <= 16) LI_SK(1, 1, 8); else if (M <= 32) LI_SK(2, 1, 4); else LI_SK(4, 2, 8);
+    } else if (M <= 16) {                                   // few columns: a block a compute unit, eight waves split K
+        a.cols = balanced_per_block(N, 16);
+        const int per = a.cols ? a.cols : 16, blocks = (N + per - 1) / per;
+        if (per > 16) gemm_bf16_skinny_kernel<1, 2, 8, false, TO><<<blocks, 8 * 64, 0, stream>>>(a);
+        else gemm_bf16_skinny_kernel<1, 1, 8, false, TO><<<blocks, 8 * 64, 0, stream>>>(a);
+    } else {
+        if (M <= 32) LI_SK(2, 1, 4); else LI_SK(4, 2, 8);
     }
 #undef LI_SK
 }
@@ -1290,7 +1333,8 @@ extern "C" int li_linear_skinny(const void* x, const void* w, const float* bias,
 // in float32, xg = bf16(gamma * out), sq_parts[block * 16 + m] = the block's share of row m's sum of
 // squares.  Up to 16 rows.  li_residual_norm_parts(N) is the number of blocks, i.e. of parts.
 extern "C" int li_residual_norm_parts(int N) {
-    const int per = N >= 8192 ? 32 : 16;               // as launch_skinny tiles the columns of few rows
+    int per = 32;                                      // as launch_skinny tiles the columns of few rows
+    if (N < 8192) { per = balanced_per_block(N, 16); per = per ? per : 16; }
     return (N + per - 1) / per;
 }
 
@@ -1518,6 +1562,10 @@ extern "C" int li_linear_rope_store(const void* x, const void* w, const float* b
                  (bf16_t*)kc, (bf16_t*)vc, nh, nkv, dh, page_size, num_pages,
                  nullptr, nullptr, nullptr, row_parts, row_parts ? nparts : 0, eps};
     if (row_parts && (nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f)) return LI_ERR_SIZE;
-    gemm_bf16_skinny_kernel<1, 1, 8, false, bf16_t, true><<<N / 16, 8 * 64, 0, stream>>>(a);
+    const int pairs = N / 2;
+    a.cols = balanced_per_block(pairs, 8);
+    const int per = a.cols ? a.cols : 8, blocks = (pairs + per - 1) / per;
+    if (per > 8) gemm_bf16_skinny_kernel<1, 2, 8, false, bf16_t, true><<<blocks, 8 * 64, 0, stream>>>(a);
+    else gemm_bf16_skinny_kernel<1, 1, 8, false, bf16_t, true><<<blocks, 8 * 64, 0, stream>>>(a);
     return li_launch_status();
 }

@@ -355,9 +355,14 @@ class RowScale:
 
 
 def residual_norm_parts(n: int) -> int:
-    """Blocks of `linear_residual_norm` over n columns, i.e. shares of a row's sum of squares."""
-    per = 32 if n >= 8192 else 16
-    return -(-n // per)
+    """Blocks of `linear_residual_norm` over n columns, i.e. shares of a row's sum of squares (the
+    library spreads a matrix of few columns evenly over the current device's compute units)."""
+    f = _fn_cache.get(("gemm", "li_residual_norm_parts"))
+    if f is None:
+        f = build.load("gemm").li_residual_norm_parts
+        f.argtypes, f.restype = [c_int], c_int
+        _fn_cache[("gemm", "li_residual_norm_parts")] = f
+    return int(f(int(n)))
 
 
 def residual_norm_takes(m: int, n: int, k: int, w_dtype: torch.dtype) -> bool:
