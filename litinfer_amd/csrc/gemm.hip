@@ -1308,8 +1308,13 @@ static void launch_skinny(SkinnyArgs a, hipStream_t stream) {
         const int per = a.cols ? a.cols : 16, blocks = (N + per - 1) / per;
         if (per > 16) gemm_bf16_skinny_kernel<1, 2, 8, false, TO><<<blocks, 8 * 64, 0, stream>>>(a);
         else gemm_bf16_skinny_kernel<1, 1, 8, false, TO><<<blocks, 8 * 64, 0, stream>>>(a);
+    } else if (M <= 32) {
+        a.cols = balanced_per_block(N, 16);
+        const int per = a.cols ? a.cols : 16, blocks = (N + per - 1) / per;
+        if (per > 16) gemm_bf16_skinny_kernel<2, 2, 4, false, TO><<<blocks, 4 * 64, 0, stream>>>(a);
+        else gemm_bf16_skinny_kernel<2, 1, 4, false, TO><<<blocks, 4 * 64, 0, stream>>>(a);
     } else {
-        if (M <= 32) LI_SK(2, 1, 4); else LI_SK(4, 2, 8);
+        LI_SK(4, 2, 8);
     }
 #undef LI_SK
 }
@@ -1353,10 +1358,16 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
 // loads straight into LDS, and, where the matrix has too few such tiles to fill the chip, K cut
 // into parts whose sums go to `work` and are added up in a fixed order.  Returns -1 when it does
 // not take the call.
+// From 17 rows on the same holds where K is long (the feed-forward's way back): every block of the
+// few-row kernel reads all of x, and what a compute unit can take in then bounds the product.
+static bool mid_rows_take(int M, int K) {
+    return M <= 64 && (M > 32 || (M > 16 && (long)M * K * 2 > 600 * 1024));
+}
+
 static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, void* out, int M, int N,
                            int K, int out_dtype, int accumulate, void* work, long work_bytes,
                            hipStream_t stream) {
-    if (M <= 32 || M > 64 || K % 64 || (out_dtype != LI_F32 && out_dtype != LI_BF16)) return -1;
+    if (!mid_rows_take(M, K) || K % 64 || (out_dtype != LI_F32 && out_dtype != LI_BF16)) return -1;
 #define LI_MID(BN, NS, TO, dst, b, acc, split) launch_dma<64, BN, 64, NS, false, TO>(x, w, b, (TO*)(dst), M, N, K, acc, stream, split)
     if ((N + 255) / 256 >= 128)
         return out_dtype == LI_F32 ? LI_MID(256, 3, float, out, bias, accumulate, 1) : LI_MID(256, 3, bf16_t, out, bias, accumulate, 1);
@@ -1392,7 +1403,8 @@ static int split_parts_many_rows(int M, int N, int K) {
 
 // Bytes of workspace with which li_linear cuts this product along K (0: it would not).
 extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
-    if (in_dtype != LI_BF16 || M <= 32 || N <= 0 || K <= 0 || K % 64) return 0;
+    if (in_dtype != LI_BF16 || M <= 16 || N <= 0 || K <= 0 || K % 64) return 0;
+    if (M <= 64 && !mid_rows_take(M, K)) return 0;
     int nsplit = 1;
     if (M <= 64) {
         const int tiles = (N + 127) / 128;
@@ -1414,7 +1426,7 @@ extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
 extern "C" int li_linear_then_norm(const void* x, const void* w, const float* bias, float* out, int M, int N, int K,
                                    void* work, long work_bytes, const float* gamma, float eps, void* xn,
                                    int xn_dtype, hipStream_t stream) {
-    if (M <= 32 || N <= 0 || K <= 0 || (K % 64) || !gamma || !xn || eps < 0.f) return -1;
+    if (M <= 16 || N <= 0 || K <= 0 || (K % 64) || !gamma || !xn || eps < 0.f) return -1;
     if (N > REDUCE_NORM_NT * REDUCE_NORM_PER || (xn_dtype != LI_BF16 && xn_dtype != LI_F32)) return -1;
     const long need = li_linear_work_bytes(M, N, K, LI_BF16);
     if (need <= 0 || !work || work_bytes < need) return -1;

@@ -279,7 +279,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     x [M, K] and w [N, K] of one dtype (float32 or bfloat16); out [M, N] of that
     dtype or float32; accumulation of the product is float32.  `ws` lends the
     memory for partial sums where the kernel cuts K into parts (33 to 64 rows
-    against a matrix of few columns); without it such a product takes a slower kernel."""
+    against a matrix of few columns, from 17 rows on where K is long); without it
+    such a product takes a slower kernel."""
     _gpu(x, w, bias, out)
     _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear: needs matrices")
     m, k = x.shape
@@ -294,7 +295,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
          "linear: bias must be float32 [N]")
     if m:
         work, work_bytes = 0, 0
-        if ws is not None and x.dtype is torch.bfloat16 and m > SKINNY_MAX_ROWS // 2:
+        if ws is not None and x.dtype is torch.bfloat16 and m > RESIDUAL_NORM_MAX_ROWS:
             # few rows over a long k and few columns: the library cuts k into parts if it is lent room for their sums
             need = _work_bytes(m, n, k, _DT[x.dtype])
             if need:
