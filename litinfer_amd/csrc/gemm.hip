@@ -1131,14 +1131,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     };
     if constexpr (AHEAD) {
         if (wave < nchunks) load_chunk(wave, wbuf[0], xbuf[0]);
+        // the rows' sums of squares: thread t adds the parts t / 16, t / 16 + G, ... of row t % 16 in
+        // that order; the epilogue adds the G sums in theirs.  The loads are issued together, behind
+        // those of the first chunk, only as many rounds as there are parts, and never conditional
+        // within a round (a part past the end reads the last one).  They are added up behind the
+        // loads of the second chunk: the wait for them is the wait the first multiplication has anyway.
+        constexpr int G = WAVES * 4, PER = SK_MAX_PARTS / G;
+        float part[PER];
         if (a.row_parts) {
-            // the rows' sums of squares: thread t adds the parts t / 16, t / 16 + G, ... of row t % 16 in
-            // that order; the epilogue adds the G sums in theirs.  The loads are issued together, behind
-            // those of the first chunk, only as many rounds as there are parts, and never conditional
-            // within a round (a part past the end reads the last one).
-            constexpr int G = WAVES * 4, PER = SK_MAX_PARTS / G;
             const int m = threadIdx.x & 15, q = threadIdx.x >> 4;
-            float part[PER];
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
                 part[i] = 0.f;
@@ -1147,17 +1148,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                     part[i] = a.row_parts[(size_t)(p < a.nparts ? p : a.nparts - 1) * 16 + m];
                 }
             }
+        }
+        if (wave + WAVES < nchunks) load_chunk(wave + WAVES, wbuf[1], xbuf[1]);
+        if (a.row_parts) {
+            const int m = threadIdx.x & 15, q = threadIdx.x >> 4;
             float mine = 0.f;
 #pragma unroll
             for (int i = 0; i < PER; ++i) mine += (q + i * G < a.nparts) ? part[i] : 0.f;
             part_sums[q][m] = mine;
         }
-        for (int c = wave; c < nchunks; c += 2 * WAVES) {          // two chunks a turn: buffer numbers are constants
-            if (c + WAVES < nchunks) load_chunk(c + WAVES, wbuf[1], xbuf[1]);
-            multiply(wbuf[0], xbuf[0]);
-            if (c + WAVES >= nchunks) break;
-            if (c + 2 * WAVES < nchunks) load_chunk(c + 2 * WAVES, wbuf[0], xbuf[0]);
+        // (the first turn is written out: its loads of the second chunk stand above, before the parts are added up)
+        if (wave < nchunks) multiply(wbuf[0], xbuf[0]);
+        if (wave + WAVES < nchunks) {
+            if (wave + 2 * WAVES < nchunks) load_chunk(wave + 2 * WAVES, wbuf[0], xbuf[0]);
             multiply(wbuf[1], xbuf[1]);
+            for (int c = wave + 2 * WAVES; c < nchunks; c += 2 * WAVES) {      // two chunks a turn: buffer numbers are constants
+                if (c + WAVES < nchunks) load_chunk(c + WAVES, wbuf[1], xbuf[1]);
+                multiply(wbuf[0], xbuf[0]);
+                if (c + WAVES >= nchunks) break;
+                if (c + 2 * WAVES < nchunks) load_chunk(c + 2 * WAVES, wbuf[0], xbuf[0]);
+                multiply(wbuf[1], xbuf[1]);
+            }
         }
     } else {
         for (int c = wave; c < nchunks; c += WAVES) {
