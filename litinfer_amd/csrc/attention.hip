@@ -590,7 +590,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ tiles, const int* __restrict__ q_start,
     const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int page_size,
-    int num_pages, int window, float scale) {
+    int num_pages, int window, float scale, int ncu) {
     constexpr int KS = DH / 16;                 // MFMA steps of K Q^T (16 head dimensions each)
     constexpr int HD = DH / 2;                  // head dimensions owned by one lane half
     constexpr int DT = DH / 32;                 // tiles of 32 output dimensions
@@ -600,13 +600,22 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
     __shared__ __attribute__((aligned(16))) uint16_t Ks[2][32 * DH];      // [key][dimension], chunks swizzled by key
     __shared__ __attribute__((aligned(16))) uint16_t Vt[2][DH * VS];      // [dimension][key position]
     __shared__ int pages[PRE_TABLE_CAP];
-    // the last tiles of a long segment have the most keys: they are started first
-    const int tile = gridDim.x - 1 - blockIdx.x;
+    // The last tiles of a long segment have the most keys: they are started first.  Blocks are handed to
+    // the compute units in the order of their numbers, one each and then again from the first unit, and
+    // a unit's blocks share it: the work is dealt in a snake (every other round of `ncu` blocks backwards),
+    // so that the unit with the longest tile of one round gets the shortest of the next.
+    const int per_tile = gridDim.y * gridDim.z;
+    const int total = gridDim.x * per_tile;
+    const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const int round = lin / ncu, pos = lin - round * ncu;
+    const int in_round = total - round * ncu < ncu ? total - round * ncu : ncu;
+    const int item = round * ncu + ((round & 1) ? in_round - 1 - pos : pos);
+    const int tile = gridDim.x - 1 - item / per_tile;
     const int s = tiles[tile * 4], t0 = tiles[tile * 4 + 1], nrows = tiles[tile * 4 + 2];
-    const int kvh = blockIdx.y;
+    const int kvh = (item % per_tile) / gridDim.z;      // (the parts of a group of heads are neighbours: they read the same keys)
     const int G = nh / nkv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hw = blockIdx.z * PRE_WAVES + wave;       // this wave's head within the group
+    const int hw = ((item % per_tile) % gridDim.z) * PRE_WAVES + wave;       // this wave's head within the group
     const bool active = hw < G;                         // (idle waves still help to fetch and keep the barriers)
     const int head = kvh * G + (active ? hw : 0);
     const int ql = lane & 31, h = lane >> 5;
@@ -833,9 +842,14 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
     const int parts = (G + PRE_WAVES - 1) / PRE_WAVES;
     if (parts > 65535) return LI_ERR_SIZE;
     dim3 grid(ntiles, nkv, parts);
+    int dev = 0, ncu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || ncu <= 0) {
+        (void)hipGetLastError();
+        ncu = 256;
+    }
 #define LI_PRE(DHV) paged_attention_prefill_mfma_kernel<DHV><<<grid, PRE_WAVES * 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
-        tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale)
+        tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
     if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
 #undef LI_PRE
 #undef LI_PRE_FETCH
