@@ -103,6 +103,11 @@ def test_linear(ops, dtype, mnk, bias, acc):
     (32, 37, 264, False, torch.bfloat16, True, False),
     (33, 130, 1160, True, torch.bfloat16, False, False),
     (64, 50, 128, False, torch.float32, True, True),
+    (7, 2049, 72, False, torch.float32, True, True),            # few columns: 9 a block, the last block ragged
+    (16, 4100, 40, False, torch.bfloat16, True, False),         # 17 a block: two tiles, the second nearly empty
+    (12, 8191, 32, False, torch.bfloat16, False, False),        # 32 a block
+    (24, 4100, 72, False, torch.float32, True, True),           # the same shares with 17 to 32 rows
+    (30, 2500, 40, False, torch.bfloat16, False, False),
     (3, 9000, 64, False, torch.bfloat16, True, False),          # wide output: two tiles a wave
     (20, 9000, 520, False, torch.bfloat16, False, False),
 ])
@@ -546,6 +551,9 @@ def test_rope_kv_store_and_plain_store(ops, dtype, dh, pad):
     (1, 3, 1, 32, 96, True),
     (16, 5, 5, 48, 120, False),         # a head size that is no power of two
     (3, 6, 2, 64, 136, True),
+    (5, 35, 1, 80, 72, True),           # 1480 rotation pairs: 6 a block, blocks that straddle heads, a ragged last one
+    (16, 40, 8, 128, 64, False),        # 3584 pairs: 14 a block, two tiles
+    (2, 70, 1, 128, 40, True),          # more pairs than two tiles a compute unit hold: whole tiles again
 ])
 def test_projection_with_rotary_encoding_and_page_write_as_its_epilogue(ops, t, nh, nkv, dh, k, bias):
     g = torch.Generator().manual_seed(16)
