@@ -161,12 +161,13 @@ __global__ __launch_bounds__(256) void gemm_f32_big_kernel(const float* __restri
 }
 
 // ------------------------------------------------------ float32, few rows (decode)
-// The product streams W once: a wave owns NT consecutive columns of the output and
-// walks K with 16 bytes a lane; the MT rows of x come from the caches (every wave of the
-// grid reads the same few rows).  More than MT rows run as passes of MT; the passes of one
-// group of columns are neighbouring blocks, so that the second finds the matrix's rows in L2.
-// Each output element is the butterfly sum of its 64 lanes' strided partial sums: an order
-// that depends on K alone.
+// The product streams W once: a block owns up to NT consecutive columns of the output, its
+// four waves split K (wave v takes the 256 k-values 1024 i + 256 v ..., 16 bytes a lane), so
+// that a block reads the MT rows of x once, not once a wave: what a compute unit can take in
+// bounds these products, and x comes through the same path as W.  More than MT rows run as
+// passes of MT; the passes of one group of columns are neighbouring blocks, so that the second
+// finds the matrix's rows in L2.  Each output element is the sum, in wave order, of the four
+// waves' butterfly sums of their 64 lanes' strided partial sums: an order that depends on K alone.
 #define F32R_WAVES 4
 
 template <int MT, int NT>
@@ -174,12 +175,13 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
                                                                         const float* __restrict__ w,
                                                                         const float* __restrict__ bias,
                                                                         float* __restrict__ out, int M, int N, int K,
-                                                                        int accumulate, int npass) {
+                                                                        int accumulate, int npass, int cols) {
+    __shared__ float part[F32R_WAVES][MT * NT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pass = blockIdx.x % npass, group = blockIdx.x / npass;
-    const int n0 = (group * F32R_WAVES + wave) * NT;
+    const int n0 = group * cols;
+    const int nend = n0 + cols < N ? n0 + cols : N;
     const int m0 = pass * MT;
-    if (n0 >= N) return;
     float acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
@@ -187,11 +189,11 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
         for (int j = 0; j < NT; ++j) acc[i][j] = 0.f;
     const float* wrow[NT];
 #pragma unroll
-    for (int j = 0; j < NT; ++j) wrow[j] = w + (size_t)(n0 + j < N ? n0 + j : N - 1) * K;
+    for (int j = 0; j < NT; ++j) wrow[j] = w + (size_t)(n0 + j < nend ? n0 + j : nend - 1) * K;
     const float* xrow[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) xrow[i] = x + (size_t)(m0 + i < M ? m0 + i : M - 1) * K;
-    for (int k = 4 * lane; k < K; k += 256) {
+    for (int k = 4 * lane + 256 * wave; k < K; k += 256 * F32R_WAVES) {
         floatx4 wv[NT], xv[MT];
 #pragma unroll
         for (int j = 0; j < NT; ++j) wv[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(wrow[j] + k));
@@ -211,45 +213,43 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
             float v = acc[i][j];
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-            acc[i][j] = v;
+            if (lane == 0) part[wave][i * NT + j] = v;
         }
-    if (lane == 0) {
+    __syncthreads();
+    for (int t = threadIdx.x; t < MT * NT; t += F32R_WAVES * 64) {
+        const int i = t / NT, j = t - i * NT;
+        if (m0 + i >= M || n0 + j >= nend) continue;
+        float v = part[0][t];
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            if (m0 + i >= M) continue;
-#pragma unroll
-            for (int j = 0; j < NT; ++j)
-                if (n0 + j < N) epilogue_store(out, (size_t)(m0 + i) * N + n0 + j, acc[i][j], bias, n0 + j, accumulate != 0);
-        }
+        for (int v2 = 1; v2 < F32R_WAVES; ++v2) v += part[v2][t];
+        epilogue_store(out, (size_t)(m0 + i) * N + n0 + j, v, bias, n0 + j, accumulate != 0);
     }
 }
 
 #define F32_ROWS_MAX 64          // up to this many rows the row kernel is taken (K a multiple of 4)
 
+static int compute_units();
+
 static int launch_f32_rows(const float* x, const float* w, const float* bias, float* out, int M, int N, int K,
                            int accumulate, hipStream_t stream) {
     const int mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-    const int nt = (mt <= 8 && N >= 8192) ? 8 : 4;            // columns a wave owns: more where the matrix has many
+    const int nt = mt <= 8 ? 8 : 4;                           // columns a block owns at most (16 and 12 were slower)
     const int npass = (M + mt - 1) / mt;
-    const long groups = (N + F32R_WAVES * nt - 1) / (F32R_WAVES * nt);
+    // as many blocks as a whole number of rounds over the compute units, each with the same share of the columns
+    const int cu = compute_units();
+    const int rounds = (N + cu * nt - 1) / (cu * nt);
+    int cols = (N + cu * rounds - 1) / (cu * rounds);
+    if (cols < 1) cols = 1;
+    const long groups = (N + cols - 1) / cols;
     if (groups * npass > 0x7fffffffL) return LI_ERR_SIZE;
     const unsigned grid = (unsigned)(groups * npass);
-#define LI_F32R(MT, NT) gemm_f32_rows_kernel<MT, NT><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass)
-    if (nt == 8) {
-        switch (mt) {
-            case 1: LI_F32R(1, 8); break;
-            case 2: LI_F32R(2, 8); break;
-            case 4: LI_F32R(4, 8); break;
-            default: LI_F32R(8, 8); break;
-        }
-    } else {
-        switch (mt) {
-            case 1: LI_F32R(1, 4); break;
-            case 2: LI_F32R(2, 4); break;
-            case 4: LI_F32R(4, 4); break;
-            case 8: LI_F32R(8, 4); break;
-            default: LI_F32R(16, 4); break;
-        }
+#define LI_F32R(MT, NT) gemm_f32_rows_kernel<MT, NT><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass, cols)
+    switch (mt) {
+        case 1: LI_F32R(1, 8); break;
+        case 2: LI_F32R(2, 8); break;
+        case 4: LI_F32R(4, 8); break;
+        case 8: LI_F32R(8, 8); break;
+        default: LI_F32R(16, 4); break;
     }
 #undef LI_F32R
     return li_launch_status();
