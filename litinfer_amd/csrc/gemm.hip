@@ -588,7 +588,7 @@ __device__ __forceinline__ void static_for(F&& f) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"                          \
                  :: "s"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(lptr)), "v"(voff), "s"(base) : "memory", "m0")
 
-template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO>
+template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO, int WLM = 2>
 __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __restrict__ x,
                                                              const bf16_t* __restrict__ w,
                                                              const float* __restrict__ bias,
@@ -596,7 +596,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                                                              int accumulate) {
     // gridDim.y > 1: block (., y) multiplies the y-th part of K and writes its sums to the y-th
     // [M, N] matrix behind `out` (float, no bias, no accumulation); splitk_reduce_kernel adds them
-    constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    // WLM: waves along the rows of the tile, 2 (two by two) or 4 (each wave 32-row bands over all columns:
+    // BN may then be any multiple of 32, for matrices whose columns no other tile divides into 256 tiles)
+    constexpr int WLN = 4 / WLM;
+    constexpr int WM = BM / WLM, WN = BN / WLN, TM = WM / 32, TN = WN / 32;
+    static_assert(WM % 32 == 0 && WN % 32 == 0 && (WLM == 2 || WLM == 4), "a wave's part of the tile is made of 32 x 32 tiles");
+    static_assert(BM % 32 == 0 && BN % 32 == 0 && (BM / 4) % (64 / (BK / 8)) == 0 && (BN / 4) % (64 / (BK / 8)) == 0, "whole load instructions a wave");
     constexpr int CPR = BK / 8, WRAP = 128 / BK;                 // chunks in a row; rows that fill all banks once
     constexpr int RPI = 64 / CPR;                                // rows one load instruction of a wave covers
     constexpr int IA = BM / 4 / RPI, IB = BN / 4 / RPI;          // load instructions per wave and step for A and B
@@ -604,7 +609,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     constexpr int LPW = IA + IB;                                 // loads a wave issues per step
     extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    const int wm = (wave / WLN) * WM, wn = (wave % WLN) * WN;
     const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
     int mt, nt;
     if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, mt, nt)) return;
@@ -740,11 +745,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
             });
         });
         constexpr int BL = (KS - 1) & 1;           // the buffer with the fragments of the last 16 columns
+        constexpr int HALF = (TM / 2) * TN > 0 ? (TM / 2) * TN : GM / 2;       // MFMAs of the last group before the wait
 #pragma unroll
-        for (int i = 0; i < TM / 2; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][i], bfr[BL][j], acc[i][j], 0, 0, 0);
+        for (int m = 0; m < HALF; ++m)
+            acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][m / TN], bfr[BL][m % TN], acc[m / TN][m % TN], 0, 0, 0);
         if (kt + 1 < nk) {
             // loads of later steps that may stay in flight: steps kt + 2 .. kt + NSTAGE - 1, where they exist
             const int younger = LOADS ? NSTAGE - 2 : (nk - 2 - kt < NSTAGE - 2 ? nk - 2 - kt : NSTAGE - 2);
@@ -757,10 +761,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
             LI_FREAD((kt + 1) % NSTAGE, 0, 0)
         }
 #pragma unroll
-        for (int i = TM / 2; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][i], bfr[BL][j], acc[i][j], 0, 0, 0);
+        for (int m = HALF; m < GM; ++m)
+            acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[BL][m / TN], bfr[BL][m % TN], acc[m / TN][m % TN], 0, 0, 0);
     };
     int kt = 0;
     if constexpr (SPREAD)
@@ -771,6 +773,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     __syncthreads();                               // the main loop's LDS is free now
     constexpr int EW = SWIGLU ? WN / 2 : WN;        // output columns of a wave
     constexpr int ESTRIDE = EW + 4;
+    static_assert(4 * 32 * ESTRIDE * 4 <= NSTAGE * STAGE * 2, "the waves' bands fit the main loop's LDS");
     float* band = reinterpret_cast<float*>(lds) + wave * 32 * ESTRIDE;
     const int ccol = lane & 31, crow = (lane >> 5) * 4;
     constexpr int LPR = EW / 8, RPP = 64 / LPR;     // lanes a row of the band takes; rows a pass of the wave covers
@@ -835,7 +838,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     }
 }
 
-template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO>
+template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO, int WLM = 2>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream, int nsplit = 1) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
@@ -848,12 +851,12 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
     constexpr int lds_bytes = NSTAGE * (BM + BN) * BK * 2;
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO>,
+        if (hipFuncSetAttribute((const void*)gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO, WLM>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
             return LI_ERR_LAUNCH;
         configured = true;
     }
-    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO><<<dim3((unsigned)(per_xcd * 8), nsplit), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
+    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO, WLM><<<dim3((unsigned)(per_xcd * 8), nsplit), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
     return li_launch_status();
 }
 
@@ -1492,7 +1495,7 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
             if (out_dtype != LI_F32 && out_dtype != LI_BF16) return LI_ERR_DTYPE;
 #define LI_DMA(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, false, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                                : launch_dma<BM, BN, BK, NS, false, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
-            // Four tilings; the one with the least (rounds of blocks over the 256 compute units) x
+            // Six tilings; the one with the least (rounds of blocks over the 256 compute units) x
             // (area of a tile) / (its measured relative speed) is taken: large tiles are the fastest
             // per multiply-add but leave compute units idle when the matrix has few of them.
             if (K % 64 == 0) {
@@ -1513,7 +1516,16 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
                 };
                 const double c_large = cost(256, 256, 1.0), c_wide = cost(256, 192, 0.97), c_mid = cost(256, 128, 0.95),
                              c_small = cost(128, 128, 0.8);
-                const double best = std::min(std::min(c_large, c_wide), std::min(c_mid, c_small));
+#define LI_DMA4(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, false, float, 4>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
+                                                : launch_dma<BM, BN, BK, NS, false, bf16_t, 4>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
+                // (tiles of 128 rows with four waves one above the other: slower per multiply-add, their LDS reads
+                // take as long as their MFMAs, but 224 or 288 columns cut 3,584 or 4,608 into exactly as many
+                // tiles as 2,048 rows need to give every compute unit one)
+                const double c_224 = cost(128, 224, 0.87), c_288 = cost(128, 288, 0.87);
+                const double best = std::min(std::min(std::min(c_large, c_wide), std::min(c_mid, c_small)), std::min(c_224, c_288));
+                if (c_224 == best) return LI_DMA4(128, 224, 64, 3);
+                if (c_288 == best) return LI_DMA4(128, 288, 64, 3);
+#undef LI_DMA4
                 if (c_large == best) return LI_DMA(256, 256, 64, 2);
                 if (c_wide == best) return LI_DMA(256, 192, 64, 2);
                 if (c_mid == best) return LI_DMA(256, 128, 64, 3);

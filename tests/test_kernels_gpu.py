@@ -73,7 +73,8 @@ def test_rmsnorm_zero_row_is_zero_not_nan(ops):
     ((8, 4608, 3584), True, False), ((65, 50, 128), False, True),
     ((1, 1000, 3584), True, False), ((16, 70, 260), True, True), ((40, 19, 100), False, True),      # few rows in 32-bit
     ((9, 18, 4), True, False),
-    ((300, 200, 130), True, True), ((256, 128, 64), False, False), ((1000, 333, 1027), True, False)])     # the large 32-bit tile
+    ((300, 200, 130), True, True), ((256, 128, 64), False, False), ((1000, 333, 1027), True, False),     # the large 32-bit tile
+    ((2048, 3584, 128), True, True), ((2000, 4600, 64), True, False)])          # tiles of 128 x 224 and 128 x 288, ragged
 def test_linear(ops, dtype, mnk, bias, acc):
     m, n, k = mnk
     g = torch.Generator().manual_seed(2)
