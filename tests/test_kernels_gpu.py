@@ -110,6 +110,10 @@ def test_linear(ops, dtype, mnk, bias, acc):
     (24, 4100, 72, False, torch.float32, True, True),           # the same shares with 17 to 32 rows
     (30, 2500, 40, False, torch.bfloat16, False, False),
     (3, 9000, 64, False, torch.bfloat16, True, False),          # wide output: two tiles a wave
+    (16, 8200, 1160, False, torch.float32, True, True),         # wide outputs at other sizes
+    (7, 40000, 264, False, torch.float32, False, False),
+    (11, 8300, 520, True, torch.bfloat16, False, False),
+    (1, 152064, 64, False, torch.float32, False, False),
     (20, 9000, 520, False, torch.bfloat16, False, False),
 ])
 def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, acc):
@@ -247,6 +251,8 @@ def test_linear_with_swiglu_epilogue(ops, m, n, k):
     (1, 40, 8, 24, 1e-5),
     (16, 8200, 64, 48, 1e-5),        # a width from which the product before takes 32 columns a block; ragged
     (5, 200, 136, 301, 0.1),         # a ragged last block of 16 columns; an eps that counts
+    (9, 264, 72, 8210, 1e-5),        # many outputs, ragged; fewer chunks of K than waves
+    (4, 1096, 40, 9000, 1e-6),
 ])
 def test_rms_norm_shared_between_the_products_on_its_two_sides(ops, m, n, kprev, inter, eps):
     """x += h Wo^T leaves gamma * x and the shares of the rows' sums of squares; the gate/up product
