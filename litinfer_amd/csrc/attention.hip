@@ -829,10 +829,13 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
         }
 }
 
+#undef LI_PRE_FETCH
+#undef LI_PRE_ROW
+#undef LI_PRE_STASH
 // The same with the loads of K and V going straight into LDS (no registers, no transposing on the way in:
 // that way of filling LDS took as long as the arithmetic) and V turned by the LDS read that transposes
 // 16-bit elements (ds_read_b64_tr_b16).  Three stages of LDS, so a block of keys has two turns to arrive.
-#define PRE2_TABLE_CAP 4096
+#define PRE2_TABLE_CAP 2048
 typedef short tr4 __attribute__((ext_vector_type(4)));
 #define LI_ATT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 // (inline assembly, so that the compiler neither counts these loads nor waits for them before LDS
@@ -840,7 +843,8 @@ typedef short tr4 __attribute__((ext_vector_type(4)));
 #define LI_ATT_LOAD_TO_LDS(gptr, lptr)                                                                    \
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"                        \
                  :: "s"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(lptr)), "v"(gptr) : "memory", "m0")
-template <int DH>
+// P32: the page size divides 32, so a row keeps its place in its page from block to block
+template <int DH, bool P32>
 __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
@@ -855,7 +859,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     constexpr int NST = 3;                      // stages of LDS: one worked on, two on their way
     __shared__ __attribute__((aligned(16))) uint16_t Ks[NST][32 * DH];    // [key][dimension], chunks swizzled by key
     __shared__ __attribute__((aligned(16))) uint16_t Vs[NST][32 * DH];    // the same for V, another swizzle
-    __shared__ int pages[PRE2_TABLE_CAP];
+    __shared__ unsigned long long pageoff[PRE2_TABLE_CAP];                // byte offset of each page of the tile's part of the table
     // The last tiles of a long segment have the most keys: they are started first.  Blocks are handed to
     // the compute units in the order of their numbers, one each and then again from the first unit, and
     // a unit's blocks share it: the work is dealt in a snake (every other round of `ncu` blocks backwards),
@@ -882,7 +886,13 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     const int first_block = lo0 / page_size;
     const int nblocks = (k_end - 1) / page_size - first_block + 1;     // <= PRE2_TABLE_CAP (checked by the host)
     const int* table = block_table + (size_t)s * max_blocks + first_block;
-    for (int i = tid; i < nblocks; i += NT) pages[i] = table[i];
+    const size_t page_bytes = (size_t)nkv * page_size * DH * 2;
+    for (int i = tid; i < nblocks; i += NT) {
+        int pg = table[i];
+        pg = pg < 0 ? 0 : (pg >= num_pages ? num_pages - 1 : pg);
+        pageoff[i] = (unsigned long long)(unsigned)pg * page_bytes;
+    }
+    const int last_entry = nblocks - 1;
     __syncthreads();
     // ---- fetching a block of 32 keys: the loads go straight into LDS (16 bytes a lane, a wave's
     // 64 lanes to 1 KB in a row), so a stage's K and V are [key][16-byte chunk] in the order of
@@ -897,6 +907,10 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     constexpr int NL = (32 * CPR) / NT;                 // loads of K (and of V) a thread makes per block
     static_assert(NL * NT == 32 * CPR, "whole load instructions a block of keys");
     int row_blk[NL], row_in[NL], kcol[NL], vcol[NL];
+    const char* kbase = reinterpret_cast<const char*>(kc) + (size_t)kvh * page_size * DH * 2;
+    const char* vbase = reinterpret_cast<const char*>(vc) + (size_t)kvh * page_size * DH * 2;
+    const char* krow[NL];                               // P32: the row's place in its page and its chunk, once and for all
+    const char* vrow[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         const int ci = 64 * (NL * wave + i) + lane, key = ci / CPR, place = ci % CPR;
@@ -905,25 +919,32 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
         const int kk = k_begin + key;
         row_blk[i] = kk / page_size - first_block;
         row_in[i] = kk % page_size;
+        krow[i] = kbase + (size_t)(row_in[i] * DH + kcol[i]) * 2;
+        vrow[i] = vbase + (size_t)(row_in[i] * DH + vcol[i]) * 2;
     }
     const int step_blk = 32 / page_size, step_in = 32 % page_size;      // a turn moves every row 32 keys on
-    const size_t page_bytes = (size_t)nkv * page_size * DH * 2;
-    const char* kbase = reinterpret_cast<const char*>(kc) + (size_t)kvh * page_size * DH * 2;
-    const char* vbase = reinterpret_cast<const char*>(vc) + (size_t)kvh * page_size * DH * 2;
     const int uwave = __builtin_amdgcn_readfirstlane(wave);
     // (fetches are made for consecutive blocks: k_begin, k_begin + 32, ...)
 #define LI_PRE_FETCH(stage)                                                                          \
     {                                                                                                \
+        unsigned long long off_[NL];                                                                 \
         _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                             \
-            int ix_ = row_blk[i] < 0 ? 0 : (row_blk[i] > PRE2_TABLE_CAP - 1 ? PRE2_TABLE_CAP - 1 : row_blk[i]); \
-            int page_ = pages[ix_];                                                                  \
-            page_ = page_ < 0 ? 0 : (page_ >= num_pages ? num_pages - 1 : page_);                    \
-            const size_t off_ = (size_t)(unsigned)page_ * page_bytes + (unsigned)(row_in[i] * DH * 2); \
-            row_in[i] += step_in;                                                                    \
-            row_blk[i] += step_blk;                                                                  \
-            if (row_in[i] >= page_size) { row_in[i] -= page_size; row_blk[i] += 1; }                 \
-            LI_ATT_LOAD_TO_LDS(kbase + off_ + 2 * kcol[i], &Ks[stage][512 * (NL * uwave + i)]);      \
-            LI_ATT_LOAD_TO_LDS(vbase + off_ + 2 * vcol[i], &Vs[stage][512 * (NL * uwave + i)]);      \
+            const int ix_ = row_blk[i] < 0 ? 0 : (row_blk[i] > last_entry ? last_entry : row_blk[i]); \
+            off_[i] = pageoff[ix_];                                                                  \
+        }                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                             \
+            if constexpr (P32) {                                                                     \
+                row_blk[i] += step_blk;                                                              \
+                LI_ATT_LOAD_TO_LDS(krow[i] + off_[i], &Ks[stage][512 * (NL * uwave + i)]);           \
+                LI_ATT_LOAD_TO_LDS(vrow[i] + off_[i], &Vs[stage][512 * (NL * uwave + i)]);           \
+            } else {                                                                                 \
+                const size_t o_ = off_[i] + (unsigned)(row_in[i] * DH * 2);                          \
+                row_in[i] += step_in;                                                                \
+                row_blk[i] += step_blk;                                                              \
+                if (row_in[i] >= page_size) { row_in[i] -= page_size; row_blk[i] += 1; }             \
+                LI_ATT_LOAD_TO_LDS(kbase + o_ + 2 * kcol[i], &Ks[stage][512 * (NL * uwave + i)]);    \
+                LI_ATT_LOAD_TO_LDS(vbase + o_ + 2 * vcol[i], &Vs[stage][512 * (NL * uwave + i)]);    \
+            }                                                                                        \
         }                                                                                            \
     }
     // ---- this wave's queries
@@ -1090,12 +1111,14 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
 #define LI_PRE(DHV) paged_attention_prefill_mfma_kernel<DHV><<<grid, PRE_WAVES * 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
         tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
-#define LI_PRE2(DHV) paged_attention_prefill_dma_kernel<DHV><<<grid, PRE_WAVES * 64, 0, stream>>>( \
+#define LI_PRE2(DHV, P32V) paged_attention_prefill_dma_kernel<DHV, P32V><<<grid, PRE_WAVES * 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
         tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
-    static const bool old_form = getenv("LI_EXP_OLDPRE") != nullptr;
-    if (max_blocks <= PRE2_TABLE_CAP && !old_form) {          // (longer block tables: the form that keeps 8,192 entries in LDS)
-        if (dh == 128) LI_PRE2(128); else if (dh == 64) LI_PRE2(64); else return LI_ERR_SIZE;
+    if (max_blocks <= PRE2_TABLE_CAP) {                       // (longer block tables: the form that keeps 8,192 entries in LDS)
+        const bool p32 = 32 % page_size == 0;
+        if (dh == 128) { if (p32) LI_PRE2(128, true); else LI_PRE2(128, false); }
+        else if (dh == 64) { if (p32) LI_PRE2(64, true); else LI_PRE2(64, false); }
+        else return LI_ERR_SIZE;
     } else
     if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
 #undef LI_PRE2
