@@ -459,6 +459,11 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
     ([(700, 700), (40, 3), (513, 1), (300, 17)], 28, 4, 128, 16, 0),    # portions on the matrix cores
     ([(257, 100), (90, 90), (64, 33)], 20, 2, 64, 8, 50),           # 10 heads a group (two turns of waves), window
     ([(2, 2), (17, 16), (33, 2)], 3, 3, 128, 16, 0),
+    ([(500, 300), (70, 70), (45, 2)], 8, 2, 128, 12, 0),            # page sizes that do not divide a block of 32 keys
+    ([(400, 150), (130, 130)], 6, 3, 128, 64, 90),                  # pages longer than a block of keys, window
+    ([(333, 200), (64, 5)], 10, 2, 64, 5, 0),
+    ([(300, 300), (100, 9)], 4, 1, 64, 24, 40),
+    ([(1, 1), (3000, 700)], 14, 2, 128, 1, 0),                      # one key a page: a long table
 ])
 def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     out, ref = _paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=6)
