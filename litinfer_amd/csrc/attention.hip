@@ -835,7 +835,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
 // The same with the loads of K and V going straight into LDS (no registers, no transposing on the way in:
 // that way of filling LDS took as long as the arithmetic) and V turned by the LDS read that transposes
 // 16-bit elements (ds_read_b64_tr_b16).  Three stages of LDS, so a block of keys has two turns to arrive.
-#define PRE2_TABLE_CAP 2048
+#define PRE2_TABLE_CAP 4096
 typedef short tr4 __attribute__((ext_vector_type(4)));
 #define LI_ATT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | 0x0F70)
 // (inline assembly, so that the compiler neither counts these loads nor waits for them before LDS
@@ -859,7 +859,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     constexpr int NST = 3;                      // stages of LDS: one worked on, two on their way
     __shared__ __attribute__((aligned(16))) uint16_t Ks[NST][32 * DH];    // [key][dimension], chunks swizzled by key
     __shared__ __attribute__((aligned(16))) uint16_t Vs[NST][32 * DH];    // the same for V, another swizzle
-    __shared__ unsigned long long pageoff[PRE2_TABLE_CAP];                // byte offset of each page of the tile's part of the table
+    __shared__ uint32_t pageoff[PRE2_TABLE_CAP];                          // byte offset / 128 of each page of the tile's part of the table
     // The last tiles of a long segment have the most keys: they are started first.  Blocks are handed to
     // the compute units in the order of their numbers, one each and then again from the first unit, and
     // a unit's blocks share it: the work is dealt in a snake (every other round of `ncu` blocks backwards),
@@ -890,7 +890,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     for (int i = tid; i < nblocks; i += NT) {
         int pg = table[i];
         pg = pg < 0 ? 0 : (pg >= num_pages ? num_pages - 1 : pg);
-        pageoff[i] = (unsigned long long)(unsigned)pg * page_bytes;
+        pageoff[i] = (uint32_t)(((unsigned long long)(unsigned)pg * page_bytes) >> 7);     // (a page is a multiple of 128 bytes: dh >= 64; 512 GB of cache)
     }
     const int last_entry = nblocks - 1;
     __syncthreads();
@@ -930,7 +930,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
         unsigned long long off_[NL];                                                                 \
         _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                             \
             const int ix_ = row_blk[i] < 0 ? 0 : (row_blk[i] > last_entry ? last_entry : row_blk[i]); \
-            off_[i] = pageoff[ix_];                                                                  \
+            off_[i] = (unsigned long long)pageoff[ix_] << 7;                                         \
         }                                                                                            \
         _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                             \
             if constexpr (P32) {                                                                     \
