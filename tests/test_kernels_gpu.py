@@ -463,7 +463,8 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
     ([(400, 150), (130, 130)], 6, 3, 128, 64, 90),                  # pages longer than a block of keys, window
     ([(333, 200), (64, 5)], 10, 2, 64, 5, 0),
     ([(300, 300), (100, 9)], 4, 1, 64, 24, 40),
-    ([(1, 1), (3000, 700)], 14, 2, 128, 1, 0),                      # one key a page: a table too long for the kernel that keeps offsets in LDS
+    ([(1, 1), (3000, 700)], 14, 2, 128, 1, 0),                      # one key a page: a long table
+    ([(5000, 300)], 4, 2, 128, 1, 0),                               # a table too long for the kernel that keeps the pages' offsets in LDS
     ([(1500, 400), (9, 9)], 7, 1, 128, 1, 0),                       # one key a page, within its table
 ])
 def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
