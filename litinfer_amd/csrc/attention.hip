@@ -1090,6 +1090,284 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
         }
 }
 
+#undef LI_PRE_FETCH
+// The same for prompts of so few tiles that a compute unit holds one or two blocks and the time is that of
+// the longest tile, one block of keys after the other: eight waves a block, two groups of four, each group
+// with its own stages of LDS takes half of the tile's blocks of keys (the first half, the second half), and
+// at the end the second group hands its sums, maxima and outputs to the first through LDS.
+template <int DH, bool P32>
+__global__ __launch_bounds__(2 * PRE_WAVES * 64) void paged_attention_prefill_split_kernel(
+    const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
+    const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
+    int max_blocks, const int* __restrict__ tiles, const int* __restrict__ q_start,
+    const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int page_size,
+    int num_pages, int window, float scale, int ncu) {
+    constexpr int KS = DH / 16;                 // MFMA steps of K Q^T (16 head dimensions each)
+    constexpr int HD = DH / 2;                  // head dimensions owned by one lane half
+    constexpr int DT = DH / 32;                 // tiles of 32 output dimensions
+    constexpr int CPR = DH / 8;                 // 16-byte chunks in a row of K
+    constexpr int NT = PRE_WAVES * 64;
+    constexpr int NST = 3;                      // stages of LDS: one worked on, two on their way
+    __shared__ __attribute__((aligned(16))) uint16_t kv[2][2][NST][32 * DH];   // [K, V][group][stage][key][dimension], chunks swizzled by key
+    __shared__ uint32_t pageoff[PRE2_TABLE_CAP];                          // byte offset / 128 of each page of the tile's part of the table
+    // The last tiles of a long segment have the most keys: they are started first.  Blocks are handed to
+    // the compute units in the order of their numbers, one each and then again from the first unit, and
+    // a unit's blocks share it: the work is dealt in a snake (every other round of `ncu` blocks backwards),
+    // so that the unit with the longest tile of one round gets the shortest of the next.
+    const int per_tile = gridDim.y * gridDim.z;
+    const int total = gridDim.x * per_tile;
+    const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const int round = lin / ncu, pos = lin - round * ncu;
+    const int in_round = total - round * ncu < ncu ? total - round * ncu : ncu;
+    const int item = round * ncu + ((round & 1) ? in_round - 1 - pos : pos);
+    const int tile = gridDim.x - 1 - item / per_tile;
+    const int s = tiles[tile * 4], t0 = tiles[tile * 4 + 1], nrows = tiles[tile * 4 + 2];
+    const int kvh = (item % per_tile) / gridDim.z;      // (the parts of a group of heads are neighbours: they read the same keys)
+    const int G = nh / nkv;
+    const int tid = threadIdx.x, lane = tid & 63, half = tid >> 8, wave = (tid >> 6) & 3;     // group of waves, wave within it
+    const int hw = ((item % per_tile) % gridDim.z) * PRE_WAVES + wave;       // this wave's head within the group
+    const bool active = hw < G;                         // (idle waves still help to fetch and keep the barriers)
+    const int head = kvh * G + (active ? hw : 0);
+    const int ql = lane & 31, h = lane >> 5;
+    const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);           // position of the tile's first token
+    const int p_last = p0 + nrows - 1;
+    const int lo0 = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+    const int k_begin = lo0 & ~31, k_end = p_last + 1;
+    const int first_block = lo0 / page_size;
+    const int nblocks = (k_end - 1) / page_size - first_block + 1;     // <= PRE2_TABLE_CAP (checked by the host)
+    const int* table = block_table + (size_t)s * max_blocks + first_block;
+    const size_t page_bytes = (size_t)nkv * page_size * DH * 2;
+    for (int i = tid; i < nblocks; i += 2 * NT) {
+        int pg = table[i];
+        pg = pg < 0 ? 0 : (pg >= num_pages ? num_pages - 1 : pg);
+        pageoff[i] = (uint32_t)(((unsigned long long)(unsigned)pg * page_bytes) >> 7);     // (a page is a multiple of 128 bytes: dh >= 64; 512 GB of cache)
+    }
+    const int last_entry = nblocks - 1;
+    __syncthreads();
+    const int nblk = (k_end - k_begin + 31) / 32;        // blocks of 32 keys of the tile
+    const int n0 = (nblk + 1) / 2;                       // ... of the first group; turns of the loop
+    const int nb = half ? nblk - n0 : n0;                // ... of this group
+    const int kb0 = k_begin + 32 * n0 * half;            // this group's first key
+    // ---- fetching a block of 32 keys: the loads go straight into LDS (16 bytes a lane, a wave's
+    // 64 lanes to 1 KB in a row), so a stage's K and V are [key][16-byte chunk] in the order of
+    // the lanes: chunk index ci = 64 (NL wave + i) + lane, key ci / CPR, place ci % CPR.  The
+    // bank swizzle is made on the way in: the place holds the chunk (place ^ swizzle(key)) of the
+    // key's row, for K swizzle = key % CPR, for V 2 (key % 8) (% CPR), see the reads below.
+    // A thread fetches the same rows of every block, 32 keys further on each turn: it keeps each
+    // row's page block and place in the page and moves them on without a division; K and V of a
+    // row lie at the same place of their cache layers.  Rows before the first or past the last
+    // key of the tile (their scores are masked) read whatever page the clamped table entry
+    // names: the cache holds finite numbers everywhere.
+    constexpr int NL = (32 * CPR) / NT;                 // loads of K (and of V) a thread makes per block
+    static_assert(NL * NT == 32 * CPR, "whole load instructions a block of keys");
+    int row_blk[NL], row_in[NL], kcol[NL], vcol[NL];
+    const char* kbase = reinterpret_cast<const char*>(kc) + (size_t)kvh * page_size * DH * 2;
+    const char* vbase = reinterpret_cast<const char*>(vc) + (size_t)kvh * page_size * DH * 2;
+    const char* krow[NL];                               // P32: the row's place in its page and its chunk, once and for all
+    const char* vrow[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int ci = 64 * (NL * wave + i) + lane, key = ci / CPR, place = ci % CPR;
+        kcol[i] = 8 * (place ^ (key & (CPR - 1)));
+        vcol[i] = 8 * (place ^ ((2 * (key & 7)) & (CPR - 1)));
+        const int kk = kb0 + key;
+        row_blk[i] = kk / page_size - first_block;
+        row_in[i] = kk % page_size;
+        krow[i] = kbase + (size_t)(row_in[i] * DH + kcol[i]) * 2;
+        vrow[i] = vbase + (size_t)(row_in[i] * DH + vcol[i]) * 2;
+    }
+    const int step_blk = 32 / page_size, step_in = 32 % page_size;      // a turn moves every row 32 keys on
+    const int uwave = __builtin_amdgcn_readfirstlane(wave), uhalf = __builtin_amdgcn_readfirstlane(half);
+    // (fetches are made for consecutive blocks: k_begin, k_begin + 32, ...)
+#define LI_PRE_FETCH(stage)                                                                          \
+    {                                                                                                \
+        unsigned long long off_[NL];                                                                 \
+        _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                             \
+            const int ix_ = row_blk[i] < 0 ? 0 : (row_blk[i] > last_entry ? last_entry : row_blk[i]); \
+            off_[i] = (unsigned long long)pageoff[ix_] << 7;                                         \
+        }                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < NL; ++i) {                                             \
+            if constexpr (P32) {                                                                     \
+                row_blk[i] += step_blk;                                                              \
+                LI_ATT_LOAD_TO_LDS(krow[i] + off_[i], &kv[0][uhalf][stage][512 * (NL * uwave + i)]);           \
+                LI_ATT_LOAD_TO_LDS(vrow[i] + off_[i], &kv[1][uhalf][stage][512 * (NL * uwave + i)]);           \
+            } else {                                                                                 \
+                const size_t o_ = off_[i] + (unsigned)(row_in[i] * DH * 2);                          \
+                row_in[i] += step_in;                                                                \
+                row_blk[i] += step_blk;                                                              \
+                if (row_in[i] >= page_size) { row_in[i] -= page_size; row_blk[i] += 1; }             \
+                LI_ATT_LOAD_TO_LDS(kbase + o_ + 2 * kcol[i], &kv[0][uhalf][stage][512 * (NL * uwave + i)]);    \
+                LI_ATT_LOAD_TO_LDS(vbase + o_ + 2 * vcol[i], &kv[1][uhalf][stage][512 * (NL * uwave + i)]);    \
+            }                                                                                        \
+        }                                                                                            \
+    }
+    // ---- this wave's queries
+    frag8 qf[KS];
+    {
+        const bf16_t* qrow = q + (size_t)(t0 + (ql < nrows ? ql : nrows - 1)) * q_row_stride + (size_t)head * DH + HD * h;
+#pragma unroll
+        for (int st = 0; st < KS; ++st) qf[st].raw = *reinterpret_cast<const u32x4*>(qrow + 8 * st);
+    }
+    const int pq = p0 + (ql < nrows ? ql : nrows - 1);       // last visible key of this lane's query (lanes past the tile repeat its last row)
+    const int lq = (window > 0 && pq - window + 1 > 0) ? pq - window + 1 : 0;
+    const int l_last = (window > 0 && p_last - window + 1 > 0) ? p_last - window + 1 : 0;
+    const float scale2 = scale * 1.44269504088896341f;                       // scores in units of log 2
+    f32x16_t acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    // Order of a turn: the block two on is asked for, into the stage that the turn before read
+    // (its readers are past the barrier); then the block in this stage is worked on; then the wave
+    // waits for its own loads of the NEXT block (the loads of the block after it may stay in
+    // flight: a wave's loads retire in order) and meets the others at the barrier.
+    if (nb > 0) LI_PRE_FETCH(0);
+    if (nb > 1) { LI_PRE_FETCH(1); LI_ATT_VMCNT(2 * NL); } else { LI_ATT_VMCNT(0); }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // where this lane reads its fragments of K in a stage (the swizzle depends on the lane only)
+    int kaddr[KS];
+#pragma unroll
+    for (int st = 0; st < KS; ++st) kaddr[st] = ql * DH + ((((HD / 8) * h + st) ^ (ql & (CPR - 1))) << 3);
+    // where this lane reads V for the row operand of O^T = V^T P^T.  The transposing LDS read (64
+    // bits a lane) hands lane i of a group of 16 the element i % 4 of the 4 x 16-bit pieces that the
+    // group's lanes 4 j + i / 4 point at, j = 0 .. 3.  Lane i of a group points at key base + i / 4,
+    // dimensions d0 + 4 (i % 4) ..: it receives the keys base .. base + 3 of dimension d0 + i.  The
+    // lane's group gives d0 (16 (group % 2) within the tile of 32) and the k-group (group / 2), whose
+    // 8 keys of MFMA step st are 16 st + 4 h + {0 .. 3} and 16 st + 8 + 4 h + {0 .. 3}: two reads.
+    // With the swizzle 2 (key % 8) the four keys of a read lie in eight different 16-byte columns.
+    int vaddr[DT];
+    {
+        const int gi = lane & 15, grp = lane >> 4;
+        const int vkey = 4 * (grp >> 1) + (gi >> 2);            // + 16 st + 8 r: the swizzle does not see those
+        const int swz = (2 * (vkey & 7)) & (CPR - 1);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int chunk = 4 * dt + 2 * (grp & 1) + ((gi & 3) >> 1);
+            vaddr[dt] = vkey * DH + 8 * (chunk ^ swz) + 4 * (gi & 1);
+        }
+    }
+    // three turns a trip, so that the stage is a constant of the code and the LDS addresses are
+    // a register plus an immediate
+    for (int j3 = 0; j3 < n0; j3 += NST) {
+#pragma unroll
+      for (int stage = 0; stage < NST; ++stage) {
+        const int jb = j3 + stage;
+        if (jb >= n0) break;
+        const int kb = kb0 + 32 * jb;
+        if (jb + 2 < nb) LI_PRE_FETCH((stage + 2) % NST);
+        if (active && jb < nb) {                         // (the second group may have a block less: it keeps the barriers)
+            // ---- S^T = K Q^T
+            f32x16_t sv;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sv[r] = 0.f;
+            frag8 kf[KS];
+#pragma unroll
+            for (int st = 0; st < KS; ++st) kf[st].raw = *reinterpret_cast<const u32x4*>(&kv[0][half][stage][kaddr[st]]);
+#pragma unroll
+            for (int st = 0; st < KS; ++st) sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st].v, qf[st].v, sv, 0, 0, 0);
+            // ---- softmax over the keys of this lane's query.  The running maximum m is only moved
+            // (and the sums so far rescaled, for the whole wave) when some query's scores pass it by
+            // more than 2^8: until then the exponentials are taken against the older maximum, which
+            // changes no result (numerator and denominator carry the same factor) and stays far
+            // inside the range of float and bfloat16.
+            // A block that every query of the tile sees whole (most are) needs no masks.
+            if (!(kb + 31 <= p0 && kb >= l_last)) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = kb + 8 * (r >> 2) + 4 * h + (r & 3);
+                    sv[r] = (key <= pq && key >= lq) ? sv[r] : -INFINITY;
+                }
+            }
+            float mx = max3f(sv[0], sv[1], sv[2]);
+#pragma unroll
+            for (int r = 3; r < 15; r += 2) mx = max3f(mx, sv[r], sv[r + 1]);
+            mx = max3f(mx, sv[15], sv[15]);
+            mx = max3f(mx, __shfl_xor(mx, 32, LI_WAVE), mx) * scale2;   // (scale2 > 0)
+            if (__any(mx > m + 8.0f)) {
+                const float mn = fmaxf(m, mx);
+                const float alpha = (mn == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - mn);   // (m = -inf: nothing summed yet)
+                l *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
+                m = mn;
+            }
+            const float ms = (m == -INFINITY) ? 0.f : m;         // a query may see no key yet
+            float ps = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { sv[r] = __builtin_amdgcn_exp2f(fmaf(sv[r], scale2, -ms)); ps += sv[r]; }
+            l += ps;
+            frag8 pf[2];
+#pragma unroll
+            for (int st = 0; st < 2; ++st)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) pf[st].raw.w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+                for (int st = 0; st < 2; ++st) {
+                    frag8 vf;
+                    const tr4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr4 __attribute__((address_space(3)))*)&kv[1][half][stage][vaddr[dt] + (16 * st) * DH]);
+                    const tr4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr4 __attribute__((address_space(3)))*)&kv[1][half][stage][vaddr[dt] + (16 * st + 8) * DH]);
+                    vf.raw.w[0] = (uint32_t)(uint16_t)v0[0] | ((uint32_t)(uint16_t)v0[1] << 16);
+                    vf.raw.w[1] = (uint32_t)(uint16_t)v0[2] | ((uint32_t)(uint16_t)v0[3] << 16);
+                    vf.raw.w[2] = (uint32_t)(uint16_t)v1[0] | ((uint32_t)(uint16_t)v1[1] << 16);
+                    vf.raw.w[3] = (uint32_t)(uint16_t)v1[2] | ((uint32_t)(uint16_t)v1[3] << 16);
+                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
+                }
+            }
+        }
+        if (jb + 2 < nb) { LI_ATT_VMCNT(2 * NL); } else { LI_ATT_VMCNT(0); }
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+      }
+    }
+    // ---- the second group's results go to the first through LDS (the stages are free now)
+    __syncthreads();
+    float* mrg = reinterpret_cast<float*>(&kv[0][0][0][0]) + (size_t)wave * ((DT * 16 + 2) * 64);
+    static_assert(sizeof(kv) >= (size_t)PRE_WAVES * (DT * 16 + 2) * 64 * 4, "the groups' exchange fits the stages");
+    if (half == 1 && active) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mrg[(dt * 16 + r) * 64 + lane] = acc[dt][r];
+        mrg[(DT * 16) * 64 + lane] = m;
+        mrg[(DT * 16 + 1) * 64 + lane] = l;
+    }
+    __syncthreads();
+    if (half == 1 || !active || ql >= nrows) return;
+    {
+        const float m1 = mrg[(DT * 16) * 64 + lane], l1 = mrg[(DT * 16 + 1) * 64 + lane];
+        const float mn = fmaxf(m, m1);
+        const float a0 = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - mn);        // (a group that saw no key brings nothing)
+        const float a1 = (m1 == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m1 - mn);
+        l = l * a0 + l1 * a1;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[dt][r] = acc[dt][r] * a0 + mrg[(dt * 16 + r) * 64 + lane] * a1;
+    }
+    l += __shfl_xor(l, 32, LI_WAVE);               // (both halves of a query are past the return together)
+    const float inv = l != 0.f ? 1.0f / l : 0.f;
+    bf16_t* orow = out + (size_t)(t0 + ql) * nh * DH + (size_t)head * DH;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {           // registers 4 rg .. 4 rg + 3: dimensions 32 dt + 8 rg + 4 h ..
+            uint32_t w0 = pack2_bf16(acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv);
+            uint32_t w1 = pack2_bf16(acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv);
+            uint32_t* dst = reinterpret_cast<uint32_t*>(orow + 32 * dt + 8 * rg + 4 * h);
+            dst[0] = w0;
+            dst[1] = w1;
+        }
+}
+
+
 // tiles: int [ntiles, 4] = (segment, first token of the tile in the batch, rows <= 32, unused)
 extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void* out, const void* kc,
                                           const void* vc, const int* block_table, int max_blocks,
@@ -1114,6 +1392,15 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
 #define LI_PRE2(DHV, P32V) paged_attention_prefill_dma_kernel<DHV, P32V><<<grid, PRE_WAVES * 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
         tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
+#define LI_PRE3(DHV, P32V) paged_attention_prefill_split_kernel<DHV, P32V><<<grid, 2 * PRE_WAVES * 64, 0, stream>>>( \
+        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
+        tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
+    if (max_blocks <= PRE2_TABLE_CAP && (long)ntiles * nkv * parts <= (long)ncu) {      // at most a block a compute unit: the tile's keys in two halves
+        const bool p32 = 32 % page_size == 0;
+        if (dh == 128) { if (p32) LI_PRE3(128, true); else LI_PRE3(128, false); }
+        else if (dh == 64) { if (p32) LI_PRE3(64, true); else LI_PRE3(64, false); }
+        else return LI_ERR_SIZE;
+    } else
     if (max_blocks <= PRE2_TABLE_CAP) {                       // (longer block tables: the form that keeps 8,192 entries in LDS)
         const bool p32 = 32 % page_size == 0;
         if (dh == 128) { if (p32) LI_PRE2(128, true); else LI_PRE2(128, false); }
@@ -1122,6 +1409,7 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
     } else
     if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
 #undef LI_PRE2
+#undef LI_PRE3
 #undef LI_PRE
 #undef LI_PRE_FETCH
 #undef LI_PRE_ROW

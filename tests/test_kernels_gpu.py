@@ -464,6 +464,8 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
     ([(333, 200), (64, 5)], 10, 2, 64, 5, 0),
     ([(300, 300), (100, 9)], 4, 1, 64, 24, 40),
     ([(1, 1), (3000, 700)], 14, 2, 128, 1, 0),                      # one key a page: a long table
+    ([(1200, 1200), (40, 3)], 28, 4, 128, 16, 0),                   # more blocks than compute units: the tile's keys in one go
+    ([(1300, 1300)], 32, 8, 64, 8, 200),
     ([(5000, 300)], 4, 2, 128, 1, 0),                               # a table too long for the kernel that keeps the pages' offsets in LDS
     ([(1500, 400), (9, 9)], 7, 1, 128, 1, 0),                       # one key a page, within its table
 ])
