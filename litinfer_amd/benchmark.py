@@ -381,7 +381,7 @@ def headline(a) -> Dict[str, object]:
     if ref:
         out["reference"] = ref
     if not a.no_scheduler:
-        # BASELINE's workload through the scheduler: prompts of 2,048 tokens, then 256 greedy tokens
+        # the headline workload through the scheduler: prompts of 2,048 tokens, then 256 greedy tokens
         sch = {}
         # (in 32-bit the prompts of 64 requests alone take half a minute: the batch and one request there)
         for b in ((a.batch,) if a.no_points else (a.batch, 64, 1) if a.dtype == "bf16" else (a.batch, 1)):
@@ -402,7 +402,7 @@ def headline(a) -> Dict[str, object]:
 
 
 def serving(a) -> Dict[str, object]:
-    """BASELINE configs[3]: continuous batching at the 1.5B layer sizes."""
+    """Continuous batching at the 1.5B layer sizes: 128 requests of random lengths arriving over time, half of them sampled."""
     import numpy as np
     import torch
     from .engine import Engine
@@ -452,7 +452,7 @@ def serving(a) -> Dict[str, object]:
 
 
 def long_prompts(a) -> Dict[str, object]:
-    """BASELINE configs[4]: 8 prompts of 30,000 tokens at the 32B layer sizes."""
+    """Long prompts at the 32B layer sizes: 8 prompts of 30,000 tokens in portions, then 256 greedy tokens each."""
     import numpy as np
     import torch
     from .engine import Engine
