@@ -1368,6 +1368,171 @@ __global__ __launch_bounds__(2 * PRE_WAVES * 64) void paged_attention_prefill_sp
 }
 
 
+// ------------------------------------------------ portions of prompts, float32, FMA
+// The true 32-bit path's kernel for prompts: a block of 256 threads takes a tile of up to 32 tokens
+// of one segment and one head and walks the keys in blocks of 32 through LDS.  Scores: thread
+// (qg, kg) = (tid / 16, tid % 16) owns queries 2 qg, 2 qg + 1 and keys 2 kg, 2 kg + 1, four dot
+// products over the head size from LDS (each float4 of Q and K feeds two of them).  The 16 lanes of
+// a query pair agree on the new maximum by exchanges; probabilities go through LDS, transposed;
+// then thread (qg, dg) adds to its 2 x (dh / 16) outputs.  Every sum over keys or dimensions runs in
+// an order that depends on the sizes only.
+#define PF_T 32
+template <int DH>
+__global__ __launch_bounds__(256) void paged_attention_prefill_f32_kernel(
+    const float* __restrict__ q, int q_row_stride, float* __restrict__ out,
+    const float* __restrict__ kc, const float* __restrict__ vc, const int* __restrict__ block_table,
+    int max_blocks, const int* __restrict__ tiles, const int* __restrict__ q_start,
+    const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int page_size,
+    int num_pages, int window, float scale) {
+    constexpr int RS = DH + 4;                      // row stride in LDS: the rows of a float4 column fall into different banks
+    constexpr int C4 = DH / 4;                      // float4 pieces of a row
+    constexpr int PER = PF_T * C4 / 256;            // pieces of K (and of V) a thread fetches per block of keys
+    constexpr int DPT = DH / 16;                    // output dimensions a thread owns
+    static_assert(PER * 256 == PF_T * C4 && DPT % 4 == 0, "head sizes 64 and 128");
+    __shared__ __attribute__((aligned(16))) float Qs[PF_T * RS];
+    __shared__ __attribute__((aligned(16))) float Ks[PF_T * RS];
+    __shared__ __attribute__((aligned(16))) float Vs[PF_T * RS];
+    __shared__ __attribute__((aligned(16))) float Ps[PF_T * (PF_T + 2)];       // [key][query]
+    const int tile = gridDim.x - 1 - blockIdx.x, head = blockIdx.y;           // (the longest tiles of a segment first)
+    const int s = tiles[tile * 4], t0 = tiles[tile * 4 + 1], nrows = tiles[tile * 4 + 2];
+    const int kvh = head / (nh / nkv);
+    const int tid = threadIdx.x, qg = tid >> 4, kg = tid & 15;
+    const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);               // position of the tile's first token
+    const int p_last = p0 + nrows - 1;
+    const int lo0 = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+    const int k_begin = lo0 & ~(PF_T - 1), k_end = p_last + 1;
+    const int* table = block_table + (size_t)s * max_blocks;
+    // queries of the tile (rows past its end repeat the last one and store nothing)
+    for (int ci = tid; ci < PF_T * C4; ci += 256) {
+        const int r = ci / C4, c = ci % C4;
+        const float* src = q + (size_t)(t0 + (r < nrows ? r : nrows - 1)) * q_row_stride + (size_t)head * DH + 4 * c;
+        *reinterpret_cast<float4*>(&Qs[r * RS + 4 * c]) = *reinterpret_cast<const float4*>(src);
+    }
+    // this thread's pieces of a block of keys: key (tid + 256 i) / C4, piece (tid + 256 i) % C4
+    float4 kreg[PER], vreg[PER];
+    auto fetch = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int ci = tid + 256 * i, key = kb + ci / C4, c = ci % C4;
+            const int kk = key < k_end ? key : k_end - 1;                    // (masked below; the address stays inside the request)
+            int page = table[kk / page_size];
+            page = page < 0 ? 0 : (page >= num_pages ? num_pages - 1 : page);
+            const size_t off = (((size_t)page * nkv + kvh) * page_size + kk % page_size) * DH + 4 * c;
+            kreg[i] = *reinterpret_cast<const float4*>(kc + off);
+            vreg[i] = *reinterpret_cast<const float4*>(vc + off);
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int ci = tid + 256 * i, key = ci / C4, c = ci % C4;
+            *reinterpret_cast<float4*>(&Ks[key * RS + 4 * c]) = kreg[i];
+            *reinterpret_cast<float4*>(&Vs[key * RS + 4 * c]) = vreg[i];
+        }
+    };
+    const int q0 = 2 * qg, k0 = 2 * kg;
+    const int pq[2] = {p0 + (q0 < nrows ? q0 : nrows - 1), p0 + (q0 + 1 < nrows ? q0 + 1 : nrows - 1)};
+    int lq[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) lq[a] = (window > 0 && pq[a] - window + 1 > 0) ? pq[a] - window + 1 : 0;
+    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
+    float acc[2][DPT];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int d = 0; d < DPT; ++d) acc[a][d] = 0.f;
+    fetch(k_begin);
+    for (int kb = k_begin; kb < k_end; kb += PF_T) {
+        __syncthreads();                            // the block before is done with K, V and P (and Q is there)
+        stash();
+        __syncthreads();
+        if (kb + PF_T < k_end) fetch(kb + PF_T);    // on its way while this block is worked on
+        // ---- scores
+        float sc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+#pragma unroll 8
+        for (int c = 0; c < C4; ++c) {
+            const float4 qa = *reinterpret_cast<const float4*>(&Qs[q0 * RS + 4 * c]);
+            const float4 qb = *reinterpret_cast<const float4*>(&Qs[(q0 + 1) * RS + 4 * c]);
+            const float4 ka = *reinterpret_cast<const float4*>(&Ks[k0 * RS + 4 * c]);
+            const float4 kb4 = *reinterpret_cast<const float4*>(&Ks[(k0 + 1) * RS + 4 * c]);
+            sc[0][0] = fmaf(qa.x, ka.x, sc[0][0]); sc[0][0] = fmaf(qa.y, ka.y, sc[0][0]); sc[0][0] = fmaf(qa.z, ka.z, sc[0][0]); sc[0][0] = fmaf(qa.w, ka.w, sc[0][0]);
+            sc[0][1] = fmaf(qa.x, kb4.x, sc[0][1]); sc[0][1] = fmaf(qa.y, kb4.y, sc[0][1]); sc[0][1] = fmaf(qa.z, kb4.z, sc[0][1]); sc[0][1] = fmaf(qa.w, kb4.w, sc[0][1]);
+            sc[1][0] = fmaf(qb.x, ka.x, sc[1][0]); sc[1][0] = fmaf(qb.y, ka.y, sc[1][0]); sc[1][0] = fmaf(qb.z, ka.z, sc[1][0]); sc[1][0] = fmaf(qb.w, ka.w, sc[1][0]);
+            sc[1][1] = fmaf(qb.x, kb4.x, sc[1][1]); sc[1][1] = fmaf(qb.y, kb4.y, sc[1][1]); sc[1][1] = fmaf(qb.z, kb4.z, sc[1][1]); sc[1][1] = fmaf(qb.w, kb4.w, sc[1][1]);
+        }
+        // ---- softmax over the keys of each of the two queries: the 16 lanes that share them agree on the maximum
+        float alpha[2], pr[2][2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int key = kb + k0 + b;
+                sc[a][b] = (key <= pq[a] && key >= lq[a]) ? sc[a][b] * scale : -INFINITY;
+                mx = fmaxf(mx, sc[a][b]);
+            }
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, LI_WAVE));
+            const float mn = fmaxf(m[a], mx);
+            alpha[a] = (mn == -INFINITY) ? 1.0f : expf(m[a] - mn);           // (nothing seen yet: nothing to rescale)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) pr[a][b] = (sc[a][b] == -INFINITY) ? 0.f : expf(sc[a][b] - mn);
+            l[a] = l[a] * alpha[a] + (pr[a][0] + pr[a][1]);                  // this lane's keys; the lanes are added up at the end
+            m[a] = mn;
+        }
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            Ps[(k0 + b) * (PF_T + 2) + q0] = pr[0][b];
+            Ps[(k0 + b) * (PF_T + 2) + q0 + 1] = pr[1][b];
+        }
+        __syncthreads();
+        // ---- outputs: thread (qg, dg = kg) owns dimensions DPT dg .. of its two queries
+#pragma unroll
+        for (int d = 0; d < DPT; ++d) { acc[0][d] *= alpha[0]; acc[1][d] *= alpha[1]; }
+#pragma unroll 4
+        for (int k = 0; k < PF_T; ++k) {
+            const float pa = Ps[k * (PF_T + 2) + q0], pb = Ps[k * (PF_T + 2) + q0 + 1];
+#pragma unroll
+            for (int d4 = 0; d4 < DPT / 4; ++d4) {
+                const float4 v = *reinterpret_cast<const float4*>(&Vs[k * RS + DPT * kg + 4 * d4]);
+                acc[0][4 * d4] = fmaf(pa, v.x, acc[0][4 * d4]); acc[0][4 * d4 + 1] = fmaf(pa, v.y, acc[0][4 * d4 + 1]);
+                acc[0][4 * d4 + 2] = fmaf(pa, v.z, acc[0][4 * d4 + 2]); acc[0][4 * d4 + 3] = fmaf(pa, v.w, acc[0][4 * d4 + 3]);
+                acc[1][4 * d4] = fmaf(pb, v.x, acc[1][4 * d4]); acc[1][4 * d4 + 1] = fmaf(pb, v.y, acc[1][4 * d4 + 1]);
+                acc[1][4 * d4 + 2] = fmaf(pb, v.z, acc[1][4 * d4 + 2]); acc[1][4 * d4 + 3] = fmaf(pb, v.w, acc[1][4 * d4 + 3]);
+            }
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        float ls = l[a];
+#pragma unroll
+        for (int o = 8; o > 0; o >>= 1) ls += __shfl_xor(ls, o, LI_WAVE);
+        if (q0 + a >= nrows) continue;
+        const float inv = ls != 0.f ? 1.0f / ls : 0.f;
+        float* orow = out + (size_t)(t0 + q0 + a) * nh * DH + (size_t)head * DH + DPT * kg;
+#pragma unroll
+        for (int d4 = 0; d4 < DPT / 4; ++d4)
+            *reinterpret_cast<float4*>(orow + 4 * d4) = float4{acc[a][4 * d4] * inv, acc[a][4 * d4 + 1] * inv, acc[a][4 * d4 + 2] * inv, acc[a][4 * d4 + 3] * inv};
+    }
+}
+
+extern "C" int li_paged_attention_prefill_f32(const void* q, int q_row_stride, void* out, const void* kc,
+                                              const void* vc, const int* block_table, int max_blocks,
+                                              const int* tiles, int ntiles, const int* q_start, const int* q_len,
+                                              const int* ctx_len, int nh, int nkv, int dh, int page_size,
+                                              int num_pages, int window, float scale, hipStream_t stream) {
+    if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nh > 65535 || page_size <= 0 || max_blocks <= 0 ||
+        num_pages <= 0 || !(scale > 0.f) || (q_row_stride % 4))
+        return LI_ERR_SIZE;
+    dim3 grid(ntiles, nh);
+#define LI_PF(DHV) paged_attention_prefill_f32_kernel<DHV><<<grid, 256, 0, stream>>>( \
+        (const float*)q, q_row_stride, (float*)out, (const float*)kc, (const float*)vc, block_table, max_blocks, \
+        tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale)
+    if (dh == 128) LI_PF(128); else if (dh == 64) LI_PF(64); else return LI_ERR_SIZE;
+#undef LI_PF
+    return li_launch_status();
+}
+
 // tiles: int [ntiles, 4] = (segment, first token of the tile in the batch, rows <= 32, unused)
 extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void* out, const void* kc,
                                           const void* vc, const int* block_table, int max_blocks,

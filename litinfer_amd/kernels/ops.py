@@ -46,6 +46,7 @@ _SIGNATURES = {
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
         "li_paged_attention_prefill": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F],
+        "li_paged_attention_prefill_f32": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F],
         "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I],
     },
     "sampling": {
@@ -583,6 +584,13 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
     if (n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles
             and meta.tile_rows == PREFILL_TILE_ROWS and n_multi == meta.num_multi and meta.max_blocks <= 8192 and meta.max_blocks * page_size <= 1 << 21):
         _run("attention", "li_paged_attention_prefill", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
+             k.data_ptr(), v.data_ptr(), bt.data_ptr(), meta.max_blocks, meta.tiles.data_ptr(),
+             meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale))
+    elif (n_multi and qkv.dtype is torch.float32 and dh in (64, 128) and meta.num_tiles
+            and meta.tile_rows == PREFILL_TILE_ROWS and n_multi == meta.num_multi):
+        # the 32-bit path's tiled kernel for portions (other head sizes: the general kernel below)
+        _run("attention", "li_paged_attention_prefill_f32", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), bt.data_ptr(), meta.max_blocks, meta.tiles.data_ptr(),
              meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              nh, nkv, dh, page_size, k.shape[0], int(window), float(scale))
