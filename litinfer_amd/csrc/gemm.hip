@@ -1402,6 +1402,67 @@ static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, 
     return li_launch_status();
 }
 
+extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype);
+
+// The packed q/k/v projection of 17 to 64 rows cut along K: the kernel that adds the parts up also adds
+// the bias, rotates query and key heads (half-split pairs over the whole head, float32 tables
+// [M, dh / 2]) and writes keys and values into their page slots, so that the rotation needs no
+// kernel of its own.  Thread (row, head, pair): consecutive threads read consecutive sums.
+__global__ __launch_bounds__(256) void splitk_reduce_rope_store_kernel(
+    const float* __restrict__ part, int nsplit, size_t mn, int N, const float* __restrict__ bias, bf16_t* __restrict__ out,
+    const float* __restrict__ cosv, const float* __restrict__ sinv, const int* __restrict__ slot_map,
+    bf16_t* __restrict__ kc, bf16_t* __restrict__ vc, int nh, int nkv, int dh, int page_size, int num_pages, long total) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int half = dh / 2, heads = nh + 2 * nkv;
+    const int j = (int)(i % half), head = (int)((i / half) % heads), m = (int)(i / ((long)half * heads));
+    const size_t i0 = (size_t)m * N + (size_t)head * dh + j, i1 = i0 + half;
+    float a = part[i0], b = part[i1];
+    for (int sp = 1; sp < nsplit; ++sp) { a += part[(size_t)sp * mn + i0]; b += part[(size_t)sp * mn + i1]; }
+    if (bias) { a += bias[head * dh + j]; b += bias[head * dh + j + half]; }
+    if (head < nh + nkv) {
+        const float c = cosv[(size_t)m * half + j], sn = sinv[(size_t)m * half + j];
+        const float ra = __builtin_fmaf(a, c, -__fmul_rn(b, sn)), rb = __builtin_fmaf(b, c, __fmul_rn(a, sn));
+        a = ra; b = rb;
+    }
+    const uint16_t ba = float_to_bf16(a), bb = float_to_bf16(b);
+    out[i0].bits = ba;
+    out[i1].bits = bb;
+    if (head >= nh) {
+        const int slot = slot_map[m];
+        if (slot < 0 || slot >= num_pages * page_size) return;               // never write outside the pool
+        const bool is_k = head < nh + nkv;
+        const int kvh = is_k ? head - nh : head - nh - nkv;
+        const int page = slot / page_size, in_page = slot - page * page_size;
+        bf16_t* dst = (is_k ? kc : vc) + (((size_t)page * nkv + kvh) * page_size + in_page) * dh;
+        dst[j].bits = ba;
+        dst[j + half].bits = bb;
+    }
+}
+
+// Returns -1, having done nothing, where li_linear would not cut this product along K.
+extern "C" int li_linear_rope_store_parts(const void* x, const void* w, const float* bias, void* out, int M, int K,
+                                          const float* cos, const float* sin, const int* slot_map, void* kc, void* vc,
+                                          int nh, int nkv, int dh, int page_size, int num_pages,
+                                          void* work, long work_bytes, hipStream_t stream) {
+    if (M <= 0 || K <= 0 || nh <= 0 || nkv <= 0 || dh <= 0 || dh % 2 || page_size <= 0 || num_pages <= 0 ||
+        (long)(nh + 2 * nkv) * dh > 0x7fffffffL)
+        return LI_ERR_SIZE;
+    const int N = (nh + 2 * nkv) * dh;
+    if (!mid_rows_take(M, K) || K % 64) return -1;
+    const long need = li_linear_work_bytes(M, N, K, LI_BF16);
+    if (need <= 0 || !work || work_bytes < need) return -1;
+    const size_t mn = (size_t)M * N;
+    const int nsplit = (int)(need / (long)(mn * sizeof(float)));
+    const int rc = launch_dma<64, 128, 64, 4, false, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)work, M, N, K, 0, stream, nsplit);
+    if (rc != LI_OK) return rc;
+    const long total = (long)M * (nh + 2 * nkv) * (dh / 2);
+    splitk_reduce_rope_store_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
+        (const float*)work, nsplit, mn, N, bias, (bf16_t*)out, cos, sin, slot_map, (bf16_t*)kc, (bf16_t*)vc,
+        nh, nkv, dh, page_size, num_pages, total);
+    return li_launch_status();
+}
+
 // More than 64 rows but so few 128 x 128 tiles that half of the compute units would idle (a narrow
 // matrix with a long K, like the feed-forward's way back at 128 to 512 rows): K is cut into parts
 // here too.  Returns the number of parts, 1 for none.

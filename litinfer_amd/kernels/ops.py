@@ -42,6 +42,7 @@ _SIGNATURES = {
         "li_linear_residual_norm": [P, P, P, P, I, I, I, P, P, P],
         "li_linear_then_norm": [P, P, P, P, I, I, I, P, L, P, F, P, I],
         "li_linear_rope_store": [P, P, P, P, I, I, P, P, P, P, P, I, I, I, I, I, P, I, F],
+        "li_linear_rope_store_parts": [P, P, P, P, I, I, P, P, P, P, P, I, I, I, I, I, P, L],
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
@@ -491,6 +492,44 @@ def linear_rope_store(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Ten
     _run("gemm", "li_linear_rope_store", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
          out.data_ptr(), m, kk, cos.data_ptr(), sin.data_ptr(), slot_map.data_ptr(), k.data_ptr(), v.data_ptr(),
          nh, nkv, dh, page_size, k.shape[0], *_check_row_scale("linear_rope_store", m, row_scale))
+
+
+def linear_rope_store_parts(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                            nh: int, nkv: int, dh: int, cos: torch.Tensor, sin: torch.Tensor,
+                            slot_map: torch.Tensor, k: torch.Tensor, v: torch.Tensor, page_size: int, ws) -> bool:
+    """The same result as `linear_rope_store` for the rows of a large decoding batch, where the
+    packed projection is cut along K anyway: the kernel that adds the parts up rotates and writes
+    the pages.  Returns False, having done nothing, where `linear` would not cut this product."""
+    _gpu(x, w, bias, out, cos, sin, slot_map, k, v)
+    if ws is None or x.dtype is not torch.bfloat16 or w.dtype is not torch.bfloat16 or 2 * cos.shape[1] != dh:
+        return False
+    m, kk = x.shape
+    n = (nh + 2 * nkv) * dh
+    need = _work_bytes(m, n, kk, _DT[x.dtype])
+    if not need:
+        return False
+    _chk(w.shape == (n, kk) and out.shape == (m, n), "linear_rope_store_parts: shapes do not fit")
+    _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_rope_store_parts: contiguous operands")
+    _chk(out.dtype is torch.bfloat16, "linear_rope_store_parts: out must be bfloat16")
+    _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
+         "linear_rope_store_parts: bias must be float32 [N]")
+    _check_cache(k, v, nkv, dh, page_size, out.dtype)
+    _chk(cos.shape == (m, dh // 2) and sin.shape == cos.shape and cos.dtype is torch.float32
+         and sin.dtype is torch.float32 and cos.is_contiguous() and sin.is_contiguous(), "linear_rope_store_parts: tables")
+    _chk(slot_map.dtype is torch.int32 and slot_map.numel() == m and slot_map.is_contiguous(),
+         "linear_rope_store_parts: slot_map")
+    if m <= SKINNY_MAX_ROWS:                # one size for all row counts of a decode batch: the buffer does not move
+        need = max(need, SPLITK_MAX_PARTS * SKINNY_MAX_ROWS * n * 4)
+    buf = ws.buffer("gemm.parts", (need // 4,), torch.float32)
+    rc = _fn("gemm", "li_linear_rope_store_parts")(
+        x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(), out.data_ptr(), m, kk,
+        cos.data_ptr(), sin.data_ptr(), slot_map.data_ptr(), k.data_ptr(), v.data_ptr(), nh, nkv, dh, page_size,
+        k.shape[0], buf.data_ptr(), buf.numel() * 4, _stream())
+    if rc == -1:
+        return False
+    if rc != 0:
+        raise RuntimeError(f"li_linear_rope_store_parts: the kernel library refused the call (code {rc}): {_ERRORS.get(rc, 'unknown')}")
+    return True
 
 
 # ----------------------------------------------------------------- attention

@@ -83,10 +83,15 @@ class RopeNeox(Position):
 
     def project_encode_store(self, proj, xn, qkv, num_heads, num_kv_heads, head_dim, ctx, cache, row_scale=None):
         # few rows (decoding): the rotation and the page write are the projection's epilogue
-        if not (cache.owned and xn.dtype is ops.bfloat16 and proj.weight.dtype is ops.bfloat16
-                and ops.rope_store_takes(xn.shape[0], proj.in_features, proj.weight.dtype, head_dim,
-                                         self.rotary_dim)):
+        if not (cache.owned and xn.dtype is ops.bfloat16 and proj.weight.dtype is ops.bfloat16):
             return False
+        if not ops.rope_store_takes(xn.shape[0], proj.in_features, proj.weight.dtype, head_dim, self.rotary_dim):
+            # more rows: where the projection is cut along K anyway, the kernel that adds the parts up rotates and stores
+            if row_scale is not None or self.rotary_dim != head_dim:
+                return False
+            cos, sin = self.tables(ctx)
+            return ops.linear_rope_store_parts(xn, proj.weight, proj.bias, qkv, num_heads, num_kv_heads, head_dim, cos, sin,
+                                               ctx.slot_map(cache.group), cache.k, cache.v, cache.page_size, ctx.ws)
         cos, sin = self.tables(ctx)
         ops.linear_rope_store(xn, proj.weight, proj.bias, qkv, num_heads, num_kv_heads, head_dim, cos, sin,
                               ctx.slot_map(cache.group), cache.k, cache.v, cache.page_size, row_scale=row_scale)

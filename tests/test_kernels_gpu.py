@@ -563,6 +563,46 @@ def test_rope_kv_store_and_plain_store(ops, dtype, dh, pad):
 
 
 @pytest.mark.parametrize("t,nh,nkv,dh,k,bias", [
+    (64, 28, 4, 128, 3584, True),       # a decoding batch of 64 at the 7B layer sizes
+    (33, 12, 2, 128, 1536, True),
+    (40, 6, 2, 64, 1280, False),
+])
+def test_projection_cut_along_k_with_rotary_encoding_and_page_write_in_the_adding_up(ops, t, nh, nkv, dh, k, bias):
+    g = torch.Generator().manual_seed(31)
+    n, page, pages = (nh + 2 * nkv) * dh, 16, 8
+    x = torch.randn(t, k, generator=g).to(torch.bfloat16)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
+    b = torch.randn(n, generator=g) if bias else None
+    pos = torch.randint(0, 5000, (t,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(pages * page, generator=g)[:t].to(torch.int32)
+    cos = torch.empty(t, dh // 2, device=DEV)
+    sin = torch.empty(t, dh // 2, device=DEV)
+    ops.rope_table(pos.to(DEV), 1e6, dh, cos, sin)
+    kc = torch.full((pages, nkv, page, dh), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full_like(kc, 7.0)
+    out = torch.full((t, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    took = ops.linear_rope_store_parts(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, nh, nkv, dh, cos, sin,
+                                       slots.to(DEV), kc, vc, page, _Lender())
+    assert took
+    y = x.double().numpy() @ w.double().numpy().T + (0 if b is None else b.double().numpy())
+    y = y.reshape(t, nh + 2 * nkv, dh)
+    ref = np.concatenate([plain_impl.rope_neox(y[:, :nh + nkv], pos.numpy(), 1e6), y[:, nh + nkv:]], axis=1).reshape(t, n)
+    assert rel(out, ref) < 5e-3
+    ov = out.cpu().view(t, nh + 2 * nkv, dh)
+    touched = torch.zeros(pages, page, dtype=torch.bool)
+    for i in range(t):
+        sl = int(slots[i])
+        touched[sl // page, sl % page] = True
+        assert torch.equal(kc[sl // page, :, sl % page].cpu(), ov[i, nh:nh + nkv])
+        assert torch.equal(vc[sl // page, :, sl % page].cpu(), ov[i, nh + nkv:])
+    untouched = ~touched[:, None, :, None].expand(pages, nkv, page, dh)
+    assert (kc.cpu()[untouched] == 7.0).all() and (vc.cpu()[untouched] == 7.0).all()
+    # few rows, or no workspace: not taken
+    assert not ops.linear_rope_store_parts(x[:8].to(DEV), w.to(DEV), None, out[:8], nh, nkv, dh, cos[:8], sin[:8],
+                                           slots[:8].to(DEV), kc, vc, page, _Lender())
+
+
+@pytest.mark.parametrize("t,nh,nkv,dh,k,bias", [
     (8, 28, 4, 128, 3584, True),        # a decoding step at the 7B layer sizes
     (1, 3, 1, 32, 96, True),
     (16, 5, 5, 48, 120, False),         # a head size that is no power of two

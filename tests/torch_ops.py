@@ -179,6 +179,10 @@ def rope_store_takes(m, k, w_dtype, dh, rotary_dim):
     return w_dtype is torch.bfloat16 and 0 < m <= 16 and k % 8 == 0 and dh % 16 == 0 and rotary_dim == dh
 
 
+def linear_rope_store_parts(*args, **kwargs):
+    return False                 # (the stand-in never cuts a product along K)
+
+
 def linear_rope_store(x, w, bias, out, nh, nkv, dh, cos, sin, slot_map, k, v, page_size, row_scale=None):
     y = x.float() @ w.float().T
     if row_scale is not None:
@@ -201,7 +205,7 @@ def argmax_rows(logits, out):
 
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
-       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "rope_store_takes", "linear_rope_store", "check_attention_sizes",
+       "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "rope_store_takes", "linear_rope_store", "linear_rope_store_parts", "check_attention_sizes",
        "RowScale", "RESIDUAL_NORM_MAX_PARTS", "residual_norm_parts", "residual_norm_takes", "linear_residual_norm", "linear_then_norm",
        "paged_attention", "argmax_rows"]
 
