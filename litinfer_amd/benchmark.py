@@ -401,6 +401,66 @@ def headline(a) -> Dict[str, object]:
     return out
 
 
+def sweep(a) -> Dict[str, object]:
+    """Decode steps and prompts at further sizes of the 7B layer shape: contexts of 1,024 to 16,384
+    tokens at 1, 8 and 64 requests, prompts of 512 to 8,192 tokens and a portion of 1,024 tokens
+    behind 15,360 cached ones; each with its fraction of the published peak."""
+    import numpy as np
+    import torch
+    from .engine import Engine, StepEntry
+    from .sampling import Sampler, SamplingParams
+
+    cfg = dict(QWEN2_7B, num_hidden_layers=a.layers, max_position_embeddings=32768)
+    es = 2 if a.dtype == "bf16" else 4
+    dev = "cuda:0"
+    contexts, batches = (1024, 4096, 16384), (1, 8, 64)
+    eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
+                             num_pages=max(batches) * max(contexts) // PAGE + 1024, max_seqs=max(batches) + 1)
+    for g in eng.cache.groups:
+        for data in g.data.values():
+            flat = data.view(-1)
+            for i in range(0, flat.numel(), 1 << 28):
+                flat[i:i + (1 << 28)].normal_(0, 0.5)
+    sampler = Sampler(dev)
+    rng = np.random.default_rng(0)
+    loop = StepLoop(eng, cfg, sampler, rng)
+    decode = {}
+    for ctx in contexts:
+        for b in batches:
+            dt, ctx_tokens = loop.run(b, a.steps, a.warmup, ctx)
+            nbytes = decode_bytes(cfg, a.layers, ctx_tokens, es)
+            decode[f"ctx{ctx}_b{b}"] = {"tok_s": round(b * a.steps / dt, 1), "ms_per_step": round(dt / a.steps * 1e3, 3),
+                                        "frac": round(nbytes / dt * a.steps / HBM_PEAK, 4)}
+            log(f"decode, context {ctx}, batch {b}: {decode[f'ctx{ctx}_b{b}']}")
+    prefill = {}
+    for tokens, start in ((512, 0), (2048, 0), (8192, 0), (1024, 15360)):
+        ids = rng.integers(0, cfg["vocab_size"], start + tokens).tolist()
+        times = []
+        for i in range(4):
+            rid = f"s{tokens}_{start}_{i}"
+            if start:                                   # the cached part first, in portions; not timed
+                for o in range(0, start, 2048):
+                    eng.step([StepEntry(rid, ids[o:o + 2048], [])])
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            logits = eng.step([StepEntry(rid, ids[start:], [tokens - 1])])
+            sampler.sample(logits, [SamplingParams()], [0])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            eng.finish(rid)
+        pt = min(times[1:])
+        flops = prefill_flops(cfg, a.layers, tokens, start)
+        key = f"t{tokens}" + (f"_after{start}" if start else "")
+        prefill[key] = {"tok_s": round(tokens / pt, 1), "ms": round(pt * 1e3, 3), "frac": round(flops / pt / FLOP_PEAK[a.dtype], 4)}
+        log(f"prompt of {tokens} tokens behind {start}: {prefill[key]}")
+    best = decode["ctx4096_b8"]
+    return {"metric": "decode tok/s and prompt tok/s at further sizes (Qwen2-7B shape)", "value": best["tok_s"], "unit": "tok/s",
+            "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": best["ms_per_step"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic: seeded random token ids, random weights, random cache content",
+            "config": {"model": "Qwen2-7B shape", "num_hidden_layers": a.layers, "page_size": PAGE, "parallelism": "none (1 GPU)"},
+            "decode": decode, "prefill_at": prefill}
+
+
 def serving(a) -> Dict[str, object]:
     """Continuous batching at the 1.5B layer sizes: 128 requests of random lengths arriving over time, half of them sampled."""
     import numpy as np
@@ -513,7 +573,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in `config`)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
-    ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long"])
+    ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep"])
     ap.add_argument("--no-points", action="store_true", help="headline: skip the batch 1 and 64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-scheduler", action="store_true", help="headline: skip the runs through the scheduler")
@@ -532,6 +592,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     if a.mode == "headline":
         a.layers = a.layers or QWEN2_7B["num_hidden_layers"]
         out = headline(a)
+    elif a.mode == "sweep":
+        a.layers = a.layers or QWEN2_7B["num_hidden_layers"]
+        a.steps, a.warmup = min(a.steps, 32), min(a.warmup, 4)
+        out = sweep(a)
     elif a.mode == "serving":
         a.requests = a.requests or 128
         out = serving(a)

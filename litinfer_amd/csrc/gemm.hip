@@ -371,26 +371,35 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16_t* __restrict
 // chunk c of row r lies at position c ^ ((r >> 1) & 7), which spreads the 16
 // rows that one fragment read touches over all banks.
 // Blocks go to the 8 XCDs in turn (block b runs on XCD b % 8), and each XCD has an L2 of its
-// own.  The tiles are dealt so that the ~32 blocks an XCD runs at one time form a patch of up
-// to 8 row panels x 4 or more column panels: what the patch reads from beyond its L2 is then
-// (8 + 4) panels for 32 tiles.  Patches follow each other along the rows first, so a column
-// panel of W is read from HBM by one XCD only and stays in its L2 while the row panels go by.
+// own.  The tiles are put in one sequence: patches of up to 8 row panels x 4 or more column panels
+// (32 tiles, what an XCD runs at one time; smaller at the matrix's edges), patches along the rows
+// first, then along the columns; what a patch reads from beyond its L2 is (8 + 4) panels for 32
+// tiles.  Each XCD takes one eighth of the sequence in one piece: a run of neighbouring column
+// panels of W, which no other XCD reads but for the two panels at its ends.  Every block has a
+// tile, but for the last few of the last XCD, and no XCD has more than one tile more than another:
+// blocks that return at once in the middle of the queue, and XCDs with a column panel more than
+// others, made a matrix of fewer tiles than compute units take two rounds.
 struct TileOrder {
-    int pm, gn, mgroups;                             // row panels and column panels of a patch; patches along the rows
+    int pm, gn;                                      // row panels and column panels of a patch
     __host__ __device__ TileOrder(int mtiles) {
         pm = mtiles < 8 ? mtiles : 8;
         gn = 32 / pm;
-        mgroups = (mtiles + pm - 1) / pm;
     }
-    __host__ long blocks(long ntiles) const {        // grid size: whole patches on each of the 8 XCDs
-        return ((ntiles + 7) / 8 + gn - 1) / gn * (long)mgroups * pm * gn * 8;
+    __host__ static long blocks(long mtiles, long ntiles) {       // grid size: the same number of blocks on each XCD
+        return (mtiles * ntiles + 7) / 8 * 8;
     }
     __device__ bool tile(int block, int mtiles, int ntiles, int& mt, int& nt) const {
-        const int xcd = block & 7, idx = block >> 3;
-        const int patch = idx / (pm * gn), within = idx % (pm * gn);
-        mt = (patch % mgroups) * pm + within % pm;
-        nt = ((patch / mgroups) * gn + within / pm) * 8 + xcd;
-        return mt < mtiles && nt < ntiles;
+        const long total = (long)mtiles * ntiles, per = (total + 7) / 8;
+        const long t = (block & 7) * per + (block >> 3);
+        if (t >= total) return false;
+        const int group = mtiles * gn;               // tiles of gn column panels
+        const int cg = (int)(t / group), r = (int)(t % group);
+        const int gc = ntiles - cg * gn < gn ? ntiles - cg * gn : gn;        // column panels of this group
+        const int rg = r / (pm * gc), r2 = r % (pm * gc);
+        const int rows_in = mtiles - rg * pm < pm ? mtiles - rg * pm : pm;  // row panels of this patch
+        mt = rg * pm + r2 % rows_in;
+        nt = cg * gn + r2 / rows_in;
+        return true;
     }
 };
 
@@ -842,7 +851,7 @@ template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO, int WLM 
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream, int nsplit = 1) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    const long per_xcd = TileOrder((int)mtiles).blocks(ntiles) / 8;
+    const long per_xcd = TileOrder::blocks(mtiles, ntiles) / 8;
     if (per_xcd * 8 > 0x7fffffffL || nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
     // a lane's byte offset from its tile's first row is kept in 32 bits (the gate and up rows of a
     // SwiGLU tile lie N / 2 rows apart)
@@ -919,7 +928,7 @@ template <int BM, int BN, int BK, typename TO>
 static int launch_big(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    const long per_xcd = TileOrder((int)mtiles).blocks(ntiles) / 8;
+    const long per_xcd = TileOrder::blocks(mtiles, ntiles) / 8;
     if (per_xcd * 8 > 0x7fffffffL) return LI_ERR_SIZE;
     dim3 grid((unsigned)(per_xcd * 8));
     constexpr int lds_bytes = 2 * (BM + BN) * BK * 2;
@@ -1463,6 +1472,25 @@ extern "C" int li_linear_rope_store_parts(const void* x, const void* w, const fl
     return li_launch_status();
 }
 
+// Estimated time, in microseconds, of x w^T in tiles of bm x bn with K in steps of 64: rounds of tiles
+// over the compute units x (steps x the longer of a step's MFMAs and a step's loads + a tile's start
+// and end).  A compute unit multiplies at about 4 TFLOP/s under the chip's power limit, `speed` of
+// that in this tiling (small tiles spend more of their time between steps; with four waves one
+// above the other the LDS reads take nearly as long as the MFMAs), and takes in about 50 GB/s, rows
+// of x that other units read too included: with few rows of x a tile waits for its part of w, and
+// wide tiles read x less often.  A last round that does not fill the chip counts for less than a
+// whole one: the units that run clock higher.  Fitted to measurements of all tilings at 128 to
+// 8,192 rows of the 1.5B and 7B layer shapes: the tiling it takes is within 4 % of the best one
+// there, but for the 7B's way back from the feed-forward at 4,096 rows and more (10 %).
+static double tile_cost(int bm, int bn, double speed, int M, int N, int K) {
+    const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+    const int cu = compute_units();
+    const double filled = (double)tiles / cu, whole = (double)((tiles + cu - 1) / cu);
+    const double rounds = filled + 0.4 * (whole - filled);
+    const double mfma_us = (double)bm * bn * 64 * 2 / (4.0e6 * speed), load_us = (double)(bm + bn) * 128 / 50.0e3;
+    return rounds * ((K / 64) * (mfma_us > load_us ? mfma_us : load_us) + 2.0);
+}
+
 // More than 64 rows but so few 128 x 128 tiles that half of the compute units would idle (a narrow
 // matrix with a long K, like the feed-forward's way back at 128 to 512 rows): K is cut into parts
 // here too.  Returns the number of parts, 1 for none.
@@ -1556,9 +1584,6 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
             if (out_dtype != LI_F32 && out_dtype != LI_BF16) return LI_ERR_DTYPE;
 #define LI_DMA(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, false, float>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                                : launch_dma<BM, BN, BK, NS, false, bf16_t>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
-            // Six tilings; the one with the least (rounds of blocks over the 256 compute units) x
-            // (area of a tile) / (its measured relative speed) is taken: large tiles are the fastest
-            // per multiply-add but leave compute units idle when the matrix has few of them.
             if (K % 64 == 0) {
                 const int nsplit = split_parts_many_rows(M, N, K);
                 const size_t mn = (size_t)M * N;
@@ -1571,26 +1596,29 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
                     else splitk_reduce_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const float*)work, nsplit, mn, N, bias, (bf16_t*)out, accumulate);
                     return li_launch_status();
                 }
-                auto cost = [&](int bm, int bn, double speed) {
-                    const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-                    return (double)((tiles + 255) / 256) * bm * bn / speed;
-                };
-                const double c_large = cost(256, 256, 1.0), c_wide = cost(256, 192, 0.97), c_mid = cost(256, 128, 0.95),
-                             c_small = cost(128, 128, 0.8);
 #define LI_DMA4(BM, BN, BK, NS) (out_dtype == LI_F32 ? launch_dma<BM, BN, BK, NS, false, float, 4>((const bf16_t*)x, (const bf16_t*)w, bias, (float*)out, M, N, K, accumulate, stream) \
                                                 : launch_dma<BM, BN, BK, NS, false, bf16_t, 4>((const bf16_t*)x, (const bf16_t*)w, bias, (bf16_t*)out, M, N, K, accumulate, stream))
-                // (tiles of 128 rows with four waves one above the other: slower per multiply-add, their LDS reads
-                // take as long as their MFMAs, but 224 or 288 columns cut 3,584 or 4,608 into exactly as many
-                // tiles as 2,048 rows need to give every compute unit one)
-                const double c_224 = cost(128, 224, 0.87), c_288 = cost(128, 288, 0.87);
-                const double best = std::min(std::min(std::min(c_large, c_wide), std::min(c_mid, c_small)), std::min(c_224, c_288));
-                if (c_224 == best) return LI_DMA4(128, 224, 64, 3);
-                if (c_288 == best) return LI_DMA4(128, 288, 64, 3);
+                // Seven tilings; the one with the least estimated time is taken (tile_cost).  The two with four
+                // waves one above the other take any multiple of 32 columns: 224 or 288 columns cut 3,584 or
+                // 4,608 into exactly as many tiles as 2,048 rows need to give every compute unit one.
+                static const struct { int bm, bn; double speed; } shape[7] = {{256, 256, 1.0}, {256, 192, 0.95}, {256, 128, 1.0}, {192, 128, 0.95},
+                                                                                {128, 128, 0.8}, {128, 224, 0.9}, {128, 288, 0.9}};
+                int pick = 0;
+                double best = 0.0;
+                for (int i = 0; i < 7; ++i) {
+                    const double c = tile_cost(shape[i].bm, shape[i].bn, shape[i].speed, M, N, K);
+                    if (i == 0 || c < best) { best = c; pick = i; }
+                }
+                switch (pick) {
+                case 0: return LI_DMA(256, 256, 64, 2);
+                case 1: return LI_DMA(256, 192, 64, 2);
+                case 2: return LI_DMA(256, 128, 64, 3);
+                case 3: return LI_DMA(192, 128, 64, 3);
+                case 4: return LI_DMA(128, 128, 64, 4);
+                case 5: return LI_DMA4(128, 224, 64, 3);
+                default: return LI_DMA4(128, 288, 64, 3);
+                }
 #undef LI_DMA4
-                if (c_large == best) return LI_DMA(256, 256, 64, 2);
-                if (c_wide == best) return LI_DMA(256, 192, 64, 2);
-                if (c_mid == best) return LI_DMA(256, 128, 64, 3);
-                return LI_DMA(128, 128, 64, 4);
             }
 #undef LI_DMA
             return LI_BIG(128, 128, 64);             // K not a multiple of 64: loads staged in registers
@@ -1629,15 +1657,22 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     }
     if (M <= 64) return li_linear_skinny(x, w, nullptr, out, M, I, K, LI_BF16, 0, 1, stream);
     if (K % 64) return LI_ERR_SIZE;
-    auto cost = [&](int bm, int bn, double speed) {
-        const long tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-        return (double)((tiles + 255) / 256) * bm * bn / speed;
-    };
-#define LI_DMA(BM, BN, BK, NS) launch_dma<BM, BN, BK, NS, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream)
-    const double c_large = cost(256, 256, 1.0), c_mid = cost(256, 128, 0.95), c_small = cost(128, 128, 0.8);
-    if (c_large <= c_mid && c_large <= c_small) return LI_DMA(256, 256, 64, 2);
-    if (c_mid <= c_small) return LI_DMA(256, 128, 64, 3);
-    return LI_DMA(128, 128, 64, 4);
+#define LI_DMA(BM, BN, BK, NS, WLM) launch_dma<BM, BN, BK, NS, true, bf16_t, WLM>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream)
+    // (a tile's columns are gate and up columns in turn, 32 of each: its width is a multiple of 64)
+    static const struct { int bm, bn; double speed; } shape[5] = {{256, 256, 1.0}, {256, 128, 1.0}, {128, 256, 1.0}, {128, 128, 0.8}, {128, 192, 0.9}};
+    int pick = 0;
+    double best = 0.0;
+    for (int i = 0; i < 5; ++i) {
+        const double c = tile_cost(shape[i].bm, shape[i].bn, shape[i].speed, M, N, K);
+        if (i == 0 || c < best) { best = c; pick = i; }
+    }
+    switch (pick) {
+    case 0: return LI_DMA(256, 256, 64, 2, 2);
+    case 1: return LI_DMA(256, 128, 64, 3, 2);
+    case 2: return LI_DMA(128, 256, 64, 3, 2);
+    case 3: return LI_DMA(128, 128, 64, 4, 2);
+    default: return LI_DMA(128, 192, 64, 3, 4);
+    }
 #undef LI_DMA
 }
 

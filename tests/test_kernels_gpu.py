@@ -74,7 +74,9 @@ def test_rmsnorm_zero_row_is_zero_not_nan(ops):
     ((1, 1000, 3584), True, False), ((16, 70, 260), True, True), ((40, 19, 100), False, True),      # few rows in 32-bit
     ((9, 18, 4), True, False),
     ((300, 200, 130), True, True), ((256, 128, 64), False, False), ((1000, 333, 1027), True, False),     # the large 32-bit tile
-    ((2048, 3584, 128), True, True), ((2000, 4600, 64), True, False)])          # tiles of 128 x 224 and 128 x 288, ragged
+    ((2048, 3584, 128), True, True), ((2000, 4600, 64), True, False),           # tiles of 256 x 128 and 256 x 256, ragged
+    ((1100, 4600, 128), True, True), ((1167, 6627, 128), False, False),         # 192 x 128 and 256 x 192: a last row of tiles with few rows
+    ((585, 3979, 128), True, False), ((779, 6296, 128), False, True)])          # four waves one above the other: 128 x 224 and 128 x 288
 def test_linear(ops, dtype, mnk, bias, acc):
     m, n, k = mnk
     g = torch.Generator().manual_seed(2)
@@ -219,8 +221,11 @@ def test_linear_into_the_residual_sum_with_its_norm(ops, m, n, k, bias, taken):
     (65, 32, 64),                # one tile, one step of K
     (100, 200, 128),             # an output width that is no multiple of 32
     (300, 1000, 192),            # several tiles both ways, ragged edges
-    (700, 4700, 256),            # enough tiles for the largest tiling
-    (2048, 18944, 128),
+    (700, 4700, 256),            # tiles of 256 x 128
+    (2048, 18944, 128),          # enough tiles for the largest tiling
+    (97, 7419, 128),             # few rows against many columns: tiles of 128 x 192, four waves one above the other
+    (300, 9001, 128),            # tiles of 128 x 256
+    (1101, 2500, 192),           # nine rows of tiles: the last XCD's share of the tiles is short
 ])
 def test_linear_with_swiglu_epilogue(ops, m, n, k):
     g = torch.Generator().manual_seed(14)
