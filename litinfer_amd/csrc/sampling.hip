@@ -148,13 +148,19 @@ extern "C" int li_argmax_rows_noalloc(const float* logits, int* out, int n, int 
 }
 
 // ---------------------------------------------------------------- sampling
-// One block per row.  The candidates are ordered by (value descending, index
-// ascending); top-k keeps the first k, top-p then the shortest prefix whose
-// softmax mass (among the top-k survivors) reaches p; the survivors' softmax is
-// sampled by inverse CDF over ASCENDING ids with the given uniform number.
-// Thresholds are found by a bitwise search over the order-preserving integer
-// image of the floats, every count and mass being a block reduction in a fixed
-// order, so the same inputs always give the same token.
+// The candidates are ordered by (value descending, index ascending); top-k keeps the first k, top-p
+// then the shortest prefix whose softmax mass (among the top-k survivors) reaches p; the survivors'
+// softmax is sampled by inverse CDF over ASCENDING ids with the given uniform number.
+// Two kernels.  The first has a block for every tile of SMP_TILE ids of every row, so that a few
+// rows still use many compute units: a tile's maximum, and for rows without top-k and top-p its
+// softmax sum, for greedy rows its argmax.  The second has one block per row.  It reads the row in
+// the same tiles (thread t the 8 consecutive ids t * 8 ... of a tile: whole lines), in as few
+// passes as it can: the thresholds of top-k and top-p are found four bits a pass over the
+// order-preserving integer image of the floats (16 counts or 16 masses a thread and pass).  Every
+// count and every mass is added in a fixed order, so the same inputs always give the same token.
+constexpr int SMP_TILE = SMP_NT * 8;
+constexpr int SMP_WAVES = SMP_NT / LI_WAVE;
+
 __device__ __forceinline__ uint32_t sort_key(float z) {
     const uint32_t b = __float_as_uint(z);
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
@@ -162,6 +168,7 @@ __device__ __forceinline__ uint32_t sort_key(float z) {
 __device__ __forceinline__ float key_value(uint32_t k) {
     return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
+__device__ __forceinline__ bool sample_unfiltered(int k, float p, int V) { return !(k > 0 && k < V) && !(p > 0.f && p < 1.f); }
 
 __device__ __forceinline__ int block_sum_int(int v, int* smem) {
 #pragma unroll
@@ -172,7 +179,7 @@ __device__ __forceinline__ int block_sum_int(int v, int* smem) {
     __syncthreads();
     int t = 0;
 #pragma unroll
-    for (int i = 0; i < SMP_NT / LI_WAVE; ++i) t += smem[i];
+    for (int i = 0; i < SMP_WAVES; ++i) t += smem[i];
     return t;
 }
 
@@ -184,239 +191,407 @@ __device__ __forceinline__ float block_max_f(float v, float* smem) {
     __syncthreads();
     float t = smem[0];
 #pragma unroll
-    for (int i = 1; i < SMP_NT / LI_WAVE; ++i) t = fmaxf(t, smem[i]);
+    for (int i = 1; i < SMP_WAVES; ++i) t = fmaxf(t, smem[i]);
     return t;
 }
 
+__device__ __forceinline__ int block_min_int(int v, int* smem) {
+#pragma unroll
+    for (int o = LI_WAVE / 2; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, LI_WAVE));
+    const int lane = threadIdx.x & (LI_WAVE - 1), w = threadIdx.x / LI_WAVE;
+    __syncthreads();
+    if (lane == 0) smem[w] = v;
+    __syncthreads();
+    int t = smem[0];
+#pragma unroll
+    for (int i = 1; i < SMP_WAVES; ++i) t = min(t, smem[i]);
+    return t;
+}
+
+// The 16 sums of a pass over the whole block, left in tot[0..15] for every thread to read: within a
+// wave by the shuffle tree, then the waves in their order.  work: SMP_WAVES * 16 values.
+template <typename T>
+__device__ __forceinline__ void block_sum16(T (&c)[16], T* work, T* tot) {
+#pragma unroll
+    for (int b = 0; b < 16; ++b)
+#pragma unroll
+        for (int o = LI_WAVE / 2; o > 0; o >>= 1) c[b] += __shfl_xor(c[b], o, LI_WAVE);
+    const int lane = threadIdx.x & (LI_WAVE - 1), w = threadIdx.x / LI_WAVE;
+    __syncthreads();                                 // (the last pass's totals have been read)
+    if (lane == 0) {
+#pragma unroll
+        for (int b = 0; b < 16; ++b) work[w * 16 + b] = c[b];
+    }
+    __syncthreads();
+    if (threadIdx.x < 16) {
+        T t = 0;
+        for (int i = 0; i < SMP_WAVES; ++i) t += work[i * 16 + threadIdx.x];
+        tot[threadIdx.x] = t;
+    }
+    __syncthreads();
+}
+
+// Sum of v over the threads before this one, in thread order.  work: SMP_WAVES values.
+template <typename T>
+__device__ __forceinline__ T block_sum_before(T v, T* work) {
+    const int lane = threadIdx.x & (LI_WAVE - 1), w = threadIdx.x / LI_WAVE;
+    T inc = v;
+#pragma unroll
+    for (int o = 1; o < LI_WAVE; o <<= 1) {
+        const T t = __shfl_up(inc, o, LI_WAVE);
+        if (lane >= o) inc += t;
+    }
+    T before = __shfl_up(inc, 1, LI_WAVE);
+    if (lane == 0) before = 0;
+    __syncthreads();
+    if (lane == LI_WAVE - 1) work[w] = inc;
+    __syncthreads();
+    T base = 0;
+    for (int i = 0; i < w; ++i) base += work[i];
+    return base + before;
+}
+
+// A thread's 8 ids of a tile as z = logit / T (whole 16-byte loads where the row allows them)
+__device__ __forceinline__ void load_ids8(const float* __restrict__ row, int j0, int V, float T, bool vec, float (&z)[8]) {
+    if (vec && j0 + 8 <= V) {
+        const float4 a = *reinterpret_cast<const float4*>(row + j0), b = *reinterpret_cast<const float4*>(row + j0 + 4);
+        z[0] = a.x / T; z[1] = a.y / T; z[2] = a.z / T; z[3] = a.w / T;
+        z[4] = b.x / T; z[5] = b.y / T; z[6] = b.z / T; z[7] = b.w / T;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) z[e] = (j0 + e < V) ? row[j0 + e] / T : -INFINITY;
+    }
+}
+
+// f(z, id) for this thread's ids of all tiles, ascending
+template <typename F>
+__device__ __forceinline__ void each_id(const float* __restrict__ row, int V, float T, bool vec, int ntiles, F&& f) {
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int j0 = tile * SMP_TILE + (int)threadIdx.x * 8;
+        if (j0 >= V) break;
+        float z[8];
+        load_ids8(row, j0, V, T, vec, z);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (j0 + e < V) f(z[e], j0 + e);
+    }
+}
+
+__global__ __launch_bounds__(SMP_NT) void sample_tiles_kernel(
+    const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, float* __restrict__ tile_m, float* __restrict__ tile_s,
+    int* __restrict__ tile_i, int V) {
+    __shared__ float sf[SMP_WAVES];
+    __shared__ int si[SMP_WAVES];
+    const int tile = blockIdx.x, ntiles = gridDim.x, r = blockIdx.y, tid = threadIdx.x;
+    const float* row = logits + (size_t)r * V;
+    const float T = temperature[r];
+    const int j0 = tile * SMP_TILE + tid * 8;
+    const size_t slot = (size_t)r * ntiles + tile;
+    if (!(T > 0.f)) {                                          // greedy: the tile's (maximum, lowest index)
+        float v = -INFINITY;
+        int i = 0x7fffffff;
+        for (int e = 0; e < 8 && j0 + e < V; ++e) {
+            const float x = row[j0 + e];
+            if (x > v || i == 0x7fffffff) { v = x; i = j0 + e; }
+        }
+        block_argmax(v, i, sf, si);
+        if (tid == 0) { tile_m[slot] = v; tile_i[slot] = i; }
+        return;
+    }
+    float z[8], m = -INFINITY;
+    load_ids8(row, j0, V, T, (reinterpret_cast<uintptr_t>(row) & 15) == 0, z);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m = fmaxf(m, z[e]);
+    m = block_max_f(m, sf);
+    if (!sample_unfiltered(top_k[r], top_p[r], V)) {           // with top-k or top-p: the maximum is all
+        if (tid == 0) tile_m[slot] = m;
+        return;
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum += (j0 + e < V && m > -INFINITY) ? expf(z[e] - m) : 0.f;       // (a tile of -inf alone has no mass)
+    sum = block_sum<SMP_NT>(sum, sf);
+    if (tid == 0) { tile_m[slot] = m; tile_s[slot] = sum; }
+}
+
+// tile_m, tile_s, tile_i: what sample_tiles_kernel left for the row's ntiles tiles (ntiles <= SMP_NT)
 __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p,
-    const float* __restrict__ uniform, int* __restrict__ out, int V) {
-    __shared__ float sf[SMP_NT / LI_WAVE];
-    __shared__ int si[SMP_NT / LI_WAVE];
-    __shared__ float part_f[SMP_NT];
-    __shared__ int part_i[SMP_NT];
-    __shared__ int chosen_thread;
+    const float* __restrict__ uniform, int* __restrict__ out, int V,
+    const float* __restrict__ tile_m, const float* __restrict__ tile_s, const int* __restrict__ tile_i, int ntiles) {
+    __shared__ float sf[SMP_WAVES];
+    __shared__ int si[SMP_WAVES];
+    __shared__ float tile_sum[SMP_NT];               // the survivors' mass of every tile
+    __shared__ int ties_before[SMP_NT];              // ids at the threshold before every tile
+    __shared__ float work_f[SMP_WAVES * 16], tot_f[16];
+    __shared__ int work_i[SMP_WAVES * 16], tot_i[16];
+    __shared__ float pick_f[3];
+    __shared__ int pick_i[1];
     const int r = blockIdx.x, tid = threadIdx.x;
     const float* row = logits + (size_t)r * V;
     const float T = temperature[r];
-    if (!(T > 0.f)) {                                          // greedy
+    tile_m += (size_t)r * ntiles;
+    tile_s += (size_t)r * ntiles;
+    tile_i += (size_t)r * ntiles;
+    if (!(T > 0.f)) {                                          // greedy: the tiles' maxima, ties to the lower id
         float v = -INFINITY;
         int i = 0x7fffffff;
-        for (int j = tid; j < V; j += SMP_NT) {
-            const float x = row[j];
-            if (x > v || i == 0x7fffffff) { v = x; i = j; }
-        }
+        for (int t = tid; t < ntiles; t += SMP_NT) argmax_combine(v, i, tile_m[t], tile_i[t]);
         block_argmax(v, i, sf, si);
         if (tid == 0) out[r] = i;
         return;
     }
-    {
-        // Temperature alone (no top-k, no top-p: every id survives), the common case: no thresholds
-        // to search for and no ties to count, so the row is read three times in whole lines.
-        // Ids are taken in tiles of SMP_NT * 8: thread t holds the 8 consecutive ids t * 8 .. of a
-        // tile.  The inverse CDF runs over ascending ids: tile by tile (sums of whole tiles, each a
-        // block sum in its fixed order), then thread by thread within the tile that holds the
-        // target, then id by id within that thread.
-        const int kk = top_k[r];
-        const float pp = top_p[r];
-        constexpr int TILE = SMP_NT * 8;
-        const int ntiles = (V + TILE - 1) / TILE;
-        if (!(kk > 0 && kk < V) && !(pp > 0.f && pp < 1.f) && ntiles <= SMP_NT) {
-            float m = -INFINITY;
-            for (int j = tid; j < V; j += SMP_NT) m = fmaxf(m, row[j] / T);
-            m = block_max_f(m, sf);
-            auto mine_of = [&](int tile) {               // this thread's 8 ids of a tile, in id order
-                const int j0 = tile * TILE + tid * 8;
-                float s = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) s += (j0 + e < V) ? expf(row[j0 + e] / T - m) : 0.f;
-                return s;
-            };
-            for (int tile = 0; tile < ntiles; ++tile) {
-                const float ts = block_sum<SMP_NT>(mine_of(tile), sf);
-                if (tid == 0) part_f[tile] = ts;         // (ntiles <= SMP_NT places)
-            }
-            __syncthreads();
-            if (tid == 0) {
-                float total = 0.f;
-                for (int t = 0; t < ntiles; ++t) total += part_f[t];
-                const float target = uniform[r] * total;
-                float run = 0.f;
-                int pick = ntiles - 1;                   // rounding may leave the target just above the total
-                for (int t = 0; t < ntiles; ++t) {
-                    if (run + part_f[t] >= target) { pick = t; break; }
-                    run += part_f[t];
-                }
-                si[0] = pick;
-                sf[0] = run;
-                sf[1] = target;
-            }
-            __syncthreads();
-            const int tile = si[0];
-            const float before_tile = sf[0], target = sf[1];
-            __syncthreads();
-            part_f[tid] = mine_of(tile);
-            __syncthreads();
-            if (tid == 0) {
-                float run = before_tile;
-                int pick = -1, last = 0;
-                for (int t = 0; t < SMP_NT; ++t) {
-                    if (tile * TILE + t * 8 < V) last = t;
-                    if (pick < 0 && tile * TILE + t * 8 < V && run + part_f[t] >= target) pick = t;
-                    if (pick < 0) run += part_f[t];
-                }
-                if (pick < 0) { pick = last; run -= part_f[last]; }
-                chosen_thread = pick;
-                sf[0] = run;
-            }
-            __syncthreads();
-            if (tid == chosen_thread) {
-                float run = sf[0];
-                const int j0 = tile * TILE + tid * 8;
-                int pick = j0;
-                for (int e = 0; e < 8 && j0 + e < V; ++e) {
-                    pick = j0 + e;
-                    run += expf(row[j0 + e] / T - m);
-                    if (run >= target) break;
-                }
-                out[r] = pick;
-            }
-            return;
-        }
-    }
-    // contiguous chunk of ids per thread, so that block scans run in id order
-    const int chunk = (V + SMP_NT - 1) / SMP_NT;
-    const int c0 = min(tid * chunk, V), c1 = min(c0 + chunk, V);
+    const bool vec = (reinterpret_cast<uintptr_t>(row) & 15) == 0;
+    const int k = top_k[r];
+    const float p = top_p[r];
+    const bool filtered = !sample_unfiltered(k, p, V);
 
-    float m = -INFINITY;
-    for (int j = c0; j < c1; ++j) m = fmaxf(m, row[j] / T);
-    m = block_max_f(m, sf);
-
-    // ---- top-k: tau_k = k-th largest key, need_k = how many of its ties count
+    // The survivors are the ids with key > tau and the first `need` (in id order) of those with key == tau.
+    bool cut = false;
     uint32_t tau = 0u;
     int need = 0x7fffffff;
-    const int k = top_k[r];
-    if (k > 0 && k < V) {
-        for (int bit = 31; bit >= 0; --bit) {
-            const uint32_t cand = tau | (1u << bit);
-            int c = 0;
-            for (int j = c0; j < c1; ++j) c += sort_key(row[j] / T) >= cand;
-            if (block_sum_int(c, si) >= k) tau = cand;
+    float m = -INFINITY;                              // the maximum that masses are taken against
+    int tile = 0;                                     // the tile that holds the target,
+    float before = 0.f, target = 0.f;                 // the mass before it and the target, in units of exp(z - m)
+
+    if (filtered) {
+        for (int t = 0; t < ntiles; ++t) m = fmaxf(m, tile_m[t]);
+        if (k > 0 && k < V) {
+            // tau = the k-th largest key, four bits a pass: counts of the 16 values of the next digit among
+            // the keys that agree with the digits found so far
+            cut = true;
+            int kk = k;
+            for (int shift = 28; shift >= 0; shift -= 4) {
+                int cnt[16];
+#pragma unroll
+                for (int b = 0; b < 16; ++b) cnt[b] = 0;
+                each_id(row, V, T, vec, ntiles, [&](float z, int) {
+                    const uint32_t key = sort_key(z);
+                    if (shift == 28 || (key >> (shift + 4)) == (tau >> (shift + 4))) {
+                        const int d = (key >> shift) & 15;
+#pragma unroll
+                        for (int b = 0; b < 16; ++b) cnt[b] += (d == b);
+                    }
+                });
+                block_sum16(cnt, work_i, tot_i);
+                int above = 0, d = 15;
+                for (; d > 0; --d) {
+                    if (above + tot_i[d] >= kk) break;
+                    above += tot_i[d];
+                }
+                kk -= above;
+                tau |= (uint32_t)d << shift;
+            }
+            need = kk;                               // (>= 1) of the ids equal to the k-th largest count
         }
-        int c = 0;
-        for (int j = c0; j < c1; ++j) c += sort_key(row[j] / T) > tau;
-        need = k - block_sum_int(c, si);
-    }
-    // ---- top-p among the top-k survivors
-    const float p = top_p[r];
-    if (p > 0.f && p < 1.f) {
-        // Z_k: mass of the top-k survivors (ties at tau in id order, `need` of them)
-        int eq = 0;
-        for (int j = c0; j < c1; ++j) eq += sort_key(row[j] / T) == tau;
-        part_i[tid] = eq;
-        __syncthreads();
-        int before = 0;
-        for (int t = 0; t < tid; ++t) before += part_i[t];
-        float zk = 0.f;
-        {
-            int rank = before;
-            for (int j = c0; j < c1; ++j) {
-                const float z = row[j] / T;
+        if (p > 0.f && p < 1.f) {
+            // mass of the top-k survivors, and how many ids sit at tau
+            float zk = 0.f;
+            int eq = 0;
+            each_id(row, V, T, vec, ntiles, [&](float z, int) {
                 const uint32_t key = sort_key(z);
-                if (key > tau || (key == tau && rank++ < need)) zk += expf(z - m);
+                if (!cut || key > tau) zk += expf(z - m);
+                else if (key == tau) ++eq;
+            });
+            zk = block_sum<SMP_NT>(zk, sf);
+            const int ties = cut ? min(need, block_sum_int(eq, si)) : 0;
+            const float e_ties = cut ? (float)ties * expf(key_value(tau) - m) : 0.f;
+            float remaining = p * (zk + e_ties);      // mass that the prefix has to reach
+            // tp = the largest key c with mass(keys >= c) >= that, four bits a pass: masses by the next digit
+            uint32_t tp = 0u;
+            for (int shift = 28; shift >= 0; shift -= 4) {
+                float mass[16];
+#pragma unroll
+                for (int b = 0; b < 16; ++b) mass[b] = 0.f;
+                each_id(row, V, T, vec, ntiles, [&](float z, int) {
+                    const uint32_t key = sort_key(z);
+                    if ((!cut || key > tau) && (shift == 28 || (key >> (shift + 4)) == (tp >> (shift + 4)))) {
+                        const int d = (key >> shift) & 15;
+                        const float e = expf(z - m);
+#pragma unroll
+                        for (int b = 0; b < 16; ++b) mass[b] += (d == b) ? e : 0.f;
+                    }
+                });
+                block_sum16(mass, work_f, tot_f);
+                const bool ties_here = cut && ties > 0 && (shift == 28 || (tau >> (shift + 4)) == (tp >> (shift + 4)));
+                const int d_ties = (tau >> shift) & 15;
+                float above = 0.f;
+                int d = 15, lowest = -1;
+                bool reached = false;
+                for (; d >= 0; --d) {
+                    const float t = tot_f[d] + ((ties_here && d == d_ties) ? e_ties : 0.f);
+                    if (t > 0.f) lowest = d;
+                    if (t > 0.f && above + t >= remaining) { reached = true; break; }
+                    above += t;
+                }
+                if (!reached) {                       // rounding left the target just above the sum: the lowest digit with mass
+                    d = lowest < 0 ? 0 : lowest;
+                    above = 0.f;
+                    for (int b = 15; b > d; --b) above += tot_f[b] + ((ties_here && b == d_ties) ? e_ties : 0.f);
+                }
+                remaining -= above;
+                tp |= (uint32_t)d << shift;
             }
-        }
-        zk = block_sum<SMP_NT>(zk, sf);
-        const float target = p * zk;
-        // tp = the largest c with f(c) >= target, where f(c) = Z_k for c <= tau (the top-k
-        // survivors as a whole) and the mass of the keys >= c above it; f does not increase
-        uint32_t tp = 0u;
-        for (int bit = 31; bit >= 0; --bit) {
-            const uint32_t cand = tp | (1u << bit);
-            if (cand <= tau) { tp = cand; continue; }
-            float s = 0.f;
-            for (int j = c0; j < c1; ++j) {
-                const float z = row[j] / T;
-                if (sort_key(z) >= cand) s += expf(z - m);
+            const float e_tp = expf(key_value(tp) - m);
+            int need_p = 0x7fffffff;                  // ties without mass: all of them
+            if (e_tp > 0.f) {
+                const float q = ceilf(remaining / e_tp);
+                need_p = q < 1.f ? 1 : (q > 2.0e9f ? 0x7fffffff : (int)q);
             }
-            if (block_sum<SMP_NT>(s, sf) >= target) tp = cand;
+            need = (cut && tp == tau) ? min(need, need_p) : need_p;
+            tau = tp;
+            cut = true;
         }
-        float s = 0.f;
-        for (int j = c0; j < c1; ++j) {
-            const float z = row[j] / T;
-            if (sort_key(z) > tp) s += expf(z - m);
-        }
-        const float mass_gt = block_sum<SMP_NT>(s, sf);
-        const float e_tau = expf(key_value(tp) - m);
-        int need_p = 0x7fffffff;                               // ties without mass: all of them
-        if (e_tau > 0.f) {
-            const float q = ceilf((target - mass_gt) / e_tau);
-            need_p = q < 1.f ? 1 : (q > 2.0e9f ? 0x7fffffff : (int)q);
-        }
-        need = (tp == tau) ? min(need, need_p) : need_p;
-        tau = tp;
     }
+
     // ---- inverse CDF over ascending ids among the survivors
-    int eq = 0;
-    for (int j = c0; j < c1; ++j) eq += sort_key(row[j] / T) == tau;
-    __syncthreads();
-    part_i[tid] = eq;
-    __syncthreads();
-    int before = 0;
-    for (int t = 0; t < tid; ++t) before += part_i[t];
-    __syncthreads();                 // part_i is written again below
-    float mine = 0.f;
-    int last_in = -1;
-    {
-        int rank = before;
-        for (int j = c0; j < c1; ++j) {
-            const float z = row[j] / T;
-            const uint32_t key = sort_key(z);
-            if (key > tau || (key == tau && rank++ < need)) { mine += expf(z - m); last_in = j; }
-        }
-    }
-    part_f[tid] = mine;
-    part_i[tid] = last_in;           // (the tie counts are no longer needed: `before` is in a register)
-    if (tid == 0) chosen_thread = -1;
-    __syncthreads();
-    if (tid == 0) {                  // sequential scan in id order: 1024 additions, fixed order
-        float total = 0.f;
-        for (int t = 0; t < SMP_NT; ++t) total += part_f[t];
-        const float target = uniform[r] * total;
-        float run = 0.f;
-        int pick = -1, last_nonempty = -1;
-        for (int t = 0; t < SMP_NT; ++t) {
-            if (part_i[t] >= 0) last_nonempty = t;
-            if (pick < 0 && part_i[t] >= 0 && run + part_f[t] >= target) pick = t;
-            if (pick < 0) run += part_f[t];
-        }
-        if (pick < 0) pick = last_nonempty;               // rounding left the target just above the total
-        chosen_thread = pick;
-        sf[0] = run;                                       // mass before the chosen thread's chunk
-        sf[1] = target;
-    }
-    __syncthreads();
-    if (tid == chosen_thread) {
-        float run = sf[0];
-        const float target = sf[1];
-        int rank = before, pick = last_in;
-        for (int j = c0; j < c1; ++j) {
-            const float z = row[j] / T;
-            const uint32_t key = sort_key(z);
-            if (key > tau || (key == tau && rank++ < need)) {
-                run += expf(z - m);
-                if (run >= target) { pick = j; break; }
+    // Are there more ids at tau than count?  Then an id's place among them decides (ties_before).
+    bool ranked = false;
+    if (cut) {
+        int eq = 0;
+        each_id(row, V, T, vec, ntiles, [&](float z, int) { eq += sort_key(z) == tau; });
+        ranked = block_sum_int(eq, si) > need;
+        if (ranked) {
+            int running = 0;
+            for (int t = 0; t < ntiles; ++t) {
+                const int j0 = t * SMP_TILE + tid * 8;
+                float z[8];
+                int c = 0;
+                if (j0 < V) {
+                    load_ids8(row, j0, V, T, vec, z);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) c += (j0 + e < V) && sort_key(z[e]) == tau;
+                }
+                c = block_sum_int(c, si);
+                if (tid == 0) ties_before[t] = running;
+                running += c;
             }
+            __syncthreads();
+        }
+    }
+    // this thread's ids of a tile: their mass (sum in id order), whether any survives, and the place
+    // among the ids at tau of its first one
+    auto mine_of = [&](int t, bool& any, int& rank0) {
+        const int j0 = t * SMP_TILE + tid * 8;
+        float z[8];
+        any = false;
+        rank0 = 0;
+        if (j0 < V) load_ids8(row, j0, V, T, vec, z);
+        if (ranked) {
+            int c = 0;
+            if (j0 < V) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) c += (j0 + e < V) && sort_key(z[e]) == tau;
+            }
+            rank0 = ties_before[t] + block_sum_before(c, work_i);
+        }
+        float sum = 0.f;
+        if (j0 < V) {
+            int rank = rank0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (j0 + e >= V) continue;
+                const uint32_t key = sort_key(z[e]);
+                const bool in = !cut || key > tau || (key == tau && (!ranked || rank++ < need));
+                if (in) { sum += expf(z[e] - m); any = true; }
+            }
+        }
+        return sum;
+    };
+    if (!filtered) {
+        // The tiles' sums are there, each against its tile's own maximum: brought to the row's maximum
+        // they give the tile that holds the target; within it the search goes on in the tile's own scale.
+        if (tid == 0) {
+            float top = -INFINITY;
+            for (int t = 0; t < ntiles; ++t) top = fmaxf(top, tile_m[t]);
+            float total = 0.f;
+            for (int t = 0; t < ntiles; ++t) total += tile_s[t] * expf(tile_m[t] - top);
+            const float want = uniform[r] * total;
+            float run = 0.f;
+            int pick = -1, last = 0;                 // (a tile far below the maximum has no mass at all in float32)
+            for (int t = 0; t < ntiles; ++t) {
+                const float w = tile_s[t] * expf(tile_m[t] - top);
+                if (w > 0.f) last = t;
+                if (w > 0.f && run + w >= want) { pick = t; break; }
+                run += w;
+            }
+            const bool past = pick < 0;              // rounding left the target just above the total:
+            if (past) pick = last;                   // the last id with mass (no sum reaches infinity below)
+            pick_i[0] = pick;
+            pick_f[0] = 0.f;
+            pick_f[1] = past ? INFINITY : (want - run) / expf(tile_m[pick] - top);
+            pick_f[2] = tile_m[pick];
+        }
+        __syncthreads();
+        m = pick_f[2];
+    } else {
+        for (int t = 0; t < ntiles; ++t) {
+            bool any;
+            int rank0;
+            const float ts = block_sum<SMP_NT>(mine_of(t, any, rank0), sf);
+            if (tid == 0) tile_sum[t] = ts;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float total = 0.f;
+            for (int t = 0; t < ntiles; ++t) total += tile_sum[t];
+            const float want = uniform[r] * total;
+            float run = 0.f;
+            int pick = -1, last = 0;
+            for (int t = 0; t < ntiles; ++t) {
+                if (tile_sum[t] > 0.f) last = t;
+                if (tile_sum[t] > 0.f && run + tile_sum[t] >= want) { pick = t; break; }
+                run += tile_sum[t];
+            }
+            const bool past = pick < 0;
+            if (past) pick = last;
+            pick_i[0] = pick;
+            pick_f[0] = past ? 0.f : run;
+            pick_f[1] = past ? INFINITY : want;
+        }
+        __syncthreads();
+    }
+    tile = pick_i[0];
+    before = pick_f[0];
+    target = pick_f[1];
+    // within the tile: the first thread whose ids bring the running sum to the target, else the last one with a survivor
+    bool any;
+    int rank0;
+    const float mine = mine_of(tile, any, rank0);
+    const float run0 = before + block_sum_before(mine, work_f);
+    int chosen = block_min_int((any && run0 + mine >= target) ? tid : 0x7fffffff, si);
+    if (chosen == 0x7fffffff) chosen = -block_min_int(any ? -tid : 1, si);     // (the tile has a survivor: its sum is above zero)
+    if (tid == chosen) {
+        const int j0 = tile * SMP_TILE + tid * 8;
+        float z[8];
+        load_ids8(row, j0, V, T, vec, z);
+        float run = run0;
+        int rank = rank0, pick = j0;
+        for (int e = 0; e < 8 && j0 + e < V; ++e) {
+            const uint32_t key = sort_key(z[e]);
+            const bool in = !cut || key > tau || (key == tau && (!ranked || rank++ < need));
+            if (!in) continue;
+            pick = j0 + e;
+            run += expf(z[e] - m);
+            if (run >= target) break;
         }
         out[r] = pick;
     }
 }
 
+// tiles: room for 3 * n * ceil(V / 8192) floats, in which the first kernel leaves every tile's part.
 extern "C" int li_sample_rows(const float* logits, const float* temperature, const int* top_k,
                               const float* top_p, const float* uniform, int* out, int n, int V,
-                              hipStream_t stream) {
-    if (n <= 0 || V <= 0) return LI_ERR_SIZE;
-    sample_rows_kernel<<<n, SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V);
+                              float* tiles, long tiles_floats, hipStream_t stream) {
+    if (n <= 0 || n > 65535 || V <= 0) return LI_ERR_SIZE;
+    const int ntiles = (V + SMP_TILE - 1) / SMP_TILE;
+    if (ntiles > SMP_NT || !tiles || tiles_floats < 3l * n * ntiles) return LI_ERR_SIZE;
+    float* tm = tiles;
+    float* ts = tiles + (size_t)n * ntiles;
+    int* ti = reinterpret_cast<int*>(tiles + 2 * (size_t)n * ntiles);
+    sample_tiles_kernel<<<dim3(ntiles, n), SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, tm, ts, ti, V);
+    sample_rows_kernel<<<n, SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V, tm, ts, ti, ntiles);
     return li_launch_status();
 }

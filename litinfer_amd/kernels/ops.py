@@ -52,7 +52,7 @@ _SIGNATURES = {
     },
     "sampling": {
         "li_argmax_rows": [P, P, P, P, I, I],
-        "li_sample_rows": [P, P, P, P, P, P, I, I],
+        "li_sample_rows": [P, P, P, P, P, P, I, I, P, L],
     },
 }
 _fn_cache = {}
@@ -644,6 +644,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
 
 # ------------------------------------------------------------------ sampling
 _argmax_scratch = {}
+_sample_scratch = {}
 
 
 def argmax_rows(logits: torch.Tensor, out: torch.Tensor) -> None:
@@ -677,5 +678,10 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
                    (uniform, torch.float32), (out, torch.int32)):
         _chk(t_.dtype is dt and t_.numel() == n and t_.is_contiguous(), "sample: per-row arrays")
     if n:
+        v = logits.shape[1]
+        key = (logits.device, n, v)
+        if key not in _sample_scratch:               # the tiles' parts of the kernel's first stage
+            _sample_scratch[key] = torch.empty(3 * n * ((v + 8191) // 8192), dtype=torch.float32, device=logits.device)
+        tiles = _sample_scratch[key]
         _run("sampling", "li_sample_rows", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(),
-             top_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), n, logits.shape[1])
+             top_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), n, v, tiles.data_ptr(), tiles.numel())

@@ -740,6 +740,50 @@ def test_sample_rows_with_temperature_alone(ops, vocab):
     assert same >= n - 4
 
 
+def test_sample_rows_with_tiles_of_the_vocabulary_masked_out(ops):
+    # the rows' ids are summed in tiles of 8,192 first: a tile of -inf alone, a tile so far below the
+    # maximum that it has no mass in float32, and the last tile cut short must not disturb the pick
+    g = torch.Generator().manual_seed(16)
+    vocab, n = 3 * 8192 + 5, 16
+    logits = torch.randn(n, vocab, generator=g) * 2
+    logits[:8, 8192:16384] = float("-inf")
+    logits[8:12, :8192] -= 200.0
+    logits[12:, 16384:] = float("-inf")                      # the last two tiles, the short one among them
+    temperature = [0.0, 1.0, 0.7, 1.5] * 4
+    u = torch.rand(n, generator=g).tolist()
+    u[1], u[2], u[5], u[13] = 0.99999994, 0.0, 0.99999994, 0.99999994
+    picks = _sample(ops, logits, temperature, [0] * n, [1.0] * n, u)
+    rows = logits.double().numpy()
+    for r in range(n):
+        assert np.isfinite(rows[r][picks[r]]), r
+        if temperature[r] == 0.0:
+            assert picks[r] == plain_impl.argmax_first(rows[r])
+        else:
+            assert _pick_is_right(rows[r], temperature[r], 0, 1.0, u[r], picks[r]), r
+    assert all(p < 8192 or p >= 16384 for p in picks[:8]) and all(p >= 8192 for p in picks[9:12]) and all(p < 16384 for p in picks[12:])
+
+
+@pytest.mark.parametrize("vocab", [1000, 20000, 152064])
+def test_sample_rows_with_many_equal_logits_at_the_thresholds(ops, vocab):
+    # logits on a coarse grid: hundreds of ids share the k-th largest value and the value at which top-p
+    # cuts, spread over the threads and tiles of the kernel; which of them survive goes by ascending id
+    g = torch.Generator().manual_seed(17)
+    n = 16
+    logits = torch.round(torch.randn(n, vocab, generator=g) * 2) / 2
+    temperature = [1.0, 0.5, 2.0, 0.8] * 4
+    top_k = [50, 0, 300, 7, 1000, 0, 2, 64, 999, 0, 50, 50, 0, 5000, 20, 1][:n]
+    top_k = [min(k, vocab - 1) for k in top_k]
+    top_p = [1.0, 0.6, 0.9, 0.5, 0.95, 0.99, 1.0, 0.3, 1.0, 0.05, 0.8, 0.999, 0.9, 0.7, 1.0, 1.0]
+    u = torch.rand(n, generator=g).tolist()
+    u[0], u[1], u[2] = 0.99999994, 0.0, 0.99999994
+    picks = _sample(ops, logits, temperature, top_k, top_p, u)
+    rows = logits.double().numpy()
+    for r in range(n):
+        assert _pick_is_right(rows[r], temperature[r], top_k[r], top_p[r], u[r], picks[r]), r
+    same = sum(picks[r] == plain_impl.sample_with_uniform(rows[r], temperature[r], top_k[r], top_p[r], u[r]) for r in range(n))
+    assert same >= n - 2
+
+
 def test_sample_rows_frequencies_and_ties(ops):
     lg = torch.tensor([[2.0, 1.0, 3.0, 3.0, -1.0, 0.5, 2.5, 0.0]])
     n = 4000
