@@ -208,20 +208,33 @@ __device__ __forceinline__ int block_min_int(int v, int* smem) {
     return t;
 }
 
-// The 16 sums of a pass over the whole block, left in tot[0..15] for every thread to read: within a
-// wave by the shuffle tree, then the waves in their order.  work: SMP_WAVES * 16 values.
+// The 16 sums of a pass over the whole block, left in tot[0..15] for every thread to read.  Within a
+// wave the lanes halve what they hold step by step (a lane keeps one half of its sums and gets the
+// other lane's part of that half: 8 + 4 + 2 + 1 exchanges), until each lane holds one sum of its 16
+// lanes, then the four groups of 16 lanes are added: 17 exchanges instead of 96; then the waves in
+// their order.  The order of the additions is fixed.  work: SMP_WAVES * 16 values.
 template <typename T>
 __device__ __forceinline__ void block_sum16(T (&c)[16], T* work, T* tot) {
-#pragma unroll
-    for (int b = 0; b < 16; ++b)
-#pragma unroll
-        for (int o = LI_WAVE / 2; o > 0; o >>= 1) c[b] += __shfl_xor(c[b], o, LI_WAVE);
     const int lane = threadIdx.x & (LI_WAVE - 1), w = threadIdx.x / LI_WAVE;
-    __syncthreads();                                 // (the last pass's totals have been read)
-    if (lane == 0) {
-#pragma unroll
-        for (int b = 0; b < 16; ++b) work[w * 16 + b] = c[b];
+#define LI_HALVE(H, MASK)                                                         \
+    {                                                                             \
+        const bool upper = (lane & (MASK)) != 0;                                  \
+        _Pragma("unroll") for (int i = 0; i < (H); ++i) {                         \
+            const T give = upper ? c[i] : c[i + (H)];                             \
+            const T keep = upper ? c[i + (H)] : c[i];                             \
+            c[i] = keep + __shfl_xor(give, (MASK), LI_WAVE);                      \
+        }                                                                         \
     }
+    LI_HALVE(8, 1)
+    LI_HALVE(4, 2)
+    LI_HALVE(2, 4)
+    LI_HALVE(1, 8)
+#undef LI_HALVE
+    c[0] += __shfl_xor(c[0], 16, LI_WAVE);
+    c[0] += __shfl_xor(c[0], 32, LI_WAVE);
+    // lane l < 16 now holds the wave's sum number 8 (l & 1) + 4 (l >> 1 & 1) + 2 (l >> 2 & 1) + (l >> 3 & 1)
+    __syncthreads();                                 // (the last pass's totals have been read)
+    if (lane < 16) work[w * 16 + 8 * (lane & 1) + 4 * ((lane >> 1) & 1) + 2 * ((lane >> 2) & 1) + ((lane >> 3) & 1)] = c[0];
     __syncthreads();
     if (threadIdx.x < 16) {
         T t = 0;
@@ -277,12 +290,107 @@ __device__ __forceinline__ void each_id(const float* __restrict__ row, int V, fl
     }
 }
 
+// tau = the kk-th largest key among the z that `each` hands out (to all threads of the block together),
+// need (>= 1) = how many of the keys equal to tau are among the kk largest.  Four bits a pass: counts of
+// the 16 values of the next digit among the keys that agree with the digits found so far.
+template <typename Each>
+__device__ __forceinline__ void radix_kth(Each&& each, int kk, uint32_t& tau, int& need, int* work_i, int* tot_i) {
+    tau = 0u;
+    for (int shift = 28; shift >= 0; shift -= 4) {
+        int cnt[16];
+#pragma unroll
+        for (int b = 0; b < 16; ++b) cnt[b] = 0;
+        each([&](float z) {
+            const uint32_t key = sort_key(z);
+            if (shift == 28 || (key >> (shift + 4)) == (tau >> (shift + 4))) {
+                const int d = (key >> shift) & 15;
+#pragma unroll
+                for (int b = 0; b < 16; ++b) cnt[b] += (d == b);
+            }
+        });
+        block_sum16(cnt, work_i, tot_i);
+        int above = 0, d = 15;
+        for (; d > 0; --d) {
+            if (above + tot_i[d] >= kk) break;
+            above += tot_i[d];
+        }
+        kk -= above;
+        tau |= (uint32_t)d << shift;
+    }
+    need = kk;
+}
+
+// Top-p among the survivors of top-k (cut: the keys above tau, and `ties` keys equal to tau with
+// e_ties = their mass together; not cut: all keys): tp = the largest key c with mass(keys >= c) >=
+// `remaining`, four bits a pass (masses by the next digit); on return `remaining` is what the keys
+// equal to tp have to bring.  m: the maximum that masses are taken against.
+template <typename Each>
+__device__ __forceinline__ void radix_mass(Each&& each, bool cut, uint32_t tau, int ties, float e_ties, float m,
+                                           float& remaining, uint32_t& tp, float* work_f, float* tot_f) {
+    tp = 0u;
+    for (int shift = 28; shift >= 0; shift -= 4) {
+        float mass[16];
+#pragma unroll
+        for (int b = 0; b < 16; ++b) mass[b] = 0.f;
+        each([&](float z) {
+            const uint32_t key = sort_key(z);
+            if ((!cut || key > tau) && (shift == 28 || (key >> (shift + 4)) == (tp >> (shift + 4)))) {
+                const int d = (key >> shift) & 15;
+                const float e = expf(z - m);
+#pragma unroll
+                for (int b = 0; b < 16; ++b) mass[b] += (d == b) ? e : 0.f;
+            }
+        });
+        block_sum16(mass, work_f, tot_f);
+        const bool ties_here = cut && ties > 0 && (shift == 28 || (tau >> (shift + 4)) == (tp >> (shift + 4)));
+        const int d_ties = (tau >> shift) & 15;
+        float above = 0.f;
+        int d = 15, lowest = -1;
+        bool reached = false;
+        for (; d >= 0; --d) {
+            const float t = tot_f[d] + ((ties_here && d == d_ties) ? e_ties : 0.f);
+            if (t > 0.f) lowest = d;
+            if (t > 0.f && above + t >= remaining) { reached = true; break; }
+            above += t;
+        }
+        if (!reached) {                       // rounding left the target just above the sum: the lowest digit with mass
+            d = lowest < 0 ? 0 : lowest;
+            above = 0.f;
+            for (int b = 15; b > d; --b) above += tot_f[b] + ((ties_here && b == d_ties) ? e_ties : 0.f);
+        }
+        remaining -= above;
+        tp |= (uint32_t)d << shift;
+    }
+}
+
+// how many of the keys equal to tp count, from what they have to bring
+__device__ __forceinline__ int ties_needed(float remaining, uint32_t tp, float m) {
+    const float e_tp = expf(key_value(tp) - m);
+    if (!(e_tp > 0.f)) return 0x7fffffff;     // ties without mass: all of them
+    const float q = ceilf(remaining / e_tp);
+    return q < 1.f ? 1 : (q > 2.0e9f ? 0x7fffffff : (int)q);
+}
+
+// Rows with top-k or top-p: the first kernel hands the second one, per tile, the tile's SMP_KC
+// or fewer largest ids (in the order (value descending, id ascending)), so that the second kernel
+// searches among ntiles * kc candidates in registers instead of reading the row pass after pass.
+// With top-k <= SMP_KC the candidates hold all survivors (kc = k).  With top-p alone kc = SMP_KC_P
+// and the second kernel checks that the prefix ends above the kc-th largest id of the row, whose
+// betters are all among the candidates; otherwise it reads the row.  0: no candidates.
+constexpr int SMP_KC = 256, SMP_KC_P = 128, SMP_CAND_PER_THREAD = 8;
+__device__ __forceinline__ int sample_candidates(int k, float p, int V, int ntiles) {
+    if (sample_unfiltered(k, p, V)) return 0;
+    const int kc = (k > 0 && k < V) ? k : SMP_KC_P;
+    return (kc <= SMP_KC && (long)kc * ntiles <= (long)SMP_NT * SMP_CAND_PER_THREAD) ? kc : 0;
+}
+
 __global__ __launch_bounds__(SMP_NT) void sample_tiles_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, float* __restrict__ tile_m, float* __restrict__ tile_s,
-    int* __restrict__ tile_i, int V) {
+    int* __restrict__ tile_i, float* __restrict__ cand_z, int* __restrict__ cand_id, int V) {
     __shared__ float sf[SMP_WAVES];
     __shared__ int si[SMP_WAVES];
+    __shared__ int work_i[SMP_WAVES * 16], tot_i[16];
     const int tile = blockIdx.x, ntiles = gridDim.x, r = blockIdx.y, tid = threadIdx.x;
     const float* row = logits + (size_t)r * V;
     const float T = temperature[r];
@@ -304,23 +412,54 @@ __global__ __launch_bounds__(SMP_NT) void sample_tiles_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) m = fmaxf(m, z[e]);
     m = block_max_f(m, sf);
-    if (!sample_unfiltered(top_k[r], top_p[r], V)) {           // with top-k or top-p: the maximum is all
-        if (tid == 0) tile_m[slot] = m;
-        return;
-    }
     float sum = 0.f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) sum += (j0 + e < V && m > -INFINITY) ? expf(z[e] - m) : 0.f;       // (a tile of -inf alone has no mass)
     sum = block_sum<SMP_NT>(sum, sf);
     if (tid == 0) { tile_m[slot] = m; tile_s[slot] = sum; }
+    const int kc = sample_candidates(top_k[r], top_p[r], V, ntiles);
+    if (kc == 0) return;
+    // the tile's kc largest ids, written in id order
+    const int in_tile = min(SMP_TILE, V - tile * SMP_TILE);
+    const bool all = in_tile <= kc;
+    uint32_t tau = 0u;
+    int need = 0x7fffffff;
+    if (!all)
+        radix_kth([&](auto f) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (j0 + e < V) f(z[e]);
+        }, kc, tau, need, work_i, tot_i);
+    int eq = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) eq += (j0 + e < V) && sort_key(z[e]) == tau;
+    int rank = all ? 0 : block_sum_before(eq, si);
+    bool in[8];
+    int mine = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t key = sort_key(z[e]);
+        in[e] = (j0 + e < V) && (all || key > tau || (key == tau && rank++ < need));
+        mine += in[e];
+    }
+    int pos = block_sum_before(mine, si);
+    const size_t base = slot * SMP_KC;
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+        if (in[e]) {
+            cand_z[base + pos] = z[e];
+            cand_id[base + pos] = j0 + e;
+            ++pos;
+        }
 }
 
-// tile_m, tile_s, tile_i: what sample_tiles_kernel left for the row's ntiles tiles (ntiles <= SMP_NT)
+// tile_m, tile_s, tile_i, cand_z, cand_id: what sample_tiles_kernel left for the row's ntiles tiles (ntiles <= SMP_NT)
 __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
     const float* __restrict__ logits, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p,
     const float* __restrict__ uniform, int* __restrict__ out, int V,
-    const float* __restrict__ tile_m, const float* __restrict__ tile_s, const int* __restrict__ tile_i, int ntiles) {
+    const float* __restrict__ tile_m, const float* __restrict__ tile_s, const int* __restrict__ tile_i,
+    const float* __restrict__ cand_z, const int* __restrict__ cand_id, int ntiles) {
     __shared__ float sf[SMP_WAVES];
     __shared__ int si[SMP_WAVES];
     __shared__ float tile_sum[SMP_NT];               // the survivors' mass of every tile
@@ -347,50 +486,133 @@ __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
     const int k = top_k[r];
     const float p = top_p[r];
     const bool filtered = !sample_unfiltered(k, p, V);
+    const bool by_k = k > 0 && k < V, by_p = p > 0.f && p < 1.f;
 
     // The survivors are the ids with key > tau and the first `need` (in id order) of those with key == tau.
     bool cut = false;
     uint32_t tau = 0u;
     int need = 0x7fffffff;
     float m = -INFINITY;                              // the maximum that masses are taken against
+    if (filtered)
+        for (int t = 0; t < ntiles; ++t) m = fmaxf(m, tile_m[t]);
+
+    const int kc = sample_candidates(k, p, V, ntiles);
+    if (kc > 0) {
+        // ---- among the candidates: slot s = tile * kc + place, ascending ids; thread t has the slots t * C ...
+        const int slots = ntiles * kc, C = (slots + SMP_NT - 1) / SMP_NT;
+        float cz[SMP_CAND_PER_THREAD];
+        int cid[SMP_CAND_PER_THREAD];
+        bool have[SMP_CAND_PER_THREAD];
+        int total = 0;                                // candidates in all
+        for (int t = 0; t < ntiles; ++t) total += min(kc, V - t * SMP_TILE);
+#pragma unroll
+        for (int c = 0; c < SMP_CAND_PER_THREAD; ++c) {
+            const int s = tid * C + c;
+            have[c] = false;
+            cz[c] = -INFINITY;
+            cid[c] = 0;
+            if (c < C && s < slots) {
+                const int t = s / kc, i = s % kc;
+                if (i < min(kc, V - t * SMP_TILE)) {
+                    const size_t at = ((size_t)r * ntiles + t) * SMP_KC + i;
+                    have[c] = true;
+                    cz[c] = cand_z[at];
+                    cid[c] = cand_id[at];
+                }
+            }
+        }
+        auto each = [&](auto f) {
+#pragma unroll
+            for (int c = 0; c < SMP_CAND_PER_THREAD; ++c)
+                if (have[c]) f(cz[c]);
+        };
+        // the k-th largest (top-k), or the kc-th: above it the candidates are all there is
+        uint32_t tau_c;
+        int need_c;
+        radix_kth(each, min(by_k ? k : kc, total), tau_c, need_c, work_i, tot_i);
+        bool exact = true;
+        if (by_k) { cut = true; tau = tau_c; need = need_c; }
+        if (by_p) {
+            float zk = 0.f;
+            int eq = 0;
+            each([&](float z) {
+                const uint32_t key = sort_key(z);
+                if (!cut || key > tau) zk += expf(z - m);
+                else if (key == tau) ++eq;
+            });
+            zk = block_sum<SMP_NT>(zk, sf);
+            const int ties = cut ? min(need, block_sum_int(eq, si)) : 0;
+            const float e_ties = cut ? (float)ties * expf(key_value(tau) - m) : 0.f;
+            if (!cut && total < V) {                  // the mass of all ids, from the tiles' sums
+                zk = 0.f;
+                for (int t = 0; t < ntiles; ++t) zk += tile_s[t] * expf(tile_m[t] - m);
+            }
+            float remaining = p * (zk + e_ties);
+            uint32_t tp;
+            radix_mass(each, cut, tau, ties, e_ties, m, remaining, tp, work_f, tot_f);
+            if (!by_k && total < V && !(tp > tau_c)) exact = false;       // the prefix may go on beyond the candidates
+            const int need_p = ties_needed(remaining, tp, m);
+            need = (cut && tp == tau) ? min(need, need_p) : need_p;
+            tau = tp;
+            cut = true;
+        }
+        if (exact) {
+            // inverse CDF over the surviving candidates in id order
+            int eq = 0;
+            each([&](float z) { eq += sort_key(z) == tau; });
+            const bool ranked = block_sum_int(eq, si) > need;
+            const int rank0 = ranked ? block_sum_before(eq, work_i) : 0;
+            float mine = 0.f;
+            bool any = false;
+            {
+                int rank = rank0;
+#pragma unroll
+                for (int c = 0; c < SMP_CAND_PER_THREAD; ++c) {
+                    if (!have[c]) continue;
+                    const uint32_t key = sort_key(cz[c]);
+                    if (key > tau || (key == tau && (!ranked || rank++ < need))) { mine += expf(cz[c] - m); any = true; }
+                }
+            }
+            const float run0 = block_sum_before(mine, work_f);
+            if (tid == SMP_NT - 1) pick_f[0] = uniform[r] * (run0 + mine);
+            __syncthreads();
+            const float target = pick_f[0];
+            int chosen = block_min_int((any && run0 + mine >= target) ? tid : 0x7fffffff, si);
+            if (chosen == 0x7fffffff) chosen = -block_min_int(any ? -tid : 1, si);
+            if (tid == chosen) {
+                float run = run0;
+                int rank = rank0, pick = cid[0];
+#pragma unroll
+                for (int c = 0; c < SMP_CAND_PER_THREAD; ++c) {
+                    if (!have[c]) continue;
+                    const uint32_t key = sort_key(cz[c]);
+                    if (!(key > tau || (key == tau && (!ranked || rank++ < need)))) continue;
+                    pick = cid[c];
+                    run += expf(cz[c] - m);
+                    if (run >= target) break;
+                }
+                out[r] = pick;
+            }
+            return;
+        }
+        cut = false;                                  // from the row itself, then
+        tau = 0u;
+        need = 0x7fffffff;
+    }
+
     int tile = 0;                                     // the tile that holds the target,
     float before = 0.f, target = 0.f;                 // the mass before it and the target, in units of exp(z - m)
-
+    auto each_of_row = [&](auto f) { each_id(row, V, T, vec, ntiles, [&](float z, int) { f(z); }); };
     if (filtered) {
-        for (int t = 0; t < ntiles; ++t) m = fmaxf(m, tile_m[t]);
-        if (k > 0 && k < V) {
-            // tau = the k-th largest key, four bits a pass: counts of the 16 values of the next digit among
-            // the keys that agree with the digits found so far
+        if (by_k) {
             cut = true;
-            int kk = k;
-            for (int shift = 28; shift >= 0; shift -= 4) {
-                int cnt[16];
-#pragma unroll
-                for (int b = 0; b < 16; ++b) cnt[b] = 0;
-                each_id(row, V, T, vec, ntiles, [&](float z, int) {
-                    const uint32_t key = sort_key(z);
-                    if (shift == 28 || (key >> (shift + 4)) == (tau >> (shift + 4))) {
-                        const int d = (key >> shift) & 15;
-#pragma unroll
-                        for (int b = 0; b < 16; ++b) cnt[b] += (d == b);
-                    }
-                });
-                block_sum16(cnt, work_i, tot_i);
-                int above = 0, d = 15;
-                for (; d > 0; --d) {
-                    if (above + tot_i[d] >= kk) break;
-                    above += tot_i[d];
-                }
-                kk -= above;
-                tau |= (uint32_t)d << shift;
-            }
-            need = kk;                               // (>= 1) of the ids equal to the k-th largest count
+            radix_kth(each_of_row, k, tau, need, work_i, tot_i);
         }
-        if (p > 0.f && p < 1.f) {
+        if (by_p) {
             // mass of the top-k survivors, and how many ids sit at tau
             float zk = 0.f;
             int eq = 0;
-            each_id(row, V, T, vec, ntiles, [&](float z, int) {
+            each_of_row([&](float z) {
                 const uint32_t key = sort_key(z);
                 if (!cut || key > tau) zk += expf(z - m);
                 else if (key == tau) ++eq;
@@ -399,47 +621,9 @@ __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
             const int ties = cut ? min(need, block_sum_int(eq, si)) : 0;
             const float e_ties = cut ? (float)ties * expf(key_value(tau) - m) : 0.f;
             float remaining = p * (zk + e_ties);      // mass that the prefix has to reach
-            // tp = the largest key c with mass(keys >= c) >= that, four bits a pass: masses by the next digit
-            uint32_t tp = 0u;
-            for (int shift = 28; shift >= 0; shift -= 4) {
-                float mass[16];
-#pragma unroll
-                for (int b = 0; b < 16; ++b) mass[b] = 0.f;
-                each_id(row, V, T, vec, ntiles, [&](float z, int) {
-                    const uint32_t key = sort_key(z);
-                    if ((!cut || key > tau) && (shift == 28 || (key >> (shift + 4)) == (tp >> (shift + 4)))) {
-                        const int d = (key >> shift) & 15;
-                        const float e = expf(z - m);
-#pragma unroll
-                        for (int b = 0; b < 16; ++b) mass[b] += (d == b) ? e : 0.f;
-                    }
-                });
-                block_sum16(mass, work_f, tot_f);
-                const bool ties_here = cut && ties > 0 && (shift == 28 || (tau >> (shift + 4)) == (tp >> (shift + 4)));
-                const int d_ties = (tau >> shift) & 15;
-                float above = 0.f;
-                int d = 15, lowest = -1;
-                bool reached = false;
-                for (; d >= 0; --d) {
-                    const float t = tot_f[d] + ((ties_here && d == d_ties) ? e_ties : 0.f);
-                    if (t > 0.f) lowest = d;
-                    if (t > 0.f && above + t >= remaining) { reached = true; break; }
-                    above += t;
-                }
-                if (!reached) {                       // rounding left the target just above the sum: the lowest digit with mass
-                    d = lowest < 0 ? 0 : lowest;
-                    above = 0.f;
-                    for (int b = 15; b > d; --b) above += tot_f[b] + ((ties_here && b == d_ties) ? e_ties : 0.f);
-                }
-                remaining -= above;
-                tp |= (uint32_t)d << shift;
-            }
-            const float e_tp = expf(key_value(tp) - m);
-            int need_p = 0x7fffffff;                  // ties without mass: all of them
-            if (e_tp > 0.f) {
-                const float q = ceilf(remaining / e_tp);
-                need_p = q < 1.f ? 1 : (q > 2.0e9f ? 0x7fffffff : (int)q);
-            }
+            uint32_t tp;
+            radix_mass(each_of_row, cut, tau, ties, e_ties, m, remaining, tp, work_f, tot_f);
+            const int need_p = ties_needed(remaining, tp, m);
             need = (cut && tp == tau) ? min(need, need_p) : need_p;
             tau = tp;
             cut = true;
@@ -451,7 +635,7 @@ __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
     bool ranked = false;
     if (cut) {
         int eq = 0;
-        each_id(row, V, T, vec, ntiles, [&](float z, int) { eq += sort_key(z) == tau; });
+        each_of_row([&](float z) { eq += sort_key(z) == tau; });
         ranked = block_sum_int(eq, si) > need;
         if (ranked) {
             int running = 0;
@@ -581,17 +765,27 @@ __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
     }
 }
 
-// tiles: room for 3 * n * ceil(V / 8192) floats, in which the first kernel leaves every tile's part.
+// Floats of scratch memory that li_sample_rows needs for n rows of V logits.
+extern "C" long li_sample_rows_scratch_floats(int n, int V) {
+    if (n <= 0 || V <= 0) return 0;
+    const long ntiles = (V + SMP_TILE - 1) / SMP_TILE;
+    return (3 + 2 * (long)SMP_KC) * n * ntiles;
+}
+
+// tiles: scratch of li_sample_rows_scratch_floats(n, V) floats, in which the first kernel leaves every tile's part.
 extern "C" int li_sample_rows(const float* logits, const float* temperature, const int* top_k,
                               const float* top_p, const float* uniform, int* out, int n, int V,
                               float* tiles, long tiles_floats, hipStream_t stream) {
     if (n <= 0 || n > 65535 || V <= 0) return LI_ERR_SIZE;
     const int ntiles = (V + SMP_TILE - 1) / SMP_TILE;
-    if (ntiles > SMP_NT || !tiles || tiles_floats < 3l * n * ntiles) return LI_ERR_SIZE;
+    if (ntiles > SMP_NT || !tiles || tiles_floats < li_sample_rows_scratch_floats(n, V)) return LI_ERR_SIZE;
+    const size_t per = (size_t)n * ntiles;
     float* tm = tiles;
-    float* ts = tiles + (size_t)n * ntiles;
-    int* ti = reinterpret_cast<int*>(tiles + 2 * (size_t)n * ntiles);
-    sample_tiles_kernel<<<dim3(ntiles, n), SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, tm, ts, ti, V);
-    sample_rows_kernel<<<n, SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V, tm, ts, ti, ntiles);
+    float* ts = tiles + per;
+    int* ti = reinterpret_cast<int*>(tiles + 2 * per);
+    float* cz = tiles + 3 * per;
+    int* ci = reinterpret_cast<int*>(tiles + (3 + (size_t)SMP_KC) * per);
+    sample_tiles_kernel<<<dim3(ntiles, n), SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, tm, ts, ti, cz, ci, V);
+    sample_rows_kernel<<<n, SMP_NT, 0, stream>>>(logits, temperature, top_k, top_p, uniform, out, V, tm, ts, ti, cz, ci, ntiles);
     return li_launch_status();
 }

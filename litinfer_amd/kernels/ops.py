@@ -79,6 +79,15 @@ def _work_bytes(m: int, n: int, k: int, dtype: int) -> int:
     return int(f(m, n, k, dtype))
 
 
+def _sample_scratch_floats(n: int, v: int) -> int:
+    f = _fn_cache.get(("sampling", "li_sample_rows_scratch_floats"))
+    if f is None:
+        f = build.load("sampling").li_sample_rows_scratch_floats
+        f.argtypes, f.restype = [c_int, c_int], c_long
+        _fn_cache[("sampling", "li_sample_rows_scratch_floats")] = f
+    return int(f(n, v))
+
+
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
@@ -680,8 +689,8 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
     if n:
         v = logits.shape[1]
         key = (logits.device, n, v)
-        if key not in _sample_scratch:               # the tiles' parts of the kernel's first stage
-            _sample_scratch[key] = torch.empty(3 * n * ((v + 8191) // 8192), dtype=torch.float32, device=logits.device)
+        if key not in _sample_scratch:               # what the first of the two kernels leaves for the second
+            _sample_scratch[key] = torch.empty(_sample_scratch_floats(n, v), dtype=torch.float32, device=logits.device)
         tiles = _sample_scratch[key]
         _run("sampling", "li_sample_rows", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(),
              top_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), n, v, tiles.data_ptr(), tiles.numel())
