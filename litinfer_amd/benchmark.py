@@ -52,6 +52,27 @@ SHAPES = {
             "head_dim": 128, "intermediate_size": 27648, "vocab_size": 152064, "rope_theta": 1000000.0,
             "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "use_sliding_window": False,
             "max_position_embeddings": 32768},
+    # further members of the family, for `--mode sweep --shape ...`
+    "0.5b": {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu",
+             "num_hidden_layers": 24, "hidden_size": 896, "num_attention_heads": 14, "num_key_value_heads": 2,
+             "head_dim": 64, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
+             "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "use_sliding_window": False,
+             "max_position_embeddings": 32768},
+    "3b": {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu",
+           "num_hidden_layers": 36, "hidden_size": 2048, "num_attention_heads": 16, "num_key_value_heads": 2,
+           "head_dim": 128, "intermediate_size": 11008, "vocab_size": 151936, "rope_theta": 1000000.0,
+           "rms_norm_eps": 1e-6, "tie_word_embeddings": True, "use_sliding_window": False,
+           "max_position_embeddings": 32768},
+    "14b": {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu",
+            "num_hidden_layers": 48, "hidden_size": 5120, "num_attention_heads": 40, "num_key_value_heads": 8,
+            "head_dim": 128, "intermediate_size": 13824, "vocab_size": 152064, "rope_theta": 1000000.0,
+            "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "use_sliding_window": False,
+            "max_position_embeddings": 32768},
+    "72b": {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_act": "silu",
+            "num_hidden_layers": 80, "hidden_size": 8192, "num_attention_heads": 64, "num_key_value_heads": 8,
+            "head_dim": 128, "intermediate_size": 29568, "vocab_size": 152064, "rope_theta": 1000000.0,
+            "rms_norm_eps": 1e-6, "tie_word_embeddings": False, "use_sliding_window": False,
+            "max_position_embeddings": 32768},
 }
 QWEN2_7B = SHAPES["7b"]
 CONTEXT = 4096
@@ -410,10 +431,10 @@ def sweep(a) -> Dict[str, object]:
     from .engine import Engine, StepEntry
     from .sampling import Sampler, SamplingParams
 
-    cfg = dict(QWEN2_7B, num_hidden_layers=a.layers, max_position_embeddings=32768)
+    cfg = dict(SHAPES[a.shape], num_hidden_layers=a.layers, max_position_embeddings=32768)
     es = 2 if a.dtype == "bf16" else 4
     dev = "cuda:0"
-    contexts, batches = (1024, 4096, 16384), (1, 8, 64)
+    contexts, batches = ((1024, 4096, 16384) if a.shape == "7b" else (4096,)), (1, 8, 64)
     eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
                              num_pages=max(batches) * max(contexts) // PAGE + 1024, max_seqs=max(batches) + 1)
     for g in eng.cache.groups:
@@ -433,7 +454,7 @@ def sweep(a) -> Dict[str, object]:
                                         "frac": round(nbytes / dt * a.steps / HBM_PEAK, 4)}
             log(f"decode, context {ctx}, batch {b}: {decode[f'ctx{ctx}_b{b}']}")
     prefill = {}
-    for tokens, start in ((512, 0), (2048, 0), (8192, 0), (1024, 15360)):
+    for tokens, start in (((512, 0), (2048, 0), (8192, 0), (1024, 15360)) if a.shape == "7b" else ((2048, 0),)):
         ids = rng.integers(0, cfg["vocab_size"], start + tokens).tolist()
         times = []
         for i in range(4):
@@ -454,10 +475,11 @@ def sweep(a) -> Dict[str, object]:
         prefill[key] = {"tok_s": round(tokens / pt, 1), "ms": round(pt * 1e3, 3), "frac": round(flops / pt / FLOP_PEAK[a.dtype], 4)}
         log(f"prompt of {tokens} tokens behind {start}: {prefill[key]}")
     best = decode["ctx4096_b8"]
-    return {"metric": "decode tok/s and prompt tok/s at further sizes (Qwen2-7B shape)", "value": best["tok_s"], "unit": "tok/s",
+    return {"metric": f"decode tok/s and prompt tok/s at further sizes (Qwen2 {a.shape} shape)", "value": best["tok_s"], "unit": "tok/s",
             "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": best["ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": a.dtype, "data": "synthetic: seeded random token ids, random weights, random cache content",
-            "config": {"model": "Qwen2-7B shape", "num_hidden_layers": a.layers, "page_size": PAGE, "parallelism": "none (1 GPU)"},
+            "config": {"model": f"Qwen2 {a.shape} shape", "num_hidden_layers": a.layers, "full_num_hidden_layers": SHAPES[a.shape]["num_hidden_layers"],
+                       "page_size": PAGE, "parallelism": "none (1 GPU)"},
             "decode": decode, "prefill_at": prefill}
 
 
@@ -574,6 +596,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has (named in `config`)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep"])
+    ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="sweep: the member of the family whose layer sizes are taken")
     ap.add_argument("--no-points", action="store_true", help="headline: skip the batch 1 and 64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-scheduler", action="store_true", help="headline: skip the runs through the scheduler")
@@ -593,7 +616,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         a.layers = a.layers or QWEN2_7B["num_hidden_layers"]
         out = headline(a)
     elif a.mode == "sweep":
-        a.layers = a.layers or QWEN2_7B["num_hidden_layers"]
+        a.layers = a.layers or SHAPES[a.shape]["num_hidden_layers"]
         a.steps, a.warmup = min(a.steps, 32), min(a.warmup, 4)
         out = sweep(a)
     elif a.mode == "serving":
