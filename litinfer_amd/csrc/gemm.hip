@@ -1376,15 +1376,19 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
     return li_launch_status();
 }
 
-// Between 33 and 64 rows (a large decoding batch) the product is still bound by streaming W, but
-// x is too large to be read again by every block of a few columns: tiles of 64 rows with the
-// loads straight into LDS, and, where the matrix has too few such tiles to fill the chip, K cut
-// into parts whose sums go to `work` and are added up in a fixed order.  Returns -1 when it does
+// Between 17 and 64 rows (a large decoding batch) the product is still bound by streaming W, but
+// x is too large to be read again by every block of a few columns (every block of the few-row
+// kernel reads all of x, and what a compute unit can take in then bounds the product): tiles of
+// 64 rows with the loads straight into LDS, and, where the matrix has too few such tiles to fill
+// the chip, K cut into parts whose sums go to `work` and are added up in a fixed order, by kernels
+// that also do what follows the product (the norm of the new residual sum, the rotary encoding
+// and the page write), which the few-row kernel does in its epilogue for up to 16 rows only.
+// Measured on the 7B layer sizes, a decode step of 17 / 24 / 32 requests: 4.57 / 4.95 / 5.33 ms
+// against 4.90 / 5.33 / 5.84 ms with the few-row kernel up to 32 rows.  Returns -1 when it does
 // not take the call.
-// From 17 rows on the same holds where K is long (the feed-forward's way back): every block of the
-// few-row kernel reads all of x, and what a compute unit can take in then bounds the product.
 static bool mid_rows_take(int M, int K) {
-    return M <= 64 && (M > 32 || (M > 16 && (long)M * K * 2 > 600 * 1024));
+    (void)K;
+    return M > 16 && M <= 64;
 }
 
 static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, void* out, int M, int N,
@@ -1649,7 +1653,7 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
         launch_skinny<true, bf16_t>(a, stream);
         return li_launch_status();
     }
-    if (M > 32 && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
+    if (M > 16 && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
         if ((N + 255) / 256 >= 128)
             return launch_dma<64, 256, 64, 3, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
         if ((N + 127) / 128 >= 128)

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
@@ -289,8 +289,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     """out = x w^T + bias, or out += x w^T + bias when `accumulate`.
     x [M, K] and w [N, K] of one dtype (float32 or bfloat16); out [M, N] of that
     dtype or float32; accumulation of the product is float32.  `ws` lends the
-    memory for partial sums where the kernel cuts K into parts (33 to 64 rows
-    against a matrix of few columns, from 17 rows on where K is long); without it
+    memory for partial sums where the kernel cuts K into parts (17 rows and more
+    against a matrix of few columns); without it
     such a product takes a slower kernel."""
     _gpu(x, w, bias, out)
     _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear: needs matrices")
@@ -550,6 +550,34 @@ DECODE_MAX_SPLITS = 64       # the merge kernel keeps a weight per split
 DECODE_TABLE_CAP = 1024      # pages of one split that the matrix-core decode kernel copies into LDS
 
 
+_simds: Dict[int, int] = {}
+
+
+def _simd_count(device: torch.device) -> int:
+    """Waves of the decode kernel that run at one time: one on each SIMD, four SIMDs a compute unit."""
+    i = device.index if device.index is not None else torch.cuda.current_device()
+    if i not in _simds:
+        _simds[i] = 4 * torch.cuda.get_device_properties(i).multi_processor_count
+    return _simds[i]
+
+
+def decode_splits(pairs: int, keys: int, simds: int = _DEC_WAVES) -> int:
+    """Into how many runs the keys of a decoding token are cut.  Every (token, kv head) pair and
+    run is one wave, and a SIMD holds one wave of this kernel: the waves go over the SIMDs in
+    rounds, each as long as a run (plus a wave's start and end, about 24 keys' time), so the
+    number of runs with the least rounds x run length is taken, a run being a multiple of 32
+    keys and at least 128 where the keys allow; every run costs the merge a little (4 keys' time).
+    Few pairs: as many runs as fill the SIMDs once."""
+    most = max(1, min(-(-keys // 128), DECODE_MAX_SPLITS))
+    best, best_cost = 1, None
+    for ns in range(1, most + 1):
+        run = (-(-keys // ns) + 31) & ~31
+        cost = -(-pairs * ns // simds) * (run + 24) + 4 * ns
+        if best_cost is None or cost < best_cost:
+            best, best_cost = ns, cost
+    return best
+
+
 def decode_split_blocks(max_blocks: int, page_size: int, window: int, nsplit: int) -> int:
     """The most pages one of `nsplit` splits of the keys can touch, for block tables of
     `max_blocks` pages: the keys (at most the table's, or the window's) are cut into runs
@@ -603,7 +631,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         # block of four waves per split on the vector ALU
         mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
         if mfma:
-            nsplit = max(1, min(-(-_DEC_WAVES // (n_single * nkv)), -(-keys // 128), DECODE_MAX_SPLITS))
+            nsplit = decode_splits(n_single * nkv, keys, _simd_count(qkv.device))
             # a split's pages must fit the kernel's copy of the block table
             while nsplit <= DECODE_MAX_SPLITS and decode_split_blocks(meta.max_blocks, page_size, window, nsplit) > DECODE_TABLE_CAP:
                 nsplit += 1

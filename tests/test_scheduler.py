@@ -185,3 +185,20 @@ def test_sampling_stream_is_per_request():
     assert all(0.0 <= uniform(s, c) < 1.0 for s in range(20) for c in range(50))
     mean = sum(uniform(1, c) for c in range(4000)) / 4000
     assert abs(mean - 0.5) < 0.03
+
+
+def test_decode_attention_splits_fill_the_simds_in_whole_rounds():
+    # every (token, kv head) pair and run of keys is one wave, a SIMD holds one: the runs are chosen for
+    # the least rounds x run length
+    from litinfer_amd.kernels.ops import DECODE_MAX_SPLITS, decode_splits
+    simds = 1024
+    assert decode_splits(8 * 4, 4096, simds) == 32            # 1,024 waves: one round
+    assert decode_splits(64 * 4, 4096, simds) == 4
+    assert decode_splits(96 * 4, 4096, simds) == 8            # 3 rounds of 512 keys, not 2 of 1,376
+    assert decode_splits(24 * 4, 4096, simds) == 10           # 960 waves, not 1,056
+    assert decode_splits(256 * 4, 4096, simds) == 1
+    for pairs in (1, 3, 28, 100, 333, 1000, 5000):
+        for keys in (1, 31, 128, 1000, 4096, 100000):
+            ns = decode_splits(pairs, keys, simds)
+            assert 1 <= ns <= DECODE_MAX_SPLITS
+            assert ns == 1 or keys / ns >= 96                 # runs of about 128 keys at least
