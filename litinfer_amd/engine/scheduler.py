@@ -93,6 +93,11 @@ class Request:
         return out
 
 
+# Rows of the smallest tile that the kernels' products of more than 64 rows are cut into (csrc/gemm.hip):
+# what callers pass as `row_tile`.
+PRODUCT_ROW_TILE = 128
+
+
 @dataclass
 class Planned:
     request: Request
@@ -104,13 +109,18 @@ class Planned:
 class Scheduler:
     def __init__(self, engine, *, max_batch_tokens: int = 2048, chunk_size: int = 512,
                  max_running: Optional[int] = None, eos_token_ids: Optional[Sequence[int]] = None,
-                 sampler=None, lookahead: bool = False):
-        if max_batch_tokens <= 0 or chunk_size <= 0:
-            raise ValueError("scheduler: max_batch_tokens and chunk_size must be positive")
+                 sampler=None, lookahead: bool = False, row_tile: int = 1):
+        """row_tile: rows that the kernels of a step take at a time (the products' tiles).  A step
+        whose tokens number a few more than a multiple of it (up to half a tile) pays for a whole
+        tile more: then the last portion of a prompt in the plan that is not the prompt's end gives
+        those tokens up to the next step.  1: as planned."""
+        if max_batch_tokens <= 0 or chunk_size <= 0 or row_tile <= 0:
+            raise ValueError("scheduler: max_batch_tokens, chunk_size and row_tile must be positive")
         self.engine = engine
         self.cache = engine.cache
         self.max_batch_tokens = int(max_batch_tokens)
         self.chunk_size = int(chunk_size)
+        self.row_tile = int(row_tile)
         self.max_running = int(max_running) if max_running else self.cache.max_seqs
         self.eos = tuple(engine.spec.eos_token_ids if eos_token_ids is None else eos_token_ids)
         self.sampler = sampler if sampler is not None else Sampler(engine.rt.device)
@@ -275,13 +285,29 @@ class Scheduler:
                 slots -= 1
                 plan.append(Planned(r, 0, n, n == r.remaining))
             if plan or not movable:
-                return plan
+                return self._whole_tiles(plan)
             # requests are running, want to go on and none can (each holds pages, none is free):
             # the most recently admitted gives way
             if len(self.running) > 1:
                 self._preempt(self.running[-1])
             else:
                 self._end_lone(self.running[0])
+
+    def _whole_tiles(self, plan: List[Planned]) -> List[Planned]:
+        """See `row_tile`: shortens one portion, so that the step's tokens fill whole tiles."""
+        tile = self.row_tile
+        if tile <= 1 or not plan:
+            return plan
+        total = sum(p.n for p in plan)
+        over = total % tile
+        if total <= tile or over == 0 or over > tile // 2:
+            return plan
+        for i in range(len(plan) - 1, -1, -1):
+            p = plan[i]
+            if not p.wants_logits and p.n - over >= tile:        # a portion that stays one, and a large one
+                plan[i] = Planned(p.request, p.start, p.n - over, False)
+                break
+        return plan
 
     # ---- one step ------------------------------------------------------------
     def _ends_with_pending(self, r: Request) -> bool:

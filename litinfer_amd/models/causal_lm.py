@@ -16,7 +16,7 @@ import time
 from pathlib import Path
 from typing import Iterator, List, Optional, Sequence
 
-from ..engine import Engine, Scheduler
+from ..engine import PRODUCT_ROW_TILE, Engine, Scheduler
 from ..sampling import SamplingParams
 
 
@@ -50,7 +50,7 @@ class CausalLM:
         self.seed = int(seed)
         # lookahead: a step is started before the tokens of the one before have reached the host
         self._sched_args = dict(max_batch_tokens=max_batch_tokens, chunk_size=chunk_size,
-                                lookahead=bool(lookahead))
+                                lookahead=bool(lookahead), row_tile=PRODUCT_ROW_TILE)
         self._scheduler: Optional[Scheduler] = None
         print(f"[litinfer_amd] ready: {self.engine.spec.architecture}, "
               f"{self.engine.model.weight_bytes() / 2**20:.1f} MiB of weights", flush=True)

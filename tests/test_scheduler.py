@@ -202,3 +202,38 @@ def test_decode_attention_splits_fill_the_simds_in_whole_rounds():
             ns = decode_splits(pairs, keys, simds)
             assert 1 <= ns <= DECODE_MAX_SPLITS
             assert ns == 1 or keys / ns >= 96                 # runs of about 128 keys at least
+
+
+def test_a_step_a_few_tokens_over_whole_tiles_shortens_a_portion():
+    # row_tile 8: a portion of 16 beside one decoded token would be 17 tokens, one over two tiles; the
+    # portion gives that token up.  A prompt's last portion is never shortened, and nothing is when the
+    # step is more than half a tile over.
+    e = FakeEngine(num_pages=64, max_positions=200)
+    s = sched(e, max_batch_tokens=40, chunk_size=16, row_tile=8)
+    a = s.add_request(list(range(3)), max_new_tokens=6)
+    s.step()                                                       # a's prompt: 3 tokens, nothing to shorten
+    b = s.add_request([(7 * i) % 50 for i in range(50)], max_new_tokens=2)
+    s.step()
+    assert e.batches[0] == [(a, 3, [2])]
+    assert e.batches[1] == [(a, 1, [0]), (b, 15, [])]              # 1 + 16 = 17 -> 16
+    s.step()
+    assert e.batches[2] == [(a, 1, [0]), (b, 15, [])]
+    s.step()
+    assert e.batches[3] == [(a, 1, [0]), (b, 15, [])]
+    s.step()
+    assert e.batches[4] == [(a, 1, [0]), (b, 5, [4])]              # the prompt's end: as it is
+    s.run_to_completion()
+    assert s.output(a) == [3, 4, 5, 6, 7, 8] and s.output(b) == [44, 45]
+    assert e.cache.free_pages() == [64]
+    # five tokens over (more than half a tile): as planned
+    e2 = FakeEngine(num_pages=64, max_positions=200)
+    s2 = sched(e2, max_batch_tokens=40, chunk_size=21, row_tile=8)
+    c = s2.add_request([i % 50 for i in range(60)], max_new_tokens=1)
+    s2.step()
+    assert e2.batches[0] == [(c, 21, [])]
+    # and the default leaves every plan alone
+    e3 = FakeEngine(num_pages=64, max_positions=200)
+    s3 = sched(e3, max_batch_tokens=40, chunk_size=17)
+    d = s3.add_request([i % 50 for i in range(60)], max_new_tokens=1)
+    s3.step()
+    assert e3.batches[0] == [(d, 17, [])]
