@@ -473,6 +473,9 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
     ([(1300, 1300)], 32, 8, 64, 8, 200),
     ([(5000, 300)], 4, 2, 128, 1, 0),                               # a table too long for the kernel that keeps the pages' offsets in LDS
     ([(1500, 400), (9, 9)], 7, 1, 128, 1, 0),                       # one key a page, within its table
+    ([(1100, 1100), (40, 3)], 40, 8, 128, 16, 0),                   # groups of 5 heads: blocks of five waves
+    ([(1100, 1100)], 48, 8, 64, 12, 0),                             # groups of 6: six waves, pages that do not divide a block of keys
+    ([(2100, 2100)], 18, 2, 64, 8, 700),                            # groups of 9: two blocks of five waves, one of them with four heads
 ])
 def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     out, ref = _paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=6)
