@@ -610,6 +610,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     constexpr int WLN = 4 / WLM;
     constexpr int WM = BM / WLM, WN = BN / WLN, TM = WM / 32, TN = WN / 32;
     static_assert(WM % 32 == 0 && WN % 32 == 0 && (WLM == 2 || WLM == 4), "a wave's part of the tile is made of 32 x 32 tiles");
+    constexpr bool SWSPLIT = SWIGLU && (TN % 2 == 1);        // gates and ups in different waves (see the rows of w below)
+    static_assert(!SWSPLIT || WLN == 2, "gates in one wave, ups in the wave beside it");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && (BM / 4) % (64 / (BK / 8)) == 0 && (BN / 4) % (64 / (BK / 8)) == 0, "whole load instructions a wave");
     constexpr int CPR = BK / 8, WRAP = 128 / BK;                 // chunks in a row; rows that fill all banks once
     constexpr int RPI = 64 / CPR;                                // rows one load instruction of a wave covers
@@ -648,13 +650,20 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     for (int i = 0; i < IB; ++i) {
         const int row = (BN / 4) * wave + RPI * i + lane / CPR, c = (lane % CPR) ^ ((row / WRAP) & (CPR - 1));
         size_t rel = (n0 + row < N) ? row : N - 1 - n0;            // row of w relative to the tile's first
-        if constexpr (SWIGLU) {
+        if constexpr (SWIGLU && !SWSPLIT) {
             // w is [gate; up] with N / 2 rows each.  The tile's rows alternate in blocks of 32: 32
             // gate rows, the 32 up rows of the same outputs, the next 32 gate rows, ..., so that an
             // accumulator tile and its neighbour hold the two factors of one output tile.
             const int half = N / 2, blk = row / 32;
             const int o = n0 / 2 + (blk / 2) * 32 + row % 32;
             rel = (size_t)((o < half ? o : half - 1) - n0 / 2) + (size_t)(blk & 1) * half;
+        } else if constexpr (SWSPLIT) {
+            // (a wave's part of the tile is an odd number of blocks of 32 columns: the tile's first half
+            // are gate rows, its second half the up rows of the same outputs, so that of two waves side
+            // by side one holds the gates and the other the ups; they meet in the epilogue's LDS)
+            const int half = N / 2;
+            const int o = n0 / 2 + row % (BN / 2);
+            rel = (size_t)((o < half ? o : half - 1) - n0 / 2) + (size_t)(row / (BN / 2)) * half;
         }
         gb[i] = (uint32_t)((rel * K + 8 * c) * 2);
     }
@@ -780,6 +789,54 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #undef LI_FREAD
 #undef LI_WAIT_YOUNGER
     __syncthreads();                               // the main loop's LDS is free now
+    if constexpr (SWSPLIT) {
+        // every wave leaves its sums in its band; of two waves side by side the first then takes rows 0 .. 15
+        // of the 32 and the second rows 16 .. 31: gates from the first wave's band, ups from the second's
+        constexpr int ES = WN + 4;
+        static_assert(4 * 32 * ES * 4 <= NSTAGE * STAGE * 2, "the waves' bands fit the main loop's LDS");
+        float* bands = reinterpret_cast<float*>(lds);
+        float* band = bands + wave * 32 * ES;
+        const float* gband = bands + (wave & ~1) * 32 * ES;
+        const float* uband = bands + (wave | 1) * 32 * ES;
+        const int ccol = lane & 31, crow = (lane >> 5) * 4;
+        constexpr int LPR = WN / 8, RPP = 64 / LPR;
+        const int erow = lane / LPR, ecol = (lane % LPR) * 8;
+        const int NO = N / 2;
+        const int col = n0 / 2 + ecol;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            if (i > 0) __syncthreads();              // (the bands have been read)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    band[(8 * (r >> 2) + crow + (r & 3)) * ES + 32 * j + ccol] = acc[i][j][r];
+            __syncthreads();
+#pragma unroll
+            for (int pass = 0; pass < (16 + RPP - 1) / RPP; ++pass) {
+                const int rr = RPP * pass + erow;
+                const int row = m0 + wm + 32 * i + 16 * (wave & 1) + rr;
+                if (erow >= RPP || rr >= 16 || row >= M || col >= NO) continue;
+                const float* gs = &gband[(16 * (wave & 1) + rr) * ES + ecol];
+                const float* us = &uband[(16 * (wave & 1) + rr) * ES + ecol];
+                float v[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = us[e] * (gs[e] / (1.0f + expf(-gs[e])));
+                const size_t o_idx = (size_t)row * NO + col;
+                if (col + 8 <= NO && (NO % 8) == 0) {
+                    chunk16 o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o.w[e] = pack2_bf16(v[2 * e], v[2 * e + 1]);
+                    *reinterpret_cast<chunk16*>(reinterpret_cast<uint16_t*>(out) + o_idx) = o;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (col + e < NO) epilogue_store(out, o_idx + e, v[e], nullptr, col + e, 0);
+                }
+            }
+        }
+        return;
+    }
     constexpr int EW = SWIGLU ? WN / 2 : WN;        // output columns of a wave
     constexpr int ESTRIDE = EW + 4;
     static_assert(4 * 32 * ESTRIDE * 4 <= NSTAGE * STAGE * 2, "the waves' bands fit the main loop's LDS");
@@ -1654,10 +1711,20 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
         return li_launch_status();
     }
     if (M > 16 && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
-        if ((N + 255) / 256 >= 128)
-            return launch_dma<64, 256, 64, 3, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
-        if ((N + 127) / 128 >= 128)
-            return launch_dma<64, 128, 64, 4, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
+        // tiles of 64 rows: the width with the least estimated time that gives the chip enough tiles (a
+        // product of few rows waits for w, and a compute unit takes in only so much: more units, each
+        // with a narrower tile, stream more, until the tiles no longer fit one round)
+        const int widths[3] = {256, 192, 128};
+        int pick = -1;
+        double best = 0.0;
+        for (int i = 0; i < 3; ++i) {
+            if ((N + widths[i] - 1) / widths[i] < 128) continue;         // too few tiles: the few-row kernel
+            const double c = tile_cost(64, widths[i], 1.0, M, N, K);
+            if (pick < 0 || c < best) { best = c; pick = i; }
+        }
+        if (pick == 0) return launch_dma<64, 256, 64, 3, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
+        if (pick == 1) return launch_dma<64, 192, 64, 4, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
+        if (pick == 2) return launch_dma<64, 128, 64, 4, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
     }
     if (M <= 64) return li_linear_skinny(x, w, nullptr, out, M, I, K, LI_BF16, 0, 1, stream);
     if (K % 64) return LI_ERR_SIZE;

@@ -218,6 +218,8 @@ def test_linear_into_the_residual_sum_with_its_norm(ops, m, n, k, bias, taken):
     (8, 200, 96),                # few rows: the decode kernel
     (40, 20000, 128),            # 33 to 64 rows: tiles of 64 rows
     (64, 9500, 192),
+    (50, 18944, 128),            # tiles of 64 x 192: the gates in one wave, the ups in the wave beside it
+    (33, 12300, 192),            # the same with a ragged last tile
     (65, 32, 64),                # one tile, one step of K
     (100, 200, 128),             # an output width that is no multiple of 32
     (300, 1000, 192),            # several tiles both ways, ragged edges
