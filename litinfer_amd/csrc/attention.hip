@@ -299,12 +299,13 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 template <typename T>
 __global__ __launch_bounds__(128) void attention_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int nsplit) {
+    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int nsplit, int by_token) {
+    // by_token: the partial results lie by the token's row in the batch, not by its place in token_list
     __shared__ float wgt[MERGE_MAX_SPLITS];
     __shared__ float inv_l;
     const int ti = blockIdx.x, head = blockIdx.y;
     const int t = token_list ? token_list[ti] : ti;
-    const size_t base = ((size_t)ti * nh + head) * nsplit;
+    const size_t base = ((size_t)(by_token ? t : ti) * nh + head) * nsplit;
     // The partial results of this thread's first dimension are asked for before the weights
     // are known (up to 32 splits, all loads at once and never conditional): their way from
     // memory then runs beside the weights' way and arithmetic, not behind them.
@@ -850,7 +851,11 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ tiles, const int* __restrict__ q_start,
     const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int page_size,
-    int num_pages, int window, float scale, int ncu) {
+    int num_pages, int window, float scale, int ncu, int ksplit, float* __restrict__ part_acc,
+    float* __restrict__ part_ml) {
+    // ksplit > 1: the tile's blocks of keys are cut into ksplit runs, blockIdx.z = part of the heads x
+    // ksplit + run; a block then leaves its sums, unscaled, in part_acc [token, head, run, dh] and its
+    // (maximum, sum) in part_ml, and attention_merge_kernel joins the runs in their order
     constexpr int KS = DH / 16;                 // MFMA steps of K Q^T (16 head dimensions each)
     constexpr int HD = DH / 2;                  // head dimensions owned by one lane half
     constexpr int DT = DH / 32;                 // tiles of 32 output dimensions
@@ -875,15 +880,38 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     const int kvh = (item % per_tile) / gridDim.z;      // (the parts of a group of heads are neighbours: they read the same keys)
     const int G = nh / nkv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hw = ((item % per_tile) % gridDim.z) * PRE_WAVES + wave;       // this wave's head within the group
+    const int zz = (item % per_tile) % gridDim.z, run = zz % ksplit;
+    const int hw = (zz / ksplit) * PRE_WAVES + wave;    // this wave's head within the group
     const bool active = hw < G;                         // (idle waves still help to fetch and keep the barriers)
     const int head = kvh * G + (active ? hw : 0);
     const int ql = lane & 31, h = lane >> 5;
     const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);           // position of the tile's first token
     const int p_last = p0 + nrows - 1;
     const int lo0 = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
-    const int k_begin = lo0 & ~31, k_end = p_last + 1;
-    const int first_block = lo0 / page_size;
+    int k_begin = lo0 & ~31, k_end = p_last + 1;
+    int first_key = lo0;
+    if (ksplit > 1) {                                   // this run's blocks of 32 keys
+        const int all = (k_end - k_begin + 31) / 32, per = (all + ksplit - 1) / ksplit;
+        const int b0 = run * per, b1 = (run + 1) * per < all ? (run + 1) * per : all;
+        if (b0 >= b1) {                                 // no keys for this run: it says so and is done (before any barrier)
+            if (active && ql < nrows && h == 0) {
+                const size_t at = ((size_t)(t0 + ql) * nh + head) * ksplit + run;
+                part_ml[at * 2] = -INFINITY;
+                part_ml[at * 2 + 1] = 0.f;
+            }
+            if (active && ql < nrows) {
+                float* pa = part_acc + (((size_t)(t0 + ql) * nh + head) * ksplit + run) * DH + HD * h;
+#pragma unroll
+                for (int d = 0; d < HD; d += 4) *reinterpret_cast<float4*>(pa + d) = float4{0.f, 0.f, 0.f, 0.f};
+            }
+            return;
+        }
+        const int kb0 = k_begin + 32 * b0;
+        k_end = k_begin + 32 * b1 < k_end ? k_begin + 32 * b1 : k_end;
+        k_begin = kb0;
+        first_key = kb0 > lo0 ? kb0 : lo0;
+    }
+    const int first_block = first_key / page_size;
     const int nblocks = (k_end - 1) / page_size - first_block + 1;     // <= PRE2_TABLE_CAP (checked by the host)
     const int* table = block_table + (size_t)s * max_blocks + first_block;
     const size_t page_bytes = (size_t)nkv * page_size * DH * 2;
@@ -1076,6 +1104,21 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     }
     if (!active || ql >= nrows) return;
     l += __shfl_xor(l, 32, LI_WAVE);               // (both halves of a query are past the return together)
+    if (ksplit > 1) {
+        const size_t at = ((size_t)(t0 + ql) * nh + head) * ksplit + run;
+        if (h == 0) {
+            part_ml[at * 2] = m * 0.69314718055994531f;          // (the kernel that joins the runs counts in powers of e)
+            part_ml[at * 2 + 1] = l;
+        }
+        float* pa = part_acc + at * DH;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg)
+                *reinterpret_cast<float4*>(pa + 32 * dt + 8 * rg + 4 * h) =
+                    float4{acc[dt][4 * rg], acc[dt][4 * rg + 1], acc[dt][4 * rg + 2], acc[dt][4 * rg + 3]};
+        return;
+    }
     const float inv = l != 0.f ? 1.0f / l : 0.f;
     bf16_t* orow = out + (size_t)(t0 + ql) * nh * DH + (size_t)head * DH;
 #pragma unroll
@@ -1533,18 +1576,61 @@ extern "C" int li_paged_attention_prefill_f32(const void* q, int q_row_stride, v
     return li_launch_status();
 }
 
+// Into how many runs the keys of every tile are cut (1: not at all).  A block is one tile x kv head x
+// four heads of the group x run; a compute unit holds two blocks, each as long as its run of keys,
+// and the blocks go over the units in rounds: with few tiles against long contexts (a portion of a
+// prompt behind a long cached part, few kv heads) whole units stand idle or a few blocks make a
+// round of their own.  Estimated in blocks of 32 keys: rounds x (run + 8) + 2 per run for the
+// kernel that joins the runs; the form with eight waves a block (two halves of the keys, no joining
+// kernel), which takes up to one block a unit, is the yardstick where it applies.  Runs of at
+// least 16 blocks of keys, at most 16 runs, and the partial results within max_bytes.
+extern "C" int li_paged_attention_prefill_runs(int ntiles, int nh, int nkv, int dh, int max_blocks, int page_size,
+                                               int max_keys, int tokens, long max_bytes) {
+    if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || max_blocks > PRE2_TABLE_CAP || max_keys <= 0) return 1;
+    int dev = 0, ncu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || ncu <= 0) {
+        (void)hipGetLastError();
+        ncu = 256;
+    }
+    const int G = nh / nkv, parts = (G + PRE_WAVES - 1) / PRE_WAVES;
+    const long blocks = (long)ntiles * nkv * parts;
+    const int len = (max_keys + 31) / 32;                               // the longest tile's blocks of keys
+    auto cost = [&](int runs) {
+        const long rounds = (blocks * runs + 2l * ncu - 1) / (2l * ncu);
+        return (double)rounds * ((len + runs - 1) / runs + 8) + (runs > 1 ? 2.0 * runs : 0.0);
+    };
+    double best = cost(1);
+    if (blocks <= ncu) {                                                // the form with eight waves a block
+        const double halves = (len + 1) / 2 + 8;
+        if (halves < best) best = halves;
+    }
+    int pick = 1;
+    for (int runs = 2; runs <= 16 && len / runs >= 16; ++runs) {
+        if ((long)tokens * nh * runs * (dh + 2) * 4 > max_bytes) break;
+        const double c = cost(runs);
+        if (c < 0.9 * best) { best = c; pick = runs; }                  // (only for a clear gain)
+    }
+    return pick;
+}
+
 // tiles: int [ntiles, 4] = (segment, first token of the tile in the batch, rows <= 32, unused)
+// runs > 1 (see li_paged_attention_prefill_runs): part_acc [tokens, nh, runs, dh] and part_ml
+// [tokens, nh, runs, 2] float32 take the runs' results, which are then joined for the n_merge tokens
+// of merge_tokens (null: the tokens 0 .. n_merge - 1).
 extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void* out, const void* kc,
                                           const void* vc, const int* block_table, int max_blocks,
                                           const int* tiles, int ntiles, const int* q_start, const int* q_len,
                                           const int* ctx_len, int nh, int nkv, int dh, int page_size,
-                                          int num_pages, int window, float scale, hipStream_t stream) {
+                                          int num_pages, int window, float scale, int runs, float* part_acc,
+                                          float* part_ml, const int* merge_tokens, int n_merge, hipStream_t stream) {
     if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || page_size <= 0 || max_blocks <= 0 ||
         max_blocks > PRE_TABLE_CAP || (long long)max_blocks * page_size > (1ll << 21) || !(scale > 0.f))
         return LI_ERR_SIZE;
+    if (runs < 1 || runs > MERGE_MAX_SPLITS || (runs > 1 && (!part_acc || !part_ml || n_merge <= 0 || max_blocks > PRE2_TABLE_CAP)))
+        return LI_ERR_SIZE;
     const int G = nh / nkv;
     const int parts = (G + PRE_WAVES - 1) / PRE_WAVES;
-    if (parts > 65535) return LI_ERR_SIZE;
+    if ((long)parts * runs > 65535) return LI_ERR_SIZE;
     dim3 grid(ntiles, nkv, parts);
     int dev = 0, ncu = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || ncu <= 0) {
@@ -1556,21 +1642,26 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
         tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
 #define LI_PRE2(DHV, P32V) paged_attention_prefill_dma_kernel<DHV, P32V><<<grid, PRE_WAVES * 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
-        tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
+        tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu, runs, part_acc, part_ml)
 #define LI_PRE3(DHV, P32V) paged_attention_prefill_split_kernel<DHV, P32V><<<grid, 2 * PRE_WAVES * 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
         tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale, ncu)
-    if (max_blocks <= PRE2_TABLE_CAP && (long)ntiles * nkv * parts <= (long)ncu) {      // at most a block a compute unit: the tile's keys in two halves
+    if (runs == 1 && max_blocks <= PRE2_TABLE_CAP && (long)ntiles * nkv * parts <= (long)ncu) {      // at most a block a compute unit: the tile's keys in two halves
         const bool p32 = 32 % page_size == 0;
         if (dh == 128) { if (p32) LI_PRE3(128, true); else LI_PRE3(128, false); }
         else if (dh == 64) { if (p32) LI_PRE3(64, true); else LI_PRE3(64, false); }
         else return LI_ERR_SIZE;
     } else
     if (max_blocks <= PRE2_TABLE_CAP) {                       // (longer block tables: the form that keeps 8,192 entries in LDS)
+        grid.z = parts * runs;
         const bool p32 = 32 % page_size == 0;
         if (dh == 128) { if (p32) LI_PRE2(128, true); else LI_PRE2(128, false); }
         else if (dh == 64) { if (p32) LI_PRE2(64, true); else LI_PRE2(64, false); }
         else return LI_ERR_SIZE;
+        if (runs > 1) {
+            if (li_launch_status() != LI_OK) return LI_ERR_LAUNCH;
+            attention_merge_kernel<bf16_t><<<dim3(n_merge, nh), 128, 0, stream>>>(part_acc, part_ml, merge_tokens, (bf16_t*)out, nh, dh, runs, 1);
+        }
     } else
     if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
 #undef LI_PRE2
@@ -1609,7 +1700,7 @@ static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, cons
 #undef LI_DEC
     if (nsplit > 1) {
         dim3 g2(n_tokens, nh);
-        attention_merge_kernel<T><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit);
+        attention_merge_kernel<T><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit, 0);
     }
     return li_launch_status();
 }
@@ -1646,7 +1737,7 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
 #undef LI_DM
         if (nsplit > 1) {
             dim3 g2(n_tokens, nh);
-            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit);
+            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit, 0);
         }
         return li_launch_status();
     }

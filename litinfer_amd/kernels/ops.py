@@ -46,7 +46,7 @@ _SIGNATURES = {
     },
     "attention": {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
-        "li_paged_attention_prefill": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F],
+        "li_paged_attention_prefill": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F, I, P, P, P, I],
         "li_paged_attention_prefill_f32": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F],
         "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I],
     },
@@ -86,6 +86,18 @@ def _sample_scratch_floats(n: int, v: int) -> int:
         f.argtypes, f.restype = [c_int, c_int], c_long
         _fn_cache[("sampling", "li_sample_rows_scratch_floats")] = f
     return int(f(n, v))
+
+
+PREFILL_RUNS_MAX_BYTES = 1 << 30       # room that the runs of a prompt portion's keys may take in the workspace
+
+
+def _prefill_runs(ntiles: int, nh: int, nkv: int, dh: int, max_blocks: int, page_size: int, keys: int, tokens: int) -> int:
+    f = _fn_cache.get(("attention", "li_paged_attention_prefill_runs"))
+    if f is None:
+        f = build.load("attention").li_paged_attention_prefill_runs
+        f.argtypes, f.restype = [c_int] * 8 + [c_long], c_int
+        _fn_cache[("attention", "li_paged_attention_prefill_runs")] = f
+    return int(f(ntiles, nh, nkv, dh, max_blocks, page_size, keys, tokens, PREFILL_RUNS_MAX_BYTES))
 
 
 def _stream() -> int:
@@ -659,10 +671,23 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
     # positions by the page size in float, exact below 2^21 keys; longer tables take the general kernel
     if (n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles
             and meta.tile_rows == PREFILL_TILE_ROWS and n_multi == meta.num_multi and meta.max_blocks <= 8192 and meta.max_blocks * page_size <= 1 << 21):
+        # few tiles against long contexts: the tiles' keys in runs, joined by the kernel that joins the
+        # decode attention's (the library says how many; their results take room in the workspace)
+        hq, hc = getattr(meta, "host_q_len", None), getattr(meta, "host_ctx_len", None)
+        longest = int(hc[hq > 1].max()) if hq is not None and hc is not None and (hq > 1).any() else meta.max_ctx_len
+        keys = min(longest, window) if window > 0 else longest
+        runs = _prefill_runs(meta.num_tiles, nh, nkv, dh, meta.max_blocks, page_size, keys, t) if ws is not None else 1
+        acc = ml = lst = None
+        if runs > 1:
+            acc = ws.buffer("attn.runs_acc", (t, nh, runs, dh), torch.float32)
+            ml = ws.buffer("attn.runs_ml", (t, nh, runs, 2), torch.float32)
+            lst = meta.multi_tokens if n_multi < t else None
         _run("attention", "li_paged_attention_prefill", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), bt.data_ptr(), meta.max_blocks, meta.tiles.data_ptr(),
              meta.num_tiles, meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
-             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale))
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), runs,
+             0 if acc is None else acc.data_ptr(), 0 if ml is None else ml.data_ptr(),
+             0 if lst is None else lst.data_ptr(), n_multi)
     elif (n_multi and qkv.dtype is torch.float32 and dh in (64, 128) and meta.num_tiles
             and meta.tile_rows == PREFILL_TILE_ROWS and n_multi == meta.num_multi):
         # the 32-bit path's tiled kernel for portions (other head sizes: the general kernel below)

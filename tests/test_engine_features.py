@@ -19,7 +19,7 @@ from litinfer_amd.engine.workspace import Workspace
 from litinfer_amd.parts import (BatchNeeds, FeedForward, Mixer, PagedNeed, PagedTensor, Position, ResidualStream, Runtime,
                                 StateNeed, build_part, register_part)
 from litinfer_amd.weights import ParamSpec
-from tiny_configs import TINY_A, TINY_B, TINY_C
+from tiny_configs import TINY_A, TINY_B, TINY_C, TINY_E
 from toy_parts import ToyConfig
 
 
@@ -54,6 +54,23 @@ def test_long_decoding_rolls_the_window_and_matches(tmp_path, device, dtype):
     assert schedules.rel_err(np.concatenate(rows), ref) < (F32_TOL if dtype == "float32" else BF16_TOL)
     assert eng.cache.groups[1].pool.used <= 32 // 8 + 1          # the windowed layers keep a few pages only
     assert eng.cache.groups[0].pool.used == -(-250 // 8)
+
+
+def test_a_short_portion_behind_a_long_cached_part(tmp_path, device):
+    if device == "cpu":
+        pytest.skip("a matter of the attention kernels' choice of runs")
+    # few tiles of queries against some thousand keys: the attention of such a step cuts every tile's keys
+    # into runs over several blocks and joins them; through the engine, against the plain implementation
+    cfg = dict(TINY_E, max_position_embeddings=2304)
+    d = helpers.make_model(tmp_path, cfg, 3, torch.bfloat16)
+    toks = helpers.random_requests(cfg["vocab_size"], [2250], 9)["r0"]
+    ref = helpers.plain_logits(d, {"r0": toks})["r0"]
+    eng = engine_for(d, device, dtype="bfloat16", page=32, max_tokens=2304)
+    eng.step([StepEntry("r0", toks[:2048], [])])
+    rows = [eng.step([StepEntry("r0", toks[2048:2148], list(range(100)))]).cpu().numpy(),       # 4 tiles behind 2,048
+            eng.step([StepEntry("r0", toks[2148:2150], [0, 1])]).cpu().numpy(),                 # down to two tokens
+            eng.step([StepEntry("r0", toks[2150:], list(range(100)))]).cpu().numpy()]
+    assert schedules.rel_err(np.concatenate(rows), ref[2048:]) < BF16_TOL
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

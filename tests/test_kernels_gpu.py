@@ -379,7 +379,7 @@ def test_rope(ops, dtype, t, heads, dh, theta, start):
     assert rel(xd, ref) < tol(dtype, 2e-4 if start else 2e-6, 8e-3)
 
 
-def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_one=None, row=None):
+def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_one=None, row=None, ws=None):
     """seg_specs: list of (ctx_len, q_len).  Builds random K/V for every
     segment, scatters them into shuffled pages, and compares the kernel with
     the plain attention on the logical sequences.  `scale_one` is the index of a
@@ -436,7 +436,7 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
                          max_single_ctx=int(ctx_len[q_len == 1].max()) if len(single) else 0)
     out = torch.empty(T, nh * dh, dtype=dtype, device=DEV)
     scale = 1.0 / math.sqrt(dh)
-    ops.paged_attention(q.to(DEV), out, kc.to(DEV), vc.to(DEV), meta, nh, nkv, dh, page, window, scale)
+    ops.paged_attention(q.to(DEV), out, kc.to(DEV), vc.to(DEV), meta, nh, nkv, dh, page, window, scale, ws=ws)
     refs = []
     o = 0
     for s, (c, ql) in enumerate(seg_specs):
@@ -482,6 +482,27 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
 def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     out, ref = _paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=6)
     assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
+
+
+@pytest.mark.parametrize("segs,nh,nkv,dh,page,window", [
+    ([(3000, 64)], 28, 4, 128, 16, 0),                              # two tiles behind 2,936 cached tokens: their keys in five runs
+    ([(3000, 64), (500, 1), (1200, 40), (40, 40)], 28, 4, 128, 16, 0),   # beside a decoding token; a short tile leaves runs without keys
+    ([(6000, 96)], 12, 2, 64, 8, 3000),                             # a window, six heads a group
+    ([(2500, 33), (2600, 2)], 8, 8, 128, 12, 0),                    # pages that do not divide a block of keys; a tile of one row
+])
+def test_prompt_portions_behind_long_contexts_with_their_keys_in_runs(ops, segs, nh, nkv, dh, page, window):
+    from litinfer_amd.kernels.ops import _prefill_runs
+    keys = max(c for c, q in segs if q > 1)
+    keys = min(keys, window) if window else keys
+    tiles = sum(-(-q // 32) for _, q in segs if q > 1)
+    blocks = max(-(-c // page) for c, _ in segs)
+    assert _prefill_runs(tiles, nh, nkv, dh, blocks, page, keys, sum(q for _, q in segs)) > 1     # the case is what it says
+    out, ref = _paged_case(ops, torch.bfloat16, segs, nh, nkv, dh, page, window, seed=31, ws=_Lender())
+    assert rel(out, ref) < 1.5e-2
+    # and one far key among thousands, in a run of its own
+    for far in (5, 1000, 2900):
+        out, ref = _paged_case(ops, torch.bfloat16, [(3000, 64)], 28, 4, 128, 16, 0, seed=32, scale_one=far, row=40, ws=_Lender())
+        assert rel(out, ref) < 1.5e-2
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
