@@ -299,13 +299,12 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 template <typename T>
 __global__ __launch_bounds__(128) void attention_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int nsplit, int by_token) {
-    // by_token: the partial results lie by the token's row in the batch, not by its place in token_list
+    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int nsplit) {
     __shared__ float wgt[MERGE_MAX_SPLITS];
     __shared__ float inv_l;
     const int ti = blockIdx.x, head = blockIdx.y;
     const int t = token_list ? token_list[ti] : ti;
-    const size_t base = ((size_t)(by_token ? t : ti) * nh + head) * nsplit;
+    const size_t base = ((size_t)ti * nh + head) * nsplit;
     // The partial results of this thread's first dimension are asked for before the weights
     // are known (up to 32 splits, all loads at once and never conditional): their way from
     // memory then runs beside the weights' way and arithmetic, not behind them.
@@ -339,6 +338,48 @@ __global__ __launch_bounds__(128) void attention_merge_kernel(
             for (int sp = 0; sp < nsplit; ++sp) at += part_acc[(base + sp) * dh + d] * wgt[sp];
         }
         store_from_float(out + (size_t)t * nh * dh + (size_t)head * dh + d, at * inv_l);
+    }
+}
+
+// The same for the runs of a prompt portion's keys, whose tokens are many: a block takes four heads of a
+// token (a block per token and head, as above, is tens of thousands of blocks with little to do each).
+// The partial results lie by the token's row in the batch.  Up to MERGE_RUNS_MAX runs.
+#define MERGE_RUNS_MAX 16
+#define MERGE_RUNS_HEADS 4
+template <typename T>
+__global__ __launch_bounds__(256) void attention_merge_runs_kernel(
+    const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int runs) {
+    __shared__ float wgt[MERGE_RUNS_HEADS][MERGE_RUNS_MAX];
+    __shared__ float inv[MERGE_RUNS_HEADS];
+    const int ti = blockIdx.x, h0 = blockIdx.y * MERGE_RUNS_HEADS;
+    const int heads = nh - h0 < MERGE_RUNS_HEADS ? nh - h0 : MERGE_RUNS_HEADS;
+    const int t = token_list ? token_list[ti] : ti;
+    const size_t base = ((size_t)t * nh + h0) * runs;
+    if (threadIdx.x < heads) {
+        const float* ml = part_ml + (base + (size_t)threadIdx.x * runs) * 2;
+        float mx = -INFINITY;
+        for (int sp = 0; sp < runs; ++sp) mx = fmaxf(mx, ml[2 * sp]);
+        float lt = 0.f;                          // the sum over the runs in their order
+        for (int sp = 0; sp < runs; ++sp) {
+            const float f = (mx == -INFINITY) ? 0.f : expf(ml[2 * sp] - mx);
+            wgt[threadIdx.x][sp] = f;
+            lt += ml[2 * sp + 1] * f;
+        }
+        inv[threadIdx.x] = lt != 0.f ? 1.0f / lt : 0.f;
+    }
+    __syncthreads();
+    const int n = heads * dh;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const int hd = i / dh, d = i - hd * dh;
+        const float* pa = part_acc + (base + (size_t)hd * runs) * dh + d;
+        float v[MERGE_RUNS_MAX];
+#pragma unroll
+        for (int sp = 0; sp < MERGE_RUNS_MAX; ++sp) v[sp] = pa[(size_t)(sp < runs ? sp : runs - 1) * dh];    // (all loads at once, never conditional)
+        float at = 0.f;
+#pragma unroll
+        for (int sp = 0; sp < MERGE_RUNS_MAX; ++sp) at += sp < runs ? v[sp] * wgt[hd][sp] : 0.f;
+        store_from_float(out + ((size_t)t * nh + h0) * dh + i, at * inv[hd]);
     }
 }
 
@@ -855,7 +896,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     float* __restrict__ part_ml) {
     // ksplit > 1: the tile's blocks of keys are cut into ksplit runs, blockIdx.z = part of the heads x
     // ksplit + run; a block then leaves its sums, unscaled, in part_acc [token, head, run, dh] and its
-    // (maximum, sum) in part_ml, and attention_merge_kernel joins the runs in their order
+    // (maximum, sum) in part_ml, and attention_merge_runs_kernel joins the runs in their order
     constexpr int KS = DH / 16;                 // MFMA steps of K Q^T (16 head dimensions each)
     constexpr int HD = DH / 2;                  // head dimensions owned by one lane half
     constexpr int DT = DH / 32;                 // tiles of 32 output dimensions
@@ -1580,35 +1621,56 @@ extern "C" int li_paged_attention_prefill_f32(const void* q, int q_row_stride, v
 // four heads of the group x run; a compute unit holds two blocks, each as long as its run of keys,
 // and the blocks go over the units in rounds: with few tiles against long contexts (a portion of a
 // prompt behind a long cached part, few kv heads) whole units stand idle or a few blocks make a
-// round of their own.  Estimated in blocks of 32 keys: rounds x (run + 8) + 2 per run for the
-// kernel that joins the runs; the form with eight waves a block (two halves of the keys, no joining
-// kernel), which takes up to one block a unit, is the yardstick where it applies.  Runs of at
-// least 16 blocks of keys, at most 16 runs, and the partial results within max_bytes.
-extern "C" int li_paged_attention_prefill_runs(int ntiles, int nh, int nkv, int dh, int max_blocks, int page_size,
-                                               int max_keys, int tokens, long max_bytes) {
-    if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || max_blocks > PRE2_TABLE_CAP || max_keys <= 0) return 1;
+// round of their own, and a prompt from its start has one tile as long as all its keys while the
+// mean is half that.  q_len, ctx_len: the batch's segments in HOST memory (those with one token are
+// not the business of this kernel).  Estimated in blocks of 32 keys: the longer of the longest run
+// and (rounds of blocks over the units) x (the mean run), each with 8 for a block's start and end,
+// + what writing the runs' results and joining them costs; the form with eight waves a block (two halves of the
+// keys, no joining kernel), which takes up to one block a unit, is the yardstick where it applies.
+// Runs of at least 16 blocks of keys, at most 16 runs, and the partial results within max_bytes.
+extern "C" int li_paged_attention_prefill_runs(int nseg, const int* q_len, const int* ctx_len, int nh, int nkv, int dh,
+                                               int max_blocks, int window, int tokens, long max_bytes) {
+    if (nseg <= 0 || !q_len || !ctx_len || nh <= 0 || nh > 4 * 65535 || nkv <= 0 || nh % nkv || max_blocks > PRE2_TABLE_CAP) return 1;
     int dev = 0, ncu = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&ncu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || ncu <= 0) {
         (void)hipGetLastError();
         ncu = 256;
     }
+    long ntiles = 0, work = 0;
+    int len = 0;                                                        // the longest tile's blocks of keys
+    for (int i = 0; i < nseg; ++i) {
+        if (q_len[i] <= 1) continue;
+        for (int a = 0; a < q_len[i]; a += 32) {
+            const int p0 = ctx_len[i] - q_len[i] + a, rows = q_len[i] - a < 32 ? q_len[i] - a : 32;
+            const int lo0 = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+            const int blocks = (p0 + rows - (lo0 & ~31) + 31) / 32;
+            ++ntiles;
+            work += blocks;
+            len = blocks > len ? blocks : len;
+        }
+    }
+    if (ntiles == 0) return 1;
     const int G = nh / nkv, parts = (G + PRE_WAVES - 1) / PRE_WAVES;
-    const long blocks = (long)ntiles * nkv * parts;
-    const int len = (max_keys + 31) / 32;                               // the longest tile's blocks of keys
+    const long blocks = ntiles * nkv * parts;
+    const double mean = (double)work / ntiles;
     auto cost = [&](int runs) {
         const long rounds = (blocks * runs + 2l * ncu - 1) / (2l * ncu);
-        return (double)rounds * ((len + runs - 1) / runs + 8) + (runs > 1 ? 2.0 * runs : 0.0);
+        const double longest = (len + runs - 1) / runs + 8, all = (double)rounds * (mean / runs + 8);
+        // (the runs' results are written and read again, a block of keys takes about 1.1 us)
+        const double joining = runs > 1 ? 5.0 + (double)tokens * nh * runs * dh * 8.0 / 6.0e12 / 1.1e-6 : 0.0;
+        return (longest > all ? longest : all) + joining;
     };
-    double best = cost(1);
+    double base = cost(1);
     if (blocks <= ncu) {                                                // the form with eight waves a block
         const double halves = (len + 1) / 2 + 8;
-        if (halves < best) best = halves;
+        if (halves < base) base = halves;
     }
     int pick = 1;
-    for (int runs = 2; runs <= 16 && len / runs >= 16; ++runs) {
+    double best = 0.9 * base;                                           // (only for a clear gain)
+    for (int runs = 2; runs <= MERGE_RUNS_MAX && len / runs >= 16; ++runs) {
         if ((long)tokens * nh * runs * (dh + 2) * 4 > max_bytes) break;
         const double c = cost(runs);
-        if (c < 0.9 * best) { best = c; pick = runs; }                  // (only for a clear gain)
+        if (c < best) { best = c; pick = runs; }
     }
     return pick;
 }
@@ -1626,7 +1688,7 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
     if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nkv > 65535 || page_size <= 0 || max_blocks <= 0 ||
         max_blocks > PRE_TABLE_CAP || (long long)max_blocks * page_size > (1ll << 21) || !(scale > 0.f))
         return LI_ERR_SIZE;
-    if (runs < 1 || runs > MERGE_MAX_SPLITS || (runs > 1 && (!part_acc || !part_ml || n_merge <= 0 || max_blocks > PRE2_TABLE_CAP)))
+    if (runs < 1 || runs > MERGE_RUNS_MAX || (runs > 1 && (!part_acc || !part_ml || n_merge <= 0 || nh > 4 * 65535 || max_blocks > PRE2_TABLE_CAP)))
         return LI_ERR_SIZE;
     const int G = nh / nkv;
     const int parts = (G + PRE_WAVES - 1) / PRE_WAVES;
@@ -1660,7 +1722,7 @@ extern "C" int li_paged_attention_prefill(const void* q, int q_row_stride, void*
         else return LI_ERR_SIZE;
         if (runs > 1) {
             if (li_launch_status() != LI_OK) return LI_ERR_LAUNCH;
-            attention_merge_kernel<bf16_t><<<dim3(n_merge, nh), 128, 0, stream>>>(part_acc, part_ml, merge_tokens, (bf16_t*)out, nh, dh, runs, 1);
+            attention_merge_runs_kernel<bf16_t><<<dim3(n_merge, (nh + MERGE_RUNS_HEADS - 1) / MERGE_RUNS_HEADS), 256, 0, stream>>>(part_acc, part_ml, merge_tokens, (bf16_t*)out, nh, dh, runs);
         }
     } else
     if (dh == 128) LI_PRE(128); else if (dh == 64) LI_PRE(64); else return LI_ERR_SIZE;
@@ -1700,7 +1762,7 @@ static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, cons
 #undef LI_DEC
     if (nsplit > 1) {
         dim3 g2(n_tokens, nh);
-        attention_merge_kernel<T><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit, 0);
+        attention_merge_kernel<T><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit);
     }
     return li_launch_status();
 }
@@ -1737,7 +1799,7 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
 #undef LI_DM
         if (nsplit > 1) {
             dim3 g2(n_tokens, nh);
-            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit, 0);
+            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit);
         }
         return li_launch_status();
     }

@@ -91,13 +91,18 @@ def _sample_scratch_floats(n: int, v: int) -> int:
 PREFILL_RUNS_MAX_BYTES = 1 << 30       # room that the runs of a prompt portion's keys may take in the workspace
 
 
-def _prefill_runs(ntiles: int, nh: int, nkv: int, dh: int, max_blocks: int, page_size: int, keys: int, tokens: int) -> int:
+def _prefill_runs(host_q_len, host_ctx_len, nh: int, nkv: int, dh: int, max_blocks: int, window: int, tokens: int) -> int:
+    """How many runs the library cuts the keys of a prompt portion's tiles into (the batch's segments as
+    int32 arrays in host memory)."""
     f = _fn_cache.get(("attention", "li_paged_attention_prefill_runs"))
     if f is None:
         f = build.load("attention").li_paged_attention_prefill_runs
-        f.argtypes, f.restype = [c_int] * 8 + [c_long], c_int
+        f.argtypes, f.restype = [c_int, c_void_p, c_void_p] + [c_int] * 6 + [c_long], c_int
         _fn_cache[("attention", "li_paged_attention_prefill_runs")] = f
-    return int(f(ntiles, nh, nkv, dh, max_blocks, page_size, keys, tokens, PREFILL_RUNS_MAX_BYTES))
+    if host_q_len is None or host_ctx_len is None or host_q_len.dtype != "int32" or host_ctx_len.dtype != "int32":
+        return 1
+    return int(f(len(host_q_len), host_q_len.ctypes.data, host_ctx_len.ctypes.data, nh, nkv, dh, max_blocks,
+                 int(window), tokens, PREFILL_RUNS_MAX_BYTES))
 
 
 def _stream() -> int:
@@ -673,10 +678,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
             and meta.tile_rows == PREFILL_TILE_ROWS and n_multi == meta.num_multi and meta.max_blocks <= 8192 and meta.max_blocks * page_size <= 1 << 21):
         # few tiles against long contexts: the tiles' keys in runs, joined by the kernel that joins the
         # decode attention's (the library says how many; their results take room in the workspace)
-        hq, hc = getattr(meta, "host_q_len", None), getattr(meta, "host_ctx_len", None)
-        longest = int(hc[hq > 1].max()) if hq is not None and hc is not None and (hq > 1).any() else meta.max_ctx_len
-        keys = min(longest, window) if window > 0 else longest
-        runs = _prefill_runs(meta.num_tiles, nh, nkv, dh, meta.max_blocks, page_size, keys, t) if ws is not None else 1
+        runs = 1
+        if ws is not None:
+            runs = _prefill_runs(getattr(meta, "host_q_len", None), getattr(meta, "host_ctx_len", None), nh, nkv, dh,
+                                 meta.max_blocks, window, t)
         acc = ml = lst = None
         if runs > 1:
             acc = ws.buffer("attn.runs_acc", (t, nh, runs, dh), torch.float32)

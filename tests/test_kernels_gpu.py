@@ -492,11 +492,9 @@ def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
 ])
 def test_prompt_portions_behind_long_contexts_with_their_keys_in_runs(ops, segs, nh, nkv, dh, page, window):
     from litinfer_amd.kernels.ops import _prefill_runs
-    keys = max(c for c, q in segs if q > 1)
-    keys = min(keys, window) if window else keys
-    tiles = sum(-(-q // 32) for _, q in segs if q > 1)
+    ql, cl = np.array([q for _, q in segs], dtype=np.int32), np.array([c for c, _ in segs], dtype=np.int32)
     blocks = max(-(-c // page) for c, _ in segs)
-    assert _prefill_runs(tiles, nh, nkv, dh, blocks, page, keys, sum(q for _, q in segs)) > 1     # the case is what it says
+    assert _prefill_runs(ql, cl, nh, nkv, dh, blocks, window, int(ql.sum())) > 1       # the case is what it says
     out, ref = _paged_case(ops, torch.bfloat16, segs, nh, nkv, dh, page, window, seed=31, ws=_Lender())
     assert rel(out, ref) < 1.5e-2
     # and one far key among thousands, in a run of its own
