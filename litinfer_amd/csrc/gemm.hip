@@ -1474,7 +1474,7 @@ static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, 
 
 extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype);
 
-// The packed q/k/v projection of 17 to 64 rows cut along K: the kernel that adds the parts up also adds
+// The packed q/k/v projection of 17 rows and more where it is cut along K (up to some hundred rows): the kernel that adds the parts up also adds
 // the bias, rotates query and key heads (half-split pairs over the whole head, float32 tables
 // [M, dh / 2]) and writes keys and values into their page slots, so that the rotation needs no
 // kernel of its own.  Thread (row, head, pair): consecutive threads read consecutive sums.
@@ -1519,12 +1519,14 @@ extern "C" int li_linear_rope_store_parts(const void* x, const void* w, const fl
         (long)(nh + 2 * nkv) * dh > 0x7fffffffL)
         return LI_ERR_SIZE;
     const int N = (nh + 2 * nkv) * dh;
-    if (!mid_rows_take(M, K) || K % 64) return -1;
-    const long need = li_linear_work_bytes(M, N, K, LI_BF16);
+    if (M <= 16 || K % 64) return -1;
+    const long need = li_linear_work_bytes(M, N, K, LI_BF16);            // (0 where li_linear would not cut this product)
     if (need <= 0 || !work || work_bytes < need) return -1;
     const size_t mn = (size_t)M * N;
     const int nsplit = (int)(need / (long)(mn * sizeof(float)));
-    const int rc = launch_dma<64, 128, 64, 4, false, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)work, M, N, K, 0, stream, nsplit);
+    const int rc = M <= 64
+        ? launch_dma<64, 128, 64, 4, false, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)work, M, N, K, 0, stream, nsplit)
+        : launch_dma<128, 128, 64, 4, false, float>((const bf16_t*)x, (const bf16_t*)w, nullptr, (float*)work, M, N, K, 0, stream, nsplit);
     if (rc != LI_OK) return rc;
     const long total = (long)M * (nh + 2 * nkv) * (dh / 2);
     splitk_reduce_rope_store_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(

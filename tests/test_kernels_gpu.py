@@ -595,10 +595,12 @@ def test_rope_kv_store_and_plain_store(ops, dtype, dh, pad):
     (64, 28, 4, 128, 3584, True),       # a decoding batch of 64 at the 7B layer sizes
     (33, 12, 2, 128, 1536, True),
     (40, 6, 2, 64, 1280, False),
+    (100, 28, 4, 128, 3584, True),      # more than 64 rows: tiles of 128 rows, K still cut
+    (200, 12, 2, 128, 1536, False),
 ])
 def test_projection_cut_along_k_with_rotary_encoding_and_page_write_in_the_adding_up(ops, t, nh, nkv, dh, k, bias):
     g = torch.Generator().manual_seed(31)
-    n, page, pages = (nh + 2 * nkv) * dh, 16, 8
+    n, page, pages = (nh + 2 * nkv) * dh, 16, max(8, t // 16 + 3)
     x = torch.randn(t, k, generator=g).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
     b = torch.randn(n, generator=g) if bias else None
