@@ -13,16 +13,26 @@ class Workspace:
         self.device = torch.device(device)
         self._bufs: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
         self.generation = 0          # goes up whenever a buffer moves: recorded graphs are stale then
+        self._views: Dict[Tuple[str, torch.dtype, Tuple[int, ...]], torch.Tensor] = {}
 
     def buffer(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
         """A tensor of this shape; its contents are whatever the last user of
         the same name left."""
-        n = max(1, math.prod(int(s) for s in shape))
+        shape = tuple(int(s) for s in shape)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:                       # (asked for some hundred times a step, mostly with the same shapes)
+            return view
+        n = math.prod(shape)
         key = (name, dtype)
         buf = self._bufs.get(key)
-        if buf is None or buf.numel() < n:
-            cap = n if buf is None else max(n, buf.numel() * 3 // 2)
+        if buf is None or buf.numel() < max(1, n):
+            cap = max(1, n) if buf is None else max(n, buf.numel() * 3 // 2)
             buf = torch.empty(cap, dtype=dtype, device=self.device)
             self._bufs[key] = buf
             self.generation += 1
-        return buf[:math.prod(int(s) for s in shape)].view(*shape)
+            for k in [k for k in self._views if k[0] == name and k[1] is dtype]:
+                del self._views[k]                 # views of the buffer that has just moved
+        view = buf[:n].view(*shape)
+        if len(self._views) < 4096:
+            self._views[(name, dtype, shape)] = view
+        return view

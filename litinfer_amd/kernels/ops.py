@@ -105,7 +105,15 @@ def _prefill_runs(host_q_len, host_ctx_len, nh: int, nkv: int, dh: int, max_bloc
                  int(window), tokens, PREFILL_RUNS_MAX_BYTES))
 
 
+# the current stream's handle without the stream object around it (an op is called some hundred times a
+# step, and the object's way through torch's Python layers took a quarter of a step's host time)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_get_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> int:
+    if _raw_stream is not None and _get_device is not None:
+        return _raw_stream(_get_device())
     return torch.cuda.current_stream().cuda_stream
 
 
