@@ -157,11 +157,12 @@ def _rows_ok(t: torch.Tensor) -> bool:
 def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> None:
     """Sizes the attention and position kernels take; anything else is refused
     here, when the model is built."""
-    _chk(num_heads > 0 and num_kv_heads > 0 and num_heads % num_kv_heads == 0,
-         f"attention: {num_heads} heads and {num_kv_heads} kv heads: the first must be a "
-         f"multiple of the second")
-    _chk(head_dim % 2 == 0 and 2 <= head_dim <= MAX_HEAD_DIM,
-         f"attention: head size {head_dim} is not supported (even, at most {MAX_HEAD_DIM})")
+    # (the texts are made only when they are needed: these checks run with every call of an op)
+    if not (num_heads > 0 and num_kv_heads > 0 and num_heads % num_kv_heads == 0):
+        _chk(False, f"attention: {num_heads} heads and {num_kv_heads} kv heads: the first must be a "
+                    f"multiple of the second")
+    if not (head_dim % 2 == 0 and 2 <= head_dim <= MAX_HEAD_DIM):
+        _chk(False, f"attention: head size {head_dim} is not supported (even, at most {MAX_HEAD_DIM})")
 
 
 # ---------------------------------------------------------------- elementwise
@@ -321,10 +322,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
     _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear: needs matrices")
     m, k = x.shape
     n = w.shape[0]
-    _chk(w.shape[1] == k and out.shape == (m, n), f"linear: shapes x {tuple(x.shape)}, "
-         f"w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+    if not (w.shape[1] == k and out.shape == (m, n)):
+        _chk(False, f"linear: shapes x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
     _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear: contiguous operands")
-    _chk(x.dtype is w.dtype and x.dtype in _DT, f"linear: x is {x.dtype}, w is {w.dtype}")
+    if not (x.dtype is w.dtype and x.dtype in _DT):
+        _chk(False, f"linear: x is {x.dtype}, w is {w.dtype}")
     _chk(out.dtype is x.dtype or out.dtype is torch.float32, "linear: out dtype")
     _chk(not accumulate or out.dtype is torch.float32, "linear: accumulation needs a float32 out")
     _chk(bias is None or (bias.dtype is torch.float32 and bias.numel() == n and bias.is_contiguous()),
