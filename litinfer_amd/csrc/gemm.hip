@@ -1074,7 +1074,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         int row;
-        if (SWIGLU) row = ((n0 + r16 < N) ? n0 + r16 : N - 1) + nt * N;      // gate row, up row
+        if (SWIGLU) row = ((n0 + r16 < nend) ? n0 + r16 : nend - 1) + nt * N;      // gate row, up row
         else if (ROPE) {                                    // rows 0..7 of a tile: first members of 8 pairs, 8..15: their partners
             int p = n0 + 8 * nt + (r16 & 7);
             p = p < nend ? p : nend - 1;
@@ -1308,7 +1308,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int n = n0 + 4 * (l >> 4) + r;
-                if (n < N) {
+                if (n < nend) {
                     const float gv = s[0][r], uv = s[NT - 1][r];
                     store_from_float(out + (size_t)m * N + n, uv * (gv / (1.0f + expf(-gv))));
                 }
@@ -1375,12 +1375,28 @@ static int balanced_per_block(int total, int unit) {
     return per > 2 * unit ? 0 : per;
 }
 
+// Many columns in tiles of `unit`: the blocks of a product go round the compute units several times, and
+// the units with one block more than the others set the time when the matrix is small.  The columns a
+// block takes are therefore cut down until the last round is as full as the others: as many rounds as
+// whole tiles would need, and equal shares of the columns within them (at least half a tile's).
+static int balanced_round_cols(int total, int unit) {
+    const long cu = compute_units();
+    const long rounds = (total + unit * cu - 1) / (unit * cu);
+    long per = (total + rounds * cu - 1) / (rounds * cu);
+    per = per < unit / 2 ? unit / 2 : per;
+    return (int)(per > unit ? unit : per);
+}
+
 template <bool SWIGLU, typename TO>
 static void launch_skinny(SkinnyArgs a, hipStream_t stream) {
     const int M = a.M, N = a.N;
 #define LI_SK(MT, NT, WV) gemm_bf16_skinny_kernel<MT, NT, WV, SWIGLU, TO><<<(N + 16 * (SWIGLU ? 1 : NT) - 1) / (16 * (SWIGLU ? 1 : NT)), WV * 64, 0, stream>>>(a)
     if constexpr (SWIGLU) {
-        if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
+        a.cols = balanced_round_cols(N, 16);
+        const int blocks = (N + a.cols - 1) / a.cols;
+        if (M <= 16) gemm_bf16_skinny_kernel<1, 2, 4, true, TO><<<blocks, 4 * 64, 0, stream>>>(a);
+        else if (M <= 32) gemm_bf16_skinny_kernel<2, 2, 4, true, TO><<<blocks, 4 * 64, 0, stream>>>(a);
+        else gemm_bf16_skinny_kernel<4, 2, 8, true, TO><<<blocks, 8 * 64, 0, stream>>>(a);
     } else if (N >= 8192) {                                 // many columns: many blocks, two tiles share each piece of x
         if (M <= 16) LI_SK(1, 2, 4); else if (M <= 32) LI_SK(2, 2, 4); else LI_SK(4, 2, 8);
     } else if (M <= 16) {                                   // few columns: a block a compute unit, eight waves split K

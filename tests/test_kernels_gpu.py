@@ -117,6 +117,9 @@ def test_linear(ops, dtype, mnk, bias, acc):
     (11, 8300, 520, True, torch.bfloat16, False, False),
     (1, 152064, 64, False, torch.float32, False, False),
     (20, 9000, 520, False, torch.bfloat16, False, False),
+    (4, 8960, 64, True, torch.bfloat16, False, False),          # gate/up in equal shares of the columns: 12 a block,
+    (25, 4101, 40, True, torch.bfloat16, False, False),         # 9 a block with a ragged last one,
+    (40, 4864, 72, True, torch.bfloat16, False, False),         # 10 a block
 ])
 def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, acc):
     g = torch.Generator().manual_seed(12)
@@ -133,7 +136,7 @@ def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, 
         out = base.to(DEV)
         y = y + base.double().numpy()
     else:
-        out = torch.empty(m, n, dtype=out_dtype, device=DEV)
+        out = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)     # a column left out shows
     assert ops.skinny_takes(m, k, w.dtype)
     ops.linear_skinny(x.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, acc, swiglu=swiglu)
     assert rel(out, y) < (4 * math.sqrt(k) * 2.0 ** -24 if out_dtype is torch.float32 else 5e-3)
