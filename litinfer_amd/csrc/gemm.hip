@@ -385,13 +385,28 @@ struct TileOrder {
         pm = mtiles < 8 ? mtiles : 8;
         gn = 32 / pm;
     }
-    __host__ static long blocks(long mtiles, long ntiles) {       // grid size: the same number of blocks on each XCD
-        return (mtiles * ntiles + 7) / 8 * 8;
+    __host__ static long blocks(long mtiles, long ntiles, long nsplit = 1) {      // grid size: the same number of blocks on each XCD
+        return (mtiles * ntiles * nsplit + 7) / 8 * 8;
     }
-    __device__ bool tile(int block, int mtiles, int ntiles, int& mt, int& nt) const {
-        const long total = (long)mtiles * ntiles, per = (total + 7) / 8;
-        const long t = (block & 7) * per + (block >> 3);
-        if (t >= total) return false;
+    // With K in nsplit parts: where the tiles divide by 8 every XCD takes its eighth of them in every
+    // part (the same rows of w, all of K).  Otherwise the sequence is that of the tiles nsplit times
+    // over, part after part, and the XCDs share the whole of it: dealt part by part, the last XCD's
+    // few tiles fewer would come nsplit times over and the other XCDs would hold more blocks than they
+    // have compute units (36 tiles in 7 parts: 35 blocks on each of seven XCDs, 7 on the last).
+    // (All of it in 32 bits: the launch has checked that the blocks fit.)
+    __device__ bool tile(unsigned block, int mtiles, int ntiles, int nsplit, int& mt, int& nt, int& split) const {
+        const unsigned tiles = (unsigned)mtiles * (unsigned)ntiles, total = tiles * (unsigned)nsplit;
+        unsigned t;
+        if (nsplit > 1 && (tiles & 7) == 0) {
+            split = (int)(block / tiles);
+            const unsigned b = block - (unsigned)split * tiles;
+            t = (b & 7) * (tiles >> 3) + (b >> 3);
+        } else {
+            const unsigned per = (total + 7) / 8, s = (block & 7) * per + (block >> 3);
+            if (s >= total) return false;
+            split = (int)(s / tiles);
+            t = s - (unsigned)split * tiles;
+        }
         const int group = mtiles * gn;               // tiles of gn column panels
         const int cg = (int)(t / group), r = (int)(t % group);
         const int gc = ntiles - cg * gn < gn ? ntiles - cg * gn : gn;        // column panels of this group
@@ -419,8 +434,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
     const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    int mt, nt;
-    if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, mt, nt)) return;
+    int mt, nt, split;
+    if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, 1, mt, nt, split)) return;
     const int m0 = mt * BM, n0 = nt * BN;
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -602,8 +617,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                                                              const bf16_t* __restrict__ w,
                                                              const float* __restrict__ bias,
                                                              TO* __restrict__ out, int M, int N, int K,
-                                                             int accumulate) {
-    // gridDim.y > 1: block (., y) multiplies the y-th part of K and writes its sums to the y-th
+                                                             int accumulate, int nsplit) {
+    // nsplit > 1: a block multiplies one of nsplit parts of K, the y-th, and writes its sums to the y-th
     // [M, N] matrix behind `out` (float, no bias, no accumulation); splitk_reduce_kernel adds them
     // WLM: waves along the rows of the tile, 2 (two by two) or 4 (each wave 32-row bands over all columns:
     // BN may then be any multiple of 32, for matrices whose columns no other tile divides into 256 tiles)
@@ -622,8 +637,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave / WLN) * WM, wn = (wave % WLN) * WN;
     const int mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    int mt, nt;
-    if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, mt, nt)) return;
+    int mt, nt, split;
+    if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, nsplit, mt, nt, split)) return;
     const int m0 = mt * BM, n0 = nt * BN;
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -685,9 +700,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
         for (int i = 0; i < LPW; ++i) issue_one(kt, i);
     };
     const int frow = lane & 31, fh = lane >> 5;
-    const int kt_first = (int)((long)(K / BK) * blockIdx.y / gridDim.y);
-    const int nk = (int)((long)(K / BK) * (blockIdx.y + 1) / gridDim.y) - kt_first;
-    out += (size_t)blockIdx.y * M * (SWIGLU ? N / 2 : N);
+    // (the parts' steps: equal shares, the first parts one more where they do not divide)
+    const int ksteps = K / BK, kshare = ksteps / nsplit, kmore = ksteps - kshare * nsplit;
+    const int kt_first = split * kshare + (split < kmore ? split : kmore);
+    const int nk = kshare + (split < kmore ? 1 : 0);
+    out += (size_t)split * M * (SWIGLU ? N / 2 : N);
     abase += (size_t)kt_first * BK;
     bbase += (size_t)kt_first * BK;
     constexpr int KS = BK / 16;                    // MFMA groups of a step: 16 columns each
@@ -908,8 +925,9 @@ template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO, int WLM 
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream, int nsplit = 1) {
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
-    const long per_xcd = TileOrder::blocks(mtiles, ntiles) / 8;
-    if (per_xcd * 8 > 0x7fffffffL || nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
+    if (nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
+    const long blocks = TileOrder::blocks(mtiles, ntiles, nsplit);
+    if (blocks > 0x7fffffffL) return LI_ERR_SIZE;
     // a lane's byte offset from its tile's first row is kept in 32 bits (the gate and up rows of a
     // SwiGLU tile lie N / 2 rows apart)
     const unsigned long long span_rows = SWIGLU ? (unsigned long long)N / 2 + BN : (unsigned long long)(BM > BN ? BM : BN);
@@ -922,7 +940,7 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
             return LI_ERR_LAUNCH;
         configured = true;
     }
-    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO, WLM><<<dim3((unsigned)(per_xcd * 8), nsplit), 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate);
+    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO, WLM><<<(unsigned)blocks, 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate, nsplit);
     return li_launch_status();
 }
 

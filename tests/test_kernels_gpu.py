@@ -158,6 +158,10 @@ class _Lender:
     (128, 3584, 18944, torch.float32, False, True),      # more rows, but few tiles over a long K: parts again
     (200, 300, 4096, torch.bfloat16, True, False),
     (500, 1000, 1024, torch.float32, True, False),       # 32 tiles, two parts
+    (50, 4608, 3584, torch.bfloat16, True, False),       # 36 tiles in 7 parts: not whole eighths, the XCDs share one sequence
+    (384, 3584, 2048, torch.float32, False, True),       # 84 tiles in 3 parts, three rows of tiles
+    (130, 2048, 1536, torch.float32, True, True),        # 32 tiles in 3 parts: an eighth of the tiles each, part by part
+    (64, 1100, 1984, torch.bfloat16, False, False),      # 9 tiles in 3 parts of 11, 10 and 10 steps
 ])
 def test_linear_with_k_in_parts(ops, m, n, k, out_dtype, bias, acc):
     g = torch.Generator().manual_seed(15)
