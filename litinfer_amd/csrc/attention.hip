@@ -299,20 +299,32 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 template <typename T>
 __global__ __launch_bounds__(128) void attention_merge_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int nsplit) {
+    const int* __restrict__ token_list, T* __restrict__ out, int nh, int dh, int nsplit_all,
+    const int* __restrict__ nruns = nullptr) {
     __shared__ float wgt[MERGE_MAX_SPLITS];
     __shared__ float inv_l;
     const int ti = blockIdx.x, head = blockIdx.y;
     const int t = token_list ? token_list[ti] : ti;
-    const size_t base = ((size_t)ti * nh + head) * nsplit;
+    const size_t base = ((size_t)ti * nh + head) * nsplit_all;
+    // nruns: the token's runs that were written (the others of its nsplit_all places hold anything)
+    int nsplit = nsplit_all;
+    if (nruns) {
+        nsplit = nruns[ti];
+        nsplit = nsplit < 1 ? 1 : (nsplit > nsplit_all ? nsplit_all : nsplit);
+    }
     // The partial results of this thread's first dimension are asked for before the weights
     // are known (up to 32 splits, all loads at once and never conditional): their way from
     // memory then runs beside the weights' way and arithmetic, not behind them.
     constexpr int AHEAD = 32;
     float pa[AHEAD];
     const int d0 = threadIdx.x < dh ? threadIdx.x : 0;
+    if (nruns) {                                     // (the number of runs is not known yet: the first place is always written)
 #pragma unroll
-    for (int sp = 0; sp < AHEAD; ++sp) pa[sp] = part_acc[(base + (sp < nsplit ? sp : nsplit - 1)) * dh + d0];
+        for (int sp = 0; sp < AHEAD; ++sp) pa[sp] = part_acc[(base + (sp < nsplit_all ? sp : 0)) * dh + d0];
+    } else {
+#pragma unroll
+        for (int sp = 0; sp < AHEAD; ++sp) pa[sp] = part_acc[(base + (sp < nsplit ? sp : nsplit - 1)) * dh + d0];
+    }
     if (threadIdx.x < 64) {
         const int sp = threadIdx.x;
         const float ms = sp < nsplit ? part_ml[(base + sp) * 2] : -INFINITY;
@@ -429,6 +441,112 @@ extern "C" long li_decode_split_blocks(int max_blocks, int page_size, int window
     return (per + page_size - 2) / page_size + 1;
 }
 
+// The length of a run of keys for the decode kernel below, chosen on the device for the batch at hand
+// (a recorded step is replayed for other context lengths than it was recorded with).  Cut into nsplit
+// runs each, tokens with short contexts would give short waves and the longest context would set the
+// time; with one run length for all of them a short context fills few of its nsplit runs (the others
+// find no keys and end at once) and the waves that work are equally long.  Every candidate length
+// (multiples of 32, from what the longest context needs to fit nsplit runs up to what the block
+// table's width would need) costs rounds of the working waves over the SIMDs x (length + a wave's
+// start and end, 24 keys' time); the cheapest is taken, of equal ones the shortest.  out: [0] that length,
+// [1] the number of (token, run) items, i.e. of runs with keys, [2 .. 2 + n_tokens) the runs of every token,
+// then the items, token | run << 16, a token's runs in a row: the decode kernel starts a block for every
+// item the grid could hold (tokens x nsplit) and those beyond [1] end at once, without a look at their
+// token.  At most RUN_KEYS_MAX_TOKENS tokens (the host checks).
+#define RUN_KEYS_MAX_TOKENS 4096
+__global__ __launch_bounds__(256) void decode_run_keys_kernel(
+    const int* __restrict__ token_list, int n_tokens, const int* __restrict__ seg_of_token,
+    const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
+    int cap_keys, int window, int nkv, int nsplit, int simds, int* __restrict__ out) {
+    __shared__ int nkeys[RUN_KEYS_MAX_TOKENS];
+    __shared__ int red_i[4];
+    __shared__ unsigned long long red_c[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (n_tokens > RUN_KEYS_MAX_TOKENS) return;      // (refused by the host)
+    int mx = 0;
+    for (int i = tid; i < n_tokens; i += 256) {
+        const int t = token_list ? token_list[i] : i;
+        const int s = seg_of_token[t];
+        const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
+        const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+        const int n = p - lo + 1;
+        nkeys[i] = n;
+        mx = n > mx ? n : mx;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) { const int v = __shfl_xor(mx, o, 64); mx = v > mx ? v : mx; }
+    if (lane == 0) red_i[wave] = mx;
+    __syncthreads();
+    mx = red_i[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) mx = red_i[w] > mx ? red_i[w] : mx;
+    const int lower = (((mx + nsplit - 1) / nsplit) + 31) & ~31;
+    int cap = (((cap_keys + nsplit - 1) / nsplit) + 31) & ~31;
+    cap = cap < lower ? lower : cap;
+    const int ncand = (cap - lower) / 32 + 1;
+    const int stride = (ncand + 255) / 256;             // (more candidates than threads: every stride-th)
+    // cost and length in one number: the least of them is the cheapest, of equal ones the shortest
+    unsigned long long best = ~0ull;
+    const int c = lower + 32 * stride * tid;
+    if (c <= cap) {
+        long waves = 0;
+        for (int i = 0; i < n_tokens; ++i) waves += (nkeys[i] + c - 1) / c;
+        waves *= nkv;
+        const long rounds = (waves + simds - 1) / simds;
+        best = ((unsigned long long)(rounds * (c + 24)) << 32) | (unsigned)c;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long v = __shfl_xor(best, o, 64);
+        best = v < best ? v : best;
+    }
+    __syncthreads();
+    if (lane == 0) red_c[wave] = best;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < 4; ++w) best = red_c[w] < best ? red_c[w] : best;
+    const int per = (int)(unsigned)(best & 0xffffffffull);
+    // the runs of every token at that length, and the (token, run) items one after the other: thread t
+    // takes a stretch of tokens, the stretches' first items come from a scan over the threads
+    __shared__ int first[256];
+    const int each = (n_tokens + 255) / 256;
+    const int i0 = tid * each, i1 = i0 + each < n_tokens ? i0 + each : n_tokens;
+    int mine = 0;
+    for (int i = i0; i < i1; ++i) mine += (nkeys[i] + per - 1) / per;
+    first[tid] = mine;
+    __syncthreads();
+    if (tid == 0) {
+        int at = 0;
+        for (int w = 0; w < 256; ++w) { const int n = first[w]; first[w] = at; at += n; }
+        out[0] = per;
+        out[1] = at;
+    }
+    __syncthreads();
+    int at = first[tid];
+    int* nruns = out + 2;
+    int* items = out + 2 + n_tokens;
+    for (int i = i0; i < i1; ++i) {
+        const int n = (nkeys[i] + per - 1) / per;
+        nruns[i] = n;
+        for (int r = 0; r < n; ++r) items[at + r] = i | (r << 16);
+        at += n;
+    }
+}
+
+extern "C" int li_decode_run_keys(const int* token_list, int n_tokens, const int* seg_of_token, const int* q_start,
+                                  const int* q_len, const int* ctx_len, int max_blocks, int page_size, int window,
+                                  int nkv, int nsplit, int simds, int* out, hipStream_t stream) {
+    if (n_tokens <= 0 || n_tokens > RUN_KEYS_MAX_TOKENS || max_blocks <= 0 || page_size <= 0 || nkv <= 0 ||
+        nsplit <= 0 || nsplit > 0x7fff || simds <= 0 || !out)
+        return LI_ERR_SIZE;
+    long keys = (long)max_blocks * page_size;
+    if (window > 0 && window < keys) keys = window;
+    if (keys > 0x7fffffffL - 64) return LI_ERR_SIZE;
+    decode_run_keys_kernel<<<1, 256, 0, stream>>>(token_list, n_tokens, seg_of_token, q_start, q_len, ctx_len,
+                                                  (int)keys, window, nkv, nsplit, simds, out);
+    return li_launch_status();
+}
+
 template <int DH>
 __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
@@ -436,21 +554,42 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
     int max_blocks, const int* __restrict__ token_list, const int* __restrict__ seg_of_token,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
     float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv, int page_size,
-    int num_pages, int window, float scale, int nsplit) {
+    int num_pages, int window, float scale, int nsplit, const int* __restrict__ run_keys, int n_list) {
     constexpr int KS = DH / 32;                 // MFMA steps of Q K^T
     constexpr int NS = (DH + 127) / 128;        // slabs of 128 output dimensions
     constexpr int QD = DH / 4;                  // head dimensions owned by one lane group in Q K^T
     constexpr int PSTRIDE = 40;                 // halves per row of P in LDS (32 keys + pad, 80 bytes)
     __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * PSTRIDE];
     __shared__ int pages[DEC_TABLE_CAP];
-    const int ti = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z;
+    // run_keys given: block x takes the x-th (token, run) item of the list behind it, and ends at once if the
+    // list is shorter (blocks go to the XCDs in turn, in the order of their numbers, so every XCD gets its
+    // share of the runs that have keys).  Else block (token, kv head, run) of the grid.
+    int ti = blockIdx.x, split = blockIdx.z;
+    const int kvh = blockIdx.y;
+    if (run_keys) {
+        const int count = run_keys[1];
+        const int item = run_keys[2 + n_list + blockIdx.x];
+        if ((int)blockIdx.x >= count) return;
+        ti = item & 0xffff;
+        split = item >> 16;
+    }
     const int t = token_list ? token_list[ti] : ti;
     const int G = nh / nkv;
     const int s = seg_of_token[t];
     const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int nkeys = p - lo + 1;
-    const int per = (((nkeys + nsplit - 1) / nsplit) + 31) & ~31;
+    int per = (((nkeys + nsplit - 1) / nsplit) + 31) & ~31;
+    if (run_keys) {
+        // one run length for the whole batch (decode_run_keys_kernel): never shorter than this token's keys
+        // need to fit nsplit runs, never longer than the runs the host sized the page table in LDS for
+        long widest = (long)max_blocks * page_size;
+        if (window > 0 && window < widest) widest = window;
+        const int cap = (int)((((widest + nsplit - 1) / nsplit) + 31) & ~31L);
+        int given = (run_keys[0] + 31) & ~31;
+        given = given < cap ? given : cap;
+        per = given > per ? given : per;
+    }
     const int k_begin = lo + split * per;
     const int k_end = (k_begin + per < p + 1) ? k_begin + per : p + 1;
     const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
@@ -1769,13 +1908,15 @@ static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, cons
 
 // Single-query tokens of the batch (token_list, or all tokens when it is null).
 // part_acc: float [n_tokens, nh, nsplit, dh]; part_ml: float [n_tokens, nh, nsplit, 2] (unused when nsplit is 1).
+// run_keys (may be null; the matrix-core kernel with nsplit > 1 only): one int on the device, the run
+// length li_decode_run_keys chose for this batch.
 extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* out, const void* kc,
                                          const void* vc, int dtype, const int* block_table, int max_blocks,
                                          const int* token_list, int n_tokens, const int* seg_of_token,
                                          const int* q_start, const int* q_len, const int* ctx_len,
                                          float* part_acc, float* part_ml, int nh, int nkv, int dh,
                                          int page_size, int num_pages, int window, float scale, int nsplit,
-                                         int use_mfma, hipStream_t stream) {
+                                         int use_mfma, const int* run_keys, hipStream_t stream) {
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dh <= 0 || dh > ATT_MAX_DH || page_size <= 0 ||
         max_blocks <= 0)
         return LI_ERR_SIZE;
@@ -1790,16 +1931,19 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
         // a split's pages must fit the kernel's copy of the block table: `per` keys that begin
         // anywhere in a page touch at most (per + page_size - 2) / page_size + 1 pages
         if (li_decode_split_blocks(max_blocks, page_size, window, nsplit) > DEC_TABLE_CAP) return LI_ERR_SIZE;
-        dim3 grid(n_tokens, nkv, nsplit);
+        const bool listed = run_keys && nsplit > 1;
+        if (listed && (n_tokens > RUN_KEYS_MAX_TOKENS || nsplit > 0x7fff)) return LI_ERR_SIZE;
+        dim3 grid(listed ? n_tokens * nsplit : n_tokens, nkv, listed ? 1 : nsplit);
 #define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV><<<grid, 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
         token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
-        scale, nsplit)
+        scale, nsplit, listed ? run_keys : nullptr, n_tokens)
         if (dh == 128) LI_DM(128); else if (dh == 64) LI_DM(64); else return LI_ERR_SIZE;
 #undef LI_DM
         if (nsplit > 1) {
             dim3 g2(n_tokens, nh);
-            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit);
+            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit,
+                                                                   listed ? run_keys + 2 : nullptr);
         }
         return li_launch_status();
     }

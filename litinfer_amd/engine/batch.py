@@ -94,6 +94,8 @@ class StepContext:
 
     def forget_shared(self) -> None:
         self._shared.clear()
+        for meta in self._attn:
+            meta.extra.clear()
 
     def shared(self, key, make: Callable[[], Any]):
         """Per-step value shared by every part that asks with the same key."""

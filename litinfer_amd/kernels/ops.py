@@ -8,9 +8,11 @@ GPU, or without the built library, a call raises.
 from __future__ import annotations
 
 import ctypes
+import math
 from ctypes import c_float, c_int, c_long, c_void_p
 from typing import Dict, Optional
 
+import numpy as np
 import torch
 
 from . import build
@@ -48,7 +50,8 @@ _SIGNATURES = {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
         "li_paged_attention_prefill": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F, I, P, P, P, I],
         "li_paged_attention_prefill_f32": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F],
-        "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I],
+        "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "li_decode_run_keys": [P, I, P, P, P, P, I, I, I, I, I, I, P],
     },
     "sampling": {
         "li_argmax_rows": [P, P, P, P, I, I],
@@ -575,6 +578,7 @@ _DEC_WAVES = 1024
 PREFILL_TILE_ROWS = 32       # queries of one segment that a block of the matrix-core kernel for portions takes
 DECODE_MAX_SPLITS = 64       # the merge kernel keeps a weight per split
 DECODE_TABLE_CAP = 1024      # pages of one split that the matrix-core decode kernel copies into LDS
+DECODE_LIST_MAX_TOKENS = 4096    # single tokens whose runs the device lists (`decode_run_keys`)
 
 
 _simds: Dict[int, int] = {}
@@ -603,6 +607,41 @@ def decode_splits(pairs: int, keys: int, simds: int = _DEC_WAVES) -> int:
         if best_cost is None or cost < best_cost:
             best, best_cost = ns, cost
     return best
+
+
+def _ragged_splits(nsplit: int, meta, window: int) -> int:
+    """More runs for the grid of a batch whose contexts differ: `nsplit` fits contexts that are all as
+    long as the longest; with one run length for the batch (chosen on the device) the short ones fill
+    few runs, and the same number of working waves needs the longest cut into more."""
+    ql, cl = getattr(meta, "host_q_len", None), getattr(meta, "host_ctx_len", None)
+    if ql is None or cl is None or nsplit >= DECODE_MAX_SPLITS:
+        return nsplit
+    keys = cl[ql == 1]
+    if keys.size < 2:
+        return nsplit
+    if window > 0:
+        keys = np.minimum(keys, window)
+    ragged = float(keys.max()) * keys.size / max(float(keys.sum()), 1.0)
+    if ragged < 1.15:
+        return nsplit
+    return min(DECODE_MAX_SPLITS, int(math.ceil(nsplit * ragged * 1.25)))
+
+
+def decode_run_keys(meta, token_list: Optional[torch.Tensor], n_tokens: int, page_size: int, window: int,
+                    nkv: int, nsplit: int, simds: int, out: torch.Tensor) -> None:
+    """out[0] = the run length, in keys, for the split-key decode kernel over these single tokens
+    (`token_list`, or the batch's first n_tokens tokens): the multiple of 32 with the least rounds of
+    working waves over `simds` x (length + 24), between what the longest context needs to fit
+    `nsplit` runs and what the block table's width would need.  out[1] = the number of runs with
+    keys at that length, out[2 : 2 + n_tokens] = the runs of each token, then the runs themselves as
+    token | run << 16.  At most 4,096 tokens."""
+    _gpu(out, meta.ctx_len, token_list)
+    _chk(0 < n_tokens <= DECODE_LIST_MAX_TOKENS, "decode_run_keys: too many tokens")
+    _chk(out.dtype is torch.int32 and out.is_contiguous() and out.numel() >= 2 + n_tokens + n_tokens * nsplit,
+         "decode_run_keys: out must be int32 [2 + tokens + tokens * nsplit]")
+    _run("attention", "li_decode_run_keys", 0 if token_list is None else token_list.data_ptr(), n_tokens,
+         meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
+         meta.max_blocks, page_size, int(window), nkv, nsplit, simds, out.data_ptr())
 
 
 def decode_split_blocks(max_blocks: int, page_size: int, window: int, nsplit: int) -> int:
@@ -657,8 +696,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         # bfloat16 with a head size of 64 or 128: one wave per split on the matrix cores; else one
         # block of four waves per split on the vector ALU
         mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
+        planned = 0
         if mfma:
-            nsplit = decode_splits(n_single * nkv, keys, _simd_count(qkv.device))
+            planned = decode_splits(n_single * nkv, keys, _simd_count(qkv.device))
+            nsplit = _ragged_splits(planned, meta, window)
             # a split's pages must fit the kernel's copy of the block table
             while nsplit <= DECODE_MAX_SPLITS and decode_split_blocks(meta.max_blocks, page_size, window, nsplit) > DECODE_TABLE_CAP:
                 nsplit += 1
@@ -676,12 +717,27 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
                 acc = torch.empty(shape_a, dtype=torch.float32, device=qkv.device)
                 ml = torch.empty(shape_m, dtype=torch.float32, device=qkv.device)
         lst = meta.single_tokens if n_single < t else None
+        run_keys = None
+        if mfma and nsplit > planned and n_single <= DECODE_LIST_MAX_TOKENS:
+            # contexts that differ: one run length for the batch and the list of the runs that have keys, made
+            # on the device from the context lengths, once a step for all layers with these numbers (a
+            # recorded step makes them again at every replay)
+            key = ("decode_run_keys", nkv, int(window), nsplit, meta.max_blocks, n_single)
+            run_keys = meta.extra.get(key)
+            if run_keys is None:
+                name = "attn.run_keys.%d.%d.%d.%d" % (nkv, int(window), nsplit, n_single)
+                size = 2 + n_single + n_single * nsplit
+                run_keys = (ws.buffer(name, (size,), torch.int32) if ws is not None
+                            else torch.empty(size, dtype=torch.int32, device=qkv.device))
+                decode_run_keys(meta, lst, n_single, page_size, window, nkv, nsplit, _simd_count(qkv.device), run_keys)
+                meta.extra[key] = run_keys
         _run("attention", "li_paged_attention_decode", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), _DT[qkv.dtype], bt.data_ptr(), meta.max_blocks,
              0 if lst is None else lst.data_ptr(), n_single, meta.seg_of_token.data_ptr(),
              meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              0 if acc is None else acc.data_ptr(), 0 if ml is None else ml.data_ptr(),
-             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit, int(mfma))
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit, int(mfma),
+             0 if run_keys is None else run_keys.data_ptr())
     # the matrix-core kernel for portions keeps a tile's pages in LDS (8192 entries) and divides
     # positions by the page size in float, exact below 2^21 keys; longer tables take the general kernel
     if (n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles

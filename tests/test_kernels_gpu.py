@@ -491,6 +491,41 @@ def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
 
 
+@pytest.mark.parametrize("window", [0, 900])
+def test_decode_run_length_of_a_batch_with_unequal_contexts(ops, window):
+    # the run length chosen on the device against the same search written out, for contexts from 3 to 5,000
+    # keys; then the attention of that batch
+    rng = np.random.default_rng(5)
+    ctx = rng.integers(3, 5000, 37).astype(np.int32)
+    ctx[11] = 5000
+    nseg, page, nkv, nsplit, simds = len(ctx), 16, 2, 9, 128
+    ones = np.ones(nseg, dtype=np.int32)
+    dev = lambda a: torch.from_numpy(a).to(DEV)
+    max_blocks = 512
+    meta = AttentionMeta(block_table=torch.zeros(nseg, max_blocks, dtype=torch.int32, device=DEV), max_blocks=max_blocks,
+                         seg_of_token=dev(np.arange(nseg, dtype=np.int32)), q_start=dev(np.arange(nseg, dtype=np.int32)),
+                         q_len=dev(ones), ctx_len=dev(ctx), num_segments=nseg, num_tokens=nseg, max_q_len=1,
+                         max_ctx_len=int(ctx.max()), host_q_start=np.arange(nseg, dtype=np.int32), host_q_len=ones,
+                         host_ctx_len=ctx, num_single=nseg)
+    out = torch.full((2 + nseg + nseg * nsplit,), -1, dtype=torch.int32, device=DEV)
+    ops.decode_run_keys(meta, None, nseg, page, window, nkv, nsplit, simds, out)
+    keys = np.minimum(ctx, window) if window else ctx
+    widest = min(max_blocks * page, window) if window else max_blocks * page
+    lower, cap = (-(-int(keys.max()) // nsplit) + 31) & ~31, (-(-widest // nsplit) + 31) & ~31
+    cost = {c: -(-int(nkv * np.sum(-(-keys // c))) // simds) * (c + 24) for c in range(lower, max(cap, lower) + 1, 32)}
+    want = min(cost, key=lambda c: (cost[c], c))
+    got = out.cpu().numpy()
+    assert int(got[0]) == want
+    runs = -(-keys // want)
+    assert int(got[1]) == int(runs.sum()) and np.array_equal(got[2:2 + nseg], runs)
+    items = got[2 + nseg:2 + nseg + int(runs.sum())]
+    assert [(int(i) & 0xffff, int(i) >> 16) for i in items] == [(t, r) for t in range(nseg) for r in range(int(runs[t]))]
+    assert want == (832 if not window else 128)      # (without a window the shortest run, 576, is not the cheapest)
+    segs = [(int(c), 1) for c in ctx]
+    got, ref = _paged_case(ops, torch.bfloat16, segs, 12, 2, 128, 16, window, seed=41, ws=_Lender())
+    assert rel(got, ref) < 8e-3
+
+
 @pytest.mark.parametrize("segs,nh,nkv,dh,page,window", [
     ([(3000, 64)], 28, 4, 128, 16, 0),                              # two tiles behind 2,936 cached tokens: their keys in five runs
     ([(3000, 64), (500, 1), (1200, 40), (40, 40)], 28, 4, 128, 16, 0),   # beside a decoding token; a short tile leaves runs without keys
