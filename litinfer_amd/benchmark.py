@@ -332,7 +332,8 @@ def headline(a) -> Dict[str, object]:
             f"bf16 MFMA loop {ref['mfma_bf16_TFLOPs']} TFLOP/s, fp32 FMA loop {ref['fma_fp32_TFLOPs']} TFLOP/s")
     t0 = time.time()
     eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
-                             num_pages=max_b * CONTEXT // PAGE + PREFILL_TOKENS // PAGE, max_seqs=max_b + 1)
+                             num_pages=max_b * CONTEXT // PAGE + PREFILL_TOKENS // PAGE, max_seqs=max_b + 1,
+                             page_order_seed=None if a.page_order_seed < 0 else a.page_order_seed)
     for g in eng.cache.groups:                       # synthetic cache content
         for data in g.data.values():
             flat = data.view(-1)
@@ -355,7 +356,8 @@ def headline(a) -> Dict[str, object]:
         "metric": f"decode tok/s (Qwen2-7B shape, batch {a.batch}, context {CONTEXT})", "value": round(value, 2),
         "unit": "tok/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.dtype,
-        "data": "synthetic: seeded random token ids, random weights N(0, 0.02), random cache content in the loop of steps",
+        "data": "synthetic: seeded random token ids, random weights N(0, 0.02), random cache content in the loop of steps, "
+                + ("pages handed out in the order of their numbers" if a.page_order_seed < 0 else "pages handed out in a shuffled order"),
         "config": {"model": "Qwen2-7B shape", "num_hidden_layers": a.layers,
                    "full_num_hidden_layers": QWEN2_7B["num_hidden_layers"], "hidden_size": cfg["hidden_size"],
                    "num_attention_heads": cfg["num_attention_heads"],
@@ -597,6 +599,10 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--mode", default="headline", choices=["headline", "serving", "long", "sweep"])
     ap.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="sweep: the member of the family whose layer sizes are taken")
+    ap.add_argument("--page-order-seed", type=int, default=0,
+                    help="headline: the cache's pages are handed out in a shuffled order, as a pool that has served requests "
+                         "does (negative: in the order of their numbers; a request's keys then lie in one piece, and "
+                         "how the pieces of a batch fall onto the memory's channels moves a batch-64 step by 7 %%)")
     ap.add_argument("--no-points", action="store_true", help="headline: skip the batch 1 and 64 points")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-scheduler", action="store_true", help="headline: skip the runs through the scheduler")
