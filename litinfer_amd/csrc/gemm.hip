@@ -1467,7 +1467,7 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
     return li_launch_status();
 }
 
-// Between 17 and 64 rows (a large decoding batch) the product is still bound by streaming W, but
+// Between 13 and 64 rows (a large decoding batch) the product is still bound by streaming W, but
 // x is too large to be read again by every block of a few columns (every block of the few-row
 // kernel reads all of x, and what a compute unit can take in then bounds the product): tiles of
 // 64 rows with the loads straight into LDS, and, where the matrix has too few such tiles to fill
@@ -1477,9 +1477,15 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
 // Measured on the 7B layer sizes, a decode step of 17 / 24 / 32 requests: 4.57 / 4.95 / 5.33 ms
 // against 4.90 / 5.33 / 5.84 ms with the few-row kernel up to 32 rows.  Returns -1 when it does
 // not take the call.
+// The few-row kernel takes up to 16 rows with its fused epilogues, but from 13 rows on the tiles with K in
+// parts are faster (7B layer sizes, a decode step of 12 / 14 / 16 requests: 4.08 / 4.27 / 4.43 ms with the
+// few-row kernels, 4.10 / 4.17 / 4.28 ms with the tiles): callers are told to prefer the tiles from there.
+#define FEW_ROWS_FUSED 12
+extern "C" int li_few_rows_fused() { return FEW_ROWS_FUSED; }
+
 static bool mid_rows_take(int M, int K) {
     (void)K;
-    return M > 16 && M <= 64;
+    return M > FEW_ROWS_FUSED && M <= 64;
 }
 
 static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, void* out, int M, int N,
@@ -1553,7 +1559,7 @@ extern "C" int li_linear_rope_store_parts(const void* x, const void* w, const fl
         (long)(nh + 2 * nkv) * dh > 0x7fffffffL)
         return LI_ERR_SIZE;
     const int N = (nh + 2 * nkv) * dh;
-    if (M <= 16 || K % 64) return -1;
+    if (M <= FEW_ROWS_FUSED || K % 64) return -1;
     const long need = li_linear_work_bytes(M, N, K, LI_BF16);            // (0 where li_linear would not cut this product)
     if (need <= 0 || !work || work_bytes < need) return -1;
     const size_t mn = (size_t)M * N;
@@ -1603,7 +1609,7 @@ static int split_parts_many_rows(int M, int N, int K) {
 
 // Bytes of workspace with which li_linear cuts this product along K (0: it would not).
 extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
-    if (in_dtype != LI_BF16 || M <= 16 || N <= 0 || K <= 0 || K % 64) return 0;
+    if (in_dtype != LI_BF16 || M <= FEW_ROWS_FUSED || N <= 0 || K <= 0 || K % 64) return 0;
     if (M <= 64 && !mid_rows_take(M, K)) return 0;
     int nsplit = 1;
     if (M <= 64) {
@@ -1626,7 +1632,7 @@ extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
 extern "C" int li_linear_then_norm(const void* x, const void* w, const float* bias, float* out, int M, int N, int K,
                                    void* work, long work_bytes, const float* gamma, float eps, void* xn,
                                    int xn_dtype, hipStream_t stream) {
-    if (M <= 16 || N <= 0 || K <= 0 || (K % 64) || !gamma || !xn || eps < 0.f) return -1;
+    if (M <= FEW_ROWS_FUSED || N <= 0 || K <= 0 || (K % 64) || !gamma || !xn || eps < 0.f) return -1;
     if (N > REDUCE_NORM_NT * REDUCE_NORM_PER || (xn_dtype != LI_BF16 && xn_dtype != LI_F32)) return -1;
     const long need = li_linear_work_bytes(M, N, K, LI_BF16);
     if (need <= 0 || !work || work_bytes < need) return -1;
@@ -1746,7 +1752,7 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
         launch_skinny<true, bf16_t>(a, stream);
         return li_launch_status();
     }
-    if (M > 16 && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
+    if (M > FEW_ROWS_FUSED && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
         // tiles of 64 rows: the width with the least estimated time that gives the chip enough tiles (a
         // product of few rows waits for w, and a compute unit takes in only so much: more units, each
         // with a narrower tile, stream more, until the tiles no longer fit one round)

@@ -336,7 +336,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
          "linear: bias must be float32 [N]")
     if m:
         work, work_bytes = 0, 0
-        if ws is not None and x.dtype is torch.bfloat16 and m > RESIDUAL_NORM_MAX_ROWS:
+        if ws is not None and x.dtype is torch.bfloat16 and m > FEW_ROWS_PREFERRED:
             # few rows over a long k and few columns: the library cuts k into parts if it is lent room for their sums
             need = _work_bytes(m, n, k, _DT[x.dtype])
             if need:
@@ -387,6 +387,14 @@ def swiglu_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
 # `linear_swiglu` and `linear_rope_store`).
 RESIDUAL_NORM_MAX_ROWS = 16
 RESIDUAL_NORM_MAX_PARTS = 512
+# The few-row kernels with their fused epilogues take up to 16 rows, but from 13 rows on the 64-row tiles
+# with K in parts (and the kernels that add the parts up doing the norm, the rotation and the page
+# write) are faster: parts ask `few_rows_preferred` beside the `*_takes` of the few-row kernels.
+FEW_ROWS_PREFERRED = 12
+
+
+def few_rows_preferred(m: int) -> bool:
+    return m <= FEW_ROWS_PREFERRED
 
 
 class RowScale:

@@ -158,6 +158,7 @@ class _Lender:
     (128, 3584, 18944, torch.float32, False, True),      # more rows, but few tiles over a long K: parts again
     (200, 300, 4096, torch.bfloat16, True, False),
     (500, 1000, 1024, torch.float32, True, False),       # 32 tiles, two parts
+    (13, 3584, 3584, torch.float32, True, True),         # the fewest rows that take the tiles with K in parts
     (50, 4608, 3584, torch.bfloat16, True, False),       # 36 tiles in 7 parts: not whole eighths, the XCDs share one sequence
     (384, 3584, 2048, torch.float32, False, True),       # 84 tiles in 3 parts, three rows of tiles
     (130, 2048, 1536, torch.float32, True, True),        # 32 tiles in 3 parts: an eighth of the tiles each, part by part
@@ -191,6 +192,8 @@ def test_linear_with_k_in_parts(ops, m, n, k, out_dtype, bias, acc):
     (200, 300, 4096, True, True),        # more than 64 rows, few tiles
     (64, 37000, 64, False, False),       # no cut along K: nothing is done
     (8, 200, 1024, False, False),        # few rows: another kernel's business
+    (12, 3584, 3584, False, False),      # the most rows of that kernel's
+    (13, 3584, 3584, True, True),        # from here on: tiles with K in parts
 ])
 def test_linear_into_the_residual_sum_with_its_norm(ops, m, n, k, bias, taken):
     g = torch.Generator().manual_seed(19)
@@ -223,7 +226,8 @@ def test_linear_into_the_residual_sum_with_its_norm(ops, m, n, k, bias, taken):
 
 @pytest.mark.parametrize("m,n,k", [
     (8, 200, 96),                # few rows: the decode kernel
-    (40, 20000, 128),            # 33 to 64 rows: tiles of 64 rows
+    (13, 9500, 128),             # 13 to 64 rows: tiles of 64 rows
+    (40, 20000, 128),
     (64, 9500, 192),
     (50, 18944, 128),            # tiles of 64 x 192: the gates in one wave, the ups in the wave beside it
     (33, 12300, 192),            # the same with a ragged last tile
@@ -636,6 +640,7 @@ def test_rope_kv_store_and_plain_store(ops, dtype, dh, pad):
 @pytest.mark.parametrize("t,nh,nkv,dh,k,bias", [
     (64, 28, 4, 128, 3584, True),       # a decoding batch of 64 at the 7B layer sizes
     (33, 12, 2, 128, 1536, True),
+    (13, 28, 4, 128, 3584, True),       # the fewest rows that are cut along K
     (40, 6, 2, 64, 1280, False),
     (100, 28, 4, 128, 3584, True),      # more than 64 rows: tiles of 128 rows, K still cut
     (200, 12, 2, 128, 1536, False),

@@ -143,6 +143,10 @@ def residual_norm_parts(n):
     return -(-n // (32 if n >= 8192 else 16))
 
 
+def few_rows_preferred(m):
+    return m <= 12
+
+
 def residual_norm_takes(m, n, k, w_dtype):
     return w_dtype is torch.bfloat16 and 0 < m <= 16 and k % 8 == 0 and residual_norm_parts(n) <= RESIDUAL_NORM_MAX_PARTS
 
@@ -206,7 +210,7 @@ def argmax_rows(logits, out):
 
 ALL = ["require_gpu", "embedding", "rmsnorm", "gather_rows", "cast", "swiglu", "rope_table",
        "rope_apply", "kv_store", "rope_kv_store", "linear", "linear_skinny", "swiglu_takes", "linear_swiglu", "rope_store_takes", "linear_rope_store", "linear_rope_store_parts", "check_attention_sizes",
-       "RowScale", "RESIDUAL_NORM_MAX_PARTS", "residual_norm_parts", "residual_norm_takes", "linear_residual_norm", "linear_then_norm",
+       "RowScale", "few_rows_preferred", "RESIDUAL_NORM_MAX_PARTS", "residual_norm_parts", "residual_norm_takes", "linear_residual_norm", "linear_then_norm",
        "paged_attention", "argmax_rows"]
 
 
