@@ -56,7 +56,7 @@ class Engine:
     def __init__(self, spec: ModelSpec, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  max_seqs: int = 64, page_order_seed: Optional[int] = None,
-                 config: Any = None, use_graphs: bool = True):
+                 config: Any = None, use_graphs: bool = True, graph_after: int = 4):
         self.spec = spec
         self.config = config
         self.rt = Runtime(torch.device(device), parse_dtype(dtype))
@@ -80,6 +80,11 @@ class Engine:
         # decode steps (every request brings one token) are recorded as HIP graphs, one per batch
         # shape, and replayed: a step is some hundred small launches otherwise
         self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda" and not profiler.enabled
+        # A decode step of a shape (requests, wanted rows, table widths) is recorded at its graph_after-th
+        # occurrence and replayed from then on; before that it runs eagerly.  Recording costs about as much
+        # as a few steps and drains the queue of work once: where requests come and go and a shape lasts
+        # a few steps, recording every shape at its second step costs more than replays give back.
+        self.graph_after = max(2, int(graph_after))
         self._trace = trace_enabled()
         self._graphs: Dict[Any, Any] = {}
         self._graph_generation = (-1, -1)
@@ -268,12 +273,13 @@ class Engine:
             if self._graph_generation != gen:
                 self._graphs.clear()              # a buffer moved: recorded addresses are stale
                 state = None
-            # the first step of a shape runs eagerly (it sizes the buffers), the second is recorded
+            # the first steps of a shape run eagerly (the first sizes the buffers), the graph_after-th is recorded
             logits = self.model.forward(ctx, self.cache)
             gen = (self.ws.generation, self._uploader.generation)
             self._graph_generation = gen
-            if state is None:
-                self._graphs[key] = ("seen",)
+            seen = 1 if state is None or state[0] != "seen" else state[1] + 1
+            if seen < self.graph_after:
+                self._graphs[key] = ("seen", seen)
                 return logits
             torch.cuda.synchronize(self.rt.device)
             ctx.forget_shared()                   # what the eager pass prepared must be prepared in the graph too

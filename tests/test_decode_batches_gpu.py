@@ -111,7 +111,7 @@ def _check(d, dt, page, toks, prompts, ref, n_live, graphs, budget, label, tol=N
     steps = batch_schedule(toks, prompts, budget)
     assert max(len(e) for e, _ in steps) >= n_live
     eng = Engine.from_dir(d, dtype=dt, device="cuda:0", page_size=page, max_seqs=n_live, page_order_seed=7,
-                          max_tokens=schedules.max_live_tokens(toks, steps, page), use_graphs=graphs)
+                          max_tokens=schedules.max_live_tokens(toks, steps, page), use_graphs=graphs, graph_after=2)
     out = schedules.run(eng, toks, steps)
     eng.cache.check_invariants()
     assert all(f == g.pool.capacity for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
