@@ -495,6 +495,23 @@ def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
 
 
+@pytest.mark.parametrize("far", [3, 1000, 1999])
+def test_a_far_key_stands_out_in_a_decode_batch_of_unequal_contexts(ops, far):
+    # contexts of 2,000 to 5,000 keys: the batch gets one run length and a list of its runs; one key of every
+    # request (in its first run or a later one) takes nearly all of the weight
+    rng = np.random.default_rng(9)
+    segs = [(int(c), 1) for c in rng.integers(2000, 5000, 24)] + [(5000, 1), (2000, 1)]
+    from litinfer_amd.kernels.ops import _ragged_splits, decode_splits
+    class _M: pass
+    m = _M()
+    m.host_q_len = np.ones(len(segs), dtype=np.int32)
+    m.host_ctx_len = np.array([c for c, _ in segs], dtype=np.int32)
+    planned = decode_splits(len(segs) * 2, 5000, 1024)
+    assert _ragged_splits(planned, m, 0) > planned                 # the case is what it says
+    got, ref = _paged_case(ops, torch.bfloat16, segs, 12, 2, 128, 16, 0, seed=43, scale_one=far, ws=_Lender())
+    assert rel(got, ref) < 8e-3
+
+
 @pytest.mark.parametrize("window", [0, 900])
 def test_decode_run_length_of_a_batch_with_unequal_contexts(ops, window):
     # the run length chosen on the device against the same search written out, for contexts from 3 to 5,000
