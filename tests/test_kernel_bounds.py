@@ -5,11 +5,19 @@ import numpy as np
 from litinfer_amd.kernels import ops
 
 
-def pages_touched_by_a_split(p, window, nsplit, page_size, split):
-    """As paged_attention_decode_mfma_kernel cuts the keys of the query at position p."""
+def pages_touched_by_a_split(p, window, nsplit, page_size, split, given=None, max_blocks=None):
+    """As paged_attention_decode_mfma_kernel cuts the keys of the query at position p; `given`: the run
+    length a batch of unequal contexts brings (never shorter than this token needs, never longer than
+    the table's width would need)."""
     lo = p - window + 1 if window > 0 and p - window + 1 > 0 else 0
     nkeys = p - lo + 1
     per = (-(-nkeys // nsplit) + 31) & ~31
+    if given is not None:
+        widest = max_blocks * page_size
+        if 0 < window < widest:
+            widest = window
+        cap = (-(-widest // nsplit) + 31) & ~31
+        per = max(per, min((given + 31) & ~31, cap))
     k_begin = lo + split * per
     k_end = min(k_begin + per, p + 1)
     if k_begin >= k_end:
@@ -28,6 +36,9 @@ def test_decode_split_bound_covers_every_split_of_every_context():
         for ctx in {max_blocks * page, int(rng.integers(1, max_blocks * page + 1)), max(1, max_blocks * page - 31)}:
             worst = max(pages_touched_by_a_split(ctx - 1, window, nsplit, page, s) for s in range(nsplit))
             assert worst <= bound, (page, max_blocks, window, nsplit, ctx)
+            given = int(rng.integers(0, 2 * max_blocks * page + 64))
+            worst = max(pages_touched_by_a_split(ctx - 1, window, nsplit, page, s, given, max_blocks) for s in range(nsplit))
+            assert worst <= bound, (page, max_blocks, window, nsplit, ctx, given)
     # pages of one token: 64 splits of 1,024 keys fill the kernel's table exactly, one key more does not fit
     assert ops.decode_split_blocks(64 * 1024, 1, 0, 64) == ops.DECODE_TABLE_CAP
     assert ops.decode_split_blocks(64 * 1024 + 1, 1, 0, 64) > ops.DECODE_TABLE_CAP
