@@ -617,7 +617,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                                                              const bf16_t* __restrict__ w,
                                                              const float* __restrict__ bias,
                                                              TO* __restrict__ out, int M, int N, int K,
-                                                             int accumulate, int nsplit) {
+                                                             int accumulate, int nsplit,
+                                                             const float* __restrict__ row_parts, int nparts, float eps) {
+    // row_parts (SwiGLU tiles of 64 rows, up to 16 rows of x): x is the xg of li_linear_residual_norm and these
+    // are its sq_parts; every row's sums are scaled by 1 / sqrt(sum of the row's parts / K + eps) before the
+    // activation, which makes the result that of the RMS norm (the factor of a row does not depend on k).
     // nsplit > 1: a block multiplies one of nsplit parts of K, the y-th, and writes its sums to the y-th
     // [M, N] matrix behind `out` (float, no bias, no accumulation); splitk_reduce_kernel adds them
     // WLM: waves along the rows of the tile, 2 (two by two) or 4 (each wave 32-row bands over all columns:
@@ -640,6 +644,24 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     int mt, nt, split;
     if (!TileOrder(mtiles).tile(blockIdx.x, mtiles, ntiles, nsplit, mt, nt, split)) return;
     const int m0 = mt * BM, n0 = nt * BN;
+    constexpr bool ROWSCALE = SWIGLU && BM == 64;
+    // The shares of the rows' sums of squares are asked for now, all at once and never conditional (a share
+    // past the last reads the last and is not added), before the first loads of the main loop: a wave's loads
+    // retire in order, so they have arrived when the first stage has, and the waits placed by hand below
+    // still count the main loop's loads only.  They are added up behind the main loop.
+    constexpr int RS_PER = ROWSCALE ? 32 : 1;          // shares a thread adds: 512 at most, 16 threads a row
+    [[maybe_unused]] float rs_part[RS_PER];
+    if constexpr (ROWSCALE) {
+        if (row_parts) {
+            const int r = threadIdx.x & 15, g = threadIdx.x >> 4;
+#pragma unroll
+            for (int i = 0; i < RS_PER; ++i) {
+                const int p = g + 16 * i;
+                rs_part[i] = 0.f;
+                if (16 * i < nparts) rs_part[i] = row_parts[(size_t)(p < nparts ? p : nparts - 1) * 16 + r];      // (the same for all lanes)
+            }
+        }
+    }
     floatx16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -806,6 +828,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 #undef LI_FREAD
 #undef LI_WAIT_YOUNGER
     __syncthreads();                               // the main loop's LDS is free now
+    [[maybe_unused]] float* row_inv = nullptr;
+    if constexpr (ROWSCALE) {
+        // the rows' factors, in the order of additions of the few-row kernel with four waves: thread t adds the
+        // shares t / 16, t / 16 + 16, ... of row t % 16, thread r < 16 the 16 sums of row r
+        __shared__ float inv_s[16], part_s[16][16];
+        row_inv = inv_s;
+        if (row_parts) {
+            const int r = threadIdx.x & 15, g = threadIdx.x >> 4;
+            float mine = 0.f;
+#pragma unroll
+            for (int i = 0; i < RS_PER; ++i) mine += (g + 16 * i < nparts) ? rs_part[i] : 0.f;
+            part_s[g][r] = mine;
+            __syncthreads();
+            if (threadIdx.x < 16) {
+                float sq = part_s[0][threadIdx.x];
+#pragma unroll
+                for (int q = 1; q < 16; ++q) sq += part_s[q][threadIdx.x];
+                inv_s[threadIdx.x] = 1.0f / sqrtf(sq / (float)K + eps);
+            }
+            __syncthreads();
+        }
+    }
     if constexpr (SWSPLIT) {
         // every wave leaves its sums in its band; of two waves side by side the first then takes rows 0 .. 15
         // of the 32 and the second rows 16 .. 31: gates from the first wave's band, ups from the second's
@@ -837,8 +881,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                 const float* gs = &gband[(16 * (wave & 1) + rr) * ES + ecol];
                 const float* us = &uband[(16 * (wave & 1) + rr) * ES + ecol];
                 float v[8];
+                float f = 1.0f;
+                if constexpr (ROWSCALE) f = row_parts ? row_inv[row & 15] : 1.0f;      // (row_parts: M <= 16, so row < 16 here)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = us[e] * (gs[e] / (1.0f + expf(-gs[e])));
+                for (int e = 0; e < 8; ++e) { const float gv = gs[e] * f; v[e] = (us[e] * f) * (gv / (1.0f + expf(-gv))); }
                 const size_t o_idx = (size_t)row * NO + col;
                 if (col + 8 <= NO && (NO % 8) == 0) {
                     chunk16 o;
@@ -871,7 +917,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
             for (int j = 0; j < TN; j += 2)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float gv = acc[i][j][r], uv = acc[i][j + 1][r];
+                    float gv = acc[i][j][r], uv = acc[i][j + 1][r];
+                    if constexpr (ROWSCALE) {
+                        if (row_parts) {                 // (M <= 16: only the tile's first 16 rows are written)
+                            const float f = row_inv[(wm + 32 * i + 8 * (r >> 2) + crow + (r & 3)) & 15];
+                            gv *= f;
+                            uv *= f;
+                        }
+                    }
                     band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 16 * j + ccol] = uv * (gv / (1.0f + expf(-gv)));
                 }
         } else {
@@ -923,7 +976,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
 
 template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO, int WLM = 2>
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
-                      int accumulate, hipStream_t stream, int nsplit = 1) {
+                      int accumulate, hipStream_t stream, int nsplit = 1, const float* row_parts = nullptr,
+                      int nparts = 0, float eps = 0.f) {
+    if (row_parts && !(SWIGLU && BM == 64 && M <= 16 && nparts > 0)) return LI_ERR_SIZE;
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
     if (nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
     const long blocks = TileOrder::blocks(mtiles, ntiles, nsplit);
@@ -940,7 +995,7 @@ static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* o
             return LI_ERR_LAUNCH;
         configured = true;
     }
-    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO, WLM><<<(unsigned)blocks, 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate, nsplit);
+    gemm_bf16_dma_kernel<BM, BN, BK, NSTAGE, SWIGLU, TO, WLM><<<(unsigned)blocks, 256, lds_bytes, stream>>>(x, w, bias, out, M, N, K, accumulate, nsplit, row_parts, nparts, eps);
     return li_launch_status();
 }
 
@@ -1477,21 +1532,26 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
 // Measured on the 7B layer sizes, a decode step of 17 / 24 / 32 requests: 4.57 / 4.95 / 5.33 ms
 // against 4.90 / 5.33 / 5.84 ms with the few-row kernel up to 32 rows.  Returns -1 when it does
 // not take the call.
-// The few-row kernel takes up to 16 rows with its fused epilogues, but from 13 rows on the tiles with K in
-// parts are faster (7B layer sizes, a decode step of 12 / 14 / 16 requests: 4.08 / 4.27 / 4.43 ms with the
-// few-row kernels, 4.10 / 4.17 / 4.28 ms with the tiles): callers are told to prefer the tiles from there.
+// The few-row kernel takes up to 16 rows with its fused epilogues.  Up to 12 rows it is the faster one for
+// every product but the largest gate/up matrices (li_linear_swiglu); at 13 to 16 rows the tiles with K in
+// parts are faster where the matrix is large (at 13 rows the 7B's way back from the feed-forward, 136 MB:
+// 29.8 us with its adding-up kernel against 33.5 us; its q/k/v, 33 MB: 11.8 against 9.2 us; the whole step
+// of 16 requests at the 7B sizes 4.28 against 4.43 ms, at the 1.5B sizes 2.22 against 1.94 ms).
 #define FEW_ROWS_FUSED 12
-extern "C" int li_few_rows_fused() { return FEW_ROWS_FUSED; }
+#define FEW_ROWS_LARGE_BYTES (100l << 20)
+#define SWIGLU_TILES_BYTES (400l << 20)      // a gate/up matrix from which on tiles of 64 rows beat the few-row kernel at any rows
+extern "C" int li_few_rows_preferred(int M, long N, long K) {
+    return M <= FEW_ROWS_FUSED || (M <= 16 && N * K * 2 < FEW_ROWS_LARGE_BYTES);
+}
 
-static bool mid_rows_take(int M, int K) {
-    (void)K;
-    return M > FEW_ROWS_FUSED && M <= 64;
+static bool mid_rows_take(int M, int N, int K) {
+    return !li_few_rows_preferred(M, N, K) && M <= 64;
 }
 
 static int linear_mid_rows(const bf16_t* x, const bf16_t* w, const float* bias, void* out, int M, int N,
                            int K, int out_dtype, int accumulate, void* work, long work_bytes,
                            hipStream_t stream) {
-    if (!mid_rows_take(M, K) || K % 64 || (out_dtype != LI_F32 && out_dtype != LI_BF16)) return -1;
+    if (!mid_rows_take(M, N, K) || K % 64 || (out_dtype != LI_F32 && out_dtype != LI_BF16)) return -1;
 #define LI_MID(BN, NS, TO, dst, b, acc, split) launch_dma<64, BN, 64, NS, false, TO>(x, w, b, (TO*)(dst), M, N, K, acc, stream, split)
     if ((N + 255) / 256 >= 128)
         return out_dtype == LI_F32 ? LI_MID(256, 3, float, out, bias, accumulate, 1) : LI_MID(256, 3, bf16_t, out, bias, accumulate, 1);
@@ -1559,7 +1619,7 @@ extern "C" int li_linear_rope_store_parts(const void* x, const void* w, const fl
         (long)(nh + 2 * nkv) * dh > 0x7fffffffL)
         return LI_ERR_SIZE;
     const int N = (nh + 2 * nkv) * dh;
-    if (M <= FEW_ROWS_FUSED || K % 64) return -1;
+    if (li_few_rows_preferred(M, N, K) || K % 64) return -1;
     const long need = li_linear_work_bytes(M, N, K, LI_BF16);            // (0 where li_linear would not cut this product)
     if (need <= 0 || !work || work_bytes < need) return -1;
     const size_t mn = (size_t)M * N;
@@ -1609,8 +1669,7 @@ static int split_parts_many_rows(int M, int N, int K) {
 
 // Bytes of workspace with which li_linear cuts this product along K (0: it would not).
 extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
-    if (in_dtype != LI_BF16 || M <= FEW_ROWS_FUSED || N <= 0 || K <= 0 || K % 64) return 0;
-    if (M <= 64 && !mid_rows_take(M, K)) return 0;
+    if (in_dtype != LI_BF16 || N <= 0 || K <= 0 || K % 64 || li_few_rows_preferred(M, N, K)) return 0;
     int nsplit = 1;
     if (M <= 64) {
         const int tiles = (N + 127) / 128;
@@ -1632,7 +1691,7 @@ extern "C" long li_linear_work_bytes(int M, int N, int K, int in_dtype) {
 extern "C" int li_linear_then_norm(const void* x, const void* w, const float* bias, float* out, int M, int N, int K,
                                    void* work, long work_bytes, const float* gamma, float eps, void* xn,
                                    int xn_dtype, hipStream_t stream) {
-    if (M <= FEW_ROWS_FUSED || N <= 0 || K <= 0 || (K % 64) || !gamma || !xn || eps < 0.f) return -1;
+    if (N <= 0 || K <= 0 || (K % 64) || li_few_rows_preferred(M, N, K) || !gamma || !xn || eps < 0.f) return -1;
     if (N > REDUCE_NORM_NT * REDUCE_NORM_PER || (xn_dtype != LI_BF16 && xn_dtype != LI_F32)) return -1;
     const long need = li_linear_work_bytes(M, N, K, LI_BF16);
     if (need <= 0 || !work || work_bytes < need) return -1;
@@ -1745,17 +1804,15 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
                                 const float* row_parts, int nparts, float eps, hipStream_t stream) {
     if (M <= 0 || I <= 0 || K <= 0 || I > 0x3fffffff) return LI_ERR_SIZE;
     const int N = 2 * I;
-    if (row_parts) {
-        if (M > 16 || (K % 8) || nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f) return LI_ERR_SIZE;
-        SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, nullptr, out, M, I, K, 0,
-                     nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, row_parts, nparts, eps};
-        launch_skinny<true, bf16_t>(a, stream);
-        return li_launch_status();
-    }
-    if (M > FEW_ROWS_FUSED && M <= 64 && K % 64 == 0) {                  // see linear_mid_rows
-        // tiles of 64 rows: the width with the least estimated time that gives the chip enough tiles (a
-        // product of few rows waits for w, and a compute unit takes in only so much: more units, each
-        // with a narrower tile, stream more, until the tiles no longer fit one round)
+    if (row_parts && (M > 16 || (K % 8) || nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f)) return LI_ERR_SIZE;
+    // Up to 64 rows the product waits for w.  From 17 rows on (more than the few-row kernel's fused form takes)
+    // it goes to tiles of 64 rows if the matrix has tiles enough to fill the chip: the width with the least
+    // estimated time (a compute unit takes in only so much: more units, each with a narrower tile, stream
+    // more, until the tiles no longer fit one round).  The largest matrices take the tiles at any number of
+    // rows: their loads straight into LDS stream w faster than the few-row kernel does (32B sizes, 566 MB, 1
+    // and 8 rows: 104 against 114 and 124 us; at the 7B's 272 MB and the 14B's 283 MB there is nothing in it:
+    // the rows' factors cost the tile kernel 2 us).
+    if (M <= 64 && K % 64 == 0 && (M > 16 || (long)N * K * 2 >= SWIGLU_TILES_BYTES)) {
         const int widths[3] = {256, 192, 128};
         int pick = -1;
         double best = 0.0;
@@ -1764,9 +1821,17 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
             const double c = tile_cost(64, widths[i], 1.0, M, N, K);
             if (pick < 0 || c < best) { best = c; pick = i; }
         }
-        if (pick == 0) return launch_dma<64, 256, 64, 3, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
-        if (pick == 1) return launch_dma<64, 192, 64, 4, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
-        if (pick == 2) return launch_dma<64, 128, 64, 4, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream);
+#define LI_SW64(BN, NS) launch_dma<64, BN, 64, NS, true, bf16_t>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream, 1, row_parts, nparts, eps)
+        if (pick == 0) return LI_SW64(256, 3);
+        if (pick == 1) return LI_SW64(192, 4);
+        if (pick == 2) return LI_SW64(128, 4);
+#undef LI_SW64
+    }
+    if (row_parts) {
+        SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, nullptr, out, M, I, K, 0,
+                     nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, nullptr, nullptr, nullptr, row_parts, nparts, eps};
+        launch_skinny<true, bf16_t>(a, stream);
+        return li_launch_status();
     }
     if (M <= 64) return li_linear_skinny(x, w, nullptr, out, M, I, K, LI_BF16, 0, 1, stream);
     if (K % 64) return LI_ERR_SIZE;

@@ -336,7 +336,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
          "linear: bias must be float32 [N]")
     if m:
         work, work_bytes = 0, 0
-        if ws is not None and x.dtype is torch.bfloat16 and m > FEW_ROWS_PREFERRED:
+        if ws is not None and x.dtype is torch.bfloat16 and not few_rows_preferred(m, n, k):
             # few rows over a long k and few columns: the library cuts k into parts if it is lent room for their sums
             need = _work_bytes(m, n, k, _DT[x.dtype])
             if need:
@@ -387,14 +387,20 @@ def swiglu_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
 # `linear_swiglu` and `linear_rope_store`).
 RESIDUAL_NORM_MAX_ROWS = 16
 RESIDUAL_NORM_MAX_PARTS = 512
-# The few-row kernels with their fused epilogues take up to 16 rows, but from 13 rows on the 64-row tiles
-# with K in parts (and the kernels that add the parts up doing the norm, the rotation and the page
-# write) are faster: parts ask `few_rows_preferred` beside the `*_takes` of the few-row kernels.
-FEW_ROWS_PREFERRED = 12
+# The few-row kernels with their fused epilogues take up to 16 rows; at 13 to 16 rows the 64-row tiles with
+# K in parts (and the kernels that add the parts up doing the norm, the rotation and the page write) are
+# faster where the matrix is large.  Parts ask `few_rows_preferred` beside the `*_takes` of the few-row
+# kernels; the kernel library holds the rule (its own entry points decide by it too).
 
 
-def few_rows_preferred(m: int) -> bool:
-    return m <= FEW_ROWS_PREFERRED
+def few_rows_preferred(m: int, n: int, k: int) -> bool:
+    """Whether m rows against a matrix [n, k] should take the few-row kernels."""
+    f = _fn_cache.get(("gemm", "li_few_rows_preferred"))
+    if f is None:
+        f = build.load("gemm").li_few_rows_preferred
+        f.argtypes, f.restype = [c_int, c_long, c_long], c_int
+        _fn_cache[("gemm", "li_few_rows_preferred")] = f
+    return bool(f(int(m), int(n), int(k)))
 
 
 class RowScale:

@@ -26,7 +26,8 @@ class Linear:
     def takes_scaling(self, x: torch.Tensor, out: torch.Tensor) -> bool:
         """Whether out += x W^T + b can also leave out times a norm's weights and the
         shares of the rows' sums of squares (few rows, bfloat16 operands)."""
-        return (x.dtype is torch.bfloat16 and out.dtype is torch.float32 and ops.few_rows_preferred(x.shape[0])
+        return (x.dtype is torch.bfloat16 and out.dtype is torch.float32
+                and ops.few_rows_preferred(x.shape[0], self.out_features, self.in_features)
                 and ops.residual_norm_takes(x.shape[0], self.out_features, self.in_features, self.weight.dtype))
 
     def add_with_scaling(self, x: torch.Tensor, out: torch.Tensor, scaling, rows: torch.Tensor, ws):

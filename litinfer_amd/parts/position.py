@@ -85,7 +85,7 @@ class RopeNeox(Position):
         # few rows (decoding): the rotation and the page write are the projection's epilogue
         if not (cache.owned and xn.dtype is ops.bfloat16 and proj.weight.dtype is ops.bfloat16):
             return False
-        if not (ops.few_rows_preferred(xn.shape[0])
+        if not (ops.few_rows_preferred(xn.shape[0], proj.out_features, proj.in_features)
                 and ops.rope_store_takes(xn.shape[0], proj.in_features, proj.weight.dtype, head_dim, self.rotary_dim)):
             # more rows: where the projection is cut along K anyway, the kernel that adds the parts up rotates and stores
             if row_scale is not None or self.rotary_dim != head_dim:

@@ -158,7 +158,8 @@ class _Lender:
     (128, 3584, 18944, torch.float32, False, True),      # more rows, but few tiles over a long K: parts again
     (200, 300, 4096, torch.bfloat16, True, False),
     (500, 1000, 1024, torch.float32, True, False),       # 32 tiles, two parts
-    (13, 3584, 3584, torch.float32, True, True),         # the fewest rows that take the tiles with K in parts
+    (13, 3584, 18944, torch.float32, True, True),        # the fewest rows that take the tiles with K in parts (a large matrix)
+    (16, 3584, 3584, torch.float32, True, True),         # a small one at 16 rows: the few-row kernel
     (50, 4608, 3584, torch.bfloat16, True, False),       # 36 tiles in 7 parts: not whole eighths, the XCDs share one sequence
     (384, 3584, 2048, torch.float32, False, True),       # 84 tiles in 3 parts, three rows of tiles
     (130, 2048, 1536, torch.float32, True, True),        # 32 tiles in 3 parts: an eighth of the tiles each, part by part
@@ -192,8 +193,9 @@ def test_linear_with_k_in_parts(ops, m, n, k, out_dtype, bias, acc):
     (200, 300, 4096, True, True),        # more than 64 rows, few tiles
     (64, 37000, 64, False, False),       # no cut along K: nothing is done
     (8, 200, 1024, False, False),        # few rows: another kernel's business
-    (12, 3584, 3584, False, False),      # the most rows of that kernel's
-    (13, 3584, 3584, True, True),        # from here on: tiles with K in parts
+    (12, 3584, 18944, False, False),     # the most rows of that kernel's whatever the matrix
+    (13, 3584, 3584, True, False),       # 13 to 16 rows against a small matrix: still the few-row kernel
+    (13, 3584, 18944, True, True),       # against a large one (136 MB): tiles with K in parts
 ])
 def test_linear_into_the_residual_sum_with_its_norm(ops, m, n, k, bias, taken):
     g = torch.Generator().manual_seed(19)
@@ -266,6 +268,8 @@ def test_linear_with_swiglu_epilogue(ops, m, n, k):
 
 @pytest.mark.parametrize("m,n,kprev,inter,eps", [
     (8, 3584, 512, 1024, 1e-6),      # a decoding step at the 7B width
+    (8, 5120, 256, 27648, 1e-6),     # the 32B's gate/up matrix (566 MB): tiles of 64 x 256 scale the rows
+    (16, 8192, 128, 18944, 1e-5),    # 620 MB: tiles of 64 x 192, gates and ups in two waves
     (1, 40, 8, 24, 1e-5),
     (16, 8200, 64, 48, 1e-5),        # a width from which the product before takes 32 columns a block; ragged
     (5, 200, 136, 301, 0.1),         # a ragged last block of 16 columns; an eps that counts
@@ -657,7 +661,7 @@ def test_rope_kv_store_and_plain_store(ops, dtype, dh, pad):
 @pytest.mark.parametrize("t,nh,nkv,dh,k,bias", [
     (64, 28, 4, 128, 3584, True),       # a decoding batch of 64 at the 7B layer sizes
     (33, 12, 2, 128, 1536, True),
-    (13, 28, 4, 128, 3584, True),       # the fewest rows that are cut along K
+    (13, 64, 8, 128, 8192, True),       # the fewest rows that are cut along K, against a large matrix (168 MB)
     (40, 6, 2, 64, 1280, False),
     (100, 28, 4, 128, 3584, True),      # more than 64 rows: tiles of 128 rows, K still cut
     (200, 12, 2, 128, 1536, False),

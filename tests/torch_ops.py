@@ -143,8 +143,8 @@ def residual_norm_parts(n):
     return -(-n // (32 if n >= 8192 else 16))
 
 
-def few_rows_preferred(m):
-    return m <= 12
+def few_rows_preferred(m, n, k):
+    return m <= 12 or (m <= 16 and n * k * 2 < (100 << 20))
 
 
 def residual_norm_takes(m, n, k, w_dtype):
