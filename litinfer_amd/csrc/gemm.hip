@@ -1539,7 +1539,7 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
 // of 16 requests at the 7B sizes 4.28 against 4.43 ms, at the 1.5B sizes 2.22 against 1.94 ms).
 #define FEW_ROWS_FUSED 12
 #define FEW_ROWS_LARGE_BYTES (100l << 20)
-#define SWIGLU_TILES_BYTES (400l << 20)      // a gate/up matrix from which on tiles of 64 rows beat the few-row kernel at any rows
+#define SWIGLU_TILES_BYTES (400l << 20)      // (see li_linear_swiglu)
 extern "C" int li_few_rows_preferred(int M, long N, long K) {
     return M <= FEW_ROWS_FUSED || (M <= 16 && N * K * 2 < FEW_ROWS_LARGE_BYTES);
 }
@@ -1808,11 +1808,13 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     // Up to 64 rows the product waits for w.  From 17 rows on (more than the few-row kernel's fused form takes)
     // it goes to tiles of 64 rows if the matrix has tiles enough to fill the chip: the width with the least
     // estimated time (a compute unit takes in only so much: more units, each with a narrower tile, stream
-    // more, until the tiles no longer fit one round).  The largest matrices take the tiles at any number of
-    // rows: their loads straight into LDS stream w faster than the few-row kernel does (32B sizes, 566 MB, 1
-    // and 8 rows: 104 against 114 and 124 us; at the 7B's 272 MB and the 14B's 283 MB there is nothing in it:
-    // the rows' factors cost the tile kernel 2 us).
-    if (M <= 64 && K % 64 == 0 && (M > 16 || (long)N * K * 2 >= SWIGLU_TILES_BYTES)) {
+    // more, until the tiles no longer fit one round).  Below that the few-row kernel, but for one corner that
+    // was measured: a very large matrix of short rows (the 32B sizes, 55,296 x 5,120: the few-row kernel
+    // streams it at 4.6-4.9 TB/s, 115-124 us at 8 rows, the tiles at 5.5, 104 us with the rows' factors).
+    // Against long rows or smaller matrices the few-row kernel is as fast or faster (72B sizes, 59,136 x
+    // 8,192: 173 against 181 us; 73,728 x 4,096: 109 against 130 us; the 7B's and 14B's: the same).
+    const bool large_short_rows = (long)N * K * 2 >= SWIGLU_TILES_BYTES && K >= 4608 && K <= 6144;
+    if (M <= 64 && K % 64 == 0 && (M > 16 || large_short_rows)) {
         const int widths[3] = {256, 192, 128};
         int pick = -1;
         double best = 0.0;
