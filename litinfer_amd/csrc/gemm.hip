@@ -1805,7 +1805,8 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     if (M <= 0 || I <= 0 || K <= 0 || I > 0x3fffffff) return LI_ERR_SIZE;
     const int N = 2 * I;
     if (row_parts && (M > 16 || (K % 8) || nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f)) return LI_ERR_SIZE;
-    // Up to 64 rows the product waits for w.  From 17 rows on (more than the few-row kernel's fused form takes)
+    // Up to 64 rows the product waits for w.  From 17 rows on (more than the few-row kernel's fused form takes),
+    // and from 13 on where the matrix is large (li_few_rows_preferred: the 7B's at 16 rows 51.8 against 59.6 us),
     // it goes to tiles of 64 rows if the matrix has tiles enough to fill the chip: the width with the least
     // estimated time (a compute unit takes in only so much: more units, each with a narrower tile, stream
     // more, until the tiles no longer fit one round).  Below that the few-row kernel, but for one corner that
@@ -1814,7 +1815,7 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     // Against long rows or smaller matrices the few-row kernel is as fast or faster (72B sizes, 59,136 x
     // 8,192: 173 against 181 us; 73,728 x 4,096: 109 against 130 us; the 7B's and 14B's: the same).
     const bool large_short_rows = (long)N * K * 2 >= SWIGLU_TILES_BYTES && K >= 4608 && K <= 6144;
-    if (M <= 64 && K % 64 == 0 && (M > 16 || large_short_rows)) {
+    if (M <= 64 && K % 64 == 0 && (!li_few_rows_preferred(M, N, K) || large_short_rows)) {
         const int widths[3] = {256, 192, 128};
         int pick = -1;
         double best = 0.0;
