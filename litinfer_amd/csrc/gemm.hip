@@ -1539,7 +1539,7 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
 // of 16 requests at the 7B sizes 4.28 against 4.43 ms, at the 1.5B sizes 2.22 against 1.94 ms).
 #define FEW_ROWS_FUSED 12
 #define FEW_ROWS_LARGE_BYTES (100l << 20)
-#define SWIGLU_TILES_BYTES (400l << 20)      // (see li_linear_swiglu)
+#define SWIGLU_TILES_BYTES (160l << 20)      // (see li_linear_swiglu)
 extern "C" int li_few_rows_preferred(int M, long N, long K) {
     return M <= FEW_ROWS_FUSED || (M <= 16 && N * K * 2 < FEW_ROWS_LARGE_BYTES);
 }
@@ -1809,18 +1809,27 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     // and from 13 on where the matrix is large (li_few_rows_preferred: the 7B's at 16 rows 51.8 against 59.6 us),
     // it goes to tiles of 64 rows if the matrix has tiles enough to fill the chip: the width with the least
     // estimated time (a compute unit takes in only so much: more units, each with a narrower tile, stream
-    // more, until the tiles no longer fit one round).  Below that the few-row kernel, but for one corner that
-    // was measured: a very large matrix of short rows (the 32B sizes, 55,296 x 5,120: the few-row kernel
-    // streams it at 4.6-4.9 TB/s, 115-124 us at 8 rows, the tiles at 5.5, 104 us with the rows' factors).
-    // Against long rows or smaller matrices the few-row kernel is as fast or faster (72B sizes, 59,136 x
-    // 8,192: 173 against 181 us; 73,728 x 4,096: 109 against 130 us; the 7B's and 14B's: the same).
-    const bool large_short_rows = (long)N * K * 2 >= SWIGLU_TILES_BYTES && K >= 4608 && K <= 6144;
-    if (M <= 64 && K % 64 == 0 && (!li_few_rows_preferred(M, N, K) || large_short_rows)) {
+    // more, until the tiles no longer fit one round).
+    // Below that the few-row kernel, but for a large matrix of rows that are not too long whose tiles fit ONE
+    // round over the compute units: there the tiles' loads straight into LDS stream w at the rate of a kernel
+    // that only reads (7B sizes, 272 MB: 48.8 us; the few-row kernel 49 to 54 us at 1 to 12 rows), and the
+    // rows' factors of a fused RMS norm are applied in the tile kernel's epilogue.  Measured on one machine in
+    // turn, whole decode steps: 7B sizes 3.34 -> 3.32 ms at 1 request, 3.72 -> 3.62 at 8, 4.06 -> 3.90 at 12;
+    // 14B 6.5 -> 6.57 / 7.66 -> 7.45 / 8.49 -> 8.09; 32B (566 MB) 13.98 -> 13.05 at 1.  Not taken where it
+    // loses: small matrices (3B's 90 MB, 1.5B's 55 MB: steps 4-5 % longer), rows of 8,192 (72B sizes 173
+    // against 181 us; 28,672 x 8,192: 86 against 96), or no width whose tiles fit one round (73,728 x 4,096:
+    // 109 against 130 us).
+    const int cu = compute_units();
+    const bool few = li_few_rows_preferred(M, N, K);
+    const bool stream_tiles = (long)N * K * 2 >= SWIGLU_TILES_BYTES && K <= 6144;
+    if (M <= 64 && K % 64 == 0 && (!few || stream_tiles)) {
         const int widths[3] = {256, 192, 128};
         int pick = -1;
         double best = 0.0;
         for (int i = 0; i < 3; ++i) {
-            if ((N + widths[i] - 1) / widths[i] < 128) continue;         // too few tiles: the few-row kernel
+            const int tiles = (N + widths[i] - 1) / widths[i];
+            if (tiles < 128) continue;                                   // too few tiles: the few-row kernel
+            if (few && tiles > cu) continue;                             // (few rows: one round only, see above)
             const double c = tile_cost(64, widths[i], 1.0, M, N, K);
             if (pick < 0 || c < best) { best = c; pick = i; }
         }

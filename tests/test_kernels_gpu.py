@@ -269,6 +269,7 @@ def test_linear_with_swiglu_epilogue(ops, m, n, k):
 @pytest.mark.parametrize("m,n,kprev,inter,eps", [
     (8, 3584, 512, 1024, 1e-6),      # a decoding step at the 7B width
     (8, 5120, 256, 27648, 1e-6),     # the 32B's gate/up matrix (566 MB): tiles of 64 x 256 scale the rows
+    (3, 3584, 512, 18944, 1e-6),     # the 7B's (272 MB): tiles of 64 x 192
     (16, 5120, 128, 20480, 1e-5),    # 419 MB: tiles of 64 x 192, gates and ups in two waves
     (1, 40, 8, 24, 1e-5),
     (16, 8200, 64, 48, 1e-5),        # a width from which the product before takes 32 columns a block; ragged
