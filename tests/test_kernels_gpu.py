@@ -366,6 +366,17 @@ def test_linear_rows_do_not_depend_on_the_batch(ops, dtype):
         assert rel(part, full[rows].double().cpu().numpy()) < 4 * math.sqrt(264) * 2.0 ** -24
 
 
+def test_the_rule_for_few_rows_is_the_same_in_the_library_and_in_the_host_stand_in(ops):
+    # parts ask the kernel library which kernels few rows should take; the stand-in that the host-side tests
+    # run the parts with answers the same
+    import torch_ops
+    for m in (1, 8, 12, 13, 16, 17, 64, 65):
+        for n, k in ((1536, 1536), (3584, 18944), (18944, 3584), (4608, 3584), (5120, 27648), (10240, 8192), (14000, 3745)):
+            assert ops.few_rows_preferred(m, n, k) == torch_ops.few_rows_preferred(m, n, k), (m, n, k)
+    assert ops.few_rows_preferred(12, 3584, 18944) and not ops.few_rows_preferred(13, 3584, 18944)
+    assert ops.few_rows_preferred(16, 3584, 3584) and not ops.few_rows_preferred(17, 3584, 3584)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(2, 3), (33, 200), (512, 4096)])
 def test_swiglu(ops, dtype, shape):
