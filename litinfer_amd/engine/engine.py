@@ -56,10 +56,14 @@ class Engine:
     def __init__(self, spec: ModelSpec, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  max_seqs: int = 64, page_order_seed: Optional[int] = None,
-                 config: Any = None, use_graphs: bool = True, graph_after: int = 4):
+                 config: Any = None, use_graphs: bool = True, graph_after: int = 4,
+                 keep_stored_precision: bool = False):
+        """keep_stored_precision: with dtype bfloat16, leave matrices that the checkpoint stores in
+        32-bit or half precision in 32-bit (their products then run in the 32-bit kernels) instead of
+        rounding them once to bfloat16 when they are bound."""
         self.spec = spec
         self.config = config
-        self.rt = Runtime(torch.device(device), parse_dtype(dtype))
+        self.rt = Runtime(torch.device(device), parse_dtype(dtype), bool(keep_stored_precision))
         if self.rt.device.type == "cuda":
             from ..kernels import ops
             ops.require_gpu(self.rt.device)
@@ -105,7 +109,9 @@ class Engine:
     @classmethod
     def from_random(cls, config: Dict[str, Any], seed: int, **kw) -> "Engine":
         """Random weights drawn straight on the device (no files): for
-        measurements at sizes where writing a checkpoint first would only cost time."""
+        measurements at sizes where writing a checkpoint first would only cost time.
+        The numbers differ from those that `weights.write_random_model` writes for the
+        same seed: the device's and the host's random generators are two different ones."""
         arch = lookup(architecture_name(config))
         cfg = arch.config_from_dict(config)
         spec = arch.model_spec(cfg)

@@ -38,14 +38,15 @@ class CausalLM:
     def __init__(self, model_path, device: str = "cuda:0", quantize: Optional[str] = None, *,
                  dtype: str = "bfloat16", page_size: int = 16, num_pages: Optional[int] = None,
                  max_tokens: Optional[int] = None, max_seqs: int = 64, max_batch_tokens: int = 2048,
-                 chunk_size: int = 512, seed: int = 0, lookahead: bool = True, strict_weights: bool = False):
+                 chunk_size: int = 512, seed: int = 0, lookahead: bool = True, strict_weights: bool = False,
+                 keep_stored_precision: bool = False):
         if quantize is not None:
             raise NotImplementedError("quantized weights are not supported")
         self.model_path = Path(model_path)
         print(f"[litinfer_amd] loading {self.model_path} ({dtype}) ...", flush=True)
         self.engine = Engine.from_dir(self.model_path, dtype=dtype, device=device, page_size=page_size,
                                       num_pages=num_pages, max_tokens=max_tokens, max_seqs=max_seqs,
-                                      strict_weights=strict_weights)
+                                      strict_weights=strict_weights, keep_stored_precision=keep_stored_precision)
         self.meta = self.engine.config
         self.seed = int(seed)
         # lookahead: a step is started before the tokens of the one before have reached the host

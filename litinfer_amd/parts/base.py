@@ -25,7 +25,7 @@ Interfaces (T = tokens of the step, H = hidden size):
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, Optional, Tuple
 
 import torch
@@ -38,17 +38,28 @@ from ..weights.loader import ParamSpec
 class Runtime:
     """Where and in which precision a model runs.  `dtype` is the activation and
     matrix dtype: torch.bfloat16 (serving) or torch.float32 (everything in true
-    32-bit)."""
+    32-bit).  One dtype holds for every matrix of the model, whatever the checkpoint
+    stores them in, as the reference decides one dtype for the whole model and
+    converts every tensor to it (python/llaisys/models/qwen2.py:88-110, 253-264).
+    `keep_stored_precision` (off by default) leaves a matrix that is stored in 32-bit
+    (or in half precision, which is widened) in 32-bit inside the bfloat16 engine;
+    its products then run in the 32-bit kernels, slower and on twice the bytes."""
     device: torch.device
     dtype: torch.dtype
+    keep_stored_precision: bool = False
+    # stored dtype -> number of matrices that were rounded to bfloat16 when they were bound
+    rounded: Dict[str, int] = field(default_factory=dict, compare=False, hash=False)
 
     def matrix(self, t: torch.Tensor) -> torch.Tensor:
         """A stored matrix as this runtime multiplies with it.  In 32-bit mode
-        everything is widened (exactly); in bfloat16 mode a bfloat16 matrix stays
-        and a matrix stored in 32-bit stays 32-bit (its product then runs in
-        32-bit)."""
+        everything is widened (exactly).  In bfloat16 mode a matrix stored in
+        another precision is rounded once, to nearest even, to bfloat16, so that
+        every product takes the bfloat16 kernels (unless `keep_stored_precision`)."""
         if self.dtype is torch.float32:
             t = t.to(torch.float32)
+        elif t.dtype is not torch.bfloat16 and t.is_floating_point() and not self.keep_stored_precision:
+            self.rounded[str(t.dtype)] = self.rounded.get(str(t.dtype), 0) + 1
+            t = t.to(self.device).to(torch.bfloat16)      # (rounded on the device: a large table takes a moment on the host)
         return t.to(self.device).contiguous()
 
     def vector(self, t: torch.Tensor) -> torch.Tensor:

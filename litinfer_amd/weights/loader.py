@@ -7,10 +7,14 @@ tensor and every wrong shape (and, when asked to be strict, every stored tensor
 that the model does not know).  Stored names may be aliases that the
 architecture declares; a stored tensor that the model does not use is counted
 and reported in one line, as the reference lets unknown names fall through
-(python/llaisys/models/qwen2.py:139-194).  Tensors keep their
-stored precision: bfloat16 stays bfloat16, a tensor stored in 32-bit stays
-32-bit, half precision is widened to 32-bit (exactly); integer tables become
-int32.  What the engine's dtype then needs is the parts' business.
+(python/llaisys/models/qwen2.py:139-194).  The loader hands
+tensors on in their stored precision: bfloat16 stays bfloat16, a tensor stored
+in 32-bit stays 32-bit, half precision is widened to 32-bit (exactly); integer
+tables become int32.  The model's runtime then binds every MATRIX in the
+engine's one dtype (`parts.Runtime.matrix`: the reference converts every tensor
+to the model's dtype, python/llaisys/models/qwen2.py:88-110, 253-264) and
+holds norm weights and biases in 32-bit; when matrices had to be rounded for
+that, one line says so.
 """
 from __future__ import annotations
 
@@ -178,12 +182,22 @@ def load_into(model, model_dir, aliases: Optional[Mapping[str, str]] = None, str
             shown = ", ".join(unused[:8]) + (f", ... and {len(unused) - 8} more" if len(unused) > 8 else "")
             note(f"{len(unused)} stored tensor(s) are not used by {model.spec.architecture}: {shown}")
 
+        fetched = set()
+
         def get(name: str):
             if name not in ckpt.entries:
                 return None
+            if not expected[name].integer:
+                fetched.add(ckpt.entries[name][0])
             return stored_precision(ckpt.tensor(name), expected[name].integer)
 
+        rounded = getattr(getattr(model, "rt", None), "rounded", None)
+        before = sum(rounded.values()) if rounded is not None else 0
         model.load_params(TensorSource(get, note))
+        if rounded is not None and sum(rounded.values()) > before:
+            stored = ", ".join(sorted(fetched - {"BF16"}))
+            note(f"{sum(rounded.values()) - before} matrices stored as {stored} were rounded once (to nearest even) to "
+                 f"bfloat16, the engine's dtype; keep_stored_precision=True keeps them in 32-bit")
         return unused
     finally:
         ckpt.close()

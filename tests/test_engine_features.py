@@ -166,15 +166,38 @@ def test_step_refuses_bad_batches_and_leaves_the_cache_alone(tmp_path, device):
     assert eng.cache.free_pages() == [4]
 
 
-def test_matrices_stored_in_32_bit_stay_32_bit_in_the_bfloat16_engine(tmp_path, device):
-    d = helpers.make_model(tmp_path, TINY_A, 0, torch.float32)
+@pytest.mark.parametrize("stored", [torch.float32, torch.float16])
+def test_matrices_are_bound_in_the_engines_dtype_whatever_the_checkpoint_stores(tmp_path, device, stored, capsys):
+    """A bfloat16 engine rounds matrices stored in 32-bit or half precision once to bfloat16 (every
+    product then takes the bfloat16 kernels) and says so in one line; norm weights and biases stay
+    32-bit; `keep_stored_precision` keeps the matrices in 32-bit; a 32-bit engine widens everything."""
+    d = helpers.make_model(tmp_path, TINY_A, 0, stored)
     toks = helpers.random_requests(256, [40], 1)["r0"]
-    ref = helpers.plain_logits(d, {"r0": toks})["r0"]
+    rounded = helpers.plain_logits(d, {"r0": toks}, matrices_as_bfloat16=True)["r0"]
+    as_stored = helpers.plain_logits(d, {"r0": toks})["r0"]
+    assert schedules.rel_err(rounded, as_stored) > 1e-4          # the two references can be told apart
     eng = engine_for(d, device, dtype="bfloat16")
-    assert eng.model.layers[0].mixer.qkv.weight.dtype is torch.float32
-    assert eng.model.layers[0].norm1.weight.dtype is torch.float32
+    notes = [l for l in capsys.readouterr().err.splitlines() if "rounded once" in l]
+    assert len(notes) == 1 and ("F32" if stored is torch.float32 else "F16") in notes[0]
+    mixer, ffn = eng.model.layers[0].mixer, eng.model.layers[0].ffn
+    for w in (mixer.qkv.weight, mixer.out.weight, ffn.gate_up.weight, ffn.down.weight, eng.model.embedding.table,
+              eng.model.head.proj.weight):
+        assert w.dtype is torch.bfloat16
+    assert mixer.qkv.bias.dtype is torch.float32 and eng.model.layers[0].norm1.weight.dtype is torch.float32
+    want = torch.from_numpy(helpers.round_to_bfloat16(
+        helpers.plain_impl.load_folder(d, np.float32)[1]["model.layers.0.mlp.down_proj.weight"]))
+    assert torch.equal(ffn.down.weight.float().cpu(), want)     # the engine's rounding is nearest-even, once
     out = eng.step([StepEntry("a", toks, list(range(40)))]).cpu().numpy()
-    assert schedules.rel_err(out, ref) < BF16_TOL
+    assert schedules.rel_err(out, rounded) < BF16_TOL
+    kept = engine_for(d, device, dtype="bfloat16", keep_stored_precision=True)
+    assert not [l for l in capsys.readouterr().err.splitlines() if "rounded once" in l]
+    assert kept.model.layers[0].mixer.qkv.weight.dtype is torch.float32
+    out = kept.step([StepEntry("a", toks, list(range(40)))]).cpu().numpy()
+    assert schedules.rel_err(out, as_stored) < BF16_TOL
+    wide = engine_for(d, device, dtype="float32")
+    assert wide.model.layers[0].mixer.qkv.weight.dtype is torch.float32
+    out = wide.step([StepEntry("a", toks, list(range(40)))]).cpu().numpy()
+    assert schedules.rel_err(out, as_stored) < F32_TOL
 
 
 # ------------------------------------------------------ each part on its own

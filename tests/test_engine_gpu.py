@@ -134,3 +134,24 @@ def test_a_long_prompt_in_portions_then_decoding(tmp_path, dt, name):
     worst = max(schedules.rel_err(v, ref[p]) for p, v in got.items())
     print(f"[observed] long prompt {name} {dt}: {worst:.3e}")
     assert worst < TOL[dt], f"{name} {dt}: {worst}"
+
+
+@pytest.mark.parametrize("stored", [torch.float16, torch.float32])
+@pytest.mark.parametrize("name", ["D", "E"])
+def test_a_checkpoint_in_another_precision_runs_the_bfloat16_kernels(tmp_path, name, stored):
+    """A checkpoint stored in half precision (the reference's own benchmark model is) or in 32-bit,
+    in the bfloat16 engine: every matrix is bound as bfloat16, and the mixed schedule matches the
+    plain implementation computed from the stored matrices rounded once to bfloat16."""
+    cfg, page, seed = CASES[name]
+    d = helpers.make_model(tmp_path, cfg, seed + 40, stored)
+    reqs = helpers.random_requests(cfg["vocab_size"], LENGTHS, seed + 50)
+    ref = helpers.plain_logits(d, reqs, matrices_as_bfloat16=True)
+    steps = schedules.mixed(reqs)
+    eng = _engine(d, "bfloat16", page, schedules.max_live_tokens(reqs, steps, page))
+    layer = eng.model.layers[0]
+    assert layer.mixer.qkv.weight.dtype is torch.bfloat16 and layer.ffn.gate_up.weight.dtype is torch.bfloat16
+    assert eng.model.head.proj.weight.dtype is torch.bfloat16 and layer.norm1.weight.dtype is torch.float32
+    out = schedules.run(eng, reqs, steps)
+    worst = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
+    print(f"[observed] {name} stored {stored} in the bfloat16 engine, mixed: {worst:.3e}")
+    assert worst < TOL["bfloat16"], f"{name} {stored}: {worst}"
