@@ -256,8 +256,8 @@ def run_scheduler(eng, cfg, requests, *, max_batch_tokens: int, chunk_size: int,
     arrival times if given (seconds from the start) or all at once, and run it dry.
     Returns wall tokens a second and the distributions the reference's harness reports."""
     import torch
-    from .engine import PRODUCT_ROW_TILE, Scheduler
-    sched = Scheduler(eng, max_batch_tokens=max_batch_tokens, chunk_size=chunk_size, lookahead=True, row_tile=PRODUCT_ROW_TILE)
+    from .engine import Scheduler
+    sched = Scheduler(eng, max_batch_tokens=max_batch_tokens, chunk_size=chunk_size, lookahead=True)
     order = sorted(range(len(requests)), key=lambda i: arrivals[i] if arrivals else 0.0)
     submitted, first_at, last_at, count = {}, {}, {}, {}
     step_log = []                                    # (time after the step, tokens it produced)

@@ -13,7 +13,13 @@ addressed again.  All pages of a request go back when it is released.
 
 Beside the pages there are `max_seqs` state slots.  A request holds one slot
 from admission to release; mixers with a `StateNeed` get a tensor
-[max_seqs, *shape] indexed by the slot, zeroed at admission.
+[max_seqs, *shape] indexed by the slot, zeroed at admission.  An entry may
+need both: one paged need and any number of named states (its view then has
+`tensors` and `state`/`states`).
+
+Every group's pool has its own number of pages: a windowed group holds a few
+pages a request whatever the context, so it can be far smaller than a group
+that keeps all keys.
 
 The bookkeeping itself (pools, tables, slots, the window's give-back) is done by
 the host library in C++ (csrc/host.cpp); this class owns the device tensors,
@@ -33,7 +39,7 @@ import ctypes
 import numpy as np
 import torch
 
-from ..parts.base import PagedNeed, StateNeed
+from ..parts.base import PagedNeed, StateNeed, needs_of
 from . import native
 from .pool import PagePool, PagePoolError
 
@@ -49,7 +55,8 @@ class CacheView:
     group: Optional[int] = None      # index of the page group (paged needs)
     tensors: Optional[Dict[str, torch.Tensor]] = None    # name -> [pages, *leading sizes, page_size, last size]
     page_size: int = 0
-    state: Optional[torch.Tensor] = None  # [max_seqs, *shape] (state needs)
+    state: Optional[torch.Tensor] = None  # [max_seqs, *shape]: the entry's state (its first, if it has several)
+    states: Optional[Dict[str, torch.Tensor]] = None     # name -> [max_seqs, *shape], all of them
 
     @property
     def k(self) -> Optional[torch.Tensor]:
@@ -72,55 +79,78 @@ class _Group:
         return sum(t.numel() * t.element_size() for t in self.data.values())
 
 
+def group_needs(needs: Sequence[object], sources: Sequence[Optional[int]]) -> List[PagedNeed]:
+    """The page groups that a cache manager makes for these entries, in its order: the distinct
+    paged needs in the order in which the entries first ask for them."""
+    out: List[PagedNeed] = []
+    for need, src in zip(needs, sources):
+        if src is None and need is not None:
+            paged, _ = needs_of(need)
+            if paged is not None and paged not in out:
+                out.append(paged)
+    return out
+
+
 class CacheManager:
     def __init__(self, needs: Sequence[object], sources: Sequence[Optional[int]], *,
-                 page_size: int, num_pages: int, max_seqs: int, dtype: torch.dtype,
+                 page_size: int, num_pages, max_seqs: int, dtype: torch.dtype,
                  device, page_order_seed: Optional[int] = None):
         """`needs[i]` is what entry i of the execution order needs (None for
-        nothing), `sources[i]` the entry whose cache it reads instead of its own.
-        `num_pages` is the number of pages of EVERY group."""
+        nothing; a PagedNeed, a StateNeed, or a tuple of one paged need and state
+        needs), `sources[i]` the entry whose cache it reads instead of its own.
+        `num_pages` is the number of pages of every group, or a sequence with one
+        number per group (groups are numbered in the order in which the entries
+        first ask for them; `group_needs(needs, sources)` lists them)."""
         if page_size <= 0:
             raise ValueError("cache: page_size must be positive")
-        if int(num_pages) * int(page_size) >= 1 << 31:
-            raise ValueError("cache: more than 2^31 token slots in a group")
         self.page_size = int(page_size)
         self.max_seqs = int(max_seqs)
         self.device = torch.device(device)
         self.groups: List[_Group] = []
         self._entry_group: Dict[int, Tuple[int, int]] = {}     # entry -> (group, index in group)
-        self._entry_state: Dict[int, torch.Tensor] = {}
+        self._entry_state: Dict[int, Dict[str, torch.Tensor]] = {}
         self._sources = list(sources)
         by_need: Dict[PagedNeed, int] = {}
         for i, need in enumerate(needs):
             if sources[i] is not None or need is None:
                 continue
-            if isinstance(need, PagedNeed):
-                names = [t.name for t in need.tensors]
-                if not names or len(set(names)) != len(names) or any(not t.shape or min(t.shape) <= 0 for t in need.tensors):
-                    raise ValueError(f"cache: entry {i} asks for paged tensors {need.tensors!r}: they need "
+            try:
+                paged, states = needs_of(need)
+            except (TypeError, ValueError) as e:
+                raise type(e)(f"cache: entry {i}: {e}") from None
+            if paged is not None:
+                names = [t.name for t in paged.tensors]
+                if not names or len(set(names)) != len(names) or any(not t.shape or min(t.shape) <= 0 for t in paged.tensors):
+                    raise ValueError(f"cache: entry {i} asks for paged tensors {paged.tensors!r}: they need "
                                      f"distinct names and positive sizes")
-                if need not in by_need:
-                    by_need[need] = len(self.groups)
-                    self.groups.append(_Group(need, [], None, None))
-                g = by_need[need]
+                if paged not in by_need:
+                    by_need[paged] = len(self.groups)
+                    self.groups.append(_Group(paged, [], None, None))
+                g = by_need[paged]
                 self._entry_group[i] = (g, len(self.groups[g].entries))
                 self.groups[g].entries.append(i)
-            elif isinstance(need, StateNeed):
-                self._entry_state[i] = torch.zeros((self.max_seqs, *need.shape), dtype=need.dtype,
-                                                   device=self.device)
-            else:
-                raise TypeError(f"cache: entry {i} has an unknown cache need {need!r}")
+            if states:
+                self._entry_state[i] = {s.name: torch.zeros((self.max_seqs, *s.shape), dtype=s.dtype, device=self.device)
+                                        for s in states}
+        ng = len(self.groups)
+        if isinstance(num_pages, (int, np.integer)):
+            counts = [int(num_pages)] * ng
+        else:
+            counts = [int(n) for n in num_pages]
+            if len(counts) != ng:
+                raise ValueError(f"cache: {len(counts)} page counts for {ng} page groups")
+        if any(n * self.page_size >= 1 << 31 for n in counts):
+            raise ValueError("cache: more than 2^31 token slots in a group")
         orders = None
         if page_order_seed is not None and self.groups:
             orders = []
-            for gi in range(len(self.groups)):
+            for gi in range(ng):
                 gen = torch.Generator().manual_seed(page_order_seed + gi)
-                orders += torch.randperm(num_pages, generator=gen).tolist()
+                orders += torch.randperm(counts[gi], generator=gen).tolist()
         self._lib = native.lib()
-        ng = len(self.groups)
         self._book = self._lib.li_book_create(self.page_size, self.max_seqs, ng,
                                               native.int_array([g.need.window for g in self.groups]),
-                                              int(num_pages), native.int_array(orders) if orders else None)
+                                              native.int_array(counts), native.int_array(orders) if orders else None)
         err = self._lib.li_book_error(self._book).decode()
         if err:
             self._lib.li_book_destroy(self._book)
@@ -128,8 +158,8 @@ class CacheManager:
             raise ValueError(err)
         self._ints = (ctypes.c_int * max(ng, 1))()
         for gi, g in enumerate(self.groups):
-            g.pool = PagePool(num_pages, _borrowed=self._lib.li_book_pool(self._book, gi))
-            g.data = {t.name: torch.zeros((len(g.entries), num_pages, *t.page_shape(self.page_size)),
+            g.pool = PagePool(counts[gi], _borrowed=self._lib.li_book_pool(self._book, gi))
+            g.data = {t.name: torch.zeros((len(g.entries), counts[gi], *t.page_shape(self.page_size)),
                                           dtype=t.dtype or dtype, device=self.device) for t in g.need.tensors}
         # requests are named by any hashable; the book knows them by number
         self._handles: Dict[Hashable, int] = {}
@@ -153,13 +183,15 @@ class CacheManager:
     def view(self, entry: int) -> CacheView:
         src = self._sources[entry]
         owner = entry if src is None else src
+        view = CacheView(owned=src is None)
         if owner in self._entry_group:
             g, j = self._entry_group[owner]
-            return CacheView(owned=src is None, group=g, page_size=self.page_size,
-                             tensors={name: d[j] for name, d in self.groups[g].data.items()})
+            view.group, view.page_size = g, self.page_size
+            view.tensors = {name: d[j] for name, d in self.groups[g].data.items()}
         if owner in self._entry_state:
-            return CacheView(owned=src is None, state=self._entry_state[owner])
-        return CacheView(owned=src is None)
+            view.states = self._entry_state[owner]
+            view.state = next(iter(view.states.values()))
+        return view
 
     # ---- requests --------------------------------------------------------
     def has(self, rid) -> bool:
@@ -194,8 +226,9 @@ class CacheManager:
             raise RuntimeError(self._error())
         self._next_handle += 1
         self._handles[rid] = h
-        for st in self._entry_state.values():
-            st[slot].zero_()
+        for states in self._entry_state.values():
+            for st in states.values():
+                st[slot].zero_()
         return slot
 
     def slot(self, rid) -> int:
@@ -280,7 +313,11 @@ class CacheManager:
     def rewind(self, rid, n: int) -> None:
         """Forget the last `n` tokens of `rid`: their positions will be computed and written
         again.  The pages stay with the request.  Refused (ValueError) where a windowed group has
-        already given back a page that the earlier position still sees."""
+        already given back a page that the earlier position still sees, and where any entry keeps
+        state of fixed size: such a state has moved on with the tokens and cannot be taken back."""
+        if self._entry_state and n:
+            raise ValueError("cache: a request's last tokens cannot be forgotten where a mixer keeps state of fixed "
+                             "size (the state has moved on with them)")
         if self._lib.li_book_rewind(self._book, self._handle(rid), int(n)) < 0:
             raise ValueError(self._error())
 

@@ -22,7 +22,7 @@ def lib() -> ctypes.CDLL:
             "li_pool_free": ([c_void_p], c_int), "li_pool_total_allocations": ([c_void_p], c_long),
             "li_pool_alloc": ([c_void_p], c_int), "li_pool_release": ([c_void_p, c_int], c_int),
             "li_pool_is_held": ([c_void_p, c_int], c_int),
-            "li_book_create": ([c_int, c_int, c_int, IP, c_int, IP], c_void_p),
+            "li_book_create": ([c_int, c_int, c_int, IP, IP, IP], c_void_p),
             "li_book_destroy": ([c_void_p], None), "li_book_error": ([c_void_p], c_char_p),
             "li_book_pool": ([c_void_p, c_int], c_void_p), "li_book_has": ([c_void_p, c_int64], c_int),
             "li_book_num_live": ([c_void_p], c_int), "li_book_free_slots": ([c_void_p], c_int),

@@ -708,12 +708,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     // load `idx` of a wave's LPW loads of step kt: first its rows of A, then its rows of B
     auto issue_one = [&](int kt, int idx) {
         uint16_t* st = lds + (kt % NSTAGE) * STAGE;
-#ifdef LI_EXPT_NO_LOADS
-        return;
-#endif
-#ifdef LI_EXPT_SAME_COLUMNS
-        kt = 0;
-#endif
         if (idx < IA) LI_LOAD_TO_LDS_AT(abase + (size_t)kt * BK, ga[idx], st + ((BM / 4) * uwave + RPI * idx) * BK);
         else LI_LOAD_TO_LDS_AT(bbase + (size_t)kt * BK, gb[idx - IA], st + BM * BK + ((BN / 4) * uwave + RPI * (idx - IA)) * BK);
     };
@@ -1712,6 +1706,11 @@ extern "C" int li_linear_then_norm(const void* x, const void* w, const float* bi
 }
 
 // `work` (may be null): device memory of work_bytes for the partial sums of a product cut along K.
+// Rows of the smallest tile that a product of more than 64 rows is cut into in this dtype: a
+// product of a few rows more than a multiple of it pays for a whole tile more.  Whoever cuts work
+// into steps (a scheduler) asks here instead of knowing the kernels' tilings.
+extern "C" int li_linear_row_tile(int in_dtype) { return in_dtype == LI_F32 ? F32_BM : BF_BM; }
+
 extern "C" int li_linear(const void* x, const void* w, const float* bias, void* out, int M, int N,
                          int K, int in_dtype, int out_dtype, int accumulate, void* work, long work_bytes,
                          hipStream_t stream) {

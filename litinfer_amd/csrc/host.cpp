@@ -134,8 +134,10 @@ int li_pool_is_held(void* p, int page) {
 }
 
 // ------------------------------------------------------------------ the book
-// windows [ngroups]; orders null or [ngroups * num_pages] (a permutation of the page ids per group)
-void* li_book_create(int page_size, int max_seqs, int ngroups, const int* windows, int num_pages, const int* orders) {
+// windows [ngroups]; num_pages [ngroups]: every group has a pool of its own size (a windowed group
+// holds a few pages a request, whatever the context); orders null or the groups' permutations of
+// their page ids one after the other (num_pages[0] ids, then num_pages[1], ...)
+void* li_book_create(int page_size, int max_seqs, int ngroups, const int* windows, const int* num_pages, const int* orders) {
     Book* b = new Book();
     b->page_size = page_size;
     b->max_seqs = max_seqs;
@@ -143,11 +145,14 @@ void* li_book_create(int page_size, int max_seqs, int ngroups, const int* window
     if (max_seqs <= 0 || ngroups < 0) { b->error = "cache: max_seqs must be positive"; return b; }
     b->windows.assign(windows, windows + ngroups);
     b->pools.resize(ngroups);
-    for (int g = 0; g < ngroups; ++g)
-        if (!b->pools[g].init(num_pages, orders ? orders + (size_t)g * num_pages : nullptr)) {
+    size_t at = 0;
+    for (int g = 0; g < ngroups; ++g) {
+        if (!b->pools[g].init(num_pages[g], orders ? orders + at : nullptr)) {
             b->error = b->pools[g].error;
             return b;
         }
+        at += (size_t)num_pages[g];
+    }
     b->free_slots.resize(max_seqs);
     for (int i = 0; i < max_seqs; ++i) b->free_slots[i] = max_seqs - 1 - i;
     return b;

@@ -1,7 +1,6 @@
 // The one entry point of the kernel libraries that allocates nothing.
 //
-// It has no counterpart in the reference (whose argmax, src/ops/argmax/op.cpp:26-33, is a
-// host loop without buffers of its own).  It is for callers that cannot allocate device
+// It has no counterpart in the reference.  It is for callers that cannot allocate device
 // memory: code under HIP graph capture, tight serving loops, harnesses that forbid
 // hipMalloc.  li_argmax_rows, the entry point it is a variant of, takes two buffers for the
 // partial results of its first stage from the caller; this one keeps them in a device array

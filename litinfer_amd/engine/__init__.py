@@ -1,7 +1,7 @@
 from .batch import StepContext, StepEntry
 from .engine import Engine, StepError, parse_dtype
 from .model import Model, expected_params_of_spec
-from .scheduler import PRODUCT_ROW_TILE, Request, Scheduler
+from .scheduler import Request, Scheduler
 
 __all__ = ["StepContext", "StepEntry", "Engine", "StepError", "parse_dtype", "Model",
            "expected_params_of_spec", "Request", "Scheduler"]

@@ -61,6 +61,7 @@ class AttentionMeta:
     num_tiles: int = 0
     tile_rows: int = 0
     max_single_ctx: int = 0
+    group: int = 0                   # the page group whose tables these are
     extra: Dict[Any, Any] = field(default_factory=dict)    # what kernels derive and keep for the step
 
 
@@ -190,7 +191,7 @@ def build_context(cache, entries: Sequence[StepEntry], ws, uploader: "BatchUploa
             host_q_start=ctx.host_q_start, host_q_len=ctx.host_q_len, host_ctx_len=ctx.host_ctx_len,
             single_tokens=d_single if nmulti else None, num_single=nsingle,
             multi_tokens=d_multi if nsingle else None, num_multi=nmulti,
-            tiles=d_tiles, num_tiles=ntiles, tile_rows=tile_rows,
+            tiles=d_tiles, num_tiles=ntiles, tile_rows=tile_rows, group=gi,
             # with padded tables the split count must not follow the context either
             max_single_ctx=(mb * P if pad_blocks is not None else max_single_ctx)))
     return ctx

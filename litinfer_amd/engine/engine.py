@@ -15,13 +15,14 @@ from __future__ import annotations
 
 import os
 import sys
+from collections import OrderedDict
 from pathlib import Path
 from typing import Any, Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
 
-from ..cache import CacheFull, CacheManager
+from ..cache import CacheFull, CacheManager, group_needs
 from ..config import load_config, lookup, architecture_name
 from ..config.spec import ModelSpec
 from ..parts.base import Runtime
@@ -57,7 +58,7 @@ class Engine:
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  max_seqs: int = 64, page_order_seed: Optional[int] = None,
                  config: Any = None, use_graphs: bool = True, graph_after: int = 4,
-                 keep_stored_precision: bool = False):
+                 keep_stored_precision: bool = False, max_graphs: int = 64, step_tokens: int = 2048):
         """keep_stored_precision: with dtype bfloat16, leave matrices that the checkpoint stores in
         32-bit or half precision in 32-bit (their products then run in the 32-bit kernels) instead of
         rounding them once to bfloat16 when they are bound."""
@@ -71,6 +72,8 @@ class Engine:
         self.page_size = int(page_size)
         self.max_seqs = int(max_seqs)
         self._num_pages = num_pages
+        # the most tokens a step is expected to bring: sizes the pools of windowed groups (see _make_cache)
+        self.step_tokens = max(1, int(step_tokens))
         self._max_tokens = max_tokens
         self._page_order_seed = page_order_seed
         self.cache: Optional[CacheManager] = None
@@ -90,9 +93,13 @@ class Engine:
         # a few steps, recording every shape at its second step costs more than replays give back.
         self.graph_after = max(2, int(graph_after))
         self._trace = trace_enabled()
-        self._graphs: Dict[Any, Any] = {}
+        # shape -> ("seen", times) | ("graph", graph, its output), least recently used first; at most
+        # `max_graphs` recorded ones are kept
+        self._graphs: "OrderedDict[Any, Any]" = OrderedDict()
+        self.max_graphs = max(1, int(max_graphs))
         self._graph_generation = (-1, -1)
         self.graph_replays = 0
+        self.graphs_recorded = 0
 
     # ---- construction -----------------------------------------------------
     @classmethod
@@ -126,14 +133,27 @@ class Engine:
         eng._make_cache()
         return eng
 
-    def _bytes_per_page(self) -> int:
+    def _group_page_bytes(self) -> List[int]:
+        """Bytes that one page takes in every entry of each page group."""
         needs, sources = self.model.cache_needs()
-        from ..parts.base import PagedNeed
-        return sum(n.bytes_per_token(self.rt.dtype) * self.page_size
-                   for n, s in zip(needs, sources) if s is None and isinstance(n, PagedNeed))
+        groups = group_needs(needs, sources)
+        from ..parts.base import needs_of
+        out = [0] * len(groups)
+        for n, s in zip(needs, sources):
+            paged = needs_of(n)[0] if s is None and n is not None else None
+            if paged is not None:
+                out[groups.index(paged)] += paged.bytes_per_token(self.rt.dtype) * self.page_size
+        return out
 
     def _make_cache(self) -> None:
+        """The pools' sizes.  Given `num_pages` (a number for every group, or one per group),
+        `max_tokens` or LLAISYS_NUM_BLOCKS, every group gets that many pages.  Otherwise the memory
+        that is free decides: a windowed group gets what `max_seqs` requests can hold at a time,
+        ceil(window / page) + 2 pages each, plus the pages of `step_tokens` new tokens (a step's
+        portions are held whole until the step is over); the groups that keep all keys share the rest,
+        up to `max_seqs` requests of the model's full length."""
         needs, sources = self.model.cache_needs()
+        groups = group_needs(needs, sources)
         pages = self._num_pages
         env_pages = os.environ.get("LLAISYS_NUM_BLOCKS", "").strip()
         if pages is None and self._max_tokens is None and env_pages:
@@ -144,15 +164,32 @@ class Engine:
         if pages is None and self._max_tokens is not None:
             pages = -(-int(self._max_tokens) // self.page_size)
         if pages is None:
-            per_seq = -(-self.spec.max_positions // self.page_size)
-            pages = per_seq * self.max_seqs
-            if self.rt.device.type == "cuda":
+            P = self.page_size
+            per_seq = -(-self.spec.max_positions // P)
+            full = per_seq * self.max_seqs
+            pages = [full if g.window <= 0 else
+                     min(full, self.max_seqs * (-(-g.window // P) + 2) + -(-self.step_tokens // P)) for g in groups]
+            if self.rt.device.type == "cuda" and groups:
                 free, _ = torch.cuda.mem_get_info(self.rt.device)
-                bpp = max(1, self._bytes_per_page())
-                pages = max(1, min(pages, int(free * 0.85) // bpp))
-        self.cache = CacheManager(needs, sources, page_size=self.page_size, num_pages=int(pages),
+                bpp = [max(1, b) for b in self._group_page_bytes()]
+                budget = int(free * 0.85)
+                windowed = sum(n * b for n, b, g in zip(pages, bpp, groups) if g.window > 0)
+                if windowed > budget // 2:                # (windows as long as the contexts: no group is small)
+                    share = max(1, budget // sum(bpp))
+                    pages = [min(n, share) for n in pages]
+                else:
+                    rest = sum(b for b, g in zip(bpp, groups) if g.window <= 0)
+                    share = max(1, (budget - windowed) // max(1, rest))
+                    pages = [n if g.window > 0 else min(n, share) for n, g in zip(pages, groups)]
+        self.cache = CacheManager(needs, sources, page_size=self.page_size, num_pages=pages,
                                   max_seqs=self.max_seqs, dtype=self.rt.dtype, device=self.rt.device,
                                   page_order_seed=self._page_order_seed)
+
+    @property
+    def row_tile(self) -> int:
+        """Rows that the model's kernels take at a time, as its parts report it: what a scheduler
+        rounds a step's tokens to."""
+        return self.model.batch_needs().row_tile
 
     # ---- the step ---------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]):
@@ -272,33 +309,59 @@ class Engine:
         widths = tuple(max(16, 1 << (max(need, 1) - 1).bit_length()) for need in self.cache.max_table_len(handles))
         return (len(entries), sum(len(e.want) for e in entries), widths)
 
+    def _buffers_at(self):
+        """Changes whenever a buffer that a recorded step may address has moved."""
+        return (self.ws.generation, self._uploader.generation)
+
+    def _drop_graphs(self) -> None:
+        """Recorded addresses are stale: every shape is recorded anew at its next step (which
+        runs eagerly first); how often a shape was seen is kept."""
+        for k, state in list(self._graphs.items()):
+            if state[0] == "graph":
+                self._graphs[k] = ("seen", self.graph_after - 1)
+
     def _forward_graphed(self, key, ctx: StepContext):
-        gen = (self.ws.generation, self._uploader.generation)
-        state = self._graphs.get(key)
-        if state is None or state[0] != "graph" or self._graph_generation != gen:
-            if self._graph_generation != gen:
-                self._graphs.clear()              # a buffer moved: recorded addresses are stale
-                state = None
-            # the first steps of a shape run eagerly (the first sizes the buffers), the graph_after-th is recorded
-            logits = self.model.forward(ctx, self.cache)
-            gen = (self.ws.generation, self._uploader.generation)
-            self._graph_generation = gen
-            seen = 1 if state is None or state[0] != "seen" else state[1] + 1
-            if seen < self.graph_after:
-                self._graphs[key] = ("seen", seen)
-                return logits
+        if self._graph_generation != self._buffers_at():
+            self._drop_graphs()                   # a buffer moved since the last decode step
+            self._graph_generation = self._buffers_at()
+        graphs = self._graphs
+        state = graphs.get(key)
+        if state is not None and state[0] == "graph":
+            graphs.move_to_end(key)
+            state[1].replay()
+            self.graph_replays += 1
+            return state[2]
+        # the first steps of a shape run eagerly (the first sizes the buffers), the graph_after-th is recorded
+        logits = self.model.forward(ctx, self.cache)
+        if self._graph_generation != self._buffers_at():
+            # this pass itself made a buffer grow (a larger batch than any before): what was
+            # recorded for OTHER shapes addresses the old one
+            self._drop_graphs()
+            self._graph_generation = self._buffers_at()
+        seen = 1 if state is None else state[1] + 1
+        graphs[key] = ("seen", seen)
+        graphs.move_to_end(key)
+        if seen >= self.graph_after:
+            made = self.ws.allocations
             torch.cuda.synchronize(self.rt.device)
             ctx.forget_shared()                   # what the eager pass prepared must be prepared in the graph too
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 out = self.model.forward(ctx, self.cache)
-            if (self.ws.generation, self._uploader.generation) != gen:
-                self._graphs.clear()              # recording itself moved a buffer: do not keep it
-                self._graph_generation = (self.ws.generation, self._uploader.generation)
-                return logits
-            self._graphs[key] = ("graph", graph, out)
-            return logits
-        _, graph, out = state
-        graph.replay()
-        self.graph_replays += 1
-        return out
+            if self._graph_generation != self._buffers_at() or self.ws.allocations != made:
+                # recording itself allocated (the buffer would live in the graph's own pool) or
+                # moved a buffer: do not keep it, and nothing recorded before it either
+                self._drop_graphs()
+                self._graph_generation = self._buffers_at()
+            else:
+                graphs[key] = ("graph", graph, out)
+                self.graphs_recorded += 1
+        # the least recently used shapes go: a long-lived engine sees hundreds of them, and every
+        # recorded one holds its graph and its output buffer
+        recorded = sum(1 for s in graphs.values() if s[0] == "graph")
+        for k in list(graphs):
+            if recorded <= self.max_graphs and len(graphs) <= 8 * self.max_graphs:
+                break
+            if k != key:
+                recorded -= graphs.pop(k)[0] == "graph"
+        return logits

@@ -33,6 +33,7 @@ class Model:
         return e
 
     def load_params(self, get) -> None:
+        self._batch_needs = None                     # parts may answer differently once they hold their tensors
         self.embedding.load_params(get)
         for layer in self.layers:
             layer.load_params(get)

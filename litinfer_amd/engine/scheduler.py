@@ -93,11 +93,6 @@ class Request:
         return out
 
 
-# Rows of the smallest tile that the kernels' products of more than 64 rows are cut into (csrc/gemm.hip):
-# what callers pass as `row_tile`.
-PRODUCT_ROW_TILE = 128
-
-
 @dataclass
 class Planned:
     request: Request
@@ -109,11 +104,14 @@ class Planned:
 class Scheduler:
     def __init__(self, engine, *, max_batch_tokens: int = 2048, chunk_size: int = 512,
                  max_running: Optional[int] = None, eos_token_ids: Optional[Sequence[int]] = None,
-                 sampler=None, lookahead: bool = False, row_tile: int = 1):
+                 sampler=None, lookahead: bool = False, row_tile: Optional[int] = None):
         """row_tile: rows that the kernels of a step take at a time (the products' tiles).  A step
         whose tokens number a few more than a multiple of it (up to half a tile) pays for a whole
         tile more: then the last portion of a prompt in the plan that is not the prompt's end gives
-        those tokens up to the next step.  1: as planned."""
+        those tokens up to the next step.  1: as planned.  None: what the engine's model says
+        (`Engine.row_tile`, the largest `BatchNeeds.row_tile` of its parts)."""
+        if row_tile is None:
+            row_tile = int(getattr(engine, "row_tile", 1) or 1)
         if max_batch_tokens <= 0 or chunk_size <= 0 or row_tile <= 0:
             raise ValueError("scheduler: max_batch_tokens, chunk_size and row_tile must be positive")
         self.engine = engine
@@ -153,7 +151,9 @@ class Scheduler:
                              f"length ({limit})")
         need = self.cache.pages_needed(None, len(prompt) + max_new_tokens - 1, cached=0)
         for g, n in zip(self.cache.groups, need):
-            if g.need.window <= 0 and n > g.pool.capacity:
+            if g.need.window > 0:                      # there a request goes on token by token if it must
+                n = min(n, -(-g.need.window // self.cache.page_size) + 1)
+            if n > g.pool.capacity:
                 raise ValueError(f"add_request: the request needs {n} cache pages, the pool has "
                                  f"{g.pool.capacity}: it could never run")
         if rid is None:
@@ -201,8 +201,33 @@ class Scheduler:
         self.preemptions += 1
         self.waiting.appendleft(req)
 
-    def _fits(self, free: List[int], rid, n: int, cached: Optional[int] = None) -> Optional[List[int]]:
+    def _at_a_time(self, need, portion: Optional[int] = None):
+        """`need` (pages per group, a list or an array [requests, groups]) counts every page that a
+        request's further tokens fill.  A windowed group gives pages back as the window passes them:
+        there a request holds at most the window's pages and those of the portion that a step brings
+        (up to `chunk_size` tokens) at a time, and that is what has to be free for it; a pool smaller
+        than that serves one request at a time, in shorter portions."""
+        P = self.cache.page_size
+        portion = self.chunk_size if portion is None else portion
+        caps = [min(-(-(g.need.window - 1 + portion) // P) + 1, g.pool.capacity) if g.need.window > 0 else None
+                for g in self.cache.groups]
+        if all(c is None for c in caps):
+            return need
+        if isinstance(need, np.ndarray):
+            need = need.copy()
+            for gi, c in enumerate(caps):
+                if c is not None:
+                    np.minimum(need[:, gi], c, out=need[:, gi])
+            return need
+        return [n if c is None else min(n, c) for n, c in zip(need, caps)]
+
+    def _fits(self, free: List[int], rid, n: int, cached: Optional[int] = None, whole: bool = False) -> Optional[List[int]]:
+        """The pages that n more tokens of the request take, if they are free (else None).  `whole`:
+        the n tokens will come in portions over several steps; then windowed groups count with what
+        the request holds at a time, not with every page it will ever fill."""
         need = self.cache.pages_needed(rid, n, cached)
+        if whole:
+            need = self._at_a_time(need)
         return need if all(a <= b for a, b in zip(need, free)) else None
 
     def _largest_fitting(self, free: List[int], rid, n: int, cached: Optional[int]) -> int:
@@ -268,15 +293,20 @@ class Scheduler:
             if self.waiting and budget > 0 and slots > 0 and len(self.running) < self.max_running:
                 going = [r for r in self.running if left[id(r)] > 0]
                 if going:
-                    need = self.cache.pages_needed_many(self.cache.handles_of([r.rid for r in going]),
-                                                        np.asarray([left[id(r)] for r in going], dtype=np.int32))
+                    need = self._at_a_time(self.cache.pages_needed_many(
+                        self.cache.handles_of([r.rid for r in going]), np.asarray([left[id(r)] for r in going], dtype=np.int32)))
                     spare = [int(a - b) for a, b in zip(spare, need.sum(axis=0))]
             while self.waiting and budget > 0 and slots > 0 and len(self.running) < self.max_running:
                 r = self.waiting[0]
-                whole = self._fits(spare, None, r.remaining, 0)
+                whole = self._fits(spare, None, r.remaining, 0, whole=True)
                 if whole is None:
                     break                               # first come first served: nobody overtakes
-                n = min(r.remaining, self.chunk_size, budget)
+                # (its first portion must fit what is free in this very step, which the windowed
+                # groups' pools may cut short)
+                n = self._largest_fitting(free, None, min(r.remaining, self.chunk_size, budget), 0)
+                if n <= 0:
+                    break
+                free = [a - b for a, b in zip(free, self.cache.pages_needed(None, n, cached=0))]
                 self.waiting.popleft()
                 r.state = RUNNING
                 self.running.append(r)

@@ -12,7 +12,8 @@ class Workspace:
     def __init__(self, device):
         self.device = torch.device(device)
         self._bufs: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
-        self.generation = 0          # goes up whenever a buffer moves: recorded graphs are stale then
+        self.generation = 0          # goes up whenever a buffer MOVES (is allocated anew, larger): recorded graphs are stale then
+        self.allocations = 0         # goes up with every allocation, a name's first included
         self._views: Dict[Tuple[str, torch.dtype, Tuple[int, ...]], torch.Tensor] = {}
 
     def buffer(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
@@ -27,9 +28,12 @@ class Workspace:
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < max(1, n):
             cap = max(1, n) if buf is None else max(n, buf.numel() * 3 // 2)
+            moved = buf is not None
             buf = torch.empty(cap, dtype=dtype, device=self.device)
             self._bufs[key] = buf
-            self.generation += 1
+            self.allocations += 1
+            if moved:                              # a name's first buffer moves nothing that a graph may have recorded
+                self.generation += 1
             for k in [k for k in self._views if k[0] == name and k[1] is dtype]:
                 del self._views[k]                 # views of the buffer that has just moved
         view = buf[:n].view(*shape)

@@ -174,8 +174,8 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor,
     """out[t, :] = table[id(t), :] as float32 with id(t) = ids[t], or
     feedback[id_src[t]] where id_src is given and id_src[t] >= 0 (a token chosen
     on the device that the host has not seen yet).  Ids given by the host must
-    already be inside the table (the step checks them); an id outside it leaves
-    the row as it is."""
+    already be inside the table (the step checks them); an id outside it (one
+    that the device chose) gives a row of zeros, never a read outside the table."""
     _gpu(ids, table, out, id_src, feedback)
     t, h = out.shape
     _chk(ids.dtype is torch.int32 and ids.numel() == t and ids.is_contiguous(), "embedding: ids")
@@ -347,6 +347,17 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: 
         _run("gemm", "li_linear", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
              out.data_ptr(), m, n, k, _DT[x.dtype], _DT[out.dtype], int(bool(accumulate)), work, work_bytes)
 
+
+
+def linear_row_tile(dtype: torch.dtype) -> int:
+    """Rows of the smallest tile that `linear` cuts a product of many rows of this dtype into (the
+    kernel library says): a few rows more than a multiple of it cost a whole tile more."""
+    f = _fn_cache.get(("gemm", "li_linear_row_tile"))
+    if f is None:
+        f = build.load("gemm").li_linear_row_tile
+        f.argtypes, f.restype = [c_int], c_int
+        _fn_cache[("gemm", "li_linear_row_tile")] = f
+    return int(f(_DT[dtype]))
 
 
 def skinny_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
@@ -739,8 +750,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
             key = ("decode_run_keys", nkv, int(window), nsplit, meta.max_blocks, n_single)
             run_keys = meta.extra.get(key)
             if run_keys is None:
-                name = "attn.run_keys.%d.%d.%d.%d" % (nkv, int(window), nsplit, n_single)
-                size = 2 + n_single + n_single * nsplit
+                # one buffer for every number of runs and (growing only with the batch) of tokens: a
+                # name per combination would pile up over a serving run
+                name = "attn.run_keys.%d.%d.%d" % (getattr(meta, "group", 0), nkv, int(window))
+                size = 2 + n_single + n_single * DECODE_MAX_SPLITS
                 run_keys = (ws.buffer(name, (size,), torch.int32) if ws is not None
                             else torch.empty(size, dtype=torch.int32, device=qkv.device))
                 decode_run_keys(meta, lst, n_single, page_size, window, nkv, nsplit, _simd_count(qkv.device), run_keys)

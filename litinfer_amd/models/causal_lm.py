@@ -16,7 +16,7 @@ import time
 from pathlib import Path
 from typing import Iterator, List, Optional, Sequence
 
-from ..engine import PRODUCT_ROW_TILE, Engine, Scheduler
+from ..engine import Engine, Scheduler
 from ..sampling import SamplingParams
 
 
@@ -46,12 +46,13 @@ class CausalLM:
         print(f"[litinfer_amd] loading {self.model_path} ({dtype}) ...", flush=True)
         self.engine = Engine.from_dir(self.model_path, dtype=dtype, device=device, page_size=page_size,
                                       num_pages=num_pages, max_tokens=max_tokens, max_seqs=max_seqs,
-                                      strict_weights=strict_weights, keep_stored_precision=keep_stored_precision)
+                                      strict_weights=strict_weights, keep_stored_precision=keep_stored_precision,
+                                      step_tokens=max_batch_tokens)
         self.meta = self.engine.config
         self.seed = int(seed)
         # lookahead: a step is started before the tokens of the one before have reached the host
         self._sched_args = dict(max_batch_tokens=max_batch_tokens, chunk_size=chunk_size,
-                                lookahead=bool(lookahead), row_tile=PRODUCT_ROW_TILE)
+                                lookahead=bool(lookahead))
         self._scheduler: Optional[Scheduler] = None
         print(f"[litinfer_amd] ready: {self.engine.spec.architecture}, "
               f"{self.engine.model.weight_bytes() / 2**20:.1f} MiB of weights", flush=True)

@@ -1,5 +1,5 @@
 from .base import (BatchNeeds, Block, FeedForward, Mixer, Norm, PagedKVNeed, PagedNeed, PagedTensor, Part,
-                   Runtime, StateNeed, build_part, register_part)
+                   Runtime, StateNeed, build_part, needs_of, register_part)
 from .position import Position, RopeNeox
 from .linear import Linear
 from .stream import ResidualStream
@@ -10,6 +10,6 @@ from .block import PreNormBlock
 from .embedding import LinearHead, TokenEmbedding
 
 __all__ = ["BatchNeeds", "Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "PagedNeed", "PagedTensor",
-           "Part", "Runtime", "StateNeed",
+           "Part", "Runtime", "StateNeed", "needs_of",
            "build_part", "register_part", "Position", "RopeNeox", "Linear", "ResidualStream", "RMSNorm",
            "GQAttention", "SwiGLUMLP", "PreNormBlock", "LinearHead", "TokenEmbedding"]

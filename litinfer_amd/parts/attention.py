@@ -52,7 +52,8 @@ class GQAttention(Mixer):
 
     def batch_needs(self):
         # the kernels take single-token segments (split keys) and the others (tiles of queries) apart
-        return BatchNeeds(tile_rows=ops.PREFILL_TILE_ROWS, token_kinds=True)
+        return BatchNeeds(tile_rows=ops.PREFILL_TILE_ROWS, token_kinds=True,
+                          row_tile=self.qkv.row_tile() if self.qkv is not None else 1)
 
     def expected_params(self):
         p = self.prefix

@@ -10,7 +10,8 @@ Interfaces (T = tokens of the step, H = hidden size):
 
 * Norm.forward(x [T, H] float32, out) -> out [T, H] in the activation dtype.
 * Mixer.cache_need() -> PagedNeed (named tensors per token, in pages; PagedKVNeed(...)
-  builds the usual keys and values) | StateNeed | None;
+  builds the usual keys and values) | StateNeed | None, or a tuple of them (pages AND
+  state of fixed size: one paged need and any number of named state needs);
   Mixer.forward(xn [T, H], residual, ctx, cache): ADDS its output to the
   residual stream in 32-bit.  `residual` is a `ResidualStream`
   (parts/stream.py): `residual.add_linear(linear, h)` adds h W^T + b, and
@@ -112,22 +113,47 @@ class BatchNeeds:
     """Index arrays, beyond the basic ones, that a part's kernels want laid out with a
     step's batch (they travel in the step's one upload).  `tile_rows` > 0: the tokens of
     segments with several tokens cut into tiles of up to that many consecutive tokens of one
-    segment; `token_kinds`: the lists of tokens of single-token segments and of the others."""
+    segment; `token_kinds`: the lists of tokens of single-token segments and of the others.
+    `row_tile` is no array but a hint for whoever cuts prompts into steps: the part's kernels take
+    a step's rows that many at a time, so a step of a few rows more than a multiple of it costs a
+    whole tile more (1: no such tile).  The model's is the largest of its parts'."""
     tile_rows: int = 0
     token_kinds: bool = False
+    row_tile: int = 1
 
     def merged(self, other: "BatchNeeds") -> "BatchNeeds":
         if self.tile_rows and other.tile_rows and self.tile_rows != other.tile_rows:
             raise ValueError(f"parts ask for tiles of {self.tile_rows} and of {other.tile_rows} tokens; "
                              f"a step's batch is laid out with one tile size")
-        return BatchNeeds(self.tile_rows or other.tile_rows, self.token_kinds or other.token_kinds)
+        return BatchNeeds(self.tile_rows or other.tile_rows, self.token_kinds or other.token_kinds,
+                          max(self.row_tile, other.row_tile))
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """Per-request state of fixed size, zero when a request is admitted."""
+    """Per-request state of fixed size, zero when a request is admitted.  A mixer that keeps
+    several gives them different names."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    name: str = "state"
+
+
+def needs_of(need) -> Tuple[Optional[PagedNeed], Tuple[StateNeed, ...]]:
+    """What `cache_need()` returned (None, one need, or a tuple or list of needs), taken apart:
+    the paged need (at most one per entry of the execution order; its tensors are any number) and
+    the state needs (any number, with distinct names)."""
+    items = () if need is None else tuple(need) if isinstance(need, (tuple, list)) else (need,)
+    paged = [n for n in items if isinstance(n, PagedNeed)]
+    states = tuple(n for n in items if isinstance(n, StateNeed))
+    if len(paged) + len(states) != len(items):
+        bad = [n for n in items if not isinstance(n, (PagedNeed, StateNeed))]
+        raise TypeError(f"cache need {bad[0]!r} is neither a PagedNeed nor a StateNeed")
+    if len(paged) > 1:
+        raise ValueError("a mixer keeps ONE paged need (of any number of tensors); two page groups for one entry "
+                         "of the execution order are not supported")
+    if len({s.name for s in states}) != len(states):
+        raise ValueError(f"state needs of one mixer need distinct names, found {[s.name for s in states]}")
+    return (paged[0] if paged else None), states
 
 
 class Part:

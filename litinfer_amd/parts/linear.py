@@ -17,6 +17,10 @@ class Linear:
         self.bias = None if bias is None else rt.vector(bias)
         self.out_features, self.in_features = self.weight.shape
 
+    def row_tile(self) -> int:
+        """Rows that the kernels of this product take at a time (for `BatchNeeds.row_tile`)."""
+        return ops.linear_row_tile(self.rt.dtype) if self.rt.device.type == "cuda" else 1
+
     def takes_swiglu(self, x: torch.Tensor) -> bool:
         """Whether the product of these rows can have the SwiGLU activation as its
         epilogue (bfloat16, no bias, a width the kernels take)."""

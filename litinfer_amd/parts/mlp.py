@@ -8,7 +8,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import ParamSpec
-from .base import FeedForward, register_part
+from .base import BatchNeeds, FeedForward, register_part
 from .linear import Linear
 
 
@@ -27,6 +27,9 @@ class SwiGLUMLP(FeedForward):
         return {p + "gate_proj.weight": ParamSpec((self.inter, self.hidden)),
                 p + "up_proj.weight": ParamSpec((self.inter, self.hidden)),
                 p + "down_proj.weight": ParamSpec((self.hidden, self.inter))}
+
+    def batch_needs(self):
+        return BatchNeeds(row_tile=self.down.row_tile() if self.down is not None else 1)
 
     def load_params(self, get):
         p = self.prefix

@@ -200,3 +200,57 @@ def test_random_orders_lose_no_page(seed):
     assert m.free_pages() == [10] * len(m.groups) and m.free_slots() == 3
     with pytest.raises(KeyError):
         m.release("r0")                                 # a request cannot be released twice
+
+
+def test_an_entry_may_keep_pages_and_states_of_fixed_size_together():
+    """One paged need and any number of named states for one entry: its view has both."""
+    both = (PagedKVNeed(1, 4, 0), StateNeed((3, 2), torch.float32, name="tail"), StateNeed((5,), torch.int32, name="count"))
+    m = CacheManager([both, PagedKVNeed(1, 4, 0), StateNeed((2,))], [None, None, None], page_size=4, num_pages=5,
+                     max_seqs=2, dtype=torch.float32, device="cpu")
+    assert len(m.groups) == 1 and m.groups[0].entries == [0, 1]          # the paged part joins its group as ever
+    v = m.view(0)
+    assert v.k.shape == (5, 1, 4, 4) and set(v.states) == {"tail", "count"}
+    assert v.state is v.states["tail"] and v.states["tail"].shape == (2, 3, 2) and v.states["count"].dtype is torch.int32
+    assert m.view(1).states is None and m.view(1).k is not None
+    assert m.view(2).tensors is None and m.view(2).state.shape == (2, 2)
+    s = m.admit("a")
+    v.states["tail"][s] += 1
+    v.states["count"][s] += 7
+    m.release("a")
+    assert m.admit("b") == s and not v.states["tail"][s].any() and not v.states["count"][s].any()
+    m.reserve("b", 3)
+    m.commit("b", 3)
+    with pytest.raises(ValueError, match="state of fixed size"):
+        m.rewind("b", 1)                                                   # the states have moved on with the tokens
+    with pytest.raises(ValueError, match="ONE paged need"):
+        CacheManager([(PagedKVNeed(1, 4, 0), PagedKVNeed(1, 4, 3))], [None], page_size=4, num_pages=5, max_seqs=2,
+                     dtype=torch.float32, device="cpu")
+    with pytest.raises(ValueError, match="distinct names"):
+        CacheManager([(StateNeed((1,)), StateNeed((2,)))], [None], page_size=4, num_pages=5, max_seqs=2,
+                     dtype=torch.float32, device="cpu")
+    with pytest.raises(TypeError, match="neither"):
+        CacheManager([("pages",)], [None], page_size=4, num_pages=5, max_seqs=2, dtype=torch.float32, device="cpu")
+
+
+def test_every_group_has_a_pool_of_its_own_size():
+    from litinfer_amd.cache import group_needs
+    needs = [PagedKVNeed(2, 8, 0), PagedKVNeed(2, 8, 6), PagedKVNeed(2, 8, 6), None]
+    assert [n.window for n in group_needs(needs, [None] * 4)] == [0, 6]
+    m = CacheManager(needs, [None] * 4, page_size=4, num_pages=[12, 4], max_seqs=2, dtype=torch.float32, device="cpu",
+                     page_order_seed=3)
+    assert [g.pool.capacity for g in m.groups] == [12, 4] and m.free_pages() == [12, 4]
+    assert m.groups[0].data["k"].shape[1] == 12 and m.groups[1].data["k"].shape == (2, 4, 2, 4, 8)
+    m.admit("a")
+    with pytest.raises(CacheFull, match="of 4 are free"):
+        m.reserve("a", 17)                           # five pages at once: the full group could, the windowed cannot
+    assert m.free_pages() == [12, 4]
+    for _ in range(10):                              # 40 tokens, four at a time: the window's pages go round
+        m.reserve("a", 4)
+        m.commit("a", 4)
+        m.check_invariants()
+    assert m.free_pages() == [2, 2] and m.groups[1].pool.total_allocations == 10
+    assert all(0 <= p < 4 for p in m.block_table("a", 1) if p >= 0)
+    m.release("a")
+    assert m.free_pages() == [12, 4]
+    with pytest.raises(ValueError, match="page counts"):
+        CacheManager(needs, [None] * 4, page_size=4, num_pages=[12], max_seqs=2, dtype=torch.float32, device="cpu")

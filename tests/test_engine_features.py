@@ -422,6 +422,31 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path, device
     eng.cache.check_invariants()
 
 
+def test_a_toy_mixer_keeps_pages_and_a_state_of_fixed_size(tmp_path, device):
+    """Keys and values in pages beside a tail of the last three inputs in the request's state slot
+    (tests/toy_parts.py): one mixer, both kinds of cache, no framework file touched.  The toy's
+    pages form a group of their own beside the attention layer's; slots and pages are used again."""
+    import toy_parts
+    cfg = dict(TINY_A, architectures=["ToyTailLM"], toy_decay=0.0)
+    d = helpers.make_model(tmp_path, cfg, 16)
+    pcfg, w = P.load_folder(d)
+    assert "model.layers.0.tail.wk" in w and "model.layers.0.self_attn.q_proj.weight" not in w
+    reqs = helpers.random_requests(256, [21, 40, 3, 30, 12, 1, 2], 17)
+    ref = {r: toy_parts.plain_toy_tail_logits(pcfg, w, t) for r, t in reqs.items()}
+    for kind in ("whole", "tail", "chunks", "mixed"):
+        steps = getattr(schedules, kind)(reqs)
+        eng = engine_for(d, device, page=8, max_tokens=schedules.max_live_tokens(reqs, steps, 8 if kind == "mixed" else 64),
+                         page_order_seed=5)
+        assert [g.entries for g in eng.cache.groups] == [[0], [1]] and set(eng.cache.groups[0].data) == {"k", "v"}
+        v = eng.cache.view(0)
+        assert v.tensors["k"].shape[1:] == (8, 12) and v.states["tail"].shape == (4, 3, 64) and v.state is v.states["tail"]
+        out = schedules.run(eng, reqs, steps)
+        assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind
+        eng.cache.check_invariants()
+        if kind == "mixed":
+            assert all(g.pool.total_allocations > g.pool.capacity for g in eng.cache.groups)
+
+
 # ------------- a toy mixer with a cache of its own shape: one latent vector per token, in pages
 class ToyLatentAttention(Mixer):
     """One head over a compressed cache: c_t = xn_t Wc (a latent of `rank` numbers, kept in

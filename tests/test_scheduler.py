@@ -18,9 +18,10 @@ class FakeEngine:
     """Owns a real cache manager; `step` does the bookkeeping of the real one
     and returns logits whose argmax is (last token + 1) % VOCAB."""
 
-    def __init__(self, num_pages=8, page=4, max_seqs=4, max_positions=64, eos=()):
-        self.cache = CacheManager([PagedKVNeed(1, 4, 0)], [None], page_size=page, num_pages=num_pages,
-                                  max_seqs=max_seqs, dtype=torch.float32, device="cpu")
+    def __init__(self, num_pages=8, page=4, max_seqs=4, max_positions=64, eos=(), windows=(0,)):
+        """`windows`: one page group per entry (0: all keys); `num_pages` a number for all or one per group."""
+        self.cache = CacheManager([PagedKVNeed(1, 4, w) for w in windows], [None] * len(windows), page_size=page,
+                                  num_pages=num_pages, max_seqs=max_seqs, dtype=torch.float32, device="cpu")
         self.spec = SimpleNamespace(vocab_size=VOCAB, max_positions=max_positions, eos_token_ids=tuple(eos))
         self.rt = SimpleNamespace(device=torch.device("cpu"))
         self.batches = []
@@ -237,3 +238,70 @@ def test_a_step_a_few_tokens_over_whole_tiles_shortens_a_portion():
     d = s3.add_request([i % 50 for i in range(60)], max_new_tokens=1)
     s3.step()
     assert e3.batches[0] == [(d, 17, [])]
+
+
+def test_the_scheduler_takes_the_row_tile_from_the_engine_when_none_is_given():
+    e = FakeEngine(num_pages=64, max_positions=200)
+    e.row_tile = 8                                                 # what `Engine.row_tile` reports from the model's parts
+    s = sched(e, max_batch_tokens=40, chunk_size=16)
+    a = s.add_request(list(range(3)), max_new_tokens=6)
+    s.step()
+    b = s.add_request([(7 * i) % 50 for i in range(50)], max_new_tokens=2)
+    s.step()
+    assert s.row_tile == 8 and e.batches[1] == [(a, 1, [0]), (b, 15, [])]
+    assert sched(FakeEngine(), row_tile=1).row_tile == 1 and sched(FakeEngine()).row_tile == 1
+
+
+def test_a_small_pool_of_a_windowed_group_admits_long_prompts():
+    """The windowed group's pool (6 pages) is smaller than the pages a 40-token prompt fills (10): the
+    request is admitted all the same, because at a time it holds the window's pages and a portion's."""
+    e = FakeEngine(num_pages=[32, 6], windows=(0, 6), max_positions=200)
+    s = sched(e, max_batch_tokens=8, chunk_size=8)
+    a = s.add_request([i % 50 for i in range(40)], max_new_tokens=5)
+    s.run_to_completion()
+    assert s.requests[a].finish_reason == "length" and s.output(a) == [40, 41, 42, 43, 44]
+    assert s.preemptions == 0 and e.cache.free_pages() == [32, 6]
+    assert e.cache.groups[1].pool.total_allocations >= 11          # its pages went round
+    # a portion larger than the windowed pool can hold is cut to what fits
+    e2 = FakeEngine(num_pages=[32, 3], windows=(0, 6), max_positions=200)
+    s2 = sched(e2, max_batch_tokens=16, chunk_size=16)
+    with pytest.raises(ValueError, match="could never run"):
+        sched(FakeEngine(num_pages=[32, 2], windows=(0, 6), max_positions=200)).add_request([1] * 9, 2)
+    b = s2.add_request([i % 50 for i in range(30)], max_new_tokens=2)
+    s2.run_to_completion()
+    assert s2.output(b) == [30, 31] and max(n for batch in e2.batches for _, n, _ in batch) <= 12
+    assert e2.cache.free_pages() == [32, 3]
+
+
+def test_unequal_pools_admission_waits_and_preemption_frees_the_windowed_group():
+    """Two page groups of unequal pools.  A request is admitted only when BOTH groups have room for what
+    it holds at a time; when the windowed group runs out among decoding requests, the last admitted
+    gives way and is computed again; tokens are as without the squeeze."""
+    prompts = [[(3 * i + k) % 50 for i in range(n)] for k, n in enumerate((14, 9, 11))]
+
+    def run(pages):
+        e = FakeEngine(num_pages=pages, windows=(0, 8), max_positions=200, max_seqs=3)
+        s = sched(e, max_batch_tokens=12, chunk_size=4)
+        ids = [s.add_request(p, max_new_tokens=12) for p in prompts]
+        steps = 0
+        while s.has_unfinished():
+            s.step()
+            steps += 1
+            assert steps < 400
+            e.cache.check_invariants()
+        assert e.cache.free_pages() == list(pages)
+        return e, s, [s.output(i) for i in ids]
+    roomy_e, roomy_s, want = run([64, 64])
+    assert roomy_s.preemptions == 0 and all(len(t) == 12 for t in want)
+    # window 8, page 4, portions of 4: a request holds up to ceil(11 / 4) + 1 = 4 pages at a time; seven pages
+    # do not hold three requests, so the third waits although the full group has room for all
+    e, s, got = run([64, 7])
+    assert got == want
+    first_batches = [sorted(r for r, _, _ in b) for b in e.batches[:3]]
+    assert all(len(b) <= 2 for b in first_batches), first_batches
+    # a full group too small for all three: the same through the other pool
+    e, s, got = run([12, 64])
+    assert got == want and (s.preemptions > 0 or any(len(b) < 3 for b in e.batches))
+    # both tight: preemption happens and nothing is lost
+    e, s, got = run([9, 5])
+    assert got == want

@@ -31,6 +31,14 @@ def test_argmax_without_allocation_equals_the_one_with_buffers_twice_in_a_row():
     stream = torch.cuda.current_stream().cuda_stream
     assert lib.li_argmax_rows_noalloc_init() == 0, lib.li_argmax_rows_noalloc_error().decode()
     g = torch.Generator().manual_seed(5)
+    # a first small call of both entry points: what the runtime sets up at a kernel's first launch
+    # (its code, its queue) is in place before free memory is compared
+    warm = torch.randn(2, 64, generator=g).to(dev)
+    w_out = torch.empty(2, dtype=torch.int32, device=dev)
+    w_sv, w_si = torch.empty(64, dtype=torch.float32, device=dev), torch.empty(64, dtype=torch.int32, device=dev)
+    assert lib.li_argmax_rows(warm.data_ptr(), w_out.data_ptr(), w_sv.data_ptr(), w_si.data_ptr(), 2, 64, stream) == 0
+    assert lib.li_argmax_rows_noalloc(warm.data_ptr(), w_out.data_ptr(), 2, 64, stream) == 0
+    torch.cuda.synchronize()
     for n, v in ((64, 152064), (5, 301)):                     # the second call is the smaller one
         logits = torch.randn(n, v, generator=g).to(dev)
         logits[1, min(7, v - 1)] = logits[1, v - 1] = 50.0    # a tie: the lower index wins
@@ -38,12 +46,15 @@ def test_argmax_without_allocation_equals_the_one_with_buffers_twice_in_a_row():
         sv = torch.empty(n * 32, dtype=torch.float32, device=dev)
         si = torch.empty(n * 32, dtype=torch.int32, device=dev)
         got = torch.full((n,), -7, dtype=torch.int32, device=dev)
-        torch.cuda.synchronize()
-        before = torch.cuda.memory_allocated(dev)
         assert lib.li_argmax_rows(logits.data_ptr(), want.data_ptr(), sv.data_ptr(), si.data_ptr(), n, v, stream) == 0
+        torch.cuda.synchronize()
+        # the device's own count of free memory sees any hipMalloc or hipFree, also one made inside the
+        # library; torch's counter sees its own allocator only
+        before, free_before = torch.cuda.memory_allocated(dev), torch.cuda.mem_get_info(dev)[0]
         rc = lib.li_argmax_rows_noalloc(logits.data_ptr(), got.data_ptr(), n, v, stream)
         assert rc == 0, lib.li_argmax_rows_noalloc_error().decode()
         torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info(dev)[0] == free_before, "the device's free memory changed during the call"
         assert torch.cuda.memory_allocated(dev) == before
         assert torch.equal(got, want)
         assert torch.equal(got.cpu().long(), torch.argmax(logits.cpu(), dim=1))
