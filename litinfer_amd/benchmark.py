@@ -123,6 +123,50 @@ def spread(values: List[float], scale: float = 1.0, digits: int = 3) -> Dict[str
             "max": round(max(values) * scale, digits)}
 
 
+def environment(dev) -> Dict[str, object]:
+    """Where the numbers were measured (the reference's harness records the same kind of block:
+    scripts/benchmark_cpu.py:306-325): the GPU, the versions of the runtime, of the driver and of
+    torch, and the commit of this tree."""
+    import os
+    import platform
+    import subprocess
+    from pathlib import Path
+
+    import torch
+    env: Dict[str, object] = {"python": platform.python_version(), "torch": torch.__version__,
+                              "hip": getattr(torch.version, "hip", None), "os": platform.platform(),
+                              "command": sys.argv}
+    try:
+        p = torch.cuda.get_device_properties(dev)
+        env.update(gpu=p.name, arch=getattr(p, "gcnArchName", None), compute_units=p.multi_processor_count,
+                   memory_GiB=round(p.total_memory / 2 ** 30, 1))
+    except Exception as e:                               # (no GPU: the block still says where it ran)
+        env["gpu"] = f"unknown ({e})"
+    for name, path in (("driver", "/sys/module/amdgpu/version"), ("rocm", "/opt/rocm/.info/version")):
+        try:
+            env[name] = Path(path).read_text().strip()
+        except OSError:
+            env[name] = None
+    root = Path(__file__).resolve().parent.parent
+    try:
+        env["git_commit"] = subprocess.run(["git", "-C", str(root), "rev-parse", "HEAD"], capture_output=True,
+                                           text=True, timeout=10).stdout.strip() or None
+        env["git_dirty"] = bool(subprocess.run(["git", "-C", str(root), "status", "--porcelain", "--untracked-files=no"],
+                                               capture_output=True, text=True, timeout=10).stdout.strip())
+    except (OSError, subprocess.SubprocessError):
+        env["git_commit"] = None
+    # the tree may be a copy without its history: a digest of the package's sources names it all the same
+    import hashlib
+    h = hashlib.sha256()
+    pkg = Path(__file__).resolve().parent
+    for f in sorted(list(pkg.rglob("*.py")) + list((pkg / "csrc").glob("*"))):
+        if f.is_file():
+            h.update(f.relative_to(pkg).as_posix().encode() + b"\0" + f.read_bytes())
+    env["source_digest"] = h.hexdigest()[:16]
+    env["omp_threads"] = os.environ.get("OMP_NUM_THREADS")
+    return env
+
+
 # ------------------------------------------------------- what the GPU reaches
 def measure_reference(dev) -> Dict[str, float]:
     """A kernel that only reads (and one that copies) 2 GiB, a loop of bfloat16 MFMAs and a
@@ -349,6 +393,12 @@ def headline(a) -> Dict[str, object]:
         return round(nbytes / seconds / HBM_PEAK, 4)
 
     dt, ctx_tokens = loop.run(a.batch, a.steps, a.warmup, CONTEXT)
+    # the headline is that first timing of exactly `steps` steps; it is repeated (each repeat: its own
+    # requests, warm-up and `steps` timed steps) for the spread
+    decode_ms = [dt / a.steps * 1e3]
+    for _ in range(max(0, a.repeats - 1)):
+        d, _ = loop.run(a.batch, a.steps, a.warmup, CONTEXT)
+        decode_ms.append(d / a.steps * 1e3)
     ms = dt / a.steps * 1e3
     value = a.batch * a.steps / dt
     nbytes = decode_bytes(cfg, a.layers, ctx_tokens, es)
@@ -370,12 +420,13 @@ def headline(a) -> Dict[str, object]:
         "roofline": {"bound": "hbm", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1), "peak": HBM_PEAK / 1e9,
                      "unit": "GB/s", "frac": frac_of(nbytes, ms * 1e-3)},
     }
+    out["repeats"] = {"n": len(decode_ms), "decode_ms_per_step": spread(decode_ms, 1.0, 4)}
     if ref:
         out["roofline"]["frac_of_measured_read"] = round(nbytes / (ms * 1e-3) / (ref["read_GBps"] * 1e9), 4)
     if not a.no_prefill:
         prompt = rng.integers(0, cfg["vocab_size"], PREFILL_TOKENS).tolist()
         times = []
-        for i in range(5 if a.dtype == "bf16" else 3):       # one to warm up, the best of the rest
+        for i in range(1 + (max(a.repeats, 4) if a.dtype == "bf16" else max(a.repeats, 2))):   # one to warm up, the best of the rest
             torch.cuda.synchronize()
             t = time.perf_counter()
             logits = eng.step([StepEntry(f"p{i}", prompt, [PREFILL_TOKENS - 1])])
@@ -389,6 +440,7 @@ def headline(a) -> Dict[str, object]:
         flops = prefill_flops(cfg, a.layers, PREFILL_TOKENS)
         out["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS,
                           "ms": round(pt * 1e3, 3), "frac": round(flops / pt / FLOP_PEAK[a.dtype], 4)}
+        out["repeats"]["prefill_ms"] = spread(times[1:], 1e3, 3)
         if ref:
             measured = ref["mfma_bf16_TFLOPs"] if a.dtype == "bf16" else ref["fma_fp32_TFLOPs"]
             out["prefill"]["frac_of_measured_loop"] = round(flops / pt / (measured * 1e12), 4)
@@ -421,7 +473,39 @@ def headline(a) -> Dict[str, object]:
             log(f"scheduler, {b} requests: {r['tok_s']} generated tok/s over all, TTFT median {r['ttft_ms']['median']} ms, "
                 f"TPOT median {tpot} ms; while all decode: {ph}")
         out["scheduler"] = sch
+    out["environment"] = environment(dev)
+    if not a.no_points and not a.no_small:
+        # the reference's own benchmark model (DeepSeek-R1-Distill-Qwen-1.5B layer sizes), same run: decode at
+        # 1, 8 and 64 requests, context 4,096, each with its fraction of the HBM peak
+        del loop, eng
+        torch.cuda.empty_cache()
+        out["points_1p5b"] = small_points(a, dev, sampler, rng)
     return out
+
+
+def small_points(a, dev, sampler, rng) -> Dict[str, object]:
+    import torch
+    from .engine import Engine
+    cfg = dict(SHAPES["1.5b"])
+    layers = cfg["num_hidden_layers"]
+    es = 2 if a.dtype == "bf16" else 4
+    t0 = time.time()
+    eng = Engine.from_random(cfg, seed=0, dtype=ENGINE_DTYPE[a.dtype], device=dev, page_size=PAGE,
+                             num_pages=64 * CONTEXT // PAGE + 64, max_seqs=65,
+                             page_order_seed=None if a.page_order_seed < 0 else a.page_order_seed)
+    for g in eng.cache.groups:
+        for data in g.data.values():
+            data.view(-1).normal_(0, 0.5)
+    loop = StepLoop(eng, cfg, sampler, rng)
+    pts: Dict[str, object] = {"model": "DeepSeek-R1-Distill-Qwen-1.5B shape", "num_hidden_layers": layers, "context_len": CONTEXT}
+    for b in (1, 8, 64):
+        n = max(8, a.steps // 2) if b != 8 else a.steps
+        d, ctx_b = loop.run(b, n, 4, CONTEXT)
+        pts[f"decode_b{b}"] = {"tok_s": round(b * n / d, 1), "ms_per_step": round(d / n * 1e3, 4),
+                               "frac": round(decode_bytes(cfg, layers, ctx_b, es) / (d / n) / HBM_PEAK, 4)}
+    torch.cuda.synchronize()
+    log(f"1.5B shape in {time.time() - t0:.1f} s: {pts}")
+    return pts
 
 
 def sweep(a) -> Dict[str, object]:
@@ -559,6 +643,7 @@ def long_prompts(a) -> Dict[str, object]:
     warm = [(rng.integers(0, cfg["vocab_size"], 3000).tolist(), 4, SamplingParams())]
     run_scheduler(eng, cfg, warm, max_batch_tokens=chunk + n, chunk_size=chunk, what="warm-up")
     r = run_scheduler(eng, cfg, reqs, max_batch_tokens=chunk + n, chunk_size=chunk, what="long")
+    checked = check_long_decode(eng, cfg, reqs[0][0], chunk)
     # the prompts run one after the other in portions; the last request's first token marks their end
     prefill_s = r["ttft_ms"]["max"] * 1e-3
     flops = sum(prefill_flops(cfg, layers, min(chunk, plen - s), s) - 2.0 * cfg["vocab_size"] * cfg["hidden_size"]
@@ -586,7 +671,38 @@ def long_prompts(a) -> Dict[str, object]:
         "prefill": {"value": round(n * plen / prefill_s, 1), "tokens": n * plen, "ms": round(prefill_s * 1e3, 1),
                     "frac": round(flops / prefill_s / FLOP_PEAK[a.dtype], 4)},
         "scheduler": r,
+        "decode_row_checked": checked,
     }
+
+
+def check_long_decode(eng, cfg, prompt, chunk) -> Dict[str, object]:
+    """One request's prompt once more through the step function in portions, a few tokens decoded until
+    its step is a recorded one, and then one decoded row twice: as the engine runs it (replayed) and
+    eagerly.  The logits must agree to rounding (the reference's own regression at its longest lengths
+    compares tokens, test/test_kv_cache.py:52-66)."""
+    import numpy as np
+    import torch
+    from .engine import StepEntry
+    from .sampling import Sampler
+    t0 = time.time()
+    rid = "long_check"
+    logits = None
+    for o in range(0, len(prompt), chunk):
+        part = prompt[o:o + chunk]
+        logits = eng.step([StepEntry(rid, part, [len(part) - 1] if o + chunk >= len(prompt) else [])])
+    sampler = Sampler(eng.rt.device)
+    loop = StepLoop(eng, cfg, sampler, np.random.default_rng(3))
+    tok = int(torch.argmax(logits[0]))
+    replays = eng.graph_replays
+    for _ in range(eng.graph_after + 1):
+        logits = eng.step([StepEntry(rid, [tok], [0])])
+        tok = int(torch.argmax(logits[0]))
+    recorded = eng.graph_replays > replays
+    loop._check_against_eager([rid], [tok], 1)
+    eng.finish(rid)
+    out = {"context": len(prompt) + eng.graph_after + 2, "recorded_step": recorded, "seconds": round(time.time() - t0, 1)}
+    log(f"long: a decoded row behind {out['context']} keys, recorded against eager: equal to rounding ({out})")
+    return out
 
 
 def main(argv: Optional[List[str]] = None) -> int:
@@ -607,6 +723,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-scheduler", action="store_true", help="headline: skip the runs through the scheduler")
     ap.add_argument("--no-reference", action="store_true", help="headline: skip the measured read / MFMA rates")
+    ap.add_argument("--no-small", action="store_true", help="headline: skip the decode points at the 1.5B layer sizes")
+    ap.add_argument("--repeats", type=int, default=3, help="headline: timings of `steps` decode steps and of the prompt (median/min/max)")
     ap.add_argument("--requests", type=int, default=None, help="serving: number of requests (128); long: 8")
     ap.add_argument("--arrival-rate", type=float, default=32.0, help="serving: requests a second")
     ap.add_argument("--pool-tokens", type=int, default=None, help="serving: tokens the cache pool holds (default: all)")
@@ -630,6 +748,8 @@ def main(argv: Optional[List[str]] = None) -> int:
         out = serving(a)
     else:
         out = long_prompts(a)
+    if "environment" not in out:
+        out["environment"] = environment("cuda:0")
     print(json.dumps(out), flush=True)
     return 0
 

@@ -20,6 +20,7 @@ def lib() -> ctypes.CDLL:
             "li_pool_create": ([c_int, IP], c_void_p), "li_pool_destroy": ([c_void_p], None),
             "li_pool_error": ([c_void_p], c_char_p), "li_pool_capacity": ([c_void_p], c_int),
             "li_pool_free": ([c_void_p], c_int), "li_pool_total_allocations": ([c_void_p], c_long),
+            "li_pool_peak_used": ([c_void_p], c_int),
             "li_pool_alloc": ([c_void_p], c_int), "li_pool_release": ([c_void_p, c_int], c_int),
             "li_pool_is_held": ([c_void_p, c_int], c_int),
             "li_book_create": ([c_int, c_int, c_int, IP, IP, IP], c_void_p),

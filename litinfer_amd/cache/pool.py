@@ -56,6 +56,11 @@ class PagePool:
     def total_allocations(self) -> int:
         return self._lib.li_pool_total_allocations(self._p)
 
+    @property
+    def peak_used(self) -> int:
+        """The most pages that were held at one time so far."""
+        return self._lib.li_pool_peak_used(self._p)
+
     def alloc(self) -> int:
         p = self._lib.li_pool_alloc(self._p)
         if p < 0:

@@ -33,6 +33,7 @@ struct Pool {
     std::vector<int> free_list;            // alloc() pops from the end
     std::vector<char> held;
     long total_allocations = 0;
+    int peak_used = 0;                     // the most pages that were ever held at one time
     std::string error;
 
     bool init(int n, const int* order) {
@@ -63,6 +64,7 @@ struct Pool {
         if (held[p]) { error = "page pool: page " + std::to_string(p) + " was on the free list while held"; return ERR_POOL; }
         held[p] = 1;
         ++total_allocations;
+        peak_used = std::max(peak_used, used());
         return p;
     }
     int release(int p) {
@@ -126,6 +128,7 @@ const char* li_pool_error(void* p) { return ((Pool*)p)->error.c_str(); }
 int li_pool_capacity(void* p) { return ((Pool*)p)->capacity; }
 int li_pool_free(void* p) { return ((Pool*)p)->free_count(); }
 long li_pool_total_allocations(void* p) { return ((Pool*)p)->total_allocations; }
+int li_pool_peak_used(void* p) { return ((Pool*)p)->peak_used; }
 int li_pool_alloc(void* p) { return ((Pool*)p)->alloc(); }
 int li_pool_release(void* p, int page) { return ((Pool*)p)->release(page); }
 int li_pool_is_held(void* p, int page) {

@@ -1,6 +1,8 @@
 // Choosing the next token from float32 logits: argmax (lowest index on ties)
 // and temperature / top-k / top-p sampling by inverse CDF with a uniform
-// number that the host derives from the request's own counter-based stream.
+// number from the request's own counter-based stream, which the host derives or,
+// for requests whose sampling state lies in the per-slot table on the device
+// (li_sample_prepare), the device itself.
 #include "common.h"
 #include "li_noalloc.h"
 #include <math.h>
@@ -763,6 +765,58 @@ __global__ __launch_bounds__(SMP_NT) void sample_rows_kernel(
         }
         out[r] = pick;
     }
+}
+
+// ------------------------------------------------- sampling state of the live requests, on the device
+// One row of eight 32-bit words for every state slot of the cache: {temperature, top_p (float bits), top_k,
+// seed low, seed high, draws so far, 0, 0}.  The host writes a row when a request is bound to its slot and
+// never again; the device counts the draws.  (The reference keeps the same per sequence on the host:
+// src/llaisys/models/qwen2.hpp:100-110.)
+//
+// li_sample_prepare turns the rows of a step, given as slot | flags << 24 (flag 1: this row is greedy
+// whatever its slot says, e.g. a request's first token), into the per-row arrays that li_sample_rows takes:
+// temperature, top_k, top_p and the uniform number of the slot's next draw, the draws-th number of the
+// stream `seed`: a splitmix64 hash of both, its upper 24 bits as a value in [0, 1).  A row that samples
+// (temperature > 0) advances its slot's count.  A slot outside the table gives a greedy row.
+#define SAMPLE_SLOT_WORDS 8
+__device__ __forceinline__ float stream_uniform(unsigned long long seed, unsigned long long counter) {
+    unsigned long long z = seed * 0x9E3779B97F4A7C15ull + (counter + 1ull) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+__global__ void sample_prepare_kernel(const int* __restrict__ rows, int n, int* __restrict__ table, int nslots,
+                                      float* __restrict__ temperature, int* __restrict__ top_k,
+                                      float* __restrict__ top_p, float* __restrict__ uniform) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int slot = rows[i] & 0xffffff, flags = (rows[i] >> 24) & 0x7f;
+    float T = 0.f, P = 1.f, U = 0.f;
+    int K = 0;
+    if (slot < nslots && !(flags & 1)) {
+        int* row = table + (size_t)slot * SAMPLE_SLOT_WORDS;
+        T = __int_as_float(row[0]);
+        P = __int_as_float(row[1]);
+        K = row[2];
+        if (T > 0.f) {
+            const unsigned long long seed = (unsigned long long)(unsigned)row[3] | ((unsigned long long)(unsigned)row[4] << 32);
+            const int draws = row[5];
+            U = stream_uniform(seed, (unsigned long long)(unsigned)draws);
+            row[5] = draws + 1;                      // (a slot stands once in a step's rows: no two threads write it)
+        } else {
+            T = 0.f;
+        }
+    }
+    temperature[i] = T; top_k[i] = K; top_p[i] = P; uniform[i] = U;
+}
+
+extern "C" int li_sample_prepare(const int* rows, int n, int* table, int nslots, float* temperature, int* top_k,
+                                 float* top_p, float* uniform, hipStream_t stream) {
+    if (n <= 0 || nslots <= 0 || !rows || !table) return LI_ERR_SIZE;
+    sample_prepare_kernel<<<(n + 255) / 256, 256, 0, stream>>>(rows, n, table, nslots, temperature, top_k, top_p, uniform);
+    return li_launch_status();
 }
 
 // Floats of scratch memory that li_sample_rows needs for n rows of V logits.

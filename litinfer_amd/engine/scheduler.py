@@ -66,6 +66,9 @@ class Request:
     # lookahead: the request's newest token has been sampled but is not known here yet; it lies
     # at this place of the engine's feedback buffer
     pending_take: Optional[int] = None
+    # the state slot and the options that the sampler's table on the device holds for this request
+    # (None: not written yet, or the request has given its slot back)
+    bound: Optional[Tuple[int, SamplingParams]] = None
 
     @property
     def num_generated(self) -> int:
@@ -91,6 +94,15 @@ class Request:
         if len(out) < n:
             out.append(0)                              # the pending token's place
         return out
+
+
+class _Ready:
+    """Tokens that a sampler without an asynchronous call has already brought."""
+    def __init__(self, tokens):
+        self._tokens = list(tokens)
+
+    def result(self):
+        return self._tokens
 
 
 @dataclass
@@ -121,7 +133,7 @@ class Scheduler:
         self.row_tile = int(row_tile)
         self.max_running = int(max_running) if max_running else self.cache.max_seqs
         self.eos = tuple(engine.spec.eos_token_ids if eos_token_ids is None else eos_token_ids)
-        self.sampler = sampler if sampler is not None else Sampler(engine.rt.device)
+        self.sampler = sampler if sampler is not None else Sampler(engine.rt.device, slots=self.cache.max_seqs)
         self.waiting: Deque[Request] = deque()
         self.running: List[Request] = []          # in order of admission
         self.requests: Dict[Hashable, Request] = {}
@@ -196,7 +208,7 @@ class Scheduler:
     def _preempt(self, req: Request) -> None:
         self.running.remove(req)
         self.engine.finish(req.rid)
-        req.state, req.computed = WAITING, 0
+        req.state, req.computed, req.bound = WAITING, 0, None
         req.preemptions += 1
         self.preemptions += 1
         self.waiting.appendleft(req)
@@ -385,11 +397,11 @@ class Scheduler:
         if not self.lookahead:
             produced: List[Tuple[Hashable, int]] = []
             if sampled:
-                for r, tok in zip(sampled, self.sampler.sample(logits, params, counters)):
+                for r, tok in zip(sampled, self._sample(logits, sampled, params, counters, None).result()):
                     if self._append(r, int(tok)):
                         produced.append((r.rid, int(tok)))
             return produced
-        handle = self.sampler.sample_async(logits, params, counters, out=self.engine.feedback) if sampled else None
+        handle = self._sample(logits, sampled, params, counters, self.engine.feedback) if sampled else None
         produced = self._resolve()                   # the step before; the device is busy with this one
         if handle is not None:
             for i, r in enumerate(sampled):
@@ -397,6 +409,29 @@ class Scheduler:
                     r.pending_take = i
             self._inflight = (handle, sampled)
         return produced
+
+    def _sample(self, logits, sampled: List[Request], params, counters, out):
+        """Tokens for the rows of `logits`.  A sampler with a table on the device gets each row's state
+        slot and nothing else: a request's options and stream are written there once, when it first
+        samples in its slot (and again should its options change)."""
+        sampler = self.sampler
+        if getattr(sampler, "table", None) is None:
+            if hasattr(sampler, "sample_async"):
+                return sampler.sample_async(logits, params, counters, out=out) if out is not None else \
+                    sampler.sample_async(logits, params, counters)
+            return _Ready(sampler.sample(logits, params, counters))
+        slots, greedy = [], []
+        for r, sp, c in zip(sampled, params, counters):
+            if sp.greedy:
+                slots.append(0)
+                greedy.append(True)
+                continue
+            if r.bound is None or r.bound[1] is not sp and r.bound[1] != sp:
+                r.bound = (self.cache.slot(r.rid), sp)
+                sampler.bind(r.bound[0], sp, c)
+            slots.append(r.bound[0])
+            greedy.append(False)
+        return sampler.sample_bound_async(logits, slots, greedy, out=out)
 
     def _resolve(self) -> List[Tuple[Hashable, int]]:
         """The tokens of the step in flight have to be known now: wait for them and apply them."""
@@ -427,7 +462,7 @@ class Scheduler:
 
     def _finish(self, r: Request, reason: str) -> None:
         r.state, r.finish_reason = FINISHED, reason
-        r.pending_take = None
+        r.pending_take = r.bound = None
         if r in self.running:
             self.running.remove(r)
         elif r in self.waiting:                      # preempted while its last token was on its way

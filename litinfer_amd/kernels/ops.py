@@ -56,6 +56,7 @@ _SIGNATURES = {
     "sampling": {
         "li_argmax_rows": [P, P, P, P, I, I],
         "li_sample_rows": [P, P, P, P, P, P, I, I, P, L],
+        "li_sample_prepare": [P, I, P, I, P, P, P, P],
     },
 }
 _fn_cache = {}
@@ -845,3 +846,25 @@ def sample_rows(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Te
         tiles = _sample_scratch[key]
         _run("sampling", "li_sample_rows", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(),
              top_p.data_ptr(), uniform.data_ptr(), out.data_ptr(), n, v, tiles.data_ptr(), tiles.numel())
+
+
+SAMPLE_SLOT_WORDS = 8          # 32-bit words of a slot's row in the sampling table (csrc/sampling.hip)
+SAMPLE_ROW_GREEDY = 1 << 24    # flag of a step's row: greedy whatever its slot's row says
+
+
+def sample_prepare(rows: torch.Tensor, table: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+                   top_p: torch.Tensor, uniform: torch.Tensor) -> None:
+    """From the sampling table of the state slots (int32 [slots, 8]: temperature and top_p as float bits,
+    top_k, the seed's two halves, the draws so far) and a step's rows (int32: slot | flags << 24), the
+    per-row arrays that `sample_rows` takes; the uniform number of every sampling row is drawn on the
+    device from its slot's seed and count, and the count goes up."""
+    _gpu(rows, table, temperature, top_k, top_p, uniform)
+    n = rows.numel()
+    _chk(rows.dtype is torch.int32 and rows.is_contiguous(), "sample_prepare: rows must be int32")
+    _chk(table.dtype is torch.int32 and table.dim() == 2 and table.shape[1] == SAMPLE_SLOT_WORDS and table.is_contiguous(),
+         "sample_prepare: the table must be int32 [slots, 8]")
+    for t_, dt in ((temperature, torch.float32), (top_k, torch.int32), (top_p, torch.float32), (uniform, torch.float32)):
+        _chk(t_.dtype is dt and t_.numel() == n and t_.is_contiguous(), "sample_prepare: per-row arrays")
+    if n:
+        _run("sampling", "li_sample_prepare", rows.data_ptr(), n, table.data_ptr(), table.shape[0],
+             temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr())

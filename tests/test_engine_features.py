@@ -147,6 +147,39 @@ def test_seeded_sampling_does_not_depend_on_the_batch(tmp_path, device):
     assert len({tuple(t) for t in together}) == 4
 
 
+def test_the_sampling_table_on_the_device_gives_the_tokens_of_options_sent_with_every_step(tmp_path, device):
+    """The scheduler's own sampler keeps every live request's options, seed and count of draws in a table on
+    the device, a row per state slot, written once when the request first samples in its slot; each step
+    then sends the rows' slots only.  Same tokens as a sampler that is sent options and uniform numbers with
+    every step: with large and negative seeds, top-k and top-p, greedy requests in between, the first token
+    forced greedy, and with so few pages that requests are preempted and later go on in another slot."""
+    from litinfer_amd.engine import Scheduler
+    from litinfer_amd.sampling import Sampler, SamplingParams
+    d = helpers.make_model(tmp_path, TINY_B, 1)
+    prompts = list(helpers.random_requests(320, [3, 30, 70, 9, 41, 18], 21).values())
+    params = [SamplingParams(temperature=0.9, top_k=40, seed=2 ** 63 + 12345), None,
+              SamplingParams(temperature=1.3, top_p=0.8, seed=-7), SamplingParams(temperature=0.7, seed=3),
+              SamplingParams(), SamplingParams(temperature=1.0, top_k=5, top_p=0.9, seed=2 ** 40)]
+
+    def run(table, max_tokens, lookahead):
+        eng = engine_for(d, device, page=8, max_tokens=max_tokens)
+        sampler = Sampler(eng.rt.device, slots=eng.cache.max_seqs if table else 0)
+        s = Scheduler(eng, eos_token_ids=(), chunk_size=16, max_batch_tokens=40, lookahead=lookahead, sampler=sampler)
+        ids = [s.add_request(p, 20, sp, first_token_greedy=i % 2 == 0) for i, (p, sp) in enumerate(zip(prompts, params))]
+        s.run_to_completion()
+        eng.cache.check_invariants()
+        return [s.output(i) for i in ids], s.preemptions, sampler
+    want, pre, _ = run(False, 1024, False)
+    assert pre == 0 and all(len(t) == 20 for t in want)
+    got, pre, sampler = run(True, 1024, True)
+    assert got == want and pre == 0
+    assert sampler.table is not None and int(sampler.table[:, 5].max()) >= 19          # draws were counted on the device
+    got, pre, _ = run(True, 136, True)
+    assert got == want and pre > 0
+    got, pre, _ = run(True, 136, False)
+    assert got == want and pre > 0
+
+
 def test_step_refuses_bad_batches_and_leaves_the_cache_alone(tmp_path, device):
     d = helpers.make_model(tmp_path, TINY_A, 0)
     eng = engine_for(d, device, max_tokens=64)
@@ -525,12 +558,16 @@ def test_a_toy_mixer_keeps_one_latent_vector_per_token_in_pages(tmp_path, device
         g = eng.cache.groups
         assert len(g) == 1 and set(g[0].data) == {"c"} and g[0].data["c"].shape[2:] == (8, 12)
         assert g[0].data["c"].dtype is torch.float32 and g[0].entries == [0, 1]
-        assert eng.model.batch_needs() == BatchNeeds()         # nobody here wants tiles or token lists laid out
+        needs = eng.model.batch_needs()
+        assert (needs.tile_rows, needs.token_kinds) == (0, False)        # nobody here wants tiles or token lists laid out
         out = schedules.run(eng, reqs, steps)
         assert max(schedules.rel_err(out[r], ref[r]) for r in reqs) < F32_TOL, kind
         eng.cache.check_invariants()
     # the architecture's own model does ask for them, through its attention
-    assert engine_for(helpers.make_model(tmp_path / "a", TINY_A, 0), device).model.batch_needs() == BatchNeeds(32, True)
+    needs = engine_for(helpers.make_model(tmp_path / "a", TINY_A, 0), device).model.batch_needs()
+    assert (needs.tile_rows, needs.token_kinds) == (32, True)
+    # and its products say in which tiles they take a step's rows (the kernel library's number; none on the stand-ins)
+    assert needs.row_tile == (64 if device != "cpu" else 1)
 
 
 # --------- a toy feed-forward with routing and a toy position encoding, defined here

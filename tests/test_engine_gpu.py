@@ -155,3 +155,57 @@ def test_a_checkpoint_in_another_precision_runs_the_bfloat16_kernels(tmp_path, n
     worst = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
     print(f"[observed] {name} stored {stored} in the bfloat16 engine, mixed: {worst:.3e}")
     assert worst < TOL["bfloat16"], f"{name} {stored}: {worst}"
+
+
+def test_a_prompt_of_twelve_thousand_tokens_in_portions_of_2048_then_decoding(tmp_path):
+    """The lengths of the long-prompt workload at the engine's level: block tables of hundreds of pages,
+    portions of 2,048 behind up to 10,000 cached keys (their keys cut into runs), then single tokens over
+    12,000 keys; logits at a few rows of every portion and at every decoded token against the plain
+    implementation."""
+    from litinfer_amd.engine import StepEntry
+    cfg = dict(TINY_E, max_position_embeddings=16384)
+    d = helpers.make_model(tmp_path, cfg, 61, torch.bfloat16)
+    n, tail = 12000, 8
+    toks = helpers.random_requests(cfg["vocab_size"], [n + tail], 62)["r0"]
+    ref = helpers.plain_logits(d, {"r0": toks})["r0"]
+    eng = _engine(d, "bfloat16", TINY_E_PAGE, n + 64)
+    got, start = {}, 0
+    while start < n:
+        size = min(2048, n - start)
+        want = sorted({0, size // 3, size - 1})
+        out = eng.step([StepEntry("r0", toks[start:start + size], want)]).cpu().numpy()
+        got.update({start + w: row for w, row in zip(want, out)})
+        start += size
+    for i in range(tail):
+        got[n + i] = eng.step([StepEntry("r0", [toks[n + i]], [0])]).cpu().numpy()[0]
+    worst = max(schedules.rel_err(v, ref[p]) for p, v in got.items())
+    print(f"[observed] prompt of 12,000 tokens in portions of 2,048, then 8 tokens: {worst:.3e}")
+    assert worst < TOL["bfloat16"], worst
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "D"])
+def test_the_windowed_groups_pool_at_its_minimum(models, name, dt):
+    """Every page group has a pool of its own size.  The mixed schedule once with roomy pools, which shows
+    the most pages each group ever held at a time, then with exactly that many: the windowed layers' pool
+    is a fraction of the other, its pages go round many times, no step runs out, and the logits are the
+    plain implementation's."""
+    cfg, page, _ = CASES[name]
+    d, reqs, ref = models[(name, dt)]
+    steps = schedules.mixed(reqs)
+    roomy = _engine(d, dt, page, 4 * 128)
+    schedules.run(roomy, reqs, steps)
+    peaks = [g.pool.peak_used for g in roomy.cache.groups]
+    windows = [g.need.window for g in roomy.cache.groups]
+    assert windows[0] == 0 and windows[1] == cfg["sliding_window"] and peaks[1] < peaks[0]
+    from litinfer_amd.engine import Engine
+    eng = Engine.from_dir(d, dtype=dt, device="cuda:0", page_size=page, num_pages=peaks, max_seqs=4, page_order_seed=11)
+    assert [g.pool.capacity for g in eng.cache.groups] == peaks
+    assert eng.cache.groups[1].data["k"].shape[1] == peaks[1]
+    out = schedules.run(eng, reqs, steps)
+    eng.cache.check_invariants()
+    assert [g.pool.peak_used for g in eng.cache.groups] == peaks and eng.cache.free_pages() == peaks
+    assert eng.cache.groups[1].pool.total_allocations > peaks[1]          # its pages were used again
+    worst = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
+    print(f"[observed] {name} {dt} pools of {peaks} pages: {worst:.3e}")
+    assert worst < TOL[dt], worst

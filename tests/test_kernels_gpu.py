@@ -406,12 +406,15 @@ def test_rope(ops, dtype, t, heads, dh, theta, start):
     assert rel(xd, ref) < tol(dtype, 2e-4 if start else 2e-6, 8e-3)
 
 
-def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_one=None, row=None, ws=None):
+def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_one=None, row=None, ws=None,
+                pad_pow2=False):
     """seg_specs: list of (ctx_len, q_len).  Builds random K/V for every
     segment, scatters them into shuffled pages, and compares the kernel with
     the plain attention on the logical sequences.  `scale_one` is the index of a
     key that is made to stand out for query `row` of its segment (the last one
-    when `row` is None)."""
+    when `row` is None).  `pad_pow2`: the block table is widened to the next power
+    of two and the decode kernel is told the table's width as its longest context,
+    as a recorded decode step sees its batch."""
     g = torch.Generator().manual_seed(seed)
     nseg = len(seg_specs)
     blocks = [-(-c // page) for c, _ in seg_specs]
@@ -419,7 +422,8 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
     perm = torch.randperm(num_pages, generator=g).tolist()
     kc = torch.randn(num_pages, nkv, page, dh, generator=g).to(dtype)      # garbage everywhere first
     vc = torch.randn(num_pages, nkv, page, dh, generator=g).to(dtype)
-    tab = np.full((nseg, max(blocks)), -1, dtype=np.int32)
+    width = max(blocks) if not pad_pow2 else max(16, 1 << (max(blocks) - 1).bit_length())
+    tab = np.full((nseg, width), -1, dtype=np.int32)
     T = sum(q for _, q in seg_specs)
     q = (torch.randn(T, nh * dh, generator=g)).to(dtype)
     ks, vs = [], []
@@ -460,7 +464,7 @@ def _paged_case(ops, dtype, seg_specs, nh, nkv, dh, page, window, seed, scale_on
                                                for i in range(nseg) if q_len[i] > 1
                                                for a in range(0, int(q_len[i]), 32)], dtype=np.int32).reshape(-1, 4)),
                          num_tiles=sum(-(-int(n) // 32) for n in q_len if n > 1), tile_rows=32,
-                         max_single_ctx=int(ctx_len[q_len == 1].max()) if len(single) else 0)
+                         max_single_ctx=(width * page if pad_pow2 else int(ctx_len[q_len == 1].max())) if len(single) else 0)
     out = torch.empty(T, nh * dh, dtype=dtype, device=DEV)
     scale = 1.0 / math.sqrt(dh)
     ops.paged_attention(q.to(DEV), out, kc.to(DEV), vc.to(DEV), meta, nh, nkv, dh, page, window, scale, ws=ws)
@@ -580,6 +584,50 @@ def test_prompt_portions_behind_long_contexts_with_their_keys_in_runs(ops, segs,
     for far in (5, 1000, 2900):
         out, ref = _paged_case(ops, torch.bfloat16, [(3000, 64)], 28, 4, 128, 16, 0, seed=32, scale_one=far, row=40, ws=_Lender())
         assert rel(out, ref) < 1.5e-2
+
+
+# ---- the context lengths of the long workloads (8 x 30,000-token prompts in portions of 2,048, then decoding):
+# block tables of 1,875 to 2,048 pages, a portion behind 28,000 cached keys, splits of many pages
+@pytest.mark.parametrize("pad_pow2", [False, True])
+@pytest.mark.parametrize("far", [3, 15000, 29940])
+def test_decoding_over_thirty_thousand_keys_finds_one_far_key(ops, far, pad_pow2):
+    """Eight requests of 30,000 keys each, pages of 16, 40 heads on 8 kv heads of size 128: one key of every
+    request, near the start, in the middle or near the end, carries nearly all the weight.  Also with the
+    block table widened to 2,048 pages, as a recorded step sees it."""
+    segs = [(30000 - 7 * i, 1) for i in range(8)]
+    out, ref = _paged_case(ops, torch.bfloat16, segs, 40, 8, 128, 16, 0, seed=51, scale_one=far, ws=_Lender(),
+                           pad_pow2=pad_pow2)
+    assert rel(out, ref) < 8e-3
+
+
+@pytest.mark.parametrize("page,ctx,window", [(1, 5000, 0), (2, 8400, 0), (1, 6000, 4500)])
+def test_decode_splits_that_would_hold_more_pages_than_the_kernel_keeps_get_more_runs(ops, page, ctx, window):
+    """Many requests with small pages: the number of runs that fills the SIMDs once would give every run
+    more than the 1,024 pages the matrix-core decode kernel keeps in LDS, so the host raises the number
+    of runs until a run fits; a far key in the first, a middle and the last run."""
+    from litinfer_amd.kernels import ops as O
+    n, nkv = 64, 4
+    segs = [(ctx - 3 * i, 1) for i in range(n)]
+    blocks = -(-ctx // page)
+    keys = min(ctx, window) if window else ctx
+    planned = O.decode_splits(n * nkv, keys, O._simd_count(torch.device(DEV)))
+    assert O.decode_split_blocks(blocks, page, window, planned) > O.DECODE_TABLE_CAP      # the case is what it says
+    for far in (ctx - 3 * n - 5, ctx // 2, max(ctx - window, 0) + 7 if window else 2):
+        out, ref = _paged_case(ops, torch.bfloat16, segs, 8, nkv, 64, page, window, seed=52, scale_one=far, ws=_Lender())
+        assert rel(out, ref) < 8e-3
+
+
+@pytest.mark.parametrize("far", [5, 14000, 29000])
+def test_a_portion_of_2048_behind_28000_cached_keys_finds_one_far_key(ops, far):
+    """A prompt portion of 2,048 queries behind 28,000 cached keys (pages of 16: a block table of 1,878
+    pages), its tiles' keys cut into runs that are joined afterwards: one key in the first, a middle or
+    the last run stands out for one row; all rows against the plain attention."""
+    from litinfer_amd.kernels.ops import _prefill_runs
+    segs, nh, nkv, dh, page = [(30048, 2048)], 8, 2, 128, 16
+    ql, cl = np.array([2048], dtype=np.int32), np.array([30048], dtype=np.int32)
+    assert _prefill_runs(ql, cl, nh, nkv, dh, -(-30048 // page), 0, 2048) > 1             # the case is what it says
+    out, ref = _paged_case(ops, torch.bfloat16, segs, nh, nkv, dh, page, 0, seed=53, scale_one=far, row=1500, ws=_Lender())
+    assert rel(out, ref) < 1.5e-2
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -904,3 +952,31 @@ def test_sample_rows_frequencies_and_ties(ops):
     assert set(_sample(ops, lg.repeat(500, 1), [1.0] * 500, [3] * 500, [1.0] * 500, u[:500])) == {2, 3, 6}
     # top_p = 0.5: the shortest prefix reaching half the mass is {2, 3}
     assert set(_sample(ops, lg.repeat(500, 1), [1.0] * 500, [0] * 500, [0.5] * 500, u[:500])) == {2, 3}
+
+
+def test_sampling_table_rows_become_the_arrays_of_a_step_with_uniform_numbers_drawn_on_the_device(ops):
+    """li_sample_prepare against the host's stream: the same uniform numbers bit for bit for any seed and
+    count, a count that goes up for sampling rows only, greedy flags, slots outside the table."""
+    from litinfer_amd.sampling import Sampler, SamplingParams, uniform
+    smp = Sampler(DEV, slots=6)
+    opts = [SamplingParams(temperature=0.8, top_k=7, top_p=0.9, seed=0), SamplingParams(temperature=1.5, seed=2 ** 64 - 1),
+            SamplingParams(), SamplingParams(temperature=0.3, top_p=0.5, seed=-12345678901234),
+            SamplingParams(temperature=1.0, seed=0x9E3779B97F4A7C15)]
+    draws = [0, 5, 0, 2 ** 31 - 3, 1000000]
+    for slot, (sp, c) in enumerate(zip(opts, draws)):
+        smp.bind(slot, sp, c)
+    rows = torch.tensor([4, 0, 3 | ops.SAMPLE_ROW_GREEDY, 2, 1, 5, 77], dtype=torch.int32, device=DEV)
+    n = rows.numel()
+    t, p, u = (torch.full((n,), -1.0, device=DEV) for _ in range(3))
+    k = torch.full((n,), -1, dtype=torch.int32, device=DEV)
+    for step in range(3):
+        ops.sample_prepare(rows, smp.table, t, k, p, u)
+        for i, slot in enumerate((4, 0, None, 2, 1, None, None)):      # None: greedy by flag, an unbound row, outside the table
+            if slot is None or opts[slot].greedy:
+                assert float(t[i]) == 0.0 and float(u[i]) == 0.0
+                continue
+            sp = opts[slot]
+            assert float(t[i]) == np.float32(sp.temperature) and int(k[i]) == sp.top_k and float(p[i]) == np.float32(sp.top_p)
+            assert float(u[i]) == uniform(sp.seed, draws[slot] + step), (slot, step)
+    counts = smp.table[:, 5].cpu().tolist()
+    assert counts == [3, 8, 0, draws[3], 1000003, 0]               # slot 3 was greedy by flag: its count stayed

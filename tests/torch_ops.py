@@ -239,3 +239,28 @@ def sample_rows(logits, temperature, top_k, top_p, uniform, out):
 
 
 ALL.append("sample_rows")
+
+
+def sample_prepare(rows, table, temperature, top_k, top_p, uniform):
+    """The device's per-slot sampling table (csrc/sampling.hip, sample_prepare_kernel) written out on the host."""
+    import numpy as np
+    from litinfer_amd.sampling import uniform as stream_uniform
+    nslots = table.shape[0]
+    for i, word in enumerate(rows.tolist()):
+        slot, flags = word & 0xffffff, (word >> 24) & 0x7f
+        t, p, k, u = 0.0, 1.0, 0, 0.0
+        if slot < nslots and not flags & 1:
+            row = table[slot]
+            t = float(row[0:1].view(torch.float32))
+            p = float(row[1:2].view(torch.float32))
+            k = int(row[2])
+            if t > 0:
+                seed = (int(row[3]) & 0xffffffff) | ((int(row[4]) & 0xffffffff) << 32)
+                u = stream_uniform(seed, int(row[5]) & 0xffffffff)
+                row[5] += 1
+            else:
+                t = 0.0
+        temperature[i], top_k[i], top_p[i], uniform[i] = t, k, p, u
+
+
+ALL.append("sample_prepare")
