@@ -430,6 +430,34 @@ union frag8 { u32x4 raw; bf16x8_t v; };
 // probability is exactly 0 and the finite value it brings adds nothing); a lane without a head or
 // a dimension of its own repeats a neighbour's work and stores nothing.
 
+// Orders a wave's own LDS writes before its own later LDS reads (other lanes' data included: a wave's LDS
+// instructions are carried out in the order of their issue), without the block's barrier.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Stores and loads that other compute units' blocks of the SAME kernel can rely on: they go through to
+// memory (each of the chip's eight L2 caches serves its own compute units only, and ordinary stores may
+// stay in the writer's).  A device-wide fence would do the same for ordinary accesses, but it writes back
+// and invalidates a whole L2 every time: with hundreds of blocks doing so a decode attention took 27 us more.
+__device__ __forceinline__ void store_through(float* p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_through(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// two floats that lie side by side (8-byte aligned), in one load
+__device__ __forceinline__ void load_through2(const float* p, float& a, float& b) {
+    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+    a = __uint_as_float((unsigned)(v & 0xffffffffull));
+    b = __uint_as_float((unsigned)(v >> 32));
+}
+// all of this wave's loads and stores have been carried out (stores: have arrived where they go)
+#define LI_WAIT_ALL_VMEM() __builtin_amdgcn_s_waitcnt(0x0F70)
+
 #define DEC_TABLE_CAP 1024      // pages of one split that fit the kernel's copy of the block table
 
 // The most pages one of `nsplit` splits can touch, for block tables of max_blocks pages.
@@ -453,11 +481,14 @@ extern "C" long li_decode_split_blocks(int max_blocks, int page_size, int window
 // then the items, token | run << 16, a token's runs in a row: the decode kernel starts a block for every
 // item the grid could hold (tokens x nsplit) and those beyond [1] end at once, without a look at their
 // token.  At most RUN_KEYS_MAX_TOKENS tokens (the host checks).
+// `group` > 1: the decode kernel's blocks take `group` runs of a token that follow each other, one a wave
+// (a block with fewer runs still holds `group` SIMDs): the items are then the FIRST runs of such groups
+// (run 0, group, 2 group, ...), [1] counts them, and a candidate length costs its groups x `group` waves.
 #define RUN_KEYS_MAX_TOKENS 4096
 __global__ __launch_bounds__(256) void decode_run_keys_kernel(
     const int* __restrict__ token_list, int n_tokens, const int* __restrict__ seg_of_token,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
-    int cap_keys, int window, int nkv, int nsplit, int simds, int* __restrict__ out) {
+    int cap_keys, int window, int nkv, int nsplit, int simds, int group, int* __restrict__ out) {
     __shared__ int nkeys[RUN_KEYS_MAX_TOKENS];
     __shared__ int red_i[4];
     __shared__ unsigned long long red_c[4];
@@ -490,7 +521,7 @@ __global__ __launch_bounds__(256) void decode_run_keys_kernel(
     const int c = lower + 32 * stride * tid;
     if (c <= cap) {
         long waves = 0;
-        for (int i = 0; i < n_tokens; ++i) waves += (nkeys[i] + c - 1) / c;
+        for (int i = 0; i < n_tokens; ++i) waves += ((nkeys[i] + c - 1) / c + group - 1) / group * group;
         waves *= nkv;
         const long rounds = (waves + simds - 1) / simds;
         best = ((unsigned long long)(rounds * (c + 24)) << 32) | (unsigned)c;
@@ -512,7 +543,7 @@ __global__ __launch_bounds__(256) void decode_run_keys_kernel(
     const int each = (n_tokens + 255) / 256;
     const int i0 = tid * each, i1 = i0 + each < n_tokens ? i0 + each : n_tokens;
     int mine = 0;
-    for (int i = i0; i < i1; ++i) mine += (nkeys[i] + per - 1) / per;
+    for (int i = i0; i < i1; ++i) mine += ((nkeys[i] + per - 1) / per + group - 1) / group;
     first[tid] = mine;
     __syncthreads();
     if (tid == 0) {
@@ -528,71 +559,100 @@ __global__ __launch_bounds__(256) void decode_run_keys_kernel(
     for (int i = i0; i < i1; ++i) {
         const int n = (nkeys[i] + per - 1) / per;
         nruns[i] = n;
-        for (int r = 0; r < n; ++r) items[at + r] = i | (r << 16);
-        at += n;
+        const int ng = (n + group - 1) / group;
+        for (int r = 0; r < ng; ++r) items[at + r] = i | ((r * group) << 16);
+        at += ng;
     }
 }
 
 extern "C" int li_decode_run_keys(const int* token_list, int n_tokens, const int* seg_of_token, const int* q_start,
                                   const int* q_len, const int* ctx_len, int max_blocks, int page_size, int window,
-                                  int nkv, int nsplit, int simds, int* out, hipStream_t stream) {
+                                  int nkv, int nsplit, int simds, int group, int* out, hipStream_t stream) {
     if (n_tokens <= 0 || n_tokens > RUN_KEYS_MAX_TOKENS || max_blocks <= 0 || page_size <= 0 || nkv <= 0 ||
-        nsplit <= 0 || nsplit > 0x7fff || simds <= 0 || !out)
+        nsplit <= 0 || nsplit > 0x7fff || simds <= 0 || group <= 0 || !out)
         return LI_ERR_SIZE;
     long keys = (long)max_blocks * page_size;
     if (window > 0 && window < keys) keys = window;
     if (keys > 0x7fffffffL - 64) return LI_ERR_SIZE;
     decode_run_keys_kernel<<<1, 256, 0, stream>>>(token_list, n_tokens, seg_of_token, q_start, q_len, ctx_len,
-                                                  (int)keys, window, nkv, nsplit, simds, out);
+                                                  (int)keys, window, nkv, nsplit, simds, group, out);
     return li_launch_status();
 }
 
-template <int DH>
-__global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
+// WAVES is 1 or 4.  With four, a block takes four runs of the keys of its (token, kv head) that follow each
+// other, one a wave (a wave works alone through its run: no barrier in the loop, the runs' lengths may differ),
+// and joins their results in LDS, in the order of the runs; `nsplit` then counts such blocks ("quads") and is
+// the number of partial results a (token, head) has in part_acc / part_ml.  With one quad the block writes
+// the output itself.  With more, the block that finishes last for a (token, kv head) joins the quads'
+// results in quad order and writes the output, so that no second kernel is needed: every block adds 1 to
+// `done[token * nkv + kv head]` after its results have been made visible to the device, and the block that
+// finds the count complete sets it back to 0 (the array is zero before the first call and after every
+// call).  Nobody waits for anybody.
+template <int WAVES> struct DecodeJoin {
+    float ml[WAVES][16][2];                       // per wave and head of the pass: maximum, sum
+    float acc[WAVES][16][ATT_MAX_DH / 2];         // per wave and head: the unscaled output (DH <= 128)
+    int last;
+};
+template <> struct DecodeJoin<1> { int last; };
+
+template <int DH, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
     const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ token_list, const int* __restrict__ seg_of_token,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
     float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv, int page_size,
-    int num_pages, int window, float scale, int nsplit, const int* __restrict__ run_keys, int n_list) {
+    int num_pages, int window, float scale, int nsplit, const int* __restrict__ run_keys, int n_list,
+    int* __restrict__ done) {
+    static_assert(DH <= ATT_MAX_DH / 2, "the join buffer holds head sizes up to 128");
     constexpr int KS = DH / 32;                 // MFMA steps of Q K^T
     constexpr int NS = (DH + 127) / 128;        // slabs of 128 output dimensions
     constexpr int QD = DH / 4;                  // head dimensions owned by one lane group in Q K^T
     constexpr int PSTRIDE = 40;                 // halves per row of P in LDS (32 keys + pad, 80 bytes)
-    __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * PSTRIDE];
-    __shared__ int pages[DEC_TABLE_CAP];
-    // run_keys given: block x takes the x-th (token, run) item of the list behind it, and ends at once if the
-    // list is shorter (blocks go to the XCDs in turn, in the order of their numbers, so every XCD gets its
-    // share of the runs that have keys).  Else block (token, kv head, run) of the grid.
-    int ti = blockIdx.x, split = blockIdx.z;
+    __shared__ __attribute__((aligned(16))) uint16_t p_lds_all[WAVES][16 * PSTRIDE];
+    __shared__ int pages_all[WAVES][DEC_TABLE_CAP];
+    __shared__ DecodeJoin<WAVES> join;
+    const int wave = WAVES > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
+    uint16_t* p_lds = p_lds_all[wave];
+    int* pages = pages_all[wave];
+    const int nruns_all = nsplit * WAVES;       // runs that the keys are cut into at most
+    // run_keys given: block x takes the x-th item of the list behind it, a (token, first run) pair, and ends
+    // at once if the list is shorter (blocks go to the XCDs in turn, in the order of their numbers, so every
+    // XCD gets its share of the runs that have keys).  Else block (token, kv head, quad) of the grid.
+    int ti = blockIdx.x, quad = blockIdx.z;
     const int kvh = blockIdx.y;
+    int quads_of_token = nsplit;
     if (run_keys) {
         const int count = run_keys[1];
         const int item = run_keys[2 + n_list + blockIdx.x];
         if ((int)blockIdx.x >= count) return;
         ti = item & 0xffff;
-        split = item >> 16;
+        quad = (item >> 16) / WAVES;
+        const int nr = run_keys[2 + ti];
+        quads_of_token = (nr + WAVES - 1) / WAVES;
+        quads_of_token = quads_of_token < 1 ? 1 : (quads_of_token > nsplit ? nsplit : quads_of_token);
     }
+    const int split = quad * WAVES + wave;
     const int t = token_list ? token_list[ti] : ti;
     const int G = nh / nkv;
     const int s = seg_of_token[t];
     const int p = ctx_len[s] - q_len[s] + (t - q_start[s]);
     const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     const int nkeys = p - lo + 1;
-    int per = (((nkeys + nsplit - 1) / nsplit) + 31) & ~31;
+    int per = (((nkeys + nruns_all - 1) / nruns_all) + 31) & ~31;
     if (run_keys) {
         // one run length for the whole batch (decode_run_keys_kernel): never shorter than this token's keys
-        // need to fit nsplit runs, never longer than the runs the host sized the page table in LDS for
+        // need to fit the runs, never longer than the runs the host sized the page table in LDS for
         long widest = (long)max_blocks * page_size;
         if (window > 0 && window < widest) widest = window;
-        const int cap = (int)((((widest + nsplit - 1) / nsplit) + 31) & ~31L);
+        const int cap = (int)((((widest + nruns_all - 1) / nruns_all) + 31) & ~31L);
         int given = (run_keys[0] + 31) & ~31;
         given = given < cap ? given : cap;
         per = given > per ? given : per;
     }
     const int k_begin = lo + split * per;
     const int k_end = (k_begin + per < p + 1) ? k_begin + per : p + 1;
-    const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
+    const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
     // The block table of this split goes to LDS first: a page number fetched from global
     // memory in the loop would make every wait for it a wait for all loads issued before.
     const int first_block = k_begin / page_size;
@@ -601,7 +661,7 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
         const int* table = block_table + (size_t)s * max_blocks + first_block;
         for (int i = lane; i < nblocks && i < DEC_TABLE_CAP; i += 64) pages[i] = table[i];
     }
-    __syncthreads();
+    wave_lds_sync();
     auto row_of = [&](int key, bool& ok) -> size_t {       // element offset of the key's row in a cache layer
         ok = key < k_end;
         key = ok ? key : k_end - 1;                        // (only called when k_begin < k_end)
@@ -677,11 +737,11 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
                 l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];                                        \
                 m[r] = mx;                                                                           \
             }                                                                                        \
-            __syncthreads();                                    /* readers of the last block's P are done */ \
+            wave_lds_sync();                                    /* readers of the last block's P are done */ \
             _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                         \
                 _Pragma("unroll") for (int r = 0; r < 4; ++r)                                        \
                     p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = float_to_bf16(pr[tt][r]);           \
-            __syncthreads();                                                                         \
+            wave_lds_sync();                                                                         \
             frag8 pa;                                                                                \
             pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);                   \
             /* ---- O = alpha O + P V */                                                             \
@@ -709,31 +769,122 @@ __global__ __launch_bounds__(64) void paged_attention_decode_mfma_kernel(
 #undef LI_DEC_LOAD_V
 #pragma unroll
         for (int r = 0; r < 4; ++r) l[r] = row16_sum(l[r]);
+        if constexpr (WAVES == 1) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int hr = 4 * g + r;
-            if (hr >= gcount) continue;
-            const int head = kvh * G + h0 + hr;
-            if (nsplit == 1) {
-                const float inv = l[r] != 0.f ? 1.0f / l[r] : 0.f;
-                bf16_t* orow = out + (size_t)t * nh * DH + (size_t)head * DH;
+            for (int r = 0; r < 4; ++r) {
+                const int hr = 4 * g + r;
+                if (hr >= gcount) continue;
+                const int head = kvh * G + h0 + hr;
+                if (nsplit == 1) {
+                    const float inv = l[r] != 0.f ? 1.0f / l[r] : 0.f;
+                    bf16_t* orow = out + (size_t)t * nh * DH + (size_t)head * DH;
+#pragma unroll
+                    for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+                        for (int jj = 0; jj < 8; ++jj) {
+                            const int d = 128 * ns + 8 * c + jj;
+                            if (d < DH) orow[d].bits = float_to_bf16(acc[ns][jj][r] * inv);
+                        }
+                } else {
+                    const size_t pi = ((size_t)ti * nh + head) * nsplit + split;
+#pragma unroll
+                    for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+                        for (int jj = 0; jj < 8; ++jj) {
+                            const int d = 128 * ns + 8 * c + jj;
+                            if (d < DH) part_acc[pi * DH + d] = acc[ns][jj][r];
+                        }
+                    if (c == 0) { part_ml[pi * 2] = m[r]; part_ml[pi * 2 + 1] = l[r]; }
+                }
+            }
+        } else {
+            // ---- the four runs of this block, joined in LDS in the order of the runs
+            __syncthreads();                                        // (the last pass's readers are done)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int hr = 4 * g + r;
 #pragma unroll
                 for (int ns = 0; ns < NS; ++ns)
 #pragma unroll
                     for (int jj = 0; jj < 8; ++jj) {
                         const int d = 128 * ns + 8 * c + jj;
-                        if (d < DH) orow[d].bits = float_to_bf16(acc[ns][jj][r] * inv);
+                        if (d < DH) join.acc[wave][hr][d] = acc[ns][jj][r];
                     }
-            } else {
-                const size_t pi = ((size_t)ti * nh + head) * nsplit + split;
+                if (c == 0) { join.ml[wave][hr][0] = m[r]; join.ml[wave][hr][1] = l[r]; }
+            }
+            __syncthreads();
+            for (int e = threadIdx.x; e < gcount * DH; e += 64 * WAVES) {
+                const int hr = e / DH, d = e - hr * DH;
+                float mx = join.ml[0][hr][0];
 #pragma unroll
-                for (int ns = 0; ns < NS; ++ns)
+                for (int w = 1; w < WAVES; ++w) mx = fmaxf(mx, join.ml[w][hr][0]);
+                float lt = 0.f, at = 0.f;
 #pragma unroll
-                    for (int jj = 0; jj < 8; ++jj) {
-                        const int d = 128 * ns + 8 * c + jj;
-                        if (d < DH) part_acc[pi * DH + d] = acc[ns][jj][r];
-                    }
-                if (c == 0) { part_ml[pi * 2] = m[r]; part_ml[pi * 2 + 1] = l[r]; }
+                for (int w = 0; w < WAVES; ++w) {
+                    const float f = (mx == -INFINITY) ? 0.f : expf(join.ml[w][hr][0] - mx);
+                    lt += join.ml[w][hr][1] * f;
+                    at += join.acc[w][hr][d] * f;
+                }
+                const int head = kvh * G + h0 + hr;
+                if (nsplit == 1) {
+                    out[(size_t)t * nh * DH + (size_t)head * DH + d].bits = float_to_bf16(lt != 0.f ? at / lt : 0.f);
+                } else {
+                    const size_t pi = ((size_t)ti * nh + head) * nsplit + quad;
+                    store_through(&part_acc[pi * DH + d], at);
+                    if (d == 0) { store_through(&part_ml[pi * 2], mx); store_through(&part_ml[pi * 2 + 1], lt); }
+                }
+            }
+        }
+    }
+    if constexpr (WAVES > 1) {
+        if (nsplit > 1 && done) {
+            // ---- the quads of this (token, kv head): the block that finishes last joins them, in quad order.
+            // The partial results were stored through to memory; once every thread's stores have arrived,
+            // the block counts itself (an atomic carried out in memory), and the block that completes the
+            // count reads the others' results from memory, past its own L2.
+            LI_WAIT_ALL_VMEM();
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                const int before = atomicAdd(&done[ti * nkv + kvh], 1);
+                join.last = before == quads_of_token - 1;
+                if (join.last) atomicExch(&done[ti * nkv + kvh], 0);   // as the next call expects it
+            }
+            __syncthreads();
+            if (!join.last) return;
+            // A thread takes four neighbouring dimensions of one head and asks for everything it needs of all
+            // quads at once, never conditionally (a quad or head past the last repeats the last): one trip to
+            // memory for the whole join.
+            constexpr int TPH = DH / 4, HPC = 64 * WAVES / TPH;        // threads a head, heads a chunk of the block
+            for (int hb = 0; hb < G; hb += HPC) {
+                const int hg_own = hb + (int)threadIdx.x / TPH, hg = hg_own < G ? hg_own : G - 1;
+                const int d = 4 * ((int)threadIdx.x % TPH);
+                const int head = kvh * G + hg;
+                const size_t base = ((size_t)ti * nh + head) * nsplit;
+                float mq[16], lq[16], aq[16][4];                   // (quads <= MERGE_MAX_SPLITS / WAVES = 16)
+#pragma unroll
+                for (int qd = 0; qd < 16; ++qd) {
+                    const int q_ = qd < quads_of_token ? qd : quads_of_token - 1;
+                    load_through2(&part_ml[(base + q_) * 2], mq[qd], lq[qd]);
+                    load_through2(&part_acc[(base + q_) * DH + d], aq[qd][0], aq[qd][1]);
+                    load_through2(&part_acc[(base + q_) * DH + d + 2], aq[qd][2], aq[qd][3]);
+                }
+                float mx = -INFINITY;
+#pragma unroll
+                for (int qd = 0; qd < 16; ++qd) mx = fmaxf(mx, mq[qd]);
+                float lt = 0.f, at[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int qd = 0; qd < 16; ++qd) {
+                    const float f = (qd < quads_of_token && mx != -INFINITY) ? expf(mq[qd] - mx) : 0.f;
+                    lt += lq[qd] * f;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) at[i] += aq[qd][i] * f;
+                }
+                if (hg_own < G) {
+                    const float inv = lt != 0.f ? 1.0f / lt : 0.f;
+                    uint32_t* dst = reinterpret_cast<uint32_t*>(out + (size_t)t * nh * DH + (size_t)head * DH + d);
+                    dst[0] = pack2_bf16(at[0] * inv, at[1] * inv);
+                    dst[1] = pack2_bf16(at[2] * inv, at[3] * inv);
+                }
             }
         }
     }
@@ -1908,15 +2059,20 @@ static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, cons
 
 // Single-query tokens of the batch (token_list, or all tokens when it is null).
 // part_acc: float [n_tokens, nh, nsplit, dh]; part_ml: float [n_tokens, nh, nsplit, 2] (unused when nsplit is 1).
-// run_keys (may be null; the matrix-core kernel with nsplit > 1 only): one int on the device, the run
-// length li_decode_run_keys chose for this batch.
+// run_keys (may be null; the matrix-core kernel with nsplit > 1 only): what li_decode_run_keys (with group
+// LI_DECODE_QUAD) left on the device for this batch: the run length and the list of the runs that have keys.
+// The matrix-core kernel with nsplit > 1 takes nsplit as a multiple of LI_DECODE_QUAD (a block works through
+// that many runs and joins them) and needs `done`: int [n_tokens * nkv], zero before the first call; every
+// call leaves it zero.  Its blocks join their results themselves; the other kernels run a merge kernel.
+#define LI_DECODE_QUAD 4
+extern "C" int li_decode_quad(void) { return LI_DECODE_QUAD; }
 extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* out, const void* kc,
                                          const void* vc, int dtype, const int* block_table, int max_blocks,
                                          const int* token_list, int n_tokens, const int* seg_of_token,
                                          const int* q_start, const int* q_len, const int* ctx_len,
                                          float* part_acc, float* part_ml, int nh, int nkv, int dh,
                                          int page_size, int num_pages, int window, float scale, int nsplit,
-                                         int use_mfma, const int* run_keys, hipStream_t stream) {
+                                         int use_mfma, const int* run_keys, int* done, hipStream_t stream) {
     if (n_tokens <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || dh <= 0 || dh > ATT_MAX_DH || page_size <= 0 ||
         max_blocks <= 0)
         return LI_ERR_SIZE;
@@ -1931,20 +2087,47 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
         // a split's pages must fit the kernel's copy of the block table: `per` keys that begin
         // anywhere in a page touch at most (per + page_size - 2) / page_size + 1 pages
         if (li_decode_split_blocks(max_blocks, page_size, window, nsplit) > DEC_TABLE_CAP) return LI_ERR_SIZE;
-        const bool listed = run_keys && nsplit > 1;
-        if (listed && (n_tokens > RUN_KEYS_MAX_TOKENS || nsplit > 0x7fff)) return LI_ERR_SIZE;
-        dim3 grid(listed ? n_tokens * nsplit : n_tokens, nkv, listed ? 1 : nsplit);
-#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV><<<grid, 64, 0, stream>>>( \
+        if (dh != 128 && dh != 64) return LI_ERR_SIZE;
+        if (nsplit == 1) {
+            dim3 grid(n_tokens, nkv, 1);
+#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV, 1><<<grid, 64, 0, stream>>>( \
         (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
         token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
-        scale, nsplit, listed ? run_keys : nullptr, n_tokens)
-        if (dh == 128) LI_DM(128); else if (dh == 64) LI_DM(64); else return LI_ERR_SIZE;
+        scale, 1, nullptr, n_tokens, nullptr)
+            if (dh == 128) LI_DM(128); else LI_DM(64);
 #undef LI_DM
-        if (nsplit > 1) {
+            return li_launch_status();
+        }
+        if (use_mfma == 2) {
+            // single-wave blocks, one run each, and the merge kernel behind them (what the blocks of four
+            // waves that join their runs themselves are measured against)
+            const bool listed = run_keys != nullptr;
+            if (listed && (n_tokens > RUN_KEYS_MAX_TOKENS || nsplit > 0x7fff)) return LI_ERR_SIZE;
+            dim3 grid(listed ? n_tokens * nsplit : n_tokens, nkv, listed ? 1 : nsplit);
+#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV, 1><<<grid, 64, 0, stream>>>( \
+        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
+        token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
+        scale, nsplit, listed ? run_keys : nullptr, n_tokens, nullptr)
+            if (dh == 128) LI_DM(128); else LI_DM(64);
+#undef LI_DM
             dim3 g2(n_tokens, nh);
             attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit,
                                                                    listed ? run_keys + 2 : nullptr);
+            return li_launch_status();
         }
+        if (nsplit % LI_DECODE_QUAD) return LI_ERR_SIZE;
+        const int quads = nsplit / LI_DECODE_QUAD;
+        if (quads > 1 && (!done || !part_acc || !part_ml)) return LI_ERR_SIZE;
+        const bool listed = run_keys != nullptr;
+        if (listed && (n_tokens > RUN_KEYS_MAX_TOKENS || nsplit > 0x7fff)) return LI_ERR_SIZE;
+        if ((long)n_tokens * quads > 0x7fffffffL) return LI_ERR_SIZE;
+        dim3 grid(listed ? n_tokens * quads : n_tokens, nkv, listed ? 1 : quads);
+#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV, LI_DECODE_QUAD><<<grid, 64 * LI_DECODE_QUAD, 0, stream>>>( \
+        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
+        token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
+        scale, quads, listed ? run_keys : nullptr, n_tokens, done)
+        if (dh == 128) LI_DM(128); else LI_DM(64);
+#undef LI_DM
         return li_launch_status();
     }
     if (dtype == LI_BF16)

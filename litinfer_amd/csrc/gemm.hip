@@ -226,32 +226,90 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
     }
 }
 
+// The same product on the matrix cores in float32 (v_mfma_f32_16x16x4_f32: operands, products and sums
+// are float32, nothing is rounded to a shorter format).  A block owns up to 16 columns, a pass 16 rows;
+// its four waves split K in pieces of 32 k-values (a row's whole 128-byte line), wave v taking the pieces
+// v, v + 4, ...  Lane (c, q) = (lane % 16, lane / 16) loads the four values k0 + 4 q .. + 3 of column c of w
+// and of row c of x with one 16-byte load each; the MFMA e of a piece multiplies the e-th of them, i.e. its
+// four k-slots are the k-values k0 + e, k0 + 4 + e, k0 + 8 + e, k0 + 12 + e (the order within a piece does
+// not matter for a sum; it is the same for every row and column).  No vector arithmetic and few registers,
+// so a wave keeps many loads in flight: the FMA form held 8 x 8 sums a lane and one piece in flight, and
+// streamed w at 3.2 TB/s.  The four waves' sums are added in wave order: an order that depends on K alone.
+template <int AHEAD>
+__global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_mfma_kernel(const float* __restrict__ x,
+                                                                             const float* __restrict__ w,
+                                                                             const float* __restrict__ bias,
+                                                                             float* __restrict__ out, int M, int N, int K,
+                                                                             int accumulate, int npass, int cols) {
+    __shared__ float part[F32R_WAVES][16 * 16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, q = lane >> 4;
+    const int pass = blockIdx.x % npass, group = blockIdx.x / npass;
+    const int n0 = group * cols;
+    const int nend = n0 + cols < N ? n0 + cols : N;
+    const int m0 = pass * 16;
+    const float* wrow = w + (size_t)(n0 + c < nend ? n0 + c : nend - 1) * K + 4 * q;
+    const float* xrow = x + (size_t)(m0 + c < M ? m0 + c : M - 1) * K + 4 * q;
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    const int last = K - 4;                                   // (K is a multiple of 4: the last whole 16-byte piece of a row)
+    // AHEAD pieces of 32 k-values a trip: all their loads first, never conditional (a piece past the end reads
+    // the row's last 16 bytes and multiplies by zero)
+    for (int k0 = 32 * wave; k0 < K; k0 += 32 * F32R_WAVES * AHEAD) {
+        floatx4 wv[AHEAD][2], xv[AHEAD][2];
+#pragma unroll
+        for (int a = 0; a < AHEAD; ++a)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int k = k0 + 32 * F32R_WAVES * a + 16 * u;          // + 4 q is in the row pointers
+                const bool ok = k + 4 * q < K;
+                const int at = ok ? k : last - 4 * q;
+                wv[a][u] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(wrow + at));
+                xv[a][u] = *reinterpret_cast<const floatx4*>(xrow + at);
+                if (!ok) xv[a][u] = floatx4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+        for (int a = 0; a < AHEAD; ++a)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[a][u][e], wv[a][u][e], acc, 0, 0, 0);
+    }
+    // acc[r] = the sum for row 4 q + r, column c of this wave's share of K
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part[wave][(4 * q + r) * 16 + c] = acc[r];
+    __syncthreads();
+    {
+        const int t = threadIdx.x, i = t >> 4, j = t & 15;
+        if (m0 + i < M && n0 + j < nend) {
+            float v = part[0][t];
+#pragma unroll
+            for (int v2 = 1; v2 < F32R_WAVES; ++v2) v += part[v2][t];
+            epilogue_store(out, (size_t)(m0 + i) * N + n0 + j, v, bias, n0 + j, accumulate != 0);
+        }
+    }
+}
+
 #define F32_ROWS_MAX 64          // up to this many rows the row kernel is taken (K a multiple of 4)
 
 static int compute_units();
 
 static int launch_f32_rows(const float* x, const float* w, const float* bias, float* out, int M, int N, int K,
                            int accumulate, hipStream_t stream) {
-    const int mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-    const int nt = mt <= 8 ? 8 : 4;                           // columns a block owns at most (16 and 12 were slower)
-    const int npass = (M + mt - 1) / mt;
+    const int npass = (M + 15) / 16;
     // as many blocks as a whole number of rounds over the compute units, each with the same share of the columns
     const int cu = compute_units();
-    const int rounds = (N + cu * nt - 1) / (cu * nt);
+    const int rounds = (N + cu * 16 - 1) / (cu * 16);
     int cols = (N + cu * rounds - 1) / (cu * rounds);
     if (cols < 1) cols = 1;
     const long groups = (N + cols - 1) / cols;
     if (groups * npass > 0x7fffffffL) return LI_ERR_SIZE;
     const unsigned grid = (unsigned)(groups * npass);
-#define LI_F32R(MT, NT) gemm_f32_rows_kernel<MT, NT><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass, cols)
-    switch (mt) {
-        case 1: LI_F32R(1, 8); break;
-        case 2: LI_F32R(2, 8); break;
-        case 4: LI_F32R(4, 8); break;
-        case 8: LI_F32R(8, 8); break;
-        default: LI_F32R(16, 4); break;
-    }
-#undef LI_F32R
+    // (a short K has few pieces a wave: fewer of them a trip)
+    if (K >= 32 * F32R_WAVES * 8)
+        gemm_f32_rows_mfma_kernel<8><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass, cols);
+    else
+        gemm_f32_rows_mfma_kernel<2><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass, cols);
     return li_launch_status();
 }
 

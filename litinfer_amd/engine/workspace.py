@@ -16,9 +16,10 @@ class Workspace:
         self.allocations = 0         # goes up with every allocation, a name's first included
         self._views: Dict[Tuple[str, torch.dtype, Tuple[int, ...]], torch.Tensor] = {}
 
-    def buffer(self, name: str, shape, dtype: torch.dtype) -> torch.Tensor:
+    def buffer(self, name: str, shape, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
         """A tensor of this shape; its contents are whatever the last user of
-        the same name left."""
+        the same name left.  `zero`: the buffer is zero when it is allocated (and
+        again whenever it has to grow): for users that leave it as they found it."""
         shape = tuple(int(s) for s in shape)
         view = self._views.get((name, dtype, shape))
         if view is not None:                       # (asked for some hundred times a step, mostly with the same shapes)
@@ -29,7 +30,7 @@ class Workspace:
         if buf is None or buf.numel() < max(1, n):
             cap = max(1, n) if buf is None else max(n, buf.numel() * 3 // 2)
             moved = buf is not None
-            buf = torch.empty(cap, dtype=dtype, device=self.device)
+            buf = (torch.zeros if zero else torch.empty)(cap, dtype=dtype, device=self.device)
             self._bufs[key] = buf
             self.allocations += 1
             if moved:                              # a name's first buffer moves nothing that a graph may have recorded

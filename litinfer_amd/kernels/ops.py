@@ -50,8 +50,8 @@ _SIGNATURES = {
         "li_paged_attention": [P, I, P, P, P, I, P, I, P, P, P, P, P, I, I, I, I, I, I, I, I, I, I, F],
         "li_paged_attention_prefill": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F, I, P, P, P, I],
         "li_paged_attention_prefill_f32": [P, I, P, P, P, P, I, P, I, P, P, P, I, I, I, I, I, I, F],
-        "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
-        "li_decode_run_keys": [P, I, P, P, P, P, I, I, I, I, I, I, P],
+        "li_paged_attention_decode": [P, I, P, P, P, I, P, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, P],
+        "li_decode_run_keys": [P, I, P, P, P, P, I, I, I, I, I, I, I, P],
     },
     "sampling": {
         "li_argmax_rows": [P, P, P, P, I, I],
@@ -618,16 +618,22 @@ def _simd_count(device: torch.device) -> int:
     return _simds[i]
 
 
-def decode_splits(pairs: int, keys: int, simds: int = _DEC_WAVES) -> int:
+DECODE_QUAD = 4              # runs of a token's keys that one block of the matrix-core decode kernel takes, one a wave
+# measurements only: single-wave blocks and a merge kernel behind them, as before the blocks joined their runs
+_decode_single_waves = False
+
+
+def decode_splits(pairs: int, keys: int, simds: int = _DEC_WAVES, quad: int = DECODE_QUAD) -> int:
     """Into how many runs the keys of a decoding token are cut.  Every (token, kv head) pair and
     run is one wave, and a SIMD holds one wave of this kernel: the waves go over the SIMDs in
     rounds, each as long as a run (plus a wave's start and end, about 24 keys' time), so the
     number of runs with the least rounds x run length is taken, a run being a multiple of 32
-    keys and at least 128 where the keys allow; every run costs the merge a little (4 keys' time).
-    Few pairs: as many runs as fill the SIMDs once."""
+    keys and at least 128 where the keys allow; every run costs the join a little (4 keys' time).
+    The runs come in blocks of `quad` waves (a block joins its runs itself), so their number is 1
+    or a multiple of `quad`.  Few pairs: as many runs as fill the SIMDs once."""
     most = max(1, min(-(-keys // 128), DECODE_MAX_SPLITS))
     best, best_cost = 1, None
-    for ns in range(1, most + 1):
+    for ns in [1] + list(range(quad, most + 1, quad)):
         run = (-(-keys // ns) + 31) & ~31
         cost = -(-pairs * ns // simds) * (run + 24) + 4 * ns
         if best_cost is None or cost < best_cost:
@@ -635,7 +641,7 @@ def decode_splits(pairs: int, keys: int, simds: int = _DEC_WAVES) -> int:
     return best
 
 
-def _ragged_splits(nsplit: int, meta, window: int) -> int:
+def _ragged_splits(nsplit: int, meta, window: int, quad: int = DECODE_QUAD) -> int:
     """More runs for the grid of a batch whose contexts differ: `nsplit` fits contexts that are all as
     long as the longest; with one run length for the batch (chosen on the device) the short ones fill
     few runs, and the same number of working waves needs the longest cut into more."""
@@ -650,24 +656,27 @@ def _ragged_splits(nsplit: int, meta, window: int) -> int:
     ragged = float(keys.max()) * keys.size / max(float(keys.sum()), 1.0)
     if ragged < 1.15:
         return nsplit
-    return min(DECODE_MAX_SPLITS, int(math.ceil(nsplit * ragged * 1.25)))
+    more = min(DECODE_MAX_SPLITS, int(math.ceil(nsplit * ragged * 1.25)))
+    return min(DECODE_MAX_SPLITS, -(-more // quad) * quad)
 
 
 def decode_run_keys(meta, token_list: Optional[torch.Tensor], n_tokens: int, page_size: int, window: int,
-                    nkv: int, nsplit: int, simds: int, out: torch.Tensor) -> None:
+                    nkv: int, nsplit: int, simds: int, out: torch.Tensor, group: int = 1) -> None:
     """out[0] = the run length, in keys, for the split-key decode kernel over these single tokens
     (`token_list`, or the batch's first n_tokens tokens): the multiple of 32 with the least rounds of
     working waves over `simds` x (length + 24), between what the longest context needs to fit
     `nsplit` runs and what the block table's width would need.  out[1] = the number of runs with
     keys at that length, out[2 : 2 + n_tokens] = the runs of each token, then the runs themselves as
-    token | run << 16.  At most 4,096 tokens."""
+    token | run << 16.  With `group` > 1 the runs are taken `group` at a time (one block of the decode
+    kernel): the list then holds the first run of every group, out[1] counts the groups, and a length's
+    cost counts `group` waves a group.  At most 4,096 tokens."""
     _gpu(out, meta.ctx_len, token_list)
     _chk(0 < n_tokens <= DECODE_LIST_MAX_TOKENS, "decode_run_keys: too many tokens")
     _chk(out.dtype is torch.int32 and out.is_contiguous() and out.numel() >= 2 + n_tokens + n_tokens * nsplit,
          "decode_run_keys: out must be int32 [2 + tokens + tokens * nsplit]")
     _run("attention", "li_decode_run_keys", 0 if token_list is None else token_list.data_ptr(), n_tokens,
          meta.seg_of_token.data_ptr(), meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
-         meta.max_blocks, page_size, int(window), nkv, nsplit, simds, out.data_ptr())
+         meta.max_blocks, page_size, int(window), nkv, nsplit, simds, int(group), out.data_ptr())
 
 
 def decode_split_blocks(max_blocks: int, page_size: int, window: int, nsplit: int) -> int:
@@ -724,11 +733,26 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
         planned = 0
         if mfma:
-            planned = decode_splits(n_single * nkv, keys, _simd_count(qkv.device))
+            # Blocks of four waves that join their runs themselves, or single-wave blocks and a merge kernel
+            # behind them.  Four waves sit on ONE compute unit and the join is three trips to memory at the
+            # kernel's end: it pays where one block holds all runs of a (token, kv head) (no join, no second
+            # kernel: 64 requests at the 7B head layout 105 -> 96 us a layer), and where the waves fill the
+            # chip anyway and the runs are not many or long (8 requests, 4,096 keys: 22.3 -> 21.6 us; 8
+            # requests of the 1.5B layout with 64 short runs each: 17.3 -> 18.9 us, so not there).
+            simds = _simd_count(qkv.device)
+            quad = DECODE_QUAD
+            planned = decode_splits(n_single * nkv, keys, simds, quad)
             nsplit = _ragged_splits(planned, meta, window)
+            fills = n_single * nkv * nsplit >= simds
+            if _decode_single_waves or not (nsplit == DECODE_QUAD or (fills and (nsplit <= 32 or keys >= 8192))):
+                quad = 1
+                planned = decode_splits(n_single * nkv, keys, simds, quad)
+                nsplit = _ragged_splits(planned, meta, window, quad)
             # a split's pages must fit the kernel's copy of the block table
             while nsplit <= DECODE_MAX_SPLITS and decode_split_blocks(meta.max_blocks, page_size, window, nsplit) > DECODE_TABLE_CAP:
-                nsplit += 1
+                nsplit += 1 if nsplit < quad else quad
+            if 1 < nsplit < quad:
+                nsplit = quad
             _chk(nsplit <= DECODE_MAX_SPLITS, f"attention: block tables of {meta.max_blocks} pages of {page_size} "
                                               f"are too long for the decode kernel")
         else:
@@ -743,7 +767,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
                 acc = torch.empty(shape_a, dtype=torch.float32, device=qkv.device)
                 ml = torch.empty(shape_m, dtype=torch.float32, device=qkv.device)
         lst = meta.single_tokens if n_single < t else None
-        run_keys = None
+        run_keys = done = None
+        if mfma and nsplit > DECODE_QUAD and quad > 1:
+            # the blocks of a (token, kv head) count themselves here, and the last one joins their results
+            # (zero before the first call; every call leaves it zero)
+            done = (ws.buffer("attn.done", (n_single * nkv,), torch.int32, zero=True) if ws is not None
+                    else torch.zeros(n_single * nkv, dtype=torch.int32, device=qkv.device))
         if mfma and nsplit > planned and n_single <= DECODE_LIST_MAX_TOKENS:
             # contexts that differ: one run length for the batch and the list of the runs that have keys, made
             # on the device from the context lengths, once a step for all layers with these numbers (a
@@ -757,15 +786,17 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
                 size = 2 + n_single + n_single * DECODE_MAX_SPLITS
                 run_keys = (ws.buffer(name, (size,), torch.int32) if ws is not None
                             else torch.empty(size, dtype=torch.int32, device=qkv.device))
-                decode_run_keys(meta, lst, n_single, page_size, window, nkv, nsplit, _simd_count(qkv.device), run_keys)
+                decode_run_keys(meta, lst, n_single, page_size, window, nkv, nsplit, _simd_count(qkv.device), run_keys,
+                                group=quad)
                 meta.extra[key] = run_keys
         _run("attention", "li_paged_attention_decode", qkv.data_ptr(), qkv.stride(0), out.data_ptr(),
              k.data_ptr(), v.data_ptr(), _DT[qkv.dtype], bt.data_ptr(), meta.max_blocks,
              0 if lst is None else lst.data_ptr(), n_single, meta.seg_of_token.data_ptr(),
              meta.q_start.data_ptr(), meta.q_len.data_ptr(), meta.ctx_len.data_ptr(),
              0 if acc is None else acc.data_ptr(), 0 if ml is None else ml.data_ptr(),
-             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit, int(mfma),
-             0 if run_keys is None else run_keys.data_ptr())
+             nh, nkv, dh, page_size, k.shape[0], int(window), float(scale), nsplit,
+             (2 if quad == 1 and nsplit > 1 else 1) if mfma else 0,
+             0 if run_keys is None else run_keys.data_ptr(), 0 if done is None else done.data_ptr())
     # the matrix-core kernel for portions keeps a tile's pages in LDS (8192 entries) and divides
     # positions by the page size in float, exact below 2^21 keys; longer tables take the general kernel
     if (n_multi and qkv.dtype is torch.bfloat16 and dh in (64, 128) and meta.num_tiles

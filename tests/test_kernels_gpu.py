@@ -144,8 +144,8 @@ def test_linear_skinny_with_fused_swiglu(ops, m, n, k, swiglu, out_dtype, bias, 
 
 class _Lender:
     """Stands in for the engine's workspace."""
-    def buffer(self, name, shape, dtype):
-        return torch.empty(*shape, dtype=dtype, device=DEV)
+    def buffer(self, name, shape, dtype, zero=False):
+        return (torch.zeros if zero else torch.empty)(*shape, dtype=dtype, device=DEV)
 
 
 @pytest.mark.parametrize("m,n,k,out_dtype,bias,acc", [
@@ -562,6 +562,20 @@ def test_decode_run_length_of_a_batch_with_unequal_contexts(ops, window):
     items = got[2 + nseg:2 + nseg + int(runs.sum())]
     assert [(int(i) & 0xffff, int(i) >> 16) for i in items] == [(t, r) for t in range(nseg) for r in range(int(runs[t]))]
     assert want == (832 if not window else 128)      # (without a window the shortest run, 576, is not the cheapest)
+    # the same with the runs taken four at a time, as the matrix-core decode kernel's blocks do: a group of
+    # fewer runs still holds four SIMDs, and the list names the first run of every group
+    nsplit4 = 12
+    out = torch.full((2 + nseg + nseg * nsplit4,), -1, dtype=torch.int32, device=DEV)
+    ops.decode_run_keys(meta, None, nseg, page, window, nkv, nsplit4, simds, out, group=4)
+    lower, cap = (-(-int(keys.max()) // nsplit4) + 31) & ~31, (-(-widest // nsplit4) + 31) & ~31
+    cost = {c: -(-int(nkv * np.sum(-(-(-(-keys // c)) // 4) * 4)) // simds) * (c + 24) for c in range(lower, max(cap, lower) + 1, 32)}
+    want4 = min(cost, key=lambda c: (cost[c], c))
+    got = out.cpu().numpy()
+    runs = -(-keys // want4)
+    groups = -(-runs // 4)
+    assert int(got[0]) == want4 and int(got[1]) == int(groups.sum()) and np.array_equal(got[2:2 + nseg], runs)
+    items = got[2 + nseg:2 + nseg + int(groups.sum())]
+    assert [(int(i) & 0xffff, int(i) >> 16) for i in items] == [(t, 4 * r) for t in range(nseg) for r in range(int(groups[t]))]
     segs = [(int(c), 1) for c in ctx]
     got, ref = _paged_case(ops, torch.bfloat16, segs, 12, 2, 128, 16, window, seed=41, ws=_Lender())
     assert rel(got, ref) < 8e-3

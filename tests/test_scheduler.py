@@ -190,17 +190,19 @@ def test_sampling_stream_is_per_request():
 
 def test_decode_attention_splits_fill_the_simds_in_whole_rounds():
     # every (token, kv head) pair and run of keys is one wave, a SIMD holds one: the runs are chosen for
-    # the least rounds x run length
+    # the least rounds x run length, and come four to a block (1, or a multiple of 4)
     from litinfer_amd.kernels.ops import DECODE_MAX_SPLITS, decode_splits
     simds = 1024
     assert decode_splits(8 * 4, 4096, simds) == 32            # 1,024 waves: one round
     assert decode_splits(64 * 4, 4096, simds) == 4
     assert decode_splits(96 * 4, 4096, simds) == 8            # 3 rounds of 512 keys, not 2 of 1,376
-    assert decode_splits(24 * 4, 4096, simds) == 10           # 960 waves, not 1,056
+    assert decode_splits(24 * 4, 4096, simds) == 8            # 768 waves in one round, not 1,152 in two
+    assert decode_splits(24 * 4, 4096, simds, quad=1) == 10   # (single runs: 960 waves)
     assert decode_splits(256 * 4, 4096, simds) == 1
     for pairs in (1, 3, 28, 100, 333, 1000, 5000):
         for keys in (1, 31, 128, 1000, 4096, 100000):
             ns = decode_splits(pairs, keys, simds)
+            assert ns == 1 or ns % 4 == 0
             assert 1 <= ns <= DECODE_MAX_SPLITS
             assert ns == 1 or keys / ns >= 96                 # runs of about 128 keys at least
 
