@@ -139,10 +139,13 @@ def environment(dev) -> Dict[str, object]:
     try:
         p = torch.cuda.get_device_properties(dev)
         env.update(gpu=p.name, arch=getattr(p, "gcnArchName", None), compute_units=p.multi_processor_count,
-                   memory_GiB=round(p.total_memory / 2 ** 30, 1))
+                   memory_GiB=round(p.total_memory / 2 ** 30, 1),
+                   max_clock_MHz=round(getattr(p, "clock_rate", 0) / 1000) or None,
+                   memory_clock_MHz=round(getattr(p, "memory_clock_rate", 0) / 1000) or None)
     except Exception as e:                               # (no GPU: the block still says where it ran)
         env["gpu"] = f"unknown ({e})"
-    for name, path in (("driver", "/sys/module/amdgpu/version"), ("rocm", "/opt/rocm/.info/version")):
+    for name, path in (("driver", "/sys/module/amdgpu/version"), ("driver_src", "/sys/module/amdgpu/srcversion"),
+                       ("rocm", "/opt/rocm/.info/version")):
         try:
             env[name] = Path(path).read_text().strip()
         except OSError:

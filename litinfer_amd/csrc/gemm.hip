@@ -160,6 +160,102 @@ __global__ __launch_bounds__(256) void gemm_f32_big_kernel(const float* __restri
     }
 }
 
+// ------------------------------------------------------ float32 on the matrix cores
+// v_mfma_f32_32x32x2_f32 multiplies and adds in float32 (no operand is rounded to a shorter format: this
+// is not one of the reduced-precision matrix modes), at twice the rate of the vector ALU's FMA and without
+// the operands' way through registers that an 8 x 8 tile a lane needs.  Block tile 128 x 128, four waves
+// two by two, each 64 x 64 = 2 x 2 MFMA tiles; K in steps of 16 (eight MFMAs of two k-values a tile).
+// A stage holds x and w transposed, [k][row] with rows of 128 + 4 floats: lane (row, k) of an MFMA operand
+// reads consecutive words, and the transposing writes of the 16-byte global loads (lane = row / k-quarter)
+// meet no bank twice.  Two stages: the next step's global loads are in registers while this step is
+// multiplied.  K a multiple of 4; rows and columns past the end repeat the last and are not stored.
+#define F32M_BM 128
+#define F32M_BN 128
+#define F32M_BK 16
+#define F32M_LD (F32M_BM + 4)
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                             const float* __restrict__ bias, float* __restrict__ out,
+                                                             int M, int N, int K, int accumulate) {
+    __shared__ float As[2][F32M_BK * F32M_LD];
+    __shared__ float Bs[2][F32M_BK * F32M_LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m0 = blockIdx.y * F32M_BM, n0 = blockIdx.x * F32M_BN;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    // global loads: thread t takes the k-quarter t % 4 of rows t / 4 and t / 4 + 64 of both tiles
+    const int lrow = tid >> 2, lkq = tid & 3;
+    const float* xa[2];
+    const float* wb[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int ra = m0 + lrow + 64 * h, rb = n0 + lrow + 64 * h;
+        xa[h] = x + (size_t)(ra < M ? ra : M - 1) * K + 4 * lkq;
+        wb[h] = w + (size_t)(rb < N ? rb : N - 1) * K + 4 * lkq;
+    }
+    floatx4 ga[2], gb[2];
+    auto fetch = [&](int k0) {
+        const bool ok = k0 + 4 * lkq < K;                  // (K % 4 == 0: a 16-byte piece is inside the row or past its end)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            ga[h] = *reinterpret_cast<const floatx4*>(xa[h] + (ok ? k0 : 0));
+            gb[h] = *reinterpret_cast<const floatx4*>(wb[h] + (ok ? k0 : 0));
+            if (!ok) { ga[h] = floatx4{0.f, 0.f, 0.f, 0.f}; gb[h] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+        }
+    };
+    auto stash = [&](int st) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                As[st][(4 * lkq + e) * F32M_LD + lrow + 64 * h] = ga[h][e];
+                Bs[st][(4 * lkq + e) * F32M_LD + lrow + 64 * h] = gb[h][e];
+            }
+    };
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    const int frow = lane & 31, fk = lane >> 5;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    int st = 0;
+    for (int k0 = 0; k0 < K; k0 += F32M_BK) {
+        const bool more = k0 + F32M_BK < K;
+        if (more) fetch(k0 + F32M_BK);
+#pragma unroll
+        for (int s2 = 0; s2 < F32M_BK / 2; ++s2) {
+            float a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[i] = As[st][(2 * s2 + fk) * F32M_LD + wm + 32 * i + frow];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[j] = Bs[st][(2 * s2 + fk) * F32M_LD + wn + 32 * j + frow];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) stash(st ^ 1);                           // (the other stage: its readers passed the barrier a step ago)
+        __syncthreads();
+        st ^= 1;
+    }
+    // register r of lane l: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of a 32 x 32 tile
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int col = n0 + wn + 32 * j + frow;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = m0 + wm + 32 * i + 8 * (r >> 2) + 4 * fk + (r & 3);
+                if (row < M && col < N) epilogue_store(out, (size_t)row * N + col, acc[i][j][r], bias, col, accumulate != 0);
+            }
+        }
+}
+
 // ------------------------------------------------------ float32, few rows (decode)
 // The product streams W once: a block owns up to NT consecutive columns of the output, its
 // four waves split K (wave v takes the 256 k-values 1024 i + 256 v ..., 16 bytes a lane), so
@@ -228,64 +324,118 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const fl
 
 // The same product on the matrix cores in float32 (v_mfma_f32_16x16x4_f32: operands, products and sums
 // are float32, nothing is rounded to a shorter format).  A block owns up to 16 columns, a pass 16 rows;
-// its four waves split K in pieces of 32 k-values (a row's whole 128-byte line), wave v taking the pieces
-// v, v + 4, ...  Lane (c, q) = (lane % 16, lane / 16) loads the four values k0 + 4 q .. + 3 of column c of w
+// its eight waves split K in pieces of 32 k-values (a row's whole 128-byte line), wave v taking the pieces
+// v, v + 8, ...  Lane (c, q) = (lane % 16, lane / 16) loads the four values k0 + 4 q .. + 3 of column c of w
 // and of row c of x with one 16-byte load each; the MFMA e of a piece multiplies the e-th of them, i.e. its
 // four k-slots are the k-values k0 + e, k0 + 4 + e, k0 + 8 + e, k0 + 12 + e (the order within a piece does
 // not matter for a sum; it is the same for every row and column).  No vector arithmetic and few registers,
 // so a wave keeps many loads in flight: the FMA form held 8 x 8 sums a lane and one piece in flight, and
-// streamed w at 3.2 TB/s.  The four waves' sums are added in wave order: an order that depends on K alone.
-template <int AHEAD>
-__global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_mfma_kernel(const float* __restrict__ x,
-                                                                             const float* __restrict__ w,
-                                                                             const float* __restrict__ bias,
-                                                                             float* __restrict__ out, int M, int N, int K,
-                                                                             int accumulate, int npass, int cols) {
-    __shared__ float part[F32R_WAVES][16 * 16];
+// streamed w at 3.2 TB/s.  The eight waves' sums are added in wave order: an order that depends on K alone.
+#define F32RM_WAVES 8
+template <int AHEAD, int TILES, int RT, bool SWIGLU>
+__global__ __launch_bounds__(F32RM_WAVES * 64) void gemm_f32_rows_mfma_kernel(const float* __restrict__ x,
+                                                                              const float* __restrict__ w,
+                                                                              const float* __restrict__ bias,
+                                                                              float* __restrict__ out, int M, int N, int K,
+                                                                              int accumulate, int cols) {
+    // TILES: MFMA tiles of 16 columns side by side in a block (`cols` <= 16 TILES): they share the block's
+    // loads of x, which come through the same path as w (a matrix of many columns has blocks enough).
+    // RT: tiles of 16 rows one above the other (M <= 16 RT): they share the block's loads of w, which is
+    // read from memory once whatever the rows.
+    // SWIGLU: w is [gate; up] of N rows each, the tiles come in pairs (the gate columns n0 + 16 p .. and the
+    // up columns of the same outputs), `cols` <= 8 TILES outputs a block, and out [M, N] gets
+    // up * gate / (1 + exp(-gate)) from the float32 sums: the 2 N columns never go to memory.
+    static_assert(!SWIGLU || TILES % 2 == 0, "gate and up tiles in pairs");
+    __shared__ float part[F32RM_WAVES][RT * TILES * 256];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 15, q = lane >> 4;
-    const int pass = blockIdx.x % npass, group = blockIdx.x / npass;
-    const int n0 = group * cols;
+    const int n0 = blockIdx.x * cols;
     const int nend = n0 + cols < N ? n0 + cols : N;
-    const int m0 = pass * 16;
-    const float* wrow = w + (size_t)(n0 + c < nend ? n0 + c : nend - 1) * K + 4 * q;
-    const float* xrow = x + (size_t)(m0 + c < M ? m0 + c : M - 1) * K + 4 * q;
-    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+    const float* wrow[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        const int col = SWIGLU ? n0 + 16 * (t / 2) + c : n0 + 16 * t + c;
+        wrow[t] = w + ((size_t)(col < nend ? col : nend - 1) + (SWIGLU && (t & 1) ? (size_t)N : 0)) * K + 4 * q;
+    }
+    const float* xrow[RT];
+#pragma unroll
+    for (int i = 0; i < RT; ++i) xrow[i] = x + (size_t)(16 * i + c < M ? 16 * i + c : M - 1) * K + 4 * q;
+    floatx4 acc[RT][TILES][2];                                // two chains of MFMAs a tile (each waits for its own last result only)
+#pragma unroll
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) acc[i][t][0] = acc[i][t][1] = floatx4{0.f, 0.f, 0.f, 0.f};
     const int last = K - 4;                                   // (K is a multiple of 4: the last whole 16-byte piece of a row)
-    // AHEAD pieces of 32 k-values a trip: all their loads first, never conditional (a piece past the end reads
-    // the row's last 16 bytes and multiplies by zero)
-    for (int k0 = 32 * wave; k0 < K; k0 += 32 * F32R_WAVES * AHEAD) {
-        floatx4 wv[AHEAD][2], xv[AHEAD][2];
+    // A trip is AHEAD pieces of 32 k-values a wave: all their loads at once, never conditional (a piece past
+    // the end reads the row's last 16 bytes and multiplies by zero); the next trip's loads are issued before
+    // this trip is multiplied, into the other set of registers.  (Loads that pass the caches by, `nontemporal`,
+    // were 10 % slower here, as for the bfloat16 products.)
+    floatx4 wv[2][AHEAD][2][TILES], xv[2][AHEAD][2][RT];
+    constexpr int PIECE = 32 * F32RM_WAVES, TRIP = PIECE * AHEAD;
+    auto fetch = [&](int buf, int k0) {
 #pragma unroll
         for (int a = 0; a < AHEAD; ++a)
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
-                const int k = k0 + 32 * F32R_WAVES * a + 16 * u;          // + 4 q is in the row pointers
+                const int k = k0 + PIECE * a + 16 * u;                    // + 4 q is in the row pointers
                 const bool ok = k + 4 * q < K;
                 const int at = ok ? k : last - 4 * q;
-                wv[a][u] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(wrow + at));
-                xv[a][u] = *reinterpret_cast<const floatx4*>(xrow + at);
-                if (!ok) xv[a][u] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < TILES; ++t) wv[buf][a][u][t] = *reinterpret_cast<const floatx4*>(wrow[t] + at);
+#pragma unroll
+                for (int i = 0; i < RT; ++i) {
+                    xv[buf][a][u][i] = *reinterpret_cast<const floatx4*>(xrow[i] + at);
+                    if (!ok) xv[buf][a][u][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+                }
             }
+    };
+    auto multiply = [&](int buf) {
 #pragma unroll
         for (int a = 0; a < AHEAD; ++a)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[a][u][e], wv[a][u][e], acc, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < RT; ++i)
+#pragma unroll
+                        for (int t = 0; t < TILES; ++t)
+                            acc[i][t][e & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(xv[buf][a][u][i][e], wv[buf][a][u][t][e],
+                                                                                    acc[i][t][e & 1], 0, 0, 0);
+    };
+    int k0 = 32 * wave;
+    if (k0 < K) fetch(0, k0);
+    for (; k0 < K; k0 += 2 * TRIP) {
+        if (k0 + TRIP < K) fetch(1, k0 + TRIP);
+        multiply(0);
+        if (k0 + TRIP >= K) break;
+        if (k0 + 2 * TRIP < K) fetch(0, k0 + 2 * TRIP);
+        multiply(1);
     }
-    // acc[r] = the sum for row 4 q + r, column c of this wave's share of K
+    // acc[i][t][.][r] = the sum for row 16 i + 4 q + r, column c of tile t, of this wave's share of K (its even and
+    // its odd k-values)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) part[wave][(4 * q + r) * 16 + c] = acc[r];
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) part[wave][256 * (TILES * i + t) + (4 * q + r) * 16 + c] = acc[i][t][0][r] + acc[i][t][1][r];
     __syncthreads();
-    {
-        const int t = threadIdx.x, i = t >> 4, j = t & 15;
-        if (m0 + i < M && n0 + j < nend) {
-            float v = part[0][t];
+    constexpr int OT = SWIGLU ? TILES / 2 : TILES;            // tiles of outputs
+    for (int e = threadIdx.x; e < RT * OT * 256; e += F32RM_WAVES * 64) {
+        const int i = e / (OT * 256), t = (e >> 8) % OT, row = 16 * i + ((e >> 4) & 15), j = 16 * t + (e & 15);
+        if (row >= M || n0 + j >= nend) continue;
+        const int at = 256 * (TILES * i + (SWIGLU ? 2 * t : t)) + (e & 255);
+        float v = part[0][at];
 #pragma unroll
-            for (int v2 = 1; v2 < F32R_WAVES; ++v2) v += part[v2][t];
-            epilogue_store(out, (size_t)(m0 + i) * N + n0 + j, v, bias, n0 + j, accumulate != 0);
+        for (int v2 = 1; v2 < F32RM_WAVES; ++v2) v += part[v2][at];
+        if constexpr (SWIGLU) {
+            float up = part[0][at + 256];
+#pragma unroll
+            for (int v2 = 1; v2 < F32RM_WAVES; ++v2) up += part[v2][at + 256];
+            out[(size_t)row * N + n0 + j] = up * (v / (1.0f + expf(-v)));
+        } else {
+            epilogue_store(out, (size_t)row * N + n0 + j, v, bias, n0 + j, accumulate != 0);
         }
     }
 }
@@ -294,22 +444,45 @@ __global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_mfma_kernel(con
 
 static int compute_units();
 
+// swiglu: w is [gate; up] of N rows each and out [M, N] gets the activation (no bias, no accumulation)
 static int launch_f32_rows(const float* x, const float* w, const float* bias, float* out, int M, int N, int K,
-                           int accumulate, hipStream_t stream) {
-    const int npass = (M + 15) / 16;
-    // as many blocks as a whole number of rounds over the compute units, each with the same share of the columns
+                           int accumulate, hipStream_t stream, bool swiglu = false) {
+    // as many blocks as a whole number of rounds over the compute units, each with the same share of the columns;
+    // two MFMA tiles side by side where 16 columns a block would not fit one round (they share the loads of x:
+    // the 7B's gate/up matrix at 8 rows 136 -> 130 us)
     const int cu = compute_units();
-    const int rounds = (N + cu * 16 - 1) / (cu * 16);
+    const int rt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    // (four tiles side by side were slower than two: the 7B's gate/up matrix at 8 rows 148 against 130 us)
+    int tiles = N > 16 * cu ? 2 : 1;                          // tiles of 16 outputs
+    if (swiglu) tiles = 1;                                    // (a pair of gate and up tiles: two tiles of w already)
+    const int most = 16 * tiles;
+    const int rounds = (N + cu * most - 1) / (cu * most);
     int cols = (N + cu * rounds - 1) / (cu * rounds);
     if (cols < 1) cols = 1;
     const long groups = (N + cols - 1) / cols;
-    if (groups * npass > 0x7fffffffL) return LI_ERR_SIZE;
-    const unsigned grid = (unsigned)(groups * npass);
-    // (a short K has few pieces a wave: fewer of them a trip)
-    if (K >= 32 * F32R_WAVES * 8)
-        gemm_f32_rows_mfma_kernel<8><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass, cols);
-    else
-        gemm_f32_rows_mfma_kernel<2><<<grid, F32R_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, npass, cols);
+    if (groups > 0x7fffffffL) return LI_ERR_SIZE;
+    const unsigned grid = (unsigned)groups;
+    // pieces a trip: a long K keeps four a wave in flight, a short one two (measured: 3,584 columns 136 against
+    // 156 us for the 7B's gate/up matrix, 18,944 columns 68.6 against 74.0 us for its way back), a tiny one, and
+    // many rows (whose registers hold the rows' pieces too), one
+#define LI_F32RM(AH, TL, RTV, SW) gemm_f32_rows_mfma_kernel<AH, TL, RTV, SW><<<grid, F32RM_WAVES * 64, 0, stream>>>(x, w, bias, out, M, N, K, accumulate, cols)
+    const int ahead = rt == 4 ? 1 : K >= 8192 && rt == 1 ? 4 : K >= 32 * F32RM_WAVES * 4 ? 2 : 1;
+    if (swiglu) {
+        if (rt == 1) { if (ahead == 4) LI_F32RM(4, 2, 1, true); else if (ahead == 2) LI_F32RM(2, 2, 1, true); else LI_F32RM(1, 2, 1, true); }
+        else if (rt == 2) { if (ahead >= 2) LI_F32RM(2, 2, 2, true); else LI_F32RM(1, 2, 2, true); }
+        else LI_F32RM(1, 2, 4, true);
+        return li_launch_status();
+    }
+    if (rt == 1) {
+        if (tiles == 2) { if (ahead == 4) LI_F32RM(4, 2, 1, false); else if (ahead == 2) LI_F32RM(2, 2, 1, false); else LI_F32RM(1, 2, 1, false); }
+        else { if (ahead == 4) LI_F32RM(4, 1, 1, false); else if (ahead == 2) LI_F32RM(2, 1, 1, false); else LI_F32RM(1, 1, 1, false); }
+    } else if (rt == 2) {
+        if (tiles == 2) { if (ahead >= 2) LI_F32RM(2, 2, 2, false); else LI_F32RM(1, 2, 2, false); }
+        else { if (ahead >= 2) LI_F32RM(2, 1, 2, false); else LI_F32RM(1, 1, 2, false); }
+    } else {
+        if (tiles == 2) LI_F32RM(1, 2, 4, false); else LI_F32RM(1, 1, 4, false);
+    }
+#undef LI_F32RM
     return li_launch_status();
 }
 
@@ -1778,6 +1951,12 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
         if (out_dtype != LI_F32) return LI_ERR_DTYPE;
         if (M <= F32_ROWS_MAX && K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0)
             return launch_f32_rows((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate, stream);
+        if (K % 4 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0) {       // the matrix cores' float32 form
+            dim3 tiles((N + F32M_BN - 1) / F32M_BN, (M + F32M_BM - 1) / F32M_BM);
+            if (tiles.y > 65535) return LI_ERR_SIZE;
+            gemm_f32_mfma_kernel<<<tiles, 256, 0, stream>>>((const float*)x, (const float*)w, bias, (float*)out, M, N, K, accumulate);
+            return li_launch_status();
+        }
         if (M >= 2 * F32B_BM && N >= F32B_BN) {              // enough of both for the large tile to fill the chip
             dim3 big((N + F32B_BN - 1) / F32B_BN, (M + F32B_BM - 1) / F32B_BM);
             if (big.y > 65535) return LI_ERR_SIZE;
@@ -1850,6 +2029,14 @@ extern "C" int li_linear(const void* x, const void* w, const float* bias, void* 
 #undef LI_GEMM
     } else return LI_ERR_DTYPE;
     return li_launch_status();
+}
+
+// The same in float32 for up to 64 rows (K a multiple of 4): the few-row product on the float32 matrix cores with
+// the activation in its epilogue.
+extern "C" int li_linear_swiglu_f32(const float* x, const float* w, float* out, int M, int I, int K, hipStream_t stream) {
+    if (M <= 0 || M > F32_ROWS_MAX || I <= 0 || K <= 0 || K % 4 || I > 0x3fffffff) return LI_ERR_SIZE;
+    if ((((uintptr_t)x | (uintptr_t)w) & 15) != 0) return LI_ERR_SIZE;
+    return launch_f32_rows(x, w, nullptr, out, M, I, K, 0, stream, true);
 }
 
 // out[m, n] = up * gate / (1 + exp(-gate)) with [gate, up] = x w^T, w = [gate; up] of I rows each:

@@ -41,6 +41,7 @@ _SIGNATURES = {
         "li_linear": [P, P, P, P, I, I, I, I, I, I, P, L],
         "li_linear_skinny": [P, P, P, P, I, I, I, I, I, I],
         "li_linear_swiglu": [P, P, P, I, I, I, P, I, F],
+        "li_linear_swiglu_f32": [P, P, P, I, I, I],
         "li_linear_residual_norm": [P, P, P, P, I, I, I, P, P, P],
         "li_linear_then_norm": [P, P, P, P, I, I, I, P, L, P, F, P, I],
         "li_linear_rope_store": [P, P, P, P, I, I, P, P, P, P, P, I, I, I, I, I, P, I, F],
@@ -388,7 +389,12 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]
 
 
 def swiglu_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
-    """Whether `linear_swiglu` takes a product of m rows over k with such a matrix."""
+    """Whether `linear_swiglu` takes a product of m rows over k with such a matrix (float32: the few rows of
+    a decoding step)."""
+    if w_dtype is torch.float32:
+        # (more rows: a block's share of x grows with them while its gate and up columns stay 16 each; the
+        # product without the activation takes wider blocks there)
+        return 0 < m <= 16 and k % 4 == 0
     return w_dtype is torch.bfloat16 and m > 0 and (k % 8 == 0 if m <= SKINNY_MAX_ROWS else k % 64 == 0)
 
 
@@ -514,9 +520,16 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_scale
     _chk(x.dim() == 2 and w.dim() == 2 and out.dim() == 2, "linear_swiglu: needs matrices")
     m, k = x.shape
     n = out.shape[1]
-    _chk(swiglu_takes(m, k, w.dtype), "linear_swiglu: sizes or dtype not taken")
+    _chk(swiglu_takes(m, k, w.dtype) or (w.dtype is torch.float32 and 0 < m <= SKINNY_MAX_ROWS and k % 4 == 0),
+         "linear_swiglu: sizes or dtype not taken")
     _chk(w.shape == (2 * n, k) and out.shape[0] == m, "linear_swiglu: shapes do not fit")
     _chk(x.is_contiguous() and w.is_contiguous() and out.is_contiguous(), "linear_swiglu: contiguous operands")
+    if w.dtype is torch.float32:
+        _chk(x.dtype is torch.float32 and out.dtype is torch.float32 and row_scale is None,
+             "linear_swiglu: float32 w goes with float32 x and out, and no row scale")
+        _chk(x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0, "linear_swiglu: operands must start on 16 bytes")
+        _run("gemm", "li_linear_swiglu_f32", x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k)
+        return
     _chk(x.dtype is torch.bfloat16 and out.dtype is torch.bfloat16, "linear_swiglu: x and out must be bfloat16")
     _run("gemm", "li_linear_swiglu", x.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
          *_check_row_scale("linear_swiglu", m, row_scale))

@@ -23,8 +23,8 @@ class Linear:
 
     def takes_swiglu(self, x: torch.Tensor) -> bool:
         """Whether the product of these rows can have the SwiGLU activation as its
-        epilogue (bfloat16, no bias, a width the kernels take)."""
-        return (x.dtype is torch.bfloat16 and self.bias is None
+        epilogue (no bias, x and the matrix of one dtype, a size the kernels take)."""
+        return (x.dtype is self.weight.dtype and self.bias is None and x.data_ptr() % 16 == 0
                 and ops.swiglu_takes(x.shape[0], self.in_features, self.weight.dtype))
 
     def takes_scaling(self, x: torch.Tensor, out: torch.Tensor) -> bool:

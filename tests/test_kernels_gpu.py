@@ -266,6 +266,22 @@ def test_linear_with_swiglu_epilogue(ops, m, n, k):
     assert torch.count_nonzero(o).item() <= 2 * m + 1
 
 
+@pytest.mark.parametrize("m,inter,k", [(1, 300, 264), (8, 2000, 3584), (16, 37, 100), (17, 4200, 512), (33, 200, 96),
+                                       (64, 500, 128), (5, 9000, 1160), (40, 16500, 64)])
+def test_float32_few_row_product_with_swiglu_epilogue(ops, m, inter, k):
+    """The 32-bit path's gate/up product of a decoding step: on the float32 matrix cores, the activation in
+    the epilogue; one, two and four row tiles, one to four column tiles, short and long K."""
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(m, k, generator=g)
+    w = torch.randn(2 * inter, k, generator=g) / math.sqrt(k)
+    y = x.double().numpy() @ w.double().numpy().T
+    ref = plain_impl.swiglu(y[:, :inter], y[:, inter:])
+    out = torch.full((m, inter), float("nan"), device=DEV)
+    assert ops.swiglu_takes(m, k, torch.float32) == (m <= 16)         # (the parts ask; the kernel takes up to 64 rows)
+    ops.linear_swiglu(x.to(DEV), w.to(DEV), out)
+    assert rel(out, ref) < 8 * math.sqrt(k) * 2.0 ** -24
+
+
 @pytest.mark.parametrize("m,n,kprev,inter,eps", [
     (8, 3584, 512, 1024, 1e-6),      # a decoding step at the 7B width
     (8, 5120, 256, 27648, 1e-6),     # the 32B's gate/up matrix (566 MB): tiles of 64 x 256 scale the rows
