@@ -1372,8 +1372,12 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
             frag8 kf[KS];
 #pragma unroll
             for (int st = 0; st < KS; ++st) kf[st].raw = *reinterpret_cast<const u32x4*>(&Ks[stage][kaddr[st]]);
+            // (while a wave issues its MFMAs it goes before the SIMD's other wave, which then does its softmax
+            // on the vector ALU meanwhile: 1 to 3 % at 2,048 to 30,000 keys)
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int st = 0; st < KS; ++st) sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st].v, qf[st].v, sv, 0, 0, 0);
+            __builtin_amdgcn_s_setprio(0);
             // ---- softmax over the keys of this lane's query.  The running maximum m is only moved
             // (and the sums so far rescaled, for the whole wave) when some query's scores pass it by
             // more than 2^8: until then the exponentials are taken against the older maximum, which
@@ -1413,6 +1417,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
 #pragma unroll
                 for (int i = 0; i < 4; ++i) pf[st].raw.w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
             // ---- O^T += V^T P^T
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -1427,6 +1432,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
                     acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
                 }
             }
+            __builtin_amdgcn_s_setprio(0);
         }
         if (jb + 2 < nblk) { LI_ATT_VMCNT(2 * NL); } else { LI_ATT_VMCNT(0); }
         __builtin_amdgcn_s_barrier();
@@ -1742,47 +1748,57 @@ __global__ __launch_bounds__(2 * PRE_WAVES * 64) void paged_attention_prefill_sp
 }
 
 
-// ------------------------------------------------ portions of prompts, float32, FMA
-// The true 32-bit path's kernel for prompts: a block of 256 threads takes a tile of up to 32 tokens
-// of one segment and one head and walks the keys in blocks of 32 through LDS.  Scores: thread
-// (qg, kg) = (tid / 16, tid % 16) owns queries 2 qg, 2 qg + 1 and keys 2 kg, 2 kg + 1, four dot
-// products over the head size from LDS (each float4 of Q and K feeds two of them).  The 16 lanes of
-// a query pair agree on the new maximum by exchanges; probabilities go through LDS, transposed;
-// then thread (qg, dg) adds to its 2 x (dh / 16) outputs.  Every sum over keys or dimensions runs in
-// an order that depends on the sizes only.
 #define PF_T 32
+// ------------------------------------------------ portions of prompts, float32
+// The true 32-bit path's kernel for prompts, on the float32 matrix cores (v_mfma_f32_32x32x2_f32: float32
+// operands, products and sums; no
+// operand is rounded to a shorter format).  A block takes a tile of up to 32 tokens and one kv head; its four
+// waves are query heads of that kv head (blockIdx.z picks which four), so a block of 32 keys is fetched once,
+// into LDS, for all of them.  As in the bfloat16 kernel a wave works on the TRANSPOSED scores S^T = K Q^T: in
+// the result a lane holds 16 keys of ITS query (register r: key 8 (r / 4) + 4 (l / 32) + r % 4), so the softmax
+// is arithmetic inside a lane plus one exchange with lane l ^ 32, and those registers are the column operand
+// of O^T = V^T P^T as they are: MFMA step s takes register s, i.e. the keys 8 (s / 4) + s % 4 (lane half 0)
+// and that + 4 (lane half 1), and the row operand V^T reads the same two keys' values from LDS.  For the
+// scores the two k-slots of an MFMA are the head's two halves: lane half h multiplies the dimensions
+// (DH / 2) h + s, which it keeps of its query in registers and reads of the keys in 16-byte pieces.
+typedef float f32x16m_t __attribute__((ext_vector_type(16)));
 template <int DH>
-__global__ __launch_bounds__(256) void paged_attention_prefill_f32_kernel(
+__global__ __launch_bounds__(256) void paged_attention_prefill_f32_mfma_kernel(
     const float* __restrict__ q, int q_row_stride, float* __restrict__ out,
     const float* __restrict__ kc, const float* __restrict__ vc, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ tiles, const int* __restrict__ q_start,
     const int* __restrict__ q_len, const int* __restrict__ ctx_len, int nh, int nkv, int page_size,
     int num_pages, int window, float scale) {
-    constexpr int RS = DH + 4;                      // row stride in LDS: the rows of a float4 column fall into different banks
+    constexpr int RS = DH + 4;                      // row stride in LDS
     constexpr int C4 = DH / 4;                      // float4 pieces of a row
     constexpr int PER = PF_T * C4 / 256;            // pieces of K (and of V) a thread fetches per block of keys
-    constexpr int DPT = DH / 16;                    // output dimensions a thread owns
-    static_assert(PER * 256 == PF_T * C4 && DPT % 4 == 0, "head sizes 64 and 128");
-    __shared__ __attribute__((aligned(16))) float Qs[PF_T * RS];
+    constexpr int HD = DH / 2, DT = DH / 32;
+    static_assert(PER * 256 == PF_T * C4, "head sizes 64 and 128");
     __shared__ __attribute__((aligned(16))) float Ks[PF_T * RS];
     __shared__ __attribute__((aligned(16))) float Vs[PF_T * RS];
-    __shared__ __attribute__((aligned(16))) float Ps[PF_T * (PF_T + 2)];       // [key][query]
-    const int tile = gridDim.x - 1 - blockIdx.x, head = blockIdx.y;           // (the longest tiles of a segment first)
+    const int tile = gridDim.x - 1 - blockIdx.x, kvh = blockIdx.y;           // (the longest tiles of a segment first)
     const int s = tiles[tile * 4], t0 = tiles[tile * 4 + 1], nrows = tiles[tile * 4 + 2];
-    const int kvh = head / (nh / nkv);
-    const int tid = threadIdx.x, qg = tid >> 4, kg = tid & 15;
+    const int G = nh / nkv;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hw = blockIdx.z * 4 + wave;
+    const bool active = hw < G;                     // (idle waves still help to fetch and keep the barriers)
+    const int head = kvh * G + (active ? hw : 0);
+    const int ql = lane & 31, h = lane >> 5;
     const int p0 = ctx_len[s] - q_len[s] + (t0 - q_start[s]);               // position of the tile's first token
     const int p_last = p0 + nrows - 1;
     const int lo0 = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
     const int k_begin = lo0 & ~(PF_T - 1), k_end = p_last + 1;
     const int* table = block_table + (size_t)s * max_blocks;
-    // queries of the tile (rows past its end repeat the last one and store nothing)
-    for (int ci = tid; ci < PF_T * C4; ci += 256) {
-        const int r = ci / C4, c = ci % C4;
-        const float* src = q + (size_t)(t0 + (r < nrows ? r : nrows - 1)) * q_row_stride + (size_t)head * DH + 4 * c;
-        *reinterpret_cast<float4*>(&Qs[r * RS + 4 * c]) = *reinterpret_cast<const float4*>(src);
+    // this lane's half of its query (rows past the tile's end repeat the last one and store nothing)
+    float qf[HD];
+    {
+        const float* src = q + (size_t)(t0 + (ql < nrows ? ql : nrows - 1)) * q_row_stride + (size_t)head * DH + HD * h;
+#pragma unroll
+        for (int c = 0; c < HD / 4; ++c) {
+            const float4 v = *reinterpret_cast<const float4*>(src + 4 * c);
+            qf[4 * c] = v.x; qf[4 * c + 1] = v.y; qf[4 * c + 2] = v.z; qf[4 * c + 3] = v.w;
+        }
     }
-    // this thread's pieces of a block of keys: key (tid + 256 i) / C4, piece (tid + 256 i) % C4
     float4 kreg[PER], vreg[PER];
     auto fetch = [&](int kb) {
 #pragma unroll
@@ -1804,90 +1820,71 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_f32_kernel(
             *reinterpret_cast<float4*>(&Vs[key * RS + 4 * c]) = vreg[i];
         }
     };
-    const int q0 = 2 * qg, k0 = 2 * kg;
-    const int pq[2] = {p0 + (q0 < nrows ? q0 : nrows - 1), p0 + (q0 + 1 < nrows ? q0 + 1 : nrows - 1)};
-    int lq[2];
+    const int pq = p0 + (ql < nrows ? ql : nrows - 1);       // last visible key of this lane's query
+    const int lq = (window > 0 && pq - window + 1 > 0) ? pq - window + 1 : 0;
+    f32x16m_t acc[DT];
 #pragma unroll
-    for (int a = 0; a < 2; ++a) lq[a] = (window > 0 && pq[a] - window + 1 > 0) ? pq[a] - window + 1 : 0;
-    float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
-    float acc[2][DPT];
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int d = 0; d < DPT; ++d) acc[a][d] = 0.f;
+        for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
     fetch(k_begin);
     for (int kb = k_begin; kb < k_end; kb += PF_T) {
-        __syncthreads();                            // the block before is done with K, V and P (and Q is there)
+        __syncthreads();                            // the block before is done with K and V
         stash();
         __syncthreads();
         if (kb + PF_T < k_end) fetch(kb + PF_T);    // on its way while this block is worked on
-        // ---- scores
-        float sc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
-#pragma unroll 8
-        for (int c = 0; c < C4; ++c) {
-            const float4 qa = *reinterpret_cast<const float4*>(&Qs[q0 * RS + 4 * c]);
-            const float4 qb = *reinterpret_cast<const float4*>(&Qs[(q0 + 1) * RS + 4 * c]);
-            const float4 ka = *reinterpret_cast<const float4*>(&Ks[k0 * RS + 4 * c]);
-            const float4 kb4 = *reinterpret_cast<const float4*>(&Ks[(k0 + 1) * RS + 4 * c]);
-            sc[0][0] = fmaf(qa.x, ka.x, sc[0][0]); sc[0][0] = fmaf(qa.y, ka.y, sc[0][0]); sc[0][0] = fmaf(qa.z, ka.z, sc[0][0]); sc[0][0] = fmaf(qa.w, ka.w, sc[0][0]);
-            sc[0][1] = fmaf(qa.x, kb4.x, sc[0][1]); sc[0][1] = fmaf(qa.y, kb4.y, sc[0][1]); sc[0][1] = fmaf(qa.z, kb4.z, sc[0][1]); sc[0][1] = fmaf(qa.w, kb4.w, sc[0][1]);
-            sc[1][0] = fmaf(qb.x, ka.x, sc[1][0]); sc[1][0] = fmaf(qb.y, ka.y, sc[1][0]); sc[1][0] = fmaf(qb.z, ka.z, sc[1][0]); sc[1][0] = fmaf(qb.w, ka.w, sc[1][0]);
-            sc[1][1] = fmaf(qb.x, kb4.x, sc[1][1]); sc[1][1] = fmaf(qb.y, kb4.y, sc[1][1]); sc[1][1] = fmaf(qb.z, kb4.z, sc[1][1]); sc[1][1] = fmaf(qb.w, kb4.w, sc[1][1]);
+        if (!active) continue;
+        // ---- S^T = K Q^T
+        f32x16m_t sv;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = 0.f;
+#pragma unroll
+        for (int c = 0; c < HD / 4; ++c) {
+            const float4 kv = *reinterpret_cast<const float4*>(&Ks[ql * RS + HD * h + 4 * c]);
+            sv = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.x, qf[4 * c], sv, 0, 0, 0);
+            sv = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.y, qf[4 * c + 1], sv, 0, 0, 0);
+            sv = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.z, qf[4 * c + 2], sv, 0, 0, 0);
+            sv = __builtin_amdgcn_mfma_f32_32x32x2f32(kv.w, qf[4 * c + 3], sv, 0, 0, 0);
         }
-        // ---- softmax over the keys of each of the two queries: the 16 lanes that share them agree on the maximum
-        float alpha[2], pr[2][2];
+        // ---- softmax over the keys of this lane's query (its other half is lane ^ 32)
+        float mx = -INFINITY;
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
-            float mx = -INFINITY;
-#pragma unroll
-            for (int b = 0; b < 2; ++b) {
-                const int key = kb + k0 + b;
-                sc[a][b] = (key <= pq[a] && key >= lq[a]) ? sc[a][b] * scale : -INFINITY;
-                mx = fmaxf(mx, sc[a][b]);
-            }
-#pragma unroll
-            for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, LI_WAVE));
-            const float mn = fmaxf(m[a], mx);
-            alpha[a] = (mn == -INFINITY) ? 1.0f : expf(m[a] - mn);           // (nothing seen yet: nothing to rescale)
-#pragma unroll
-            for (int b = 0; b < 2; ++b) pr[a][b] = (sc[a][b] == -INFINITY) ? 0.f : expf(sc[a][b] - mn);
-            l[a] = l[a] * alpha[a] + (pr[a][0] + pr[a][1]);                  // this lane's keys; the lanes are added up at the end
-            m[a] = mn;
+        for (int r = 0; r < 16; ++r) {
+            const int key = kb + 8 * (r >> 2) + 4 * h + (r & 3);
+            sv[r] = (key <= pq && key >= lq) ? sv[r] * scale : -INFINITY;
+            mx = fmaxf(mx, sv[r]);
         }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
+        const float mn = fmaxf(m, mx);
+        const float alpha = (mn == -INFINITY) ? 1.0f : expf(m - mn);        // (nothing seen yet: nothing to rescale)
+        float ps = 0.f;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            Ps[(k0 + b) * (PF_T + 2) + q0] = pr[0][b];
-            Ps[(k0 + b) * (PF_T + 2) + q0 + 1] = pr[1][b];
-        }
-        __syncthreads();
-        // ---- outputs: thread (qg, dg = kg) owns dimensions DPT dg .. of its two queries
+        for (int r = 0; r < 16; ++r) { sv[r] = (sv[r] == -INFINITY) ? 0.f : expf(sv[r] - mn); ps += sv[r]; }
+        l = l * alpha + ps;
+        m = mn;
+        // ---- O^T = alpha O^T + V^T P^T
 #pragma unroll
-        for (int d = 0; d < DPT; ++d) { acc[0][d] *= alpha[0]; acc[1][d] *= alpha[1]; }
-#pragma unroll 4
-        for (int k = 0; k < PF_T; ++k) {
-            const float pa = Ps[k * (PF_T + 2) + q0], pb = Ps[k * (PF_T + 2) + q0 + 1];
+        for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
-            for (int d4 = 0; d4 < DPT / 4; ++d4) {
-                const float4 v = *reinterpret_cast<const float4*>(&Vs[k * RS + DPT * kg + 4 * d4]);
-                acc[0][4 * d4] = fmaf(pa, v.x, acc[0][4 * d4]); acc[0][4 * d4 + 1] = fmaf(pa, v.y, acc[0][4 * d4 + 1]);
-                acc[0][4 * d4 + 2] = fmaf(pa, v.z, acc[0][4 * d4 + 2]); acc[0][4 * d4 + 3] = fmaf(pa, v.w, acc[0][4 * d4 + 3]);
-                acc[1][4 * d4] = fmaf(pb, v.x, acc[1][4 * d4]); acc[1][4 * d4 + 1] = fmaf(pb, v.y, acc[1][4 * d4 + 1]);
-                acc[1][4 * d4 + 2] = fmaf(pb, v.z, acc[1][4 * d4 + 2]); acc[1][4 * d4 + 3] = fmaf(pb, v.w, acc[1][4 * d4 + 3]);
+            for (int r = 0; r < 16; ++r) acc[dt][r] *= alpha;
+#pragma unroll
+            for (int st = 0; st < 16; ++st) {
+                const float v = Vs[(8 * (st >> 2) + 4 * h + (st & 3)) * RS + 32 * dt + ql];
+                acc[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v, sv[st], acc[dt], 0, 0, 0);
             }
         }
     }
+    if (!active || ql >= nrows) return;
+    l += __shfl_xor(l, 32, LI_WAVE);               // (both halves of a query are past the return together)
+    const float inv = l != 0.f ? 1.0f / l : 0.f;
+    float* orow = out + (size_t)(t0 + ql) * nh * DH + (size_t)head * DH;
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
-        float ls = l[a];
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int o = 8; o > 0; o >>= 1) ls += __shfl_xor(ls, o, LI_WAVE);
-        if (q0 + a >= nrows) continue;
-        const float inv = ls != 0.f ? 1.0f / ls : 0.f;
-        float* orow = out + (size_t)(t0 + q0 + a) * nh * DH + (size_t)head * DH + DPT * kg;
-#pragma unroll
-        for (int d4 = 0; d4 < DPT / 4; ++d4)
-            *reinterpret_cast<float4*>(orow + 4 * d4) = float4{acc[a][4 * d4] * inv, acc[a][4 * d4 + 1] * inv, acc[a][4 * d4 + 2] * inv, acc[a][4 * d4 + 3] * inv};
-    }
+        for (int rg = 0; rg < 4; ++rg)              // registers 4 rg .. 4 rg + 3: dimensions 32 dt + 8 rg + 4 h ..
+            *reinterpret_cast<float4*>(orow + 32 * dt + 8 * rg + 4 * h) =
+                float4{acc[dt][4 * rg] * inv, acc[dt][4 * rg + 1] * inv, acc[dt][4 * rg + 2] * inv, acc[dt][4 * rg + 3] * inv};
 }
 
 extern "C" int li_paged_attention_prefill_f32(const void* q, int q_row_stride, void* out, const void* kc,
@@ -1898,8 +1895,9 @@ extern "C" int li_paged_attention_prefill_f32(const void* q, int q_row_stride, v
     if (ntiles <= 0 || nh <= 0 || nkv <= 0 || nh % nkv || nh > 65535 || page_size <= 0 || max_blocks <= 0 ||
         num_pages <= 0 || !(scale > 0.f) || (q_row_stride % 4))
         return LI_ERR_SIZE;
-    dim3 grid(ntiles, nh);
-#define LI_PF(DHV) paged_attention_prefill_f32_kernel<DHV><<<grid, 256, 0, stream>>>( \
+    if (nkv > 65535 || (nh / nkv + 3) / 4 > 65535) return LI_ERR_SIZE;
+    dim3 grid(ntiles, nkv, (nh / nkv + 3) / 4);
+#define LI_PF(DHV) paged_attention_prefill_f32_mfma_kernel<DHV><<<grid, 256, 0, stream>>>( \
         (const float*)q, q_row_stride, (float*)out, (const float*)kc, (const float*)vc, block_table, max_blocks, \
         tiles, q_start, q_len, ctx_len, nh, nkv, page_size, num_pages, window, scale)
     if (dh == 128) LI_PF(128); else if (dh == 64) LI_PF(64); else return LI_ERR_SIZE;

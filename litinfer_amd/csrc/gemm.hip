@@ -257,73 +257,8 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
 }
 
 // ------------------------------------------------------ float32, few rows (decode)
-// The product streams W once: a block owns up to NT consecutive columns of the output, its
-// four waves split K (wave v takes the 256 k-values 1024 i + 256 v ..., 16 bytes a lane), so
-// that a block reads the MT rows of x once, not once a wave: what a compute unit can take in
-// bounds these products, and x comes through the same path as W.  More than MT rows run as
-// passes of MT; the passes of one group of columns are neighbouring blocks, so that the second
-// finds the matrix's rows in L2.  Each output element is the sum, in wave order, of the four
-// waves' butterfly sums of their 64 lanes' strided partial sums: an order that depends on K alone.
-#define F32R_WAVES 4
-
-template <int MT, int NT>
-__global__ __launch_bounds__(F32R_WAVES * 64) void gemm_f32_rows_kernel(const float* __restrict__ x,
-                                                                        const float* __restrict__ w,
-                                                                        const float* __restrict__ bias,
-                                                                        float* __restrict__ out, int M, int N, int K,
-                                                                        int accumulate, int npass, int cols) {
-    __shared__ float part[F32R_WAVES][MT * NT];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int pass = blockIdx.x % npass, group = blockIdx.x / npass;
-    const int n0 = group * cols;
-    const int nend = n0 + cols < N ? n0 + cols : N;
-    const int m0 = pass * MT;
-    float acc[MT][NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j) acc[i][j] = 0.f;
-    const float* wrow[NT];
-#pragma unroll
-    for (int j = 0; j < NT; ++j) wrow[j] = w + (size_t)(n0 + j < nend ? n0 + j : nend - 1) * K;
-    const float* xrow[MT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) xrow[i] = x + (size_t)(m0 + i < M ? m0 + i : M - 1) * K;
-    for (int k = 4 * lane + 256 * wave; k < K; k += 256 * F32R_WAVES) {
-        floatx4 wv[NT], xv[MT];
-#pragma unroll
-        for (int j = 0; j < NT; ++j) wv[j] = __builtin_nontemporal_load(reinterpret_cast<const floatx4*>(wrow[j] + k));
-#pragma unroll
-        for (int i = 0; i < MT; ++i) xv[i] = *reinterpret_cast<const floatx4*>(xrow[i] + k);
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int j = 0; j < NT; ++j) acc[i][j] = fmaf(xv[i][e], wv[j][e], acc[i][j]);
-    }
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-            float v = acc[i][j];
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-            if (lane == 0) part[wave][i * NT + j] = v;
-        }
-    __syncthreads();
-    for (int t = threadIdx.x; t < MT * NT; t += F32R_WAVES * 64) {
-        const int i = t / NT, j = t - i * NT;
-        if (m0 + i >= M || n0 + j >= nend) continue;
-        float v = part[0][t];
-#pragma unroll
-        for (int v2 = 1; v2 < F32R_WAVES; ++v2) v += part[v2][t];
-        epilogue_store(out, (size_t)(m0 + i) * N + n0 + j, v, bias, n0 + j, accumulate != 0);
-    }
-}
-
-// The same product on the matrix cores in float32 (v_mfma_f32_16x16x4_f32: operands, products and sums
-// are float32, nothing is rounded to a shorter format).  A block owns up to 16 columns, a pass 16 rows;
+// The product streams w once, on the matrix cores in float32 (v_mfma_f32_16x16x4_f32: operands, products and sums
+// are float32, nothing is rounded to a shorter format).  A block owns up to 16 columns a tile and 16 rows a tile;
 // its eight waves split K in pieces of 32 k-values (a row's whole 128-byte line), wave v taking the pieces
 // v, v + 8, ...  Lane (c, q) = (lane % 16, lane / 16) loads the four values k0 + 4 q .. + 3 of column c of w
 // and of row c of x with one 16-byte load each; the MFMA e of a piece multiplies the e-th of them, i.e. its
