@@ -595,25 +595,30 @@ template <int WAVES> struct DecodeJoin {
 };
 template <> struct DecodeJoin<1> { int last; };
 
-template <int DH, int WAVES>
+template <typename T, int DH, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel(
-    const bf16_t* __restrict__ q, int q_row_stride, bf16_t* __restrict__ out,
-    const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc, const int* __restrict__ block_table,
+    const T* __restrict__ q, int q_row_stride, T* __restrict__ out,
+    const T* __restrict__ kc, const T* __restrict__ vc, const int* __restrict__ block_table,
     int max_blocks, const int* __restrict__ token_list, const int* __restrict__ seg_of_token,
     const int* __restrict__ q_start, const int* __restrict__ q_len, const int* __restrict__ ctx_len,
     float* __restrict__ part_acc, float* __restrict__ part_ml, int nh, int nkv, int page_size,
     int num_pages, int window, float scale, int nsplit, const int* __restrict__ run_keys, int n_list,
     int* __restrict__ done) {
     static_assert(DH <= ATT_MAX_DH / 2, "the join buffer holds head sizes up to 128");
-    constexpr int KS = DH / 32;                 // MFMA steps of Q K^T
-    constexpr int NS = (DH + 127) / 128;        // slabs of 128 output dimensions
+    constexpr bool F32 = sizeof(T) == 4;        // float32: v_mfma_f32_16x16x4f32 on float32 operands
+    constexpr int KS = DH / 32;                 // bfloat16: MFMA steps of Q K^T
+    constexpr int NS = (DH + 127) / 128;        // bfloat16: slabs of 128 output dimensions
     constexpr int QD = DH / 4;                  // head dimensions owned by one lane group in Q K^T
-    constexpr int PSTRIDE = 40;                 // halves per row of P in LDS (32 keys + pad, 80 bytes)
-    __shared__ __attribute__((aligned(16))) uint16_t p_lds_all[WAVES][16 * PSTRIDE];
+    constexpr int KJ = QD / 4;                  // float32: 16-byte pieces of those
+    constexpr int NP = (DH + 63) / 64;          // float32: slabs of 64 output dimensions
+    // the output's registers: acc[i] holds, for the lane's four heads, dimension dim_of(i) (below)
+    constexpr int NACC = F32 ? 4 * NP : 8 * NS;
+    constexpr int PSTRIDE = F32 ? 36 : 40;      // elements per row of P in LDS (32 keys + pad; rows 16-byte aligned)
+    __shared__ __attribute__((aligned(16))) T p_lds_all[WAVES][16 * PSTRIDE];
     __shared__ int pages_all[WAVES][DEC_TABLE_CAP];
     __shared__ DecodeJoin<WAVES> join;
     const int wave = WAVES > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
-    uint16_t* p_lds = p_lds_all[wave];
+    T* p_lds = p_lds_all[wave];
     int* pages = pages_all[wave];
     const int nruns_all = nsplit * WAVES;       // runs that the keys are cut into at most
     // run_keys given: block x takes the x-th item of the list behind it, a (token, first run) pair, and ends
@@ -653,6 +658,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
     const int k_begin = lo + split * per;
     const int k_end = (k_begin + per < p + 1) ? k_begin + per : p + 1;
     const int lane = threadIdx.x & 63, g = lane >> 4, c = lane & 15;
+    auto dim_of = [&](int i) -> int { return F32 ? 64 * (i >> 2) + 4 * c + (i & 3) : 128 * (i >> 3) + 8 * c + (i & 7); };
     // The block table of this split goes to LDS first: a page number fetched from global
     // memory in the loop would make every wait for it a wait for all loads issued before.
     const int first_block = k_begin / page_size;
@@ -674,99 +680,183 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
 
     for (int h0 = 0; h0 < G; h0 += 16) {
         const int gcount = (G - h0 < 16) ? G - h0 : 16;
-        frag8 qa[KS];
+        f32x4_t acc[NACC];
 #pragma unroll
-        for (int j = 0; j < KS; ++j)
-            qa[j].raw = *reinterpret_cast<const u32x4*>(
-                q + (size_t)t * q_row_stride + (size_t)(kvh * G + h0 + (c < gcount ? c : gcount - 1)) * DH + QD * g + 8 * j);
-        f32x4_t acc[NS][8];
-#pragma unroll
-        for (int ns = 0; ns < NS; ++ns)
-#pragma unroll
-            for (int jj = 0; jj < 8; ++jj) acc[ns][jj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < NACC; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (!F32) {
+            frag8 qa[KS];
+#pragma unroll
+            for (int j = 0; j < KS; ++j)
+                qa[j].raw = *reinterpret_cast<const u32x4*>(
+                    q + (size_t)t * q_row_stride + (size_t)(kvh * G + h0 + (c < gcount ? c : gcount - 1)) * DH + QD * g + 8 * j);
 
-        // K of a block: two tiles of 16 keys; lane (c, g) holds key 16 tt + c, dimensions QD g + 8 j ..
-        frag8 kf[2][KS];
-        bool kok[2];
-        auto load_k = [&](int kb) {
+            // K of a block: two tiles of 16 keys; lane (c, g) holds key 16 tt + c, dimensions QD g + 8 j ..
+            frag8 kf[2][KS];
+            bool kok[2];
+            auto load_k = [&](int kb) {
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const size_t off = row_of(kb + 16 * tt + c, kok[tt]);
+                for (int tt = 0; tt < 2; ++tt) {
+                    const size_t off = row_of(kb + 16 * tt + c, kok[tt]);
 #pragma unroll
-                for (int j = 0; j < KS; ++j)
-                    kf[tt][j].raw = *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j);
-            }
-        };
-        // V rows of this lane: keys kb + 8g + i, dimensions 128 ns + 8c ..  Two sets of registers
-        // take turns, so that the values of the NEXT block are in flight while this one is worked on
-        u32x4 va[NS][8], vb[NS][8];
+                    for (int j = 0; j < KS; ++j)
+                        kf[tt][j].raw = *reinterpret_cast<const u32x4*>(kc + off + QD * g + 8 * j);
+                }
+            };
+            // V rows of this lane: keys kb + 8g + i, dimensions 128 ns + 8c ..  Two sets of registers
+            // take turns, so that the values of the NEXT block are in flight while this one is worked on
+            u32x4 va[NS][8], vb[NS][8];
 #define LI_DEC_LOAD_V(kbv, dst)                                                                      \
-        _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                              \
-            bool ok_;                                                                                \
-            const size_t off_ = row_of((kbv) + 8 * g + i, ok_);                                      \
-            _Pragma("unroll") for (int ns = 0; ns < NS; ++ns) {                                      \
-                const int d_ = 128 * ns + 8 * c;                                                     \
-                dst[ns][i] = *reinterpret_cast<const u32x4*>(vc + off_ + (d_ < DH ? d_ : DH - 8));   \
-            }                                                                                        \
-        }
+            _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                              \
+                bool ok_;                                                                                \
+                const size_t off_ = row_of((kbv) + 8 * g + i, ok_);                                      \
+                _Pragma("unroll") for (int ns = 0; ns < NS; ++ns) {                                      \
+                    const int d_ = 128 * ns + 8 * c;                                                     \
+                    dst[ns][i] = *reinterpret_cast<const u32x4*>(vc + off_ + (d_ < DH ? d_ : DH - 8));   \
+                }                                                                                        \
+            }
 #define LI_DEC_STEP(kbv, vcur, vnext)                                                                \
-        {                                                                                            \
-            /* ---- S = Q K^T */                                                                     \
-            f32x4_t sv[2];                                                                           \
-            const bool sok[2] = {kok[0], kok[1]};                                                    \
-            _Pragma("unroll") for (int tt = 0; tt < 2; ++tt) {                                       \
-                sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};                                                \
-                _Pragma("unroll") for (int j = 0; j < KS; ++j)                                       \
-                    sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0); \
-            }                                                                                        \
-            /* ---- the next block's K and V: in flight during the softmax and P V */                \
-            if ((kbv) + 32 < k_end) {                                                                \
-                load_k((kbv) + 32);                                                                  \
-                LI_DEC_LOAD_V((kbv) + 32, vnext)                                                     \
-            }                                                                                        \
-            /* ---- online softmax; lanes whose key is past the end hold -inf */                     \
-            float alpha[4], pr[2][4];                                                                \
-            _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                          \
-                const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;                              \
-                const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;                              \
-                const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));     /* the block has a key: mx is finite */ \
-                alpha[r] = expf(m[r] - mx);                                                          \
-                pr[0][r] = expf(s0 - mx);                                                            \
-                pr[1][r] = expf(s1 - mx);                                                            \
-                l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];                                        \
-                m[r] = mx;                                                                           \
-            }                                                                                        \
-            wave_lds_sync();                                    /* readers of the last block's P are done */ \
-            _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                         \
-                _Pragma("unroll") for (int r = 0; r < 4; ++r)                                        \
-                    p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = float_to_bf16(pr[tt][r]);           \
-            wave_lds_sync();                                                                         \
-            frag8 pa;                                                                                \
-            pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);                   \
-            /* ---- O = alpha O + P V */                                                             \
-            _Pragma("unroll") for (int ns = 0; ns < NS; ++ns) {                                      \
-                _Pragma("unroll") for (int jj = 0; jj < 8; ++jj) {                                   \
-                    frag8 vf;                                                                        \
-                    _Pragma("unroll") for (int ii = 0; ii < 4; ++ii)                                 \
-                        vf.raw.w[ii] = __builtin_amdgcn_perm(vcur[ns][2 * ii + 1].w[jj >> 1], vcur[ns][2 * ii].w[jj >> 1], \
-                                                             (jj & 1) ? 0x07060302u : 0x05040100u);  \
-                    _Pragma("unroll") for (int r = 0; r < 4; ++r) acc[ns][jj][r] *= alpha[r];        \
-                    acc[ns][jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vf.v, acc[ns][jj], 0, 0, 0); \
-                }                                                                                    \
-            }                                                                                        \
-        }
-        if (k_begin < k_end) {
-            load_k(k_begin);
-            LI_DEC_LOAD_V(k_begin, va)
-        }
-        for (int kb = k_begin; kb < k_end; kb += 64) {
-            LI_DEC_STEP(kb, va, vb)
-            if (kb + 32 >= k_end) break;
-            LI_DEC_STEP(kb + 32, vb, va)
-        }
+            {                                                                                            \
+                /* ---- S = Q K^T */                                                                     \
+                f32x4_t sv[2];                                                                           \
+                const bool sok[2] = {kok[0], kok[1]};                                                    \
+                _Pragma("unroll") for (int tt = 0; tt < 2; ++tt) {                                       \
+                    sv[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};                                                \
+                    _Pragma("unroll") for (int j = 0; j < KS; ++j)                                       \
+                        sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0); \
+                }                                                                                        \
+                /* ---- the next block's K and V: in flight during the softmax and P V */                \
+                if ((kbv) + 32 < k_end) {                                                                \
+                    load_k((kbv) + 32);                                                                  \
+                    LI_DEC_LOAD_V((kbv) + 32, vnext)                                                     \
+                }                                                                                        \
+                /* ---- online softmax; lanes whose key is past the end hold -inf */                     \
+                float alpha[4], pr[2][4];                                                                \
+                _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                          \
+                    const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;                              \
+                    const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;                              \
+                    const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));     /* the block has a key: mx is finite */ \
+                    alpha[r] = expf(m[r] - mx);                                                          \
+                    pr[0][r] = expf(s0 - mx);                                                            \
+                    pr[1][r] = expf(s1 - mx);                                                            \
+                    l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];                                        \
+                    m[r] = mx;                                                                           \
+                }                                                                                        \
+                wave_lds_sync();                                    /* readers of the last block's P are done */ \
+                _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                         \
+                    _Pragma("unroll") for (int r = 0; r < 4; ++r)                                        \
+                        p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c].bits = float_to_bf16(pr[tt][r]);           \
+                wave_lds_sync();                                                                         \
+                frag8 pa;                                                                                \
+                pa.raw = *reinterpret_cast<const u32x4*>(&p_lds[c * PSTRIDE + 8 * g]);                   \
+                /* ---- O = alpha O + P V */                                                             \
+                _Pragma("unroll") for (int ns = 0; ns < NS; ++ns) {                                      \
+                    _Pragma("unroll") for (int jj = 0; jj < 8; ++jj) {                                   \
+                        frag8 vf;                                                                        \
+                        _Pragma("unroll") for (int ii = 0; ii < 4; ++ii)                                 \
+                            vf.raw.w[ii] = __builtin_amdgcn_perm(vcur[ns][2 * ii + 1].w[jj >> 1], vcur[ns][2 * ii].w[jj >> 1], \
+                                                                 (jj & 1) ? 0x07060302u : 0x05040100u);  \
+                        _Pragma("unroll") for (int r = 0; r < 4; ++r) acc[8 * ns + jj][r] *= alpha[r];        \
+                        acc[8 * ns + jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa.v, vf.v, acc[8 * ns + jj], 0, 0, 0); \
+                    }                                                                                    \
+                }                                                                                        \
+            }
+            if (k_begin < k_end) {
+                load_k(k_begin);
+                LI_DEC_LOAD_V(k_begin, va)
+            }
+            for (int kb = k_begin; kb < k_end; kb += 64) {
+                LI_DEC_STEP(kb, va, vb)
+                if (kb + 32 >= k_end) break;
+                LI_DEC_STEP(kb + 32, vb, va)
+            }
 #undef LI_DEC_STEP
 #undef LI_DEC_LOAD_V
+        } else {
+            // ---- float32.  Lane (c, g) of v_mfma_f32_16x16x4f32 gives A[row c][k = g] and B[k = g][column c] and gets
+            // D[row 4 g + r][column c].  Q K^T: rows are heads, columns 16 keys, and the MFMA for piece jj and
+            // element i sums over the dimensions QD g + 4 jj + i of the four lane groups, so that a lane loads
+            // its keys' dimensions in 16-byte pieces.  P V: rows are heads, k the keys 16 tt + 4 g + s (s the step:
+            // a lane reads its four P values of a tile as one 16-byte LDS read), columns the dimensions
+            // 64 n + 4 c + i, which a lane loads as one 16-byte piece of a value row.
+            f32x4_t qa[KJ];
+#pragma unroll
+            for (int j = 0; j < KJ; ++j)
+                qa[j] = *reinterpret_cast<const f32x4_t*>(
+                    q + (size_t)t * q_row_stride + (size_t)(kvh * G + h0 + (c < gcount ? c : gcount - 1)) * DH + QD * g + 4 * j);
+            f32x4_t kf[2][KJ];
+            bool kok[2];
+            auto load_k = [&](int kb) {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    const size_t off = row_of(kb + 16 * tt + c, kok[tt]);
+#pragma unroll
+                    for (int j = 0; j < KJ; ++j)
+                        kf[tt][j] = *reinterpret_cast<const f32x4_t*>(kc + off + QD * g + 4 * j);
+                }
+            };
+            // V rows of this lane: keys kb + 16 tt + 4 g + s, dimensions 64 n + 4 c ..; two sets of registers in turn
+            f32x4_t va[2][4][NP], vb[2][4][NP];
+#define LI_DEC_LOAD_V(kbv, dst)                                                                      \
+            _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                         \
+                _Pragma("unroll") for (int s_ = 0; s_ < 4; ++s_) {                                   \
+                    bool ok_;                                                                        \
+                    const size_t off_ = row_of((kbv) + 16 * tt + 4 * g + s_, ok_);                   \
+                    _Pragma("unroll") for (int n = 0; n < NP; ++n) {                                 \
+                        const int d_ = 64 * n + 4 * c;                                               \
+                        dst[tt][s_][n] = *reinterpret_cast<const f32x4_t*>(vc + off_ + (d_ < DH ? d_ : DH - 4)); \
+                    }                                                                                \
+                }
+#define LI_DEC_STEP(kbv, vcur, vnext)                                                                \
+            {                                                                                        \
+                f32x4_t sv[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};          \
+                const bool sok[2] = {kok[0], kok[1]};                                                \
+                _Pragma("unroll") for (int j = 0; j < KJ; ++j)                                       \
+                    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                    \
+                        _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                             \
+                            sv[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[j][i], kf[tt][j][i], sv[tt], 0, 0, 0); \
+                if ((kbv) + 32 < k_end) {                                                            \
+                    load_k((kbv) + 32);                                                              \
+                    LI_DEC_LOAD_V((kbv) + 32, vnext)                                                 \
+                }                                                                                    \
+                float alpha[4], pr[2][4];                                                            \
+                _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                      \
+                    const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;                          \
+                    const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;                          \
+                    const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));                          \
+                    alpha[r] = expf(m[r] - mx);                                                      \
+                    pr[0][r] = expf(s0 - mx);                                                        \
+                    pr[1][r] = expf(s1 - mx);                                                        \
+                    l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];                                    \
+                    m[r] = mx;                                                                       \
+                }                                                                                    \
+                wave_lds_sync();                                                                     \
+                _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                     \
+                    _Pragma("unroll") for (int r = 0; r < 4; ++r)                                    \
+                        p_lds[(4 * g + r) * PSTRIDE + 16 * tt + c] = pr[tt][r];                      \
+                wave_lds_sync();                                                                     \
+                f32x4_t pa[2];                                                                       \
+                _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                     \
+                    pa[tt] = *reinterpret_cast<const f32x4_t*>(&p_lds[c * PSTRIDE + 16 * tt + 4 * g]); \
+                _Pragma("unroll") for (int i = 0; i < NACC; ++i)                                     \
+                    _Pragma("unroll") for (int r = 0; r < 4; ++r) acc[i][r] *= alpha[r];             \
+                _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                                     \
+                    _Pragma("unroll") for (int s_ = 0; s_ < 4; ++s_)                                 \
+                        _Pragma("unroll") for (int i = 0; i < NACC; ++i)                             \
+                            acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[tt][s_], vcur[tt][s_][i >> 2][i & 3], acc[i], 0, 0, 0); \
+            }
+            if (k_begin < k_end) {
+                load_k(k_begin);
+                LI_DEC_LOAD_V(k_begin, va)
+            }
+            for (int kb = k_begin; kb < k_end; kb += 64) {
+                LI_DEC_STEP(kb, va, vb)
+                if (kb + 32 >= k_end) break;
+                LI_DEC_STEP(kb + 32, vb, va)
+            }
+#undef LI_DEC_STEP
+#undef LI_DEC_LOAD_V
+        }
 #pragma unroll
         for (int r = 0; r < 4; ++r) l[r] = row16_sum(l[r]);
         if constexpr (WAVES == 1) {
@@ -777,23 +867,19 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                 const int head = kvh * G + h0 + hr;
                 if (nsplit == 1) {
                     const float inv = l[r] != 0.f ? 1.0f / l[r] : 0.f;
-                    bf16_t* orow = out + (size_t)t * nh * DH + (size_t)head * DH;
+                    T* orow = out + (size_t)t * nh * DH + (size_t)head * DH;
 #pragma unroll
-                    for (int ns = 0; ns < NS; ++ns)
-#pragma unroll
-                        for (int jj = 0; jj < 8; ++jj) {
-                            const int d = 128 * ns + 8 * c + jj;
-                            if (d < DH) orow[d].bits = float_to_bf16(acc[ns][jj][r] * inv);
-                        }
+                    for (int i = 0; i < NACC; ++i) {
+                        const int d = dim_of(i);
+                        if (d < DH) store_from_float(orow + d, acc[i][r] * inv);
+                    }
                 } else {
                     const size_t pi = ((size_t)ti * nh + head) * nsplit + split;
 #pragma unroll
-                    for (int ns = 0; ns < NS; ++ns)
-#pragma unroll
-                        for (int jj = 0; jj < 8; ++jj) {
-                            const int d = 128 * ns + 8 * c + jj;
-                            if (d < DH) part_acc[pi * DH + d] = acc[ns][jj][r];
-                        }
+                    for (int i = 0; i < NACC; ++i) {
+                        const int d = dim_of(i);
+                        if (d < DH) part_acc[pi * DH + d] = acc[i][r];
+                    }
                     if (c == 0) { part_ml[pi * 2] = m[r]; part_ml[pi * 2 + 1] = l[r]; }
                 }
             }
@@ -804,12 +890,10 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
             for (int r = 0; r < 4; ++r) {
                 const int hr = 4 * g + r;
 #pragma unroll
-                for (int ns = 0; ns < NS; ++ns)
-#pragma unroll
-                    for (int jj = 0; jj < 8; ++jj) {
-                        const int d = 128 * ns + 8 * c + jj;
-                        if (d < DH) join.acc[wave][hr][d] = acc[ns][jj][r];
-                    }
+                for (int i = 0; i < NACC; ++i) {
+                    const int d = dim_of(i);
+                    if (d < DH) join.acc[wave][hr][d] = acc[i][r];
+                }
                 if (c == 0) { join.ml[wave][hr][0] = m[r]; join.ml[wave][hr][1] = l[r]; }
             }
             __syncthreads();
@@ -827,7 +911,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                 }
                 const int head = kvh * G + h0 + hr;
                 if (nsplit == 1) {
-                    out[(size_t)t * nh * DH + (size_t)head * DH + d].bits = float_to_bf16(lt != 0.f ? at / lt : 0.f);
+                    store_from_float(out + (size_t)t * nh * DH + (size_t)head * DH + d, lt != 0.f ? at / lt : 0.f);
                 } else {
                     const size_t pi = ((size_t)ti * nh + head) * nsplit + quad;
                     store_through(&part_acc[pi * DH + d], at);
@@ -881,9 +965,14 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                 }
                 if (hg_own < G) {
                     const float inv = lt != 0.f ? 1.0f / lt : 0.f;
-                    uint32_t* dst = reinterpret_cast<uint32_t*>(out + (size_t)t * nh * DH + (size_t)head * DH + d);
-                    dst[0] = pack2_bf16(at[0] * inv, at[1] * inv);
-                    dst[1] = pack2_bf16(at[2] * inv, at[3] * inv);
+                    T* dst = out + (size_t)t * nh * DH + (size_t)head * DH + d;
+                    if constexpr (F32) {
+                        *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{at[0] * inv, at[1] * inv, at[2] * inv, at[3] * inv};
+                    } else {
+                        uint32_t* dw = reinterpret_cast<uint32_t*>(dst);
+                        dw[0] = pack2_bf16(at[0] * inv, at[1] * inv);
+                        dw[1] = pack2_bf16(at[2] * inv, at[3] * inv);
+                    }
                 }
             }
         }
@@ -2055,6 +2144,60 @@ static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, cons
     return li_launch_status();
 }
 
+// The matrix-core decode kernel (bfloat16 or float32, head sizes 64 and 128), in its three forms: one run a
+// (token, kv head); single-wave blocks with the merge kernel behind them (use_mfma 2); blocks of LI_DECODE_QUAD
+// waves that join their runs themselves.
+#define LI_DECODE_QUAD 4
+template <typename T>
+static int launch_decode_mfma(const T* q, int q_row_stride, T* out, const T* kc, const T* vc, const int* block_table,
+                              int max_blocks, const int* token_list, int n_tokens, const int* seg_of_token,
+                              const int* q_start, const int* q_len, const int* ctx_len, float* part_acc,
+                              float* part_ml, int nh, int nkv, int dh, int page_size, int num_pages, int window,
+                              float scale, int nsplit, int use_mfma, const int* run_keys, int* done,
+                              hipStream_t stream) {
+    if (nkv > 65535) return LI_ERR_SIZE;
+    // a split's pages must fit the kernel's copy of the block table: `per` keys that begin
+    // anywhere in a page touch at most (per + page_size - 2) / page_size + 1 pages
+    if (li_decode_split_blocks(max_blocks, page_size, window, nsplit) > DEC_TABLE_CAP) return LI_ERR_SIZE;
+    if (dh != 128 && dh != 64) return LI_ERR_SIZE;
+    if (nsplit == 1) {
+        dim3 grid(n_tokens, nkv, 1);
+#define LI_DM(DHV) paged_attention_decode_mfma_kernel<T, DHV, 1><<<grid, 64, 0, stream>>>( \
+        q, q_row_stride, out, kc, vc, block_table, max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, \
+        part_acc, part_ml, nh, nkv, page_size, num_pages, window, scale, 1, nullptr, n_tokens, nullptr)
+        if (dh == 128) LI_DM(128); else LI_DM(64);
+#undef LI_DM
+        return li_launch_status();
+    }
+    const bool listed = run_keys != nullptr;
+    if (listed && (n_tokens > RUN_KEYS_MAX_TOKENS || nsplit > 0x7fff)) return LI_ERR_SIZE;
+    if (use_mfma == 2) {
+        if (!part_acc || !part_ml) return LI_ERR_SIZE;
+        dim3 grid(listed ? n_tokens * nsplit : n_tokens, nkv, listed ? 1 : nsplit);
+#define LI_DM(DHV) paged_attention_decode_mfma_kernel<T, DHV, 1><<<grid, 64, 0, stream>>>( \
+        q, q_row_stride, out, kc, vc, block_table, max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, \
+        part_acc, part_ml, nh, nkv, page_size, num_pages, window, scale, nsplit, listed ? run_keys : nullptr, n_tokens, \
+        nullptr)
+        if (dh == 128) LI_DM(128); else LI_DM(64);
+#undef LI_DM
+        dim3 g2(n_tokens, nh);
+        attention_merge_kernel<T><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, out, nh, dh, nsplit,
+                                                          listed ? run_keys + 2 : nullptr);
+        return li_launch_status();
+    }
+    if (nsplit % LI_DECODE_QUAD) return LI_ERR_SIZE;
+    const int quads = nsplit / LI_DECODE_QUAD;
+    if (quads > 1 && (!done || !part_acc || !part_ml)) return LI_ERR_SIZE;
+    if ((long)n_tokens * quads > 0x7fffffffL) return LI_ERR_SIZE;
+    dim3 grid(listed ? n_tokens * quads : n_tokens, nkv, listed ? 1 : quads);
+#define LI_DM(DHV) paged_attention_decode_mfma_kernel<T, DHV, LI_DECODE_QUAD><<<grid, 64 * LI_DECODE_QUAD, 0, stream>>>( \
+        q, q_row_stride, out, kc, vc, block_table, max_blocks, token_list, seg_of_token, q_start, q_len, ctx_len, \
+        part_acc, part_ml, nh, nkv, page_size, num_pages, window, scale, quads, listed ? run_keys : nullptr, n_tokens, done)
+    if (dh == 128) LI_DM(128); else LI_DM(64);
+#undef LI_DM
+    return li_launch_status();
+}
+
 // Single-query tokens of the batch (token_list, or all tokens when it is null).
 // part_acc: float [n_tokens, nh, nsplit, dh]; part_ml: float [n_tokens, nh, nsplit, 2] (unused when nsplit is 1).
 // run_keys (may be null; the matrix-core kernel with nsplit > 1 only): what li_decode_run_keys (with group
@@ -2062,7 +2205,6 @@ static int launch_decode(const T* q, int q_row_stride, T* out, const T* kc, cons
 // The matrix-core kernel with nsplit > 1 takes nsplit as a multiple of LI_DECODE_QUAD (a block works through
 // that many runs and joins them) and needs `done`: int [n_tokens * nkv], zero before the first call; every
 // call leaves it zero.  Its blocks join their results themselves; the other kernels run a merge kernel.
-#define LI_DECODE_QUAD 4
 extern "C" int li_decode_quad(void) { return LI_DECODE_QUAD; }
 extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* out, const void* kc,
                                          const void* vc, int dtype, const int* block_table, int max_blocks,
@@ -2075,59 +2217,21 @@ extern "C" int li_paged_attention_decode(const void* q, int q_row_stride, void* 
         max_blocks <= 0)
         return LI_ERR_SIZE;
     if (nsplit < 1 || nsplit > MERGE_MAX_SPLITS) return LI_ERR_SIZE;      // the merge kernel keeps a weight per split in LDS
-    if (dtype == LI_F32)
+    if (dtype == LI_F32 && !use_mfma)
         return launch_decode<float>((const float*)q, q_row_stride, (float*)out, (const float*)kc, (const float*)vc,
                                     block_table, max_blocks, token_list, n_tokens, seg_of_token, q_start, q_len,
                                     ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages, window, scale,
                                     nsplit, stream);
-    if (dtype == LI_BF16 && use_mfma) {
-        if (nkv > 65535) return LI_ERR_SIZE;
-        // a split's pages must fit the kernel's copy of the block table: `per` keys that begin
-        // anywhere in a page touch at most (per + page_size - 2) / page_size + 1 pages
-        if (li_decode_split_blocks(max_blocks, page_size, window, nsplit) > DEC_TABLE_CAP) return LI_ERR_SIZE;
-        if (dh != 128 && dh != 64) return LI_ERR_SIZE;
-        if (nsplit == 1) {
-            dim3 grid(n_tokens, nkv, 1);
-#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV, 1><<<grid, 64, 0, stream>>>( \
-        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
-        token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
-        scale, 1, nullptr, n_tokens, nullptr)
-            if (dh == 128) LI_DM(128); else LI_DM(64);
-#undef LI_DM
-            return li_launch_status();
-        }
-        if (use_mfma == 2) {
-            // single-wave blocks, one run each, and the merge kernel behind them (what the blocks of four
-            // waves that join their runs themselves are measured against)
-            const bool listed = run_keys != nullptr;
-            if (listed && (n_tokens > RUN_KEYS_MAX_TOKENS || nsplit > 0x7fff)) return LI_ERR_SIZE;
-            dim3 grid(listed ? n_tokens * nsplit : n_tokens, nkv, listed ? 1 : nsplit);
-#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV, 1><<<grid, 64, 0, stream>>>( \
-        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
-        token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
-        scale, nsplit, listed ? run_keys : nullptr, n_tokens, nullptr)
-            if (dh == 128) LI_DM(128); else LI_DM(64);
-#undef LI_DM
-            dim3 g2(n_tokens, nh);
-            attention_merge_kernel<bf16_t><<<g2, 128, 0, stream>>>(part_acc, part_ml, token_list, (bf16_t*)out, nh, dh, nsplit,
-                                                                   listed ? run_keys + 2 : nullptr);
-            return li_launch_status();
-        }
-        if (nsplit % LI_DECODE_QUAD) return LI_ERR_SIZE;
-        const int quads = nsplit / LI_DECODE_QUAD;
-        if (quads > 1 && (!done || !part_acc || !part_ml)) return LI_ERR_SIZE;
-        const bool listed = run_keys != nullptr;
-        if (listed && (n_tokens > RUN_KEYS_MAX_TOKENS || nsplit > 0x7fff)) return LI_ERR_SIZE;
-        if ((long)n_tokens * quads > 0x7fffffffL) return LI_ERR_SIZE;
-        dim3 grid(listed ? n_tokens * quads : n_tokens, nkv, listed ? 1 : quads);
-#define LI_DM(DHV) paged_attention_decode_mfma_kernel<DHV, LI_DECODE_QUAD><<<grid, 64 * LI_DECODE_QUAD, 0, stream>>>( \
-        (const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc, (const bf16_t*)vc, block_table, max_blocks, \
-        token_list, seg_of_token, q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, page_size, num_pages, window, \
-        scale, quads, listed ? run_keys : nullptr, n_tokens, done)
-        if (dh == 128) LI_DM(128); else LI_DM(64);
-#undef LI_DM
-        return li_launch_status();
-    }
+    if (dtype == LI_F32)
+        return launch_decode_mfma<float>((const float*)q, q_row_stride, (float*)out, (const float*)kc, (const float*)vc,
+                                         block_table, max_blocks, token_list, n_tokens, seg_of_token, q_start, q_len,
+                                         ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages, window, scale,
+                                         nsplit, use_mfma, run_keys, done, stream);
+    if (dtype == LI_BF16 && use_mfma)
+        return launch_decode_mfma<bf16_t>((const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc,
+                                          (const bf16_t*)vc, block_table, max_blocks, token_list, n_tokens, seg_of_token,
+                                          q_start, q_len, ctx_len, part_acc, part_ml, nh, nkv, dh, page_size, num_pages,
+                                          window, scale, nsplit, use_mfma, run_keys, done, stream);
     if (dtype == LI_BF16)
         return launch_decode<bf16_t>((const bf16_t*)q, q_row_stride, (bf16_t*)out, (const bf16_t*)kc,
                                      (const bf16_t*)vc, block_table, max_blocks, token_list, n_tokens,

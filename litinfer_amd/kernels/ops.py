@@ -741,9 +741,9 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         n_single, n_multi = 0, t                      # every token through the general kernel
     if n_single:
         keys = min(meta.max_single_ctx, window) if window > 0 else meta.max_single_ctx
-        # bfloat16 with a head size of 64 or 128: one wave per split on the matrix cores; else one
-        # block of four waves per split on the vector ALU
-        mfma = qkv.dtype is torch.bfloat16 and dh in (64, 128)
+        # a head size of 64 or 128 (bfloat16, or float32 on the float32 matrix cores): one wave per split
+        # on the matrix cores; else one block of four waves per split on the vector ALU
+        mfma = dh in (64, 128)
         planned = 0
         if mfma:
             # Blocks of four waves that join their runs themselves, or single-wave blocks and a merge kernel

@@ -531,8 +531,9 @@ def test_paged_attention(ops, dtype, segs, nh, nkv, dh, page, window):
     assert rel(out, ref) < tol(dtype, 3e-6, 1.5e-2)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("far", [3, 1000, 1999])
-def test_a_far_key_stands_out_in_a_decode_batch_of_unequal_contexts(ops, far):
+def test_a_far_key_stands_out_in_a_decode_batch_of_unequal_contexts(ops, far, dtype):
     # contexts of 2,000 to 5,000 keys: the batch gets one run length and a list of its runs; one key of every
     # request (in its first run or a later one) takes nearly all of the weight
     rng = np.random.default_rng(9)
@@ -544,8 +545,8 @@ def test_a_far_key_stands_out_in_a_decode_batch_of_unequal_contexts(ops, far):
     m.host_ctx_len = np.array([c for c, _ in segs], dtype=np.int32)
     planned = decode_splits(len(segs) * 2, 5000, 1024)
     assert _ragged_splits(planned, m, 0) > planned                 # the case is what it says
-    got, ref = _paged_case(ops, torch.bfloat16, segs, 12, 2, 128, 16, 0, seed=43, scale_one=far, ws=_Lender())
-    assert rel(got, ref) < 8e-3
+    got, ref = _paged_case(ops, dtype, segs, 12, 2, 128, 16, 0, seed=43, scale_one=far, ws=_Lender())
+    assert rel(got, ref) < tol(dtype, 1e-5, 8e-3)
 
 
 @pytest.mark.parametrize("window", [0, 900])
@@ -618,16 +619,17 @@ def test_prompt_portions_behind_long_contexts_with_their_keys_in_runs(ops, segs,
 
 # ---- the context lengths of the long workloads (8 x 30,000-token prompts in portions of 2,048, then decoding):
 # block tables of 1,875 to 2,048 pages, a portion behind 28,000 cached keys, splits of many pages
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("pad_pow2", [False, True])
 @pytest.mark.parametrize("far", [3, 15000, 29940])
-def test_decoding_over_thirty_thousand_keys_finds_one_far_key(ops, far, pad_pow2):
+def test_decoding_over_thirty_thousand_keys_finds_one_far_key(ops, far, pad_pow2, dtype):
     """Eight requests of 30,000 keys each, pages of 16, 40 heads on 8 kv heads of size 128: one key of every
     request, near the start, in the middle or near the end, carries nearly all the weight.  Also with the
     block table widened to 2,048 pages, as a recorded step sees it."""
     segs = [(30000 - 7 * i, 1) for i in range(8)]
-    out, ref = _paged_case(ops, torch.bfloat16, segs, 40, 8, 128, 16, 0, seed=51, scale_one=far, ws=_Lender(),
+    out, ref = _paged_case(ops, dtype, segs, 40, 8, 128, 16, 0, seed=51, scale_one=far, ws=_Lender(),
                            pad_pow2=pad_pow2)
-    assert rel(out, ref) < 8e-3
+    assert rel(out, ref) < tol(dtype, 1e-5, 8e-3)
 
 
 @pytest.mark.parametrize("page,ctx,window", [(1, 5000, 0), (2, 8400, 0), (1, 6000, 4500)])
@@ -645,6 +647,8 @@ def test_decode_splits_that_would_hold_more_pages_than_the_kernel_keeps_get_more
     for far in (ctx - 3 * n - 5, ctx // 2, max(ctx - window, 0) + 7 if window else 2):
         out, ref = _paged_case(ops, torch.bfloat16, segs, 8, nkv, 64, page, window, seed=52, scale_one=far, ws=_Lender())
         assert rel(out, ref) < 8e-3
+    out, ref = _paged_case(ops, torch.float32, segs, 8, nkv, 64, page, window, seed=52, scale_one=ctx // 2, ws=_Lender())
+    assert rel(out, ref) < 1e-5
 
 
 @pytest.mark.parametrize("far", [5, 14000, 29000])
@@ -661,7 +665,7 @@ def test_a_portion_of_2048_behind_28000_cached_keys_finds_one_far_key(ops, far):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("dh", [32, 64, 128])          # 64 and 128 take the matrix-core kernels in bfloat16
+@pytest.mark.parametrize("dh", [32, 64, 128])          # 64 and 128 take the matrix-core kernels
 def test_paged_attention_finds_one_far_key(ops, dtype, dh):
     # one key among hundreds carries almost all the weight: a kernel that skips
     # or misplaces a page gives a visibly different output
