@@ -1461,12 +1461,11 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
             frag8 kf[KS];
 #pragma unroll
             for (int st = 0; st < KS; ++st) kf[st].raw = *reinterpret_cast<const u32x4*>(&Ks[stage][kaddr[st]]);
-            // (while a wave issues its MFMAs it goes before the SIMD's other wave, which then does its softmax
-            // on the vector ALU meanwhile: 1 to 3 % at 2,048 to 30,000 keys)
-            __builtin_amdgcn_s_setprio(1);
+            // (raising the wave's priority while it issues its MFMAs, so that the SIMD's other wave does its
+            // softmax meanwhile, was measured in turn with this form on one machine: 2 to 5 % SLOWER at 2,048 to
+            // 30,000 keys, so the waves keep the default priority)
 #pragma unroll
             for (int st = 0; st < KS; ++st) sv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[st].v, qf[st].v, sv, 0, 0, 0);
-            __builtin_amdgcn_s_setprio(0);
             // ---- softmax over the keys of this lane's query.  The running maximum m is only moved
             // (and the sums so far rescaled, for the whole wave) when some query's scores pass it by
             // more than 2^8: until then the exponentials are taken against the older maximum, which
@@ -1506,7 +1505,6 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
 #pragma unroll
                 for (int i = 0; i < 4; ++i) pf[st].raw.w[i] = pack2_bf16(sv[8 * st + 2 * i], sv[8 * st + 2 * i + 1]);
             // ---- O^T += V^T P^T
-            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
@@ -1521,7 +1519,6 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
                     acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[st].v, acc[dt], 0, 0, 0);
                 }
             }
-            __builtin_amdgcn_s_setprio(0);
         }
         if (jb + 2 < nblk) { LI_ATT_VMCNT(2 * NL); } else { LI_ATT_VMCNT(0); }
         __builtin_amdgcn_s_barrier();

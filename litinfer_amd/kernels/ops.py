@@ -751,13 +751,17 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
             # kernel's end: it pays where one block holds all runs of a (token, kv head) (no join, no second
             # kernel: 64 requests at the 7B head layout 105 -> 96 us a layer), and where the waves fill the
             # chip anyway and the runs are not many or long (8 requests, 4,096 keys: 22.3 -> 21.6 us; 8
-            # requests of the 1.5B layout with 64 short runs each: 17.3 -> 18.9 us, so not there).
+            # requests of the 1.5B layout with 64 short runs each: 17.3 -> 18.9 us, so not there).  Not for
+            # contexts that differ (one run length for the batch and a list of the runs that have keys): a
+            # token's runs then fill its last block of four only partly, and a block's waves end at different
+            # times (64 requests with 16 to 4,600 keys, 7B head layout: 73.8 us against 82.7; 1.5B: 41.3 / 52.5).
             simds = _simd_count(qkv.device)
             quad = DECODE_QUAD
             planned = decode_splits(n_single * nkv, keys, simds, quad)
             nsplit = _ragged_splits(planned, meta, window)
             fills = n_single * nkv * nsplit >= simds
-            if _decode_single_waves or not (nsplit == DECODE_QUAD or (fills and (nsplit <= 32 or keys >= 8192))):
+            if (_decode_single_waves or nsplit > planned
+                    or not (nsplit == DECODE_QUAD or (fills and (nsplit <= 32 or keys >= 8192)))):
                 quad = 1
                 planned = decode_splits(n_single * nkv, keys, simds, quad)
                 nsplit = _ragged_splits(planned, meta, window, quad)
