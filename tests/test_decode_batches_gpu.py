@@ -33,6 +33,8 @@ N_DECODE = 12
 # activations are rounded to bfloat16 between kernels, the plain side computes in float64 from
 # the same stored weights.
 TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}
+MEAN_TOL = {"float32": 5e-7, "bfloat16": 3e-3}          # the mean deviation; observed 1.6e-7 and 1.0e-3
+MEAN_TOL_7B = 6e-3                                      # observed 1.9e-3
 TOL_7B = 4e-2          # observed 1.4e-2: sums over 3,584 and 18,944 terms of bfloat16 activations
 
 
@@ -121,8 +123,10 @@ def _check(d, dt, page, toks, prompts, ref, n_live, graphs, budget, label, tol=N
         assert eng.graph_replays == 0
     worst = max(schedules.rel_err(out[r], ref[r]) for r in toks)
     worst_decode = max(schedules.rel_err(out[r][prompts[r]:], ref[r][prompts[r]:]) for r in toks)
-    print(f"[observed] {label} {dt} live={n_live} graphs={graphs}: all {worst:.3e}, decoded rows {worst_decode:.3e}")
+    mean = max(schedules.mean_err(out[r], ref[r]) for r in toks)
+    print(f"[observed] {label} {dt} live={n_live} graphs={graphs}: all {worst:.3e}, decoded rows {worst_decode:.3e}, mean {mean:.3e}")
     assert worst < (tol or TOL[dt]), f"{label} {dt} live={n_live} graphs={graphs}: {worst}"
+    assert mean < (MEAN_TOL_7B if tol else MEAN_TOL[dt]), f"{label} {dt} live={n_live} graphs={graphs}: mean deviation {mean}"
     del eng
     torch.cuda.empty_cache()
 

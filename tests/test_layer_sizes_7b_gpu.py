@@ -19,6 +19,7 @@ SHAPE_7B = {
 }
 LENGTHS = [100, 70, 40, 5]
 TOL = {"float32": 1e-4, "bfloat16": 4e-2}
+MEAN_TOL = {"float32": 4e-6, "bfloat16": 6e-3}          # the mean deviation; observed 1.2e-6 and 1.9e-3
 
 
 @pytest.fixture(scope="module")
@@ -38,7 +39,9 @@ def test_schedules_at_the_7b_layer_sizes(model, dt):
                               max_tokens=schedules.max_live_tokens(reqs, steps, 16 if kind == "mixed" else 64))
         out = schedules.run(eng, reqs, steps)
         worst = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
-        print(f"[observed] 7B sizes {dt} {kind}: {worst:.3e}")
+        mean = max(schedules.mean_err(out[r], ref[r]) for r in reqs)
+        print(f"[observed] 7B sizes {dt} {kind}: largest {worst:.3e}, mean {mean:.3e}")
         assert worst < TOL[dt], f"{dt} {kind}: {worst}"
+        assert mean < MEAN_TOL[dt], f"{dt} {kind}: mean deviation {mean}"
         del eng
         torch.cuda.empty_cache()
