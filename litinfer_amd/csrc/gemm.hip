@@ -2028,10 +2028,17 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     if (K % 64) return LI_ERR_SIZE;
 #define LI_DMA(BM, BN, BK, NS, WLM) launch_dma<BM, BN, BK, NS, true, bf16_t, WLM>((const bf16_t*)x, (const bf16_t*)w, nullptr, (bf16_t*)out, M, N, K, 0, stream)
     // (a tile's columns are gate and up columns in turn, 32 of each: its width is a multiple of 64)
-    static const struct { int bm, bn; double speed; } shape[5] = {{256, 256, 1.0}, {256, 128, 1.0}, {128, 256, 1.0}, {128, 128, 0.8}, {128, 192, 0.9}};
+    // (128 x 320: 160 gate columns in one wave, their ups in the wave beside it; for portions of a few hundred rows,
+    // where no other width comes near whole rounds of the compute units: 512 rows against the 1.5B's 17,920
+    // columns are 224 tiles of it, one round: 45.2 -> 38.7 us.  From four rows of tiles on: with two, 256 rows
+    // against the 7B's 37,888 columns, it measured 107 us against the 101 us of 148 tiles of 256 x 256, which
+    // read w once)
+    static const struct { int bm, bn; double speed; } shape[6] = {{256, 256, 1.0}, {256, 128, 1.0}, {128, 256, 1.0}, {128, 128, 0.8}, {128, 192, 0.9},
+                                                                  {128, 320, 0.9}};
     int pick = 0;
     double best = 0.0;
-    for (int i = 0; i < 5; ++i) {
+    for (int i = 0; i < 6; ++i) {
+        if (i == 5 && M <= 3 * 128) continue;
         const double c = tile_cost(shape[i].bm, shape[i].bn, shape[i].speed, M, N, K);
         if (i == 0 || c < best) { best = c; pick = i; }
     }
@@ -2040,7 +2047,8 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     case 1: return LI_DMA(256, 128, 64, 3, 2);
     case 2: return LI_DMA(128, 256, 64, 3, 2);
     case 3: return LI_DMA(128, 128, 64, 4, 2);
-    default: return LI_DMA(128, 192, 64, 3, 4);
+    case 4: return LI_DMA(128, 192, 64, 3, 4);
+    default: return LI_DMA(128, 320, 64, 2, 2);
     }
 #undef LI_DMA
 }

@@ -241,6 +241,8 @@ def test_linear_into_the_residual_sum_with_its_norm(ops, m, n, k, bias, taken):
     (97, 7419, 128),             # few rows against many columns: tiles of 128 x 192, four waves one above the other
     (300, 9001, 128),            # tiles of 128 x 256
     (1101, 2500, 192),           # nine rows of tiles: the last XCD's share of the tiles is short
+    (1024, 4800, 192),           # tiles of 128 x 320: 160 gate columns in one wave, their ups in the wave beside it
+    (2000, 4793, 192),           # the same with ragged edges both ways
 ])
 def test_linear_with_swiglu_epilogue(ops, m, n, k):
     g = torch.Generator().manual_seed(14)
