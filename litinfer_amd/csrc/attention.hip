@@ -1420,6 +1420,14 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
     const int nblk = (k_end - k_begin + 31) / 32;
     LI_PRE_FETCH(0);
     if (nblk > 1) { LI_PRE_FETCH(1); LI_ATT_VMCNT(2 * NL); } else { LI_ATT_VMCNT(0); }
+    // The queries have arrived by now: they were asked for before the blocks of keys, and a wave's loads retire
+    // in order.  The compiler counts only the loads it made itself and would wait for "its" eight at their first
+    // use, inside the loop, where the same count stands for the blocks of keys that are on their way: every turn
+    // would then wait for ALL of them (found in the kernel's code: s_waitcnt vmcnt(7) .. vmcnt(0) before the first
+    // eight MFMAs of a turn).  Using the registers here puts that wait here, once.
+#pragma unroll
+    for (int st = 0; st < KS; ++st)
+        asm volatile("" :: "v"(qf[st].raw.w[0]), "v"(qf[st].raw.w[1]), "v"(qf[st].raw.w[2]), "v"(qf[st].raw.w[3]));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     // where this lane reads its fragments of K in a stage (the swizzle depends on the lane only)
@@ -1691,6 +1699,10 @@ __global__ __launch_bounds__(2 * PRE_WAVES * 64) void paged_attention_prefill_sp
     // flight: a wave's loads retire in order) and meets the others at the barrier.
     if (nb > 0) LI_PRE_FETCH(0);
     if (nb > 1) { LI_PRE_FETCH(1); LI_ATT_VMCNT(2 * NL); } else { LI_ATT_VMCNT(0); }
+    // (the compiler's own wait for the queries, here and not inside the loop: see the kernel above)
+#pragma unroll
+    for (int st = 0; st < KS; ++st)
+        asm volatile("" :: "v"(qf[st].raw.w[0]), "v"(qf[st].raw.w[1]), "v"(qf[st].raw.w[2]), "v"(qf[st].raw.w[3]));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     // where this lane reads its fragments of K in a stage (the swizzle depends on the lane only)
