@@ -422,6 +422,16 @@ __device__ __forceinline__ float row16_max(float v) {
 }
 __device__ __forceinline__ float row16_sum(float v) { return group_sum<16>(v); }
 
+// The larger of a lane's value and that of the lane 32 further on (or back), inside the vector ALU:
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second, so that
+// with the same value in both, one result holds the lower half's value in every lane and the other the upper
+// half's.  (A shuffle across the halves goes through the LDS crossbar, and its wait is a wait for every LDS
+// read before it.)
+__device__ __forceinline__ float both_halves_max(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 union frag8 { u32x4 raw; bf16x8_t v; };
 
 // Loads in these kernels are never conditional: a load under a branch is waited for at once,
@@ -1199,7 +1209,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_mfma_k
 #pragma unroll
             for (int r = 3; r < 15; r += 2) mx = max3f(mx, sv[r], sv[r + 1]);
             mx = max3f(mx, sv[15], sv[15]);
-            mx = max3f(mx, __shfl_xor(mx, 32, LI_WAVE), mx) * scale2;   // (scale2 > 0)
+            mx = both_halves_max(mx) * scale2;                          // (scale2 > 0)
             if (__any(mx > m + 8.0f)) {
                 const float mn = fmaxf(m, mx);
                 const float alpha = (mn == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - mn);   // (m = -inf: nothing summed yet)
@@ -1491,7 +1501,7 @@ __global__ __launch_bounds__(PRE_WAVES * 64) void paged_attention_prefill_dma_ke
 #pragma unroll
             for (int r = 3; r < 15; r += 2) mx = max3f(mx, sv[r], sv[r + 1]);
             mx = max3f(mx, sv[15], sv[15]);
-            mx = max3f(mx, __shfl_xor(mx, 32, LI_WAVE), mx) * scale2;   // (scale2 > 0)
+            mx = both_halves_max(mx) * scale2;                          // (scale2 > 0)
             if (__any(mx > m + 8.0f)) {
                 const float mn = fmaxf(m, mx);
                 const float alpha = (mn == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - mn);   // (m = -inf: nothing summed yet)
@@ -1763,7 +1773,7 @@ __global__ __launch_bounds__(2 * PRE_WAVES * 64) void paged_attention_prefill_sp
 #pragma unroll
             for (int r = 3; r < 15; r += 2) mx = max3f(mx, sv[r], sv[r + 1]);
             mx = max3f(mx, sv[15], sv[15]);
-            mx = max3f(mx, __shfl_xor(mx, 32, LI_WAVE), mx) * scale2;   // (scale2 > 0)
+            mx = both_halves_max(mx) * scale2;                          // (scale2 > 0)
             if (__any(mx > m + 8.0f)) {
                 const float mn = fmaxf(m, mx);
                 const float alpha = (mn == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m - mn);   // (m = -inf: nothing summed yet)
@@ -1953,7 +1963,7 @@ __global__ __launch_bounds__(256) void paged_attention_prefill_f32_mfma_kernel(
             sv[r] = (key <= pq && key >= lq) ? sv[r] * scale : -INFINITY;
             mx = fmaxf(mx, sv[r]);
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, LI_WAVE));
+        mx = both_halves_max(mx);
         const float mn = fmaxf(m, mx);
         const float alpha = (mn == -INFINITY) ? 1.0f : expf(m - mn);        // (nothing seen yet: nothing to rescale)
         float ps = 0.f;
