@@ -671,6 +671,8 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
     auto dim_of = [&](int i) -> int { return F32 ? 64 * (i >> 2) + 4 * c + (i & 3) : 128 * (i >> 3) + 8 * c + (i & 7); };
     // The block table of this split goes to LDS first: a page number fetched from global
     // memory in the loop would make every wait for it a wait for all loads issued before.
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    const float scale2 = scale * 1.44269504088896341f;  // scores in units of log 2: the exponentials are the instruction's own
     const int first_block = k_begin / page_size;
     if (k_begin < k_end) {
         const int nblocks = (k_end - 1) / page_size - first_block + 1;       // the host keeps this <= DEC_TABLE_CAP
@@ -681,11 +683,15 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
     auto row_of = [&](int key, bool& ok) -> size_t {       // element offset of the key's row in a cache layer
         ok = key < k_end;
         key = ok ? key : k_end - 1;                        // (only called when k_begin < k_end)
-        const int blk = key / page_size;
+        // (a page size that is a power of two: a shift and a mask; the division by a number only known when
+        // the kernel runs is some twenty instructions, four of them quarter-rate multiplications, ten times a
+        // block of keys)
+        const int blk = page_shift >= 0 ? key >> page_shift : key / page_size;
+        const int in_page = page_shift >= 0 ? (key & (page_size - 1)) : key - blk * page_size;
         int page = pages[blk - first_block];
         ok = ok && page >= 0 && page < num_pages;
         page = page < 0 ? 0 : (page >= num_pages ? num_pages - 1 : page);
-        return (((size_t)page * nkv + kvh) * page_size + (key - blk * page_size)) * DH;
+        return (((size_t)page * nkv + kvh) * page_size + in_page) * DH;
     };
 
     for (int h0 = 0; h0 < G; h0 += 16) {
@@ -743,12 +749,12 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                 /* ---- online softmax; lanes whose key is past the end hold -inf */                     \
                 float alpha[4], pr[2][4];                                                                \
                 _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                          \
-                    const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;                              \
-                    const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;                              \
+                    const float s0 = sok[0] ? sv[0][r] * scale2 : -INFINITY;                             \
+                    const float s1 = sok[1] ? sv[1][r] * scale2 : -INFINITY;                             \
                     const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));     /* the block has a key: mx is finite */ \
-                    alpha[r] = expf(m[r] - mx);                                                          \
-                    pr[0][r] = expf(s0 - mx);                                                            \
-                    pr[1][r] = expf(s1 - mx);                                                            \
+                    alpha[r] = __builtin_amdgcn_exp2f(m[r] - mx);                                        \
+                    pr[0][r] = __builtin_amdgcn_exp2f(s0 - mx);                                          \
+                    pr[1][r] = __builtin_amdgcn_exp2f(s1 - mx);                                          \
                     l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];                                        \
                     m[r] = mx;                                                                           \
                 }                                                                                        \
@@ -831,12 +837,12 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                 }                                                                                    \
                 float alpha[4], pr[2][4];                                                            \
                 _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                      \
-                    const float s0 = sok[0] ? sv[0][r] * scale : -INFINITY;                          \
-                    const float s1 = sok[1] ? sv[1][r] * scale : -INFINITY;                          \
+                    const float s0 = sok[0] ? sv[0][r] * scale2 : -INFINITY;                         \
+                    const float s1 = sok[1] ? sv[1][r] * scale2 : -INFINITY;                         \
                     const float mx = fmaxf(m[r], row16_max(fmaxf(s0, s1)));                          \
-                    alpha[r] = expf(m[r] - mx);                                                      \
-                    pr[0][r] = expf(s0 - mx);                                                        \
-                    pr[1][r] = expf(s1 - mx);                                                        \
+                    alpha[r] = __builtin_amdgcn_exp2f(m[r] - mx);                                    \
+                    pr[0][r] = __builtin_amdgcn_exp2f(s0 - mx);                                      \
+                    pr[1][r] = __builtin_amdgcn_exp2f(s1 - mx);                                      \
                     l[r] = l[r] * alpha[r] + pr[0][r] + pr[1][r];                                    \
                     m[r] = mx;                                                                       \
                 }                                                                                    \
@@ -868,7 +874,10 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
 #undef LI_DEC_LOAD_V
         }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) l[r] = row16_sum(l[r]);
+        for (int r = 0; r < 4; ++r) {
+            l[r] = row16_sum(l[r]);
+            m[r] *= 0.69314718055994531f;               // (the loop counts in powers of 2, what joins the runs in powers of e)
+        }
         if constexpr (WAVES == 1) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
