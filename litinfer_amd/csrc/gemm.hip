@@ -1296,7 +1296,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     __shared__ floatx4 red[WAVES][MT * NT][64];
     __shared__ float part_sums[WAVES * 4][16];
     const int M = a.M, N = a.N, K = a.K;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // (the same for a wave's lanes: its branches are scalar)
     const int g = lane >> 4, r16 = lane & 15;
     const int per_block = a.cols > 0 ? a.cols : (ROPE ? 8 : 16) * (SWIGLU ? 1 : NT);
     const int n0 = blockIdx.x * per_block;                  // first column (with ROPE: first pair) of this block
@@ -1313,7 +1313,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
             p = p < nend ? p : nend - 1;
             row = (p / half) * a.dh + p % half + (r16 < 8 ? 0 : half);
         } else row = (n0 + 16 * nt + r16 < nend) ? n0 + 16 * nt + r16 : nend - 1;    // rows past the end repeat the last
-        wrow[nt] = a.w + (size_t)row * K + 8 * g;
+        wrow[nt] = a.w + (size_t)row * K;
     }
     // x is read with whole rows of a chunk contiguous over 16 lanes (lane l: row l / 16 + 4 i,
     // piece l % 16), which costs the load path a quarter of what reading it in the MFMA's
@@ -1334,6 +1334,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
         for (int nt = 0; nt < NT; ++nt) acc[mt][nt] = floatx4{0.f, 0.f, 0.f, 0.f};
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     const int nchunks = (K + SK_CHUNK - 1) / SK_CHUNK;
+    const int nfull = K / SK_CHUNK;                    // whole chunks
 
     // What the epilogue adds to or multiplies with the sums (bias, the residual sum, a norm's
     // weights, the rotation's cosines and sines, the page slot) is asked for now, by the wave
@@ -1385,26 +1386,32 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     constexpr bool AHEAD = MT <= 2;
     constexpr int NBUF = AHEAD ? 2 : 1;
     bf16x8 wbuf[NBUF][NT][4], xbuf[NBUF][XR];
-    auto load_chunk = [&](int c, bf16x8 (*wd)[4], bf16x8* xd) {
+    // No load of a whole chunk is conditional, and none is replaced by zeros: a load under a branch makes the
+    // compiler wait for every load in flight at the next use of any (found in this kernel's code: s_waitcnt
+    // vmcnt(0) before each multiplication, right behind the loads of the chunk after it, so that nothing was in
+    // flight while a wave multiplied), and a value chosen between what was loaded and zero is waited for at once.
+    // A row of x past the last is read from the last row (its sums are not written).  Only the last chunk of a K
+    // that is no multiple of the chunk has k-values to leave out: it is taken by itself, behind the loop (TAIL).
+    auto load_chunk = [&](int c, bf16x8 (*wd)[4], bf16x8* xd, auto tail_tag) {
+        constexpr bool TAIL = decltype(tail_tag)::value;
         const int kb = c * SK_CHUNK;
 #pragma unroll
         for (int i = 0; i < XR; ++i) {
-            if constexpr (XLDS) {
-                const int m = xl_row + 4 * i;
-                xd[i] = (m < M && kb + 8 * xl_piece < K)
-                            ? *reinterpret_cast<const bf16x8*>(a.x + (size_t)m * K + kb + 8 * xl_piece) : zero;
-            } else {                                 // operand order: row 16 mt + r16, pieces g + 4 j
-                const int m = 16 * (i >> 2) + r16;
-                xd[i] = (m < M && kb + 8 * g + 32 * (i & 3) < K)
-                            ? *reinterpret_cast<const bf16x8*>(a.x + (size_t)m * K + kb + 8 * g + 32 * (i & 3)) : zero;
-            }
+            int m, kk;
+            if constexpr (XLDS) { m = xl_row + 4 * i; kk = kb + 8 * xl_piece; }
+            else { m = 16 * (i >> 2) + r16; kk = kb + 8 * g + 32 * (i & 3); }       // operand order: row 16 mt + r16, pieces g + 4 j
+            const bf16_t* row = a.x + (size_t)(m < M ? m : M - 1) * K;
+            if constexpr (TAIL) xd[i] = kk < K ? *reinterpret_cast<const bf16x8*>(row + kk) : zero;
+            else xd[i] = *reinterpret_cast<const bf16x8*>(row + kk);
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const bool in = kb + 8 * g + 32 * j < K;
+            const int kk = kb + 8 * g + 32 * j;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-                wd[nt][j] = in ? *reinterpret_cast<const bf16x8*>(wrow[nt] + kb + 32 * j) : zero;
+            for (int nt = 0; nt < NT; ++nt) {
+                if constexpr (TAIL) wd[nt][j] = kk < K ? *reinterpret_cast<const bf16x8*>(wrow[nt] + kk) : zero;
+                else wd[nt][j] = *reinterpret_cast<const bf16x8*>(wrow[nt] + kk);
+            }
         }
     };
     auto multiply = [&](bf16x8 (*wa)[4], bf16x8* xd) {
@@ -1432,7 +1439,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
         __builtin_amdgcn_wave_barrier();
     };
     if constexpr (AHEAD) {
-        if (wave < nchunks) load_chunk(wave, wbuf[0], xbuf[0]);
+        if (wave < nfull) load_chunk(wave, wbuf[0], xbuf[0], std::false_type{});
         // the rows' sums of squares: thread t adds the parts t / 16, t / 16 + G, ... of row t % 16 in
         // that order; the epilogue adds the G sums in theirs.  The loads are issued together, behind
         // those of the first chunk, only as many rounds as there are parts, and never conditional
@@ -1451,7 +1458,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 }
             }
         }
-        if (wave + WAVES < nchunks) load_chunk(wave + WAVES, wbuf[1], xbuf[1]);
+        if (wave + WAVES < nfull) load_chunk(wave + WAVES, wbuf[1], xbuf[1], std::false_type{});
         if (a.row_parts) {
             const int m = threadIdx.x & 15, q = threadIdx.x >> 4;
             float mine = 0.f;
@@ -1460,23 +1467,37 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
             part_sums[q][m] = mine;
         }
         // (the first turn is written out: its loads of the second chunk stand above, before the parts are added up)
-        if (wave < nchunks) multiply(wbuf[0], xbuf[0]);
-        if (wave + WAVES < nchunks) {
-            if (wave + 2 * WAVES < nchunks) load_chunk(wave + 2 * WAVES, wbuf[0], xbuf[0]);
+        if (wave < nfull) multiply(wbuf[0], xbuf[0]);
+        if (wave + WAVES < nfull) {
+            if (wave + 2 * WAVES < nfull) load_chunk(wave + 2 * WAVES, wbuf[0], xbuf[0], std::false_type{});
             multiply(wbuf[1], xbuf[1]);
-            for (int c = wave + 2 * WAVES; c < nchunks; c += 2 * WAVES) {      // two chunks a turn: buffer numbers are constants
-                if (c + WAVES < nchunks) load_chunk(c + WAVES, wbuf[1], xbuf[1]);
+            // Two chunks a turn (buffer numbers are constants).  Inside the loop nothing about the loads is
+            // conditional: where a path with loads and one without meet, the compiler's count of the loads in
+            // flight is the smaller one, and the next wait is for all of them.  So the loop runs while both of
+            // a turn's loads exist, and the one or two chunks that are left are taken behind it.
+            int c = wave + 2 * WAVES;
+            for (; c + 2 * WAVES < nfull; c += 2 * WAVES) {
+                load_chunk(c + WAVES, wbuf[1], xbuf[1], std::false_type{});
                 multiply(wbuf[0], xbuf[0]);
-                if (c + WAVES >= nchunks) break;
-                if (c + 2 * WAVES < nchunks) load_chunk(c + 2 * WAVES, wbuf[0], xbuf[0]);
+                load_chunk(c + 2 * WAVES, wbuf[0], xbuf[0], std::false_type{});
                 multiply(wbuf[1], xbuf[1]);
+            }
+            if (c < nfull) {
+                const bool more = c + WAVES < nfull;
+                if (more) load_chunk(c + WAVES, wbuf[1], xbuf[1], std::false_type{});
+                multiply(wbuf[0], xbuf[0]);
+                if (more) multiply(wbuf[1], xbuf[1]);
             }
         }
     } else {
-        for (int c = wave; c < nchunks; c += WAVES) {
-            load_chunk(c, wbuf[0], xbuf[0]);
+        for (int c = wave; c < nfull; c += WAVES) {
+            load_chunk(c, wbuf[0], xbuf[0], std::false_type{});
             multiply(wbuf[0], xbuf[0]);
         }
+    }
+    if (nfull < nchunks && wave == nfull % WAVES) {     // the chunk that K ends in
+        load_chunk(nfull, wbuf[0], xbuf[0], std::true_type{});
+        multiply(wbuf[0], xbuf[0]);
     }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
