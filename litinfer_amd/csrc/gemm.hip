@@ -282,7 +282,7 @@ __global__ __launch_bounds__(F32RM_WAVES * 64) void gemm_f32_rows_mfma_kernel(co
     // up * gate / (1 + exp(-gate)) from the float32 sums: the 2 N columns never go to memory.
     static_assert(!SWIGLU || TILES % 2 == 0, "gate and up tiles in pairs");
     __shared__ float part[F32RM_WAVES][RT * TILES * 256];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // (the same for a wave's lanes: its branches are scalar)
     const int c = lane & 15, q = lane >> 4;
     const int n0 = blockIdx.x * cols;
     const int nend = n0 + cols < N ? n0 + cols : N;
@@ -307,22 +307,29 @@ __global__ __launch_bounds__(F32RM_WAVES * 64) void gemm_f32_rows_mfma_kernel(co
     // were 10 % slower here, as for the bfloat16 products.)
     floatx4 wv[2][AHEAD][2][TILES], xv[2][AHEAD][2][RT];
     constexpr int PIECE = 32 * F32RM_WAVES, TRIP = PIECE * AHEAD;
-    auto fetch = [&](int buf, int k0) {
+    // WHOLE: every piece of the trip lies inside K; nothing is then chosen or replaced (a value chosen between what
+    // was loaded and zero is waited for at once, and so is the next use of any load behind a conditional one).
+    auto fetch = [&](int buf, int k0, auto whole_tag) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
 #pragma unroll
         for (int a = 0; a < AHEAD; ++a)
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int k = k0 + PIECE * a + 16 * u;                    // + 4 q is in the row pointers
-                const bool ok = k + 4 * q < K;
+                const bool ok = WHOLE || k + 4 * q < K;
                 const int at = ok ? k : last - 4 * q;
 #pragma unroll
                 for (int t = 0; t < TILES; ++t) wv[buf][a][u][t] = *reinterpret_cast<const floatx4*>(wrow[t] + at);
 #pragma unroll
                 for (int i = 0; i < RT; ++i) {
                     xv[buf][a][u][i] = *reinterpret_cast<const floatx4*>(xrow[i] + at);
-                    if (!ok) xv[buf][a][u][i] = floatx4{0.f, 0.f, 0.f, 0.f};
+                    if constexpr (!WHOLE) { if (!ok) xv[buf][a][u][i] = floatx4{0.f, 0.f, 0.f, 0.f}; }
                 }
             }
+    };
+    auto whole = [&](int k0) { return k0 + PIECE * (AHEAD - 1) + 32 <= K; };    // (the same for a wave's lanes)
+    auto fetch_any = [&](int buf, int k0) {
+        if (whole(k0)) fetch(buf, k0, std::true_type{}); else fetch(buf, k0, std::false_type{});
     };
     auto multiply = [&](int buf) {
 #pragma unroll
@@ -339,12 +346,22 @@ __global__ __launch_bounds__(F32RM_WAVES * 64) void gemm_f32_rows_mfma_kernel(co
                                                                                     acc[i][t][e & 1], 0, 0, 0);
     };
     int k0 = 32 * wave;
-    if (k0 < K) fetch(0, k0);
+    if (k0 < K) fetch_any(0, k0);
+    // while the two trips after this one are whole, nothing about the loads is conditional (where a path with
+    // loads and one without meet, the compiler's count of the loads in flight is the smaller one, and the
+    // next wait is for all of them) ...
+    for (; whole(k0 + 2 * TRIP); k0 += 2 * TRIP) {
+        fetch(1, k0 + TRIP, std::true_type{});
+        multiply(0);
+        fetch(0, k0 + 2 * TRIP, std::true_type{});
+        multiply(1);
+    }
+    // ... and the trips that are left
     for (; k0 < K; k0 += 2 * TRIP) {
-        if (k0 + TRIP < K) fetch(1, k0 + TRIP);
+        if (k0 + TRIP < K) fetch_any(1, k0 + TRIP);
         multiply(0);
         if (k0 + TRIP >= K) break;
-        if (k0 + 2 * TRIP < K) fetch(0, k0 + 2 * TRIP);
+        if (k0 + 2 * TRIP < K) fetch_any(0, k0 + 2 * TRIP);
         multiply(1);
     }
     // acc[i][t][.][r] = the sum for row 16 i + 4 q + r, column c of tile t, of this wave's share of K (its even and
