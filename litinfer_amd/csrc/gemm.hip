@@ -2038,7 +2038,12 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
     // 109 against 130 us).
     const int cu = compute_units();
     const bool few = li_few_rows_preferred(M, N, K);
-    const bool stream_tiles = (long)N * K * 2 >= SWIGLU_TILES_BYTES && K <= 6144;
+    // (since the few-row kernel's waves have their next chunk in flight while they multiply, it is the faster one
+    // again where the rows are few: every one of its blocks reads all of x, the tiles read x once a tile.  7B sizes
+    // at 1 / 8 / 12 / 16 rows: 46.4 / 47.6 / 49.5 / 52.0 us against the tiles' 49.0 / 48.6 / 49.5 / 50.2; 14B sizes
+    // at 4 / 8: 48.8 / 50.9 against 50.4 / 50.1; 32B sizes at 1 / 4: 97.4 / 100.3 against 97.4 / 97.2: the tiles
+    // from rows x matrix bytes of 2.2 GB on)
+    const bool stream_tiles = (long)N * K * 2 >= SWIGLU_TILES_BYTES && K <= 6144 && (double)M * N * K * 2 > 2.2e9;
     if (M <= 64 && K % 64 == 0 && (!few || stream_tiles)) {
         const int widths[3] = {256, 192, 128};
         int pick = -1;
