@@ -192,13 +192,16 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
         wb[h] = w + (size_t)(rb < N ? rb : N - 1) * K + 4 * lkq;
     }
     floatx4 ga[2], gb[2];
-    auto fetch = [&](int k0) {
-        const bool ok = k0 + 4 * lkq < K;                  // (K % 4 == 0: a 16-byte piece is inside the row or past its end)
+    // WHOLE: the step's 16 k-values lie inside K; nothing is then chosen or replaced (a value chosen between what
+    // was loaded and zero is waited for at once: the loads of the next step then did not run under this step's MFMAs)
+    auto fetch = [&](int k0, auto whole_tag) {
+        constexpr bool WHOLE = decltype(whole_tag)::value;
+        const bool ok = WHOLE || k0 + 4 * lkq < K;         // (K % 4 == 0: a 16-byte piece is inside the row or past its end)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             ga[h] = *reinterpret_cast<const floatx4*>(xa[h] + (ok ? k0 : 0));
             gb[h] = *reinterpret_cast<const floatx4*>(wb[h] + (ok ? k0 : 0));
-            if (!ok) { ga[h] = floatx4{0.f, 0.f, 0.f, 0.f}; gb[h] = floatx4{0.f, 0.f, 0.f, 0.f}; }
+            if constexpr (!WHOLE) { if (!ok) { ga[h] = floatx4{0.f, 0.f, 0.f, 0.f}; gb[h] = floatx4{0.f, 0.f, 0.f, 0.f}; } }
         }
     };
     auto stash = [&](int st) {
@@ -218,13 +221,7 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
     const int frow = lane & 31, fk = lane >> 5;
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    int st = 0;
-    for (int k0 = 0; k0 < K; k0 += F32M_BK) {
-        const bool more = k0 + F32M_BK < K;
-        if (more) fetch(k0 + F32M_BK);
+    auto multiply = [&](int st) {
 #pragma unroll
         for (int s2 = 0; s2 < F32M_BK / 2; ++s2) {
             float a[2], b[2];
@@ -238,7 +235,26 @@ __global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restr
                 for (int j = 0; j < 2; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
         }
-        if (more) stash(st ^ 1);                           // (the other stage: its readers passed the barrier a step ago)
+    };
+    if (K >= F32M_BK) fetch(0, std::true_type{}); else fetch(0, std::false_type{});
+    stash(0);
+    __syncthreads();
+    int st = 0, k0 = 0;
+    // while the step after this one is whole, its loads are neither conditional nor chosen from ...
+    for (; k0 + 2 * F32M_BK <= K; k0 += F32M_BK) {
+        fetch(k0 + F32M_BK, std::true_type{});
+        __builtin_amdgcn_sched_barrier(0);                 // (left to itself the compiler moves the loads down to where their values are stored)
+        multiply(st);
+        stash(st ^ 1);                                     // (the other stage: its readers passed the barrier a step ago)
+        __syncthreads();
+        st ^= 1;
+    }
+    // ... then the last whole step and, where K is no multiple of the step, the one behind it
+    for (; k0 < K; k0 += F32M_BK) {
+        const bool more = k0 + F32M_BK < K;
+        if (more) fetch(k0 + F32M_BK, std::false_type{});
+        multiply(st);
+        if (more) stash(st ^ 1);
         __syncthreads();
         st ^= 1;
     }
