@@ -795,6 +795,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_big_kernel(const bf16_t* __rest
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(gptr),              \
                                      (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
 
+// up * gate / (1 + exp(-gate)) for a result that is rounded to bfloat16: the exponential and the reciprocal are
+// the instructions' own (v_exp_f32, v_rcp_f32: an ulp each), 5 instructions where expf and the division are some
+// 25; a tile of 256 x 256 makes 128 of them a thread, 7 % of the tile's time.  (A gate far below zero: the
+// exponential overflows to infinity, the reciprocal is 0 and so is the result, as it should be.)  The 32-bit
+// path keeps expf and the division.
+__device__ __forceinline__ float swiglu_bf16(float gate, float up) {
+    const float e = __builtin_amdgcn_exp2f(-1.44269504088896341f * gate);
+    return up * (gate * __builtin_amdgcn_rcpf(1.0f + e));
+}
+
 // f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>)
 template <typename F, int... I>
 __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
@@ -1077,7 +1087,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                 float f = 1.0f;
                 if constexpr (ROWSCALE) f = row_parts ? row_inv[row & 15] : 1.0f;      // (row_parts: M <= 16, so row < 16 here)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) { const float gv = gs[e] * f; v[e] = (us[e] * f) * (gv / (1.0f + expf(-gv))); }
+                for (int e = 0; e < 8; ++e) v[e] = swiglu_bf16(gs[e] * f, us[e] * f);
                 const size_t o_idx = (size_t)row * NO + col;
                 if (col + 8 <= NO && (NO % 8) == 0) {
                     chunk16 o;
@@ -1118,7 +1128,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                             uv *= f;
                         }
                     }
-                    band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 16 * j + ccol] = uv * (gv / (1.0f + expf(-gv)));
+                    band[(8 * (r >> 2) + crow + (r & 3)) * ESTRIDE + 16 * j + ccol] = swiglu_bf16(gv, uv);
                 }
         } else {
 #pragma unroll
@@ -1597,7 +1607,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 const int n = n0 + 4 * (l >> 4) + r;
                 if (n < nend) {
                     const float gv = s[0][r], uv = s[NT - 1][r];
-                    store_from_float(out + (size_t)m * N + n, uv * (gv / (1.0f + expf(-gv))));
+                    store_from_float(out + (size_t)m * N + n, swiglu_bf16(gv, uv));
                 }
             }
         } else {
