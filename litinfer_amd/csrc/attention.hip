@@ -671,7 +671,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
     auto dim_of = [&](int i) -> int { return F32 ? 64 * (i >> 2) + 4 * c + (i & 3) : 128 * (i >> 3) + 8 * c + (i & 7); };
     // The block table of this split goes to LDS first: a page number fetched from global
     // memory in the loop would make every wait for it a wait for all loads issued before.
-    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    const float inv_page = 1.0f / (float)page_size;
     const float scale2 = scale * 1.44269504088896341f;  // scores in units of log 2: the exponentials are the instruction's own
     const int first_block = k_begin / page_size;
     if (k_begin < k_end) {
@@ -683,11 +683,13 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
     auto row_of = [&](int key, bool& ok) -> size_t {       // element offset of the key's row in a cache layer
         ok = key < k_end;
         key = ok ? key : k_end - 1;                        // (only called when k_begin < k_end)
-        // (a page size that is a power of two: a shift and a mask; the division by a number only known when
-        // the kernel runs is some twenty instructions, four of them quarter-rate multiplications, ten times a
-        // block of keys)
-        const int blk = page_shift >= 0 ? key >> page_shift : key / page_size;
-        const int in_page = page_shift >= 0 ? (key & (page_size - 1)) : key - blk * page_size;
+        // key / page_size as a float32 product: (key + 1/2) / page_size is at least 1 / (2 page_size) away from
+        // a whole number and the product's error is below (key + 1/2) / page_size * 2^-23, so the truncation is
+        // the quotient while key < 2^22 (the host refuses longer tables).  The integer division by a number
+        // only known when the kernel runs is some twenty instructions, and a choice between it and a shift
+        // becomes a branch between the loads, behind which every wait is for all of them.
+        const int blk = (int)(((float)key + 0.5f) * inv_page);
+        const int in_page = key - __mul24(blk, page_size);
         int page = pages[blk - first_block];
         ok = ok && page >= 0 && page < num_pages;
         page = page < 0 ? 0 : (page >= num_pages ? num_pages - 1 : page);
@@ -731,7 +733,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                     dst[ns][i] = *reinterpret_cast<const u32x4*>(vc + off_ + (d_ < DH ? d_ : DH - 8));   \
                 }                                                                                        \
             }
-#define LI_DEC_STEP(kbv, vcur, vnext)                                                                \
+#define LI_DEC_STEP(kbv, vcur, vnext, more)                                                             \
             {                                                                                            \
                 /* ---- S = Q K^T */                                                                     \
                 f32x4_t sv[2];                                                                           \
@@ -741,8 +743,9 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                     _Pragma("unroll") for (int j = 0; j < KS; ++j)                                       \
                         sv[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qa[j].v, kf[tt][j].v, sv[tt], 0, 0, 0); \
                 }                                                                                        \
-                /* ---- the next block's K and V: in flight during the softmax and P V */                \
-                if ((kbv) + 32 < k_end) {                                                                \
+                /* ---- the next block's K and V: in flight during the softmax and P V (in the loop `more` */ \
+                /* is the constant: behind a branch every wait is for all loads)                         */ \
+                if (more) {                                                                              \
                     load_k((kbv) + 32);                                                                  \
                     LI_DEC_LOAD_V((kbv) + 32, vnext)                                                     \
                 }                                                                                        \
@@ -777,14 +780,20 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                     }                                                                                    \
                 }                                                                                        \
             }
+            // One condition around the first loads and the loop, and no way out of the loop between a step's
+            // loads and the step that uses them: the compiler moves loads whose values one of two paths does
+            // not use to the other path's start, where the wait for them follows at once.
             if (k_begin < k_end) {
                 load_k(k_begin);
                 LI_DEC_LOAD_V(k_begin, va)
-            }
-            for (int kb = k_begin; kb < k_end; kb += 64) {
-                LI_DEC_STEP(kb, va, vb)
-                if (kb + 32 >= k_end) break;
-                LI_DEC_STEP(kb + 32, vb, va)
+                int kb = k_begin;
+                for (; kb + 64 < k_end; kb += 64) {
+                    LI_DEC_STEP(kb, va, vb, true)
+                    LI_DEC_STEP(kb + 32, vb, va, true)
+                }
+                const bool two = kb + 32 < k_end;
+                LI_DEC_STEP(kb, va, vb, two)
+                if (two) LI_DEC_STEP(kb + 32, vb, va, false)
             }
 #undef LI_DEC_STEP
 #undef LI_DEC_LOAD_V
@@ -823,7 +832,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                         dst[tt][s_][n] = *reinterpret_cast<const f32x4_t*>(vc + off_ + (d_ < DH ? d_ : DH - 4)); \
                     }                                                                                \
                 }
-#define LI_DEC_STEP(kbv, vcur, vnext)                                                                \
+#define LI_DEC_STEP(kbv, vcur, vnext, more)                                                             \
             {                                                                                        \
                 f32x4_t sv[2] = {f32x4_t{0.f, 0.f, 0.f, 0.f}, f32x4_t{0.f, 0.f, 0.f, 0.f}};          \
                 const bool sok[2] = {kok[0], kok[1]};                                                \
@@ -831,7 +840,7 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                     _Pragma("unroll") for (int i = 0; i < 4; ++i)                                    \
                         _Pragma("unroll") for (int tt = 0; tt < 2; ++tt)                             \
                             sv[tt] = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[j][i], kf[tt][j][i], sv[tt], 0, 0, 0); \
-                if ((kbv) + 32 < k_end) {                                                            \
+                if (more) {                                                                          \
                     load_k((kbv) + 32);                                                              \
                     LI_DEC_LOAD_V((kbv) + 32, vnext)                                                 \
                 }                                                                                    \
@@ -861,14 +870,20 @@ __global__ __launch_bounds__(64 * WAVES) void paged_attention_decode_mfma_kernel
                         _Pragma("unroll") for (int i = 0; i < NACC; ++i)                             \
                             acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[tt][s_], vcur[tt][s_][i >> 2][i & 3], acc[i], 0, 0, 0); \
             }
+            // One condition around the first loads and the loop, and no way out of the loop between a step's
+            // loads and the step that uses them: the compiler moves loads whose values one of two paths does
+            // not use to the other path's start, where the wait for them follows at once.
             if (k_begin < k_end) {
                 load_k(k_begin);
                 LI_DEC_LOAD_V(k_begin, va)
-            }
-            for (int kb = k_begin; kb < k_end; kb += 64) {
-                LI_DEC_STEP(kb, va, vb)
-                if (kb + 32 >= k_end) break;
-                LI_DEC_STEP(kb + 32, vb, va)
+                int kb = k_begin;
+                for (; kb + 64 < k_end; kb += 64) {
+                    LI_DEC_STEP(kb, va, vb, true)
+                    LI_DEC_STEP(kb + 32, vb, va, true)
+                }
+                const bool two = kb + 32 < k_end;
+                LI_DEC_STEP(kb, va, vb, two)
+                if (two) LI_DEC_STEP(kb + 32, vb, va, false)
             }
 #undef LI_DEC_STEP
 #undef LI_DEC_LOAD_V
@@ -2188,6 +2203,7 @@ static int launch_decode_mfma(const T* q, int q_row_stride, T* out, const T* kc,
     // anywhere in a page touch at most (per + page_size - 2) / page_size + 1 pages
     if (li_decode_split_blocks(max_blocks, page_size, window, nsplit) > DEC_TABLE_CAP) return LI_ERR_SIZE;
     if (dh != 128 && dh != 64) return LI_ERR_SIZE;
+    if ((long)max_blocks * page_size > (1L << 21) || page_size > (1 << 16)) return LI_ERR_SIZE;   // (the kernel's key / page_size)
     if (nsplit == 1) {
         dim3 grid(n_tokens, nkv, 1);
 #define LI_DM(DHV) paged_attention_decode_mfma_kernel<T, DHV, 1><<<grid, 64, 0, stream>>>( \

@@ -746,6 +746,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
         mfma = dh in (64, 128)
         planned = 0
         if mfma:
+            # (the kernel finds a key's page by a float32 product that is exact below 2^22)
+            _chk(meta.max_blocks * page_size <= 1 << 21 and page_size <= 1 << 16,
+                 f"attention: block tables of {meta.max_blocks} pages of {page_size} keys are beyond the decode "
+                 f"kernel's {1 << 21} keys")
             # Blocks of four waves that join their runs themselves, or single-wave blocks and a merge kernel
             # behind them.  Four waves sit on ONE compute unit and the join is three trips to memory at the
             # kernel's end: it pays where one block holds all runs of a (token, kv head) (no join, no second

@@ -42,3 +42,14 @@ def test_decode_split_bound_covers_every_split_of_every_context():
     # pages of one token: 64 splits of 1,024 keys fill the kernel's table exactly, one key more does not fit
     assert ops.decode_split_blocks(64 * 1024, 1, 0, 64) == ops.DECODE_TABLE_CAP
     assert ops.decode_split_blocks(64 * 1024 + 1, 1, 0, 64) > ops.DECODE_TABLE_CAP
+
+
+def test_the_decode_kernels_float_quotient_is_the_page_of_every_key():
+    """paged_attention_decode_mfma_kernel finds a key's page as int((key + 0.5f) * (1.0f / page_size)) in
+    float32; redone here with numpy's float32 for every key the host lets through, at page sizes of every kind."""
+    keys = np.arange(0, (1 << 21) + 1, dtype=np.int64)
+    half = np.float32(0.5)
+    for page in (1, 2, 3, 5, 7, 12, 16, 17, 48, 64, 100, 127, 128, 255, 1000, 4097, 65535, 65536):
+        inv = np.float32(1.0) / np.float32(page)
+        blk = ((keys.astype(np.float32) + half) * inv).astype(np.int64)
+        assert np.array_equal(blk, keys // page), page
