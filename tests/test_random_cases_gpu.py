@@ -1,0 +1,89 @@
+"""Many small random cases, fixed seeds: mixed schedules of every tiny configuration with random request
+lengths, portions, page sizes and numbers of live requests against the plain implementation, and random
+decode batches (contexts around the edges of blocks of keys and of pages, windows, head layouts, equal and
+unequal contexts, with and without a workspace) of the attention op against the plain attention."""
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import schedules
+import test_kernels_gpu as kernel_cases
+from tiny_configs import (TINY_A, TINY_A_PAGE, TINY_B, TINY_B_PAGE, TINY_C, TINY_C_PAGE, TINY_D, TINY_D_PAGE,
+                          TINY_E, TINY_E_PAGE)
+
+pytestmark = pytest.mark.gpu
+
+CASES = {"A": (TINY_A, TINY_A_PAGE, 0), "B": (TINY_B, TINY_B_PAGE, 1), "C": (TINY_C, TINY_C_PAGE, 2),
+         "D": (TINY_D, TINY_D_PAGE, 3), "E": (TINY_E, TINY_E_PAGE, 4)}
+TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from litinfer_amd.kernels import ops
+    ops.require_gpu("cuda:0")
+    return ops
+
+
+LENGTHS = [1, 2, 3, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 90, 127, 128, 129, 200, 260]
+PORTIONS = [2, 3, 5, 8, 16, 17, 31, 32, 33, 64, 100]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(CASES))
+def test_random_mixed_schedules_match_the_plain_implementation(tmp_path, name, dt):
+    from litinfer_amd.engine import Engine
+    cfg, page0, seed = CASES[name]
+    d = helpers.make_model(tmp_path, cfg, seed, torch.float32 if dt == "float32" else torch.bfloat16)
+    worst = 0.0
+    for trial in range(5):
+        rng = np.random.default_rng(1000 * trial + seed)
+        lengths = [min(int(x), int(cfg["max_position_embeddings"])) for x in rng.choice(LENGTHS, int(rng.integers(3, 9)))]
+        reqs = helpers.random_requests(cfg["vocab_size"], lengths, 77 + trial)
+        ref = helpers.plain_logits(d, reqs)
+        portions = tuple(int(x) for x in rng.choice(PORTIONS, 5))
+        page = int(rng.choice([page0, 1, 4, 16, 32])) if trial % 2 else page0
+        steps = schedules.mixed(reqs, max_live=int(rng.integers(1, 5)), seed=trial, prefill_chunks=portions,
+                                decode_after=float(rng.choice([0.2, 0.6, 0.9])))
+        eng = Engine.from_dir(d, dtype=dt, device="cuda:0", page_size=page, max_seqs=4, page_order_seed=trial,
+                              max_tokens=schedules.max_live_tokens(reqs, steps, page))
+        out = schedules.run(eng, reqs, steps)
+        eng.cache.check_invariants()
+        assert all(f == g.pool.capacity for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
+        err = max(schedules.rel_err(out[r], ref[r]) for r in reqs)
+        assert err < TOL[dt], f"{name} {dt} trial {trial}: lengths {lengths}, portions {portions}, page {page}: {err}"
+        worst = max(worst, err)
+    print(f"[observed] {name} {dt}: {worst:.3e}")
+
+
+EDGES = [1, 2, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 255, 256, 257, 511, 513, 1023, 1024, 1025, 2047,
+         2049, 3000, 4095, 4097, 6000]
+LAYOUTS = [(28, 4, 128), (12, 2, 128), (40, 8, 128), (14, 2, 64), (7, 7, 128), (40, 2, 64), (16, 1, 128)]
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_decode_batches_match_the_plain_attention(ops, block):
+    from litinfer_amd.engine.workspace import Workspace
+    ws = Workspace("cuda:0")
+    rng = np.random.default_rng(5 + block)
+    for trial in range(30):
+        nh, nkv, dh = LAYOUTS[int(rng.integers(len(LAYOUTS)))]
+        page = int(rng.choice([1, 3, 5, 8, 12, 16, 16, 16, 24, 48, 64]))
+        window = int(rng.choice([0, 0, 0, 40, 300, 1000]))
+        nreq = int(rng.choice([1, 2, 3, 8, 17, 40]))
+        longest = 1500 if page == 1 else 10 ** 9
+        first = min(int(rng.choice(EDGES)), longest)
+        equal = rng.random() < 0.4
+        segs = [(first if equal else min(int(rng.choice(EDGES)), longest), 1) for _ in range(nreq)]
+        if rng.random() < 0.2:                         # a portion of a prompt beside the decoding requests
+            a, b = int(rng.choice([70, 300, 700])), int(rng.choice([2, 33, 70]))
+            segs.append((max(a, b), min(a, b)))
+        dtype = torch.bfloat16 if rng.random() < 0.6 else torch.float32
+        pad = bool(rng.random() < 0.3) and all(q == 1 for _, q in segs)
+        out, ref = kernel_cases._paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=100 * block + trial,
+                                            ws=ws if rng.random() < 0.8 else None, pad_pow2=pad)
+        err = kernel_cases.rel(out, ref)
+        assert err < kernel_cases.tol(dtype, 3e-6, 1.5e-2), (
+            f"block {block} trial {trial}: {dtype} heads {nh}/{nkv}/{dh} page {page} window {window} widened {pad} "
+            f"(context, tokens) {segs}: {err}")
