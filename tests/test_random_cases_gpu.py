@@ -87,3 +87,33 @@ def test_random_decode_batches_match_the_plain_attention(ops, block):
         assert err < kernel_cases.tol(dtype, 3e-6, 1.5e-2), (
             f"block {block} trial {trial}: {dtype} heads {nh}/{nkv}/{dh} page {page} window {window} widened {pad} "
             f"(context, tokens) {segs}: {err}")
+
+
+PROMPT_LAYOUTS = [(28, 4, 128), (12, 2, 128), (40, 8, 128), (14, 2, 64), (7, 7, 128), (20, 2, 64), (6, 1, 128), (9, 1, 64)]
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_random_prompt_portions_match_the_plain_attention(ops, block):
+    """Portions of 2 to 400 queries behind 0 to 4,000 cached keys, one to five requests a call, now and then a
+    decoding request beside them."""
+    from litinfer_amd.engine.workspace import Workspace
+    ws = Workspace("cuda:0")
+    rng = np.random.default_rng(11 + block)
+    for trial in range(40):
+        nh, nkv, dh = PROMPT_LAYOUTS[int(rng.integers(len(PROMPT_LAYOUTS)))]
+        page = int(rng.choice([1, 3, 5, 8, 12, 16, 16, 16, 24, 48, 64]))
+        window = int(rng.choice([0, 0, 0, 40, 300, 1000]))
+        segs = []
+        for _ in range(int(rng.choice([1, 1, 2, 3, 5]))):
+            q = int(rng.choice([2, 3, 31, 32, 33, 64, 65, 100, 257, 400]))
+            before = int(rng.choice([0, 0, 1, 31, 32, 33, 500, 1500, 4000]))
+            segs.append(((min(before, 700) if page == 1 else before) + q, q))
+        if rng.random() < 0.3:
+            segs.append((int(rng.choice([1, 33, 900])), 1))
+        dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float32
+        out, ref = kernel_cases._paged_case(ops, dtype, segs, nh, nkv, dh, page, window, seed=100 * block + trial,
+                                            ws=ws if rng.random() < 0.8 else None)
+        err = kernel_cases.rel(out, ref)
+        assert err < kernel_cases.tol(dtype, 3e-6, 1.5e-2), (
+            f"block {block} trial {trial}: {dtype} heads {nh}/{nkv}/{dh} page {page} window {window} "
+            f"(context, tokens) {segs}: {err}")
