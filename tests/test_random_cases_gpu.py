@@ -117,3 +117,54 @@ def test_random_prompt_portions_match_the_plain_attention(ops, block):
         assert err < kernel_cases.tol(dtype, 3e-6, 1.5e-2), (
             f"block {block} trial {trial}: {dtype} heads {nh}/{nkv}/{dh} page {page} window {window} "
             f"(context, tokens) {segs}: {err}")
+
+
+ROWS = [1, 2, 7, 8, 12, 13, 16, 17, 31, 32, 33, 48, 64, 65, 100, 127, 128, 129, 200, 256, 257, 384, 385, 512, 700, 1000,
+        1024, 1100, 2048, 2100]
+COLUMNS = [16, 37, 64, 100, 128, 200, 224, 288, 301, 512, 1000, 1536, 2500, 3584, 4608, 4793, 6627, 9001]
+DEPTHS = [8, 16, 40, 64, 72, 96, 128, 192, 256, 264, 320, 512, 1160]
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_random_products_match_numpy(ops, block):
+    """x w^T at random sizes on both sides of every rule that picks a kernel or a tiling (rows, columns, K a
+    multiple of 64 or not, with and without lent memory for K in parts), with bias, into a float32 sum, and with
+    the SwiGLU epilogue."""
+    import math
+    import plain_impl
+    rng = np.random.default_rng(3 + block)
+    for trial in range(80):
+        m, n, k = int(rng.choice(ROWS)), int(rng.choice(COLUMNS)), int(rng.choice(DEPTHS))
+        if rng.random() < 0.1:
+            k = int(rng.choice([4, 36, 100, 90]))
+        dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float32
+        swiglu = dtype is torch.bfloat16 and rng.random() < 0.33 and ops.swiglu_takes(m, k, dtype)
+        g = torch.Generator().manual_seed(1000 * block + trial)
+        ws = kernel_cases._Lender() if rng.random() < 0.7 else None
+        if swiglu:
+            n = min(n, 4800)
+            x = (torch.randn(m, k, generator=g) * 2).to(dtype)
+            w = (torch.randn(2 * n, k, generator=g) / math.sqrt(k)).to(dtype)
+            y = x.double().numpy() @ w.double().numpy().T
+            ref = plain_impl.swiglu(y[:, :n], y[:, n:])
+            out = torch.full((m, n), float("nan"), dtype=dtype, device="cuda:0")
+            ops.linear_swiglu(x.to("cuda:0"), w.to("cuda:0"), out)
+            limit, what = 5e-3, f"with SwiGLU {m} x {n} x {k}"
+        else:
+            bias, acc = bool(rng.random() < 0.5), bool(rng.random() < 0.4)
+            x = torch.randn(m, k, generator=g).to(dtype)
+            w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(dtype)
+            b = torch.randn(n, generator=g) if bias else None
+            ref = plain_impl.linear(x.double().numpy(), w.double().numpy(), None if b is None else b.double().numpy())
+            if acc:
+                base = torch.randn(m, n, generator=g)
+                out = base.to("cuda:0")
+                ref = ref + base.double().numpy()
+            else:
+                wide = dtype is torch.float32 or rng.random() < 0.3
+                out = torch.full((m, n), float("nan"), dtype=torch.float32 if wide else dtype, device="cuda:0")
+            ops.linear(x.to("cuda:0"), w.to("cuda:0"), None if b is None else b.to("cuda:0"), out, accumulate=acc, ws=ws)
+            limit = 4 * math.sqrt(k) * 2.0 ** -24 if out.dtype is torch.float32 else 5e-3
+            what = f"{dtype} {m} x {n} x {k}, bias {bias}, into a sum {acc}, out {out.dtype}, lent memory {ws is not None}"
+        err = kernel_cases.rel(out, ref)
+        assert err < limit, f"block {block} trial {trial}: {what}: {err}"
