@@ -168,3 +168,39 @@ def test_random_products_match_numpy(ops, block):
             what = f"{dtype} {m} x {n} x {k}, bias {bias}, into a sum {acc}, out {out.dtype}, lent memory {ws is not None}"
         err = kernel_cases.rel(out, ref)
         assert err < limit, f"block {block} trial {trial}: {what}: {err}"
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_the_scheduler_with_random_budgets_and_pools_gives_the_plain_greedy_tokens(tmp_path, name):
+    """Random prompts and limits, portions of 4 to 33 tokens, budgets of one to three portions, 2 to 8 slots, a
+    pool that just holds the largest request, twice that or plenty (so that some runs preempt), steps started
+    ahead or not; float32, where a request's greedy tokens are the plain implementation's."""
+    import plain_impl
+    from litinfer_amd.engine import Engine, Scheduler
+    cfg, page, seed = CASES[name]
+    d = helpers.make_model(tmp_path, cfg, seed)
+    pcfg, weights = plain_impl.load_folder(d)
+    preempted = 0
+    for trial in range(8):
+        rng = np.random.default_rng(100 * trial + seed)
+        n = int(rng.integers(3, 9))
+        lens = [min(int(x), int(cfg["max_position_embeddings"]) - 12) for x in rng.choice([1, 2, 7, 16, 17, 33, 40, 64, 90], n)]
+        prompts = list(helpers.random_requests(cfg["vocab_size"], lens, 50 + trial).values())
+        limits = [int(x) for x in rng.choice([1, 2, 5, 9, 12], n)]
+        need = max(-(-(a + b) // page) * page for a, b in zip(lens, limits))
+        pool = int(rng.choice([need + page, 2 * need, 4096]))
+        portion = int(rng.choice([4, 8, 16, 33]))
+        eng = Engine.from_dir(d, dtype="float32", device="cuda:0", page_size=page, max_tokens=pool,
+                              max_seqs=int(rng.choice([2, 4, 8])))
+        s = Scheduler(eng, eos_token_ids=(), chunk_size=portion, max_batch_tokens=portion * int(rng.choice([1, 2, 3])),
+                      lookahead=bool(rng.random() < 0.5))
+        ids = [s.add_request(p, m) for p, m in zip(prompts, limits)]
+        while s.has_unfinished():
+            s.step()
+            assert s.steps < 5000, "the scheduler does not come to an end"
+        eng.cache.check_invariants()
+        assert all(f == g.pool.capacity for f, g in zip(eng.cache.free_pages(), eng.cache.groups))
+        for i, p, m in zip(ids, prompts, limits):
+            assert s.output(i) == plain_impl.greedy_generate(pcfg, weights, p, m), (name, trial, len(p), m, pool, portion)
+        preempted += s.preemptions
+    print(f"[observed] {name}: {preempted} preemptions over 8 runs")
