@@ -1016,3 +1016,21 @@ def test_sampling_table_rows_become_the_arrays_of_a_step_with_uniform_numbers_dr
             assert float(u[i]) == uniform(sp.seed, draws[slot] + step), (slot, step)
     counts = smp.table[:, 5].cpu().tolist()
     assert counts == [3, 8, 0, draws[3], 1000003, 0]               # slot 3 was greedy by flag: its count stayed
+
+
+def test_decode_attention_refuses_block_tables_beyond_the_keys_its_page_quotient_is_exact_for(ops):
+    """The matrix-core decode kernel finds a key's page by a float32 product that is exact below 2^22; the host
+    refuses a table that could hold more than 2^21 keys instead of reading a wrong page."""
+    nh, nkv, dh, page = 4, 2, 128, 16
+    width = (1 << 21) // page + 1
+    tab = torch.zeros(1, width, dtype=torch.int32, device=DEV)
+    one = lambda v: torch.tensor([v], dtype=torch.int32, device=DEV)
+    ql, cl, qs = np.array([1], np.int32), np.array([40], np.int32), np.array([0], np.int32)
+    meta = AttentionMeta(block_table=tab, max_blocks=width, seg_of_token=one(0), q_start=one(0), q_len=one(1),
+                         ctx_len=one(40), num_segments=1, num_tokens=1, max_q_len=1, max_ctx_len=40, host_q_start=qs,
+                         host_q_len=ql, host_ctx_len=cl, single_tokens=None, num_single=1, multi_tokens=None,
+                         num_multi=0, max_single_ctx=40)
+    kc = torch.zeros(4, nkv, page, dh, dtype=torch.bfloat16, device=DEV)
+    q = torch.zeros(1, nh * dh, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="beyond the decode kernel"):
+        ops.paged_attention(q, torch.empty_like(q), kc, kc.clone(), meta, nh, nkv, dh, page, 0, 0.1)
