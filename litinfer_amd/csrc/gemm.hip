@@ -828,7 +828,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                                                              TO* __restrict__ out, int M, int N, int K,
                                                              int accumulate, int nsplit,
                                                              const float* __restrict__ row_parts, int nparts, float eps) {
-    // row_parts (SwiGLU tiles of 64 rows, up to 16 rows of x): x is the xg of li_linear_residual_norm and these
+    // row_parts (SwiGLU tiles of 64 rows, up to 32 rows of x): x is the xg of li_linear_residual_norm and these
     // are its sq_parts; every row's sums are scaled by 1 / sqrt(sum of the row's parts / K + eps) before the
     // activation, which makes the result that of the RMS norm (the factor of a row does not depend on k).
     // nsplit > 1: a block multiplies one of nsplit parts of K, the y-th, and writes its sums to the y-th
@@ -858,16 +858,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     // past the last reads the last and is not added), before the first loads of the main loop: a wave's loads
     // retire in order, so they have arrived when the first stage has, and the waits placed by hand below
     // still count the main loop's loads only.  They are added up behind the main loop.
-    constexpr int RS_PER = ROWSCALE ? 32 : 1;          // shares a thread adds: 512 at most, 16 threads a row
+    constexpr int RS_PER = ROWSCALE ? 64 : 1;          // shares a thread adds: 512 at most, 16 or 8 threads a row
     [[maybe_unused]] float rs_part[RS_PER];
+    [[maybe_unused]] const int rs_rows = M <= 16 ? 16 : 32;      // rows the shares are kept for (as the product before the norm wrote them)
+    [[maybe_unused]] const int rs_groups = 256 / rs_rows;
     if constexpr (ROWSCALE) {
         if (row_parts) {
-            const int r = threadIdx.x & 15, g = threadIdx.x >> 4;
+            const int r = threadIdx.x % rs_rows, g = threadIdx.x / rs_rows;
 #pragma unroll
             for (int i = 0; i < RS_PER; ++i) {
-                const int p = g + 16 * i;
+                const int p = g + rs_groups * i;
                 rs_part[i] = 0.f;
-                if (16 * i < nparts) rs_part[i] = row_parts[(size_t)(p < nparts ? p : nparts - 1) * 16 + r];      // (the same for all lanes)
+                if (rs_groups * i < nparts) rs_part[i] = row_parts[(size_t)(p < nparts ? p : nparts - 1) * rs_rows + r];      // (the same for all lanes)
             }
         }
     }
@@ -1034,20 +1036,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
     [[maybe_unused]] float* row_inv = nullptr;
     if constexpr (ROWSCALE) {
         // the rows' factors, in the order of additions of the few-row kernel with four waves: thread t adds the
-        // shares t / 16, t / 16 + 16, ... of row t % 16, thread r < 16 the 16 sums of row r
-        __shared__ float inv_s[16], part_s[16][16];
+        // shares t / R, t / R + 256 / R, ... of row t % R (R = 16 rows, or 32), thread r < R the sums of row r
+        __shared__ float inv_s[32], part_s[256];
         row_inv = inv_s;
         if (row_parts) {
-            const int r = threadIdx.x & 15, g = threadIdx.x >> 4;
+            const int r = threadIdx.x % rs_rows, g = threadIdx.x / rs_rows;
             float mine = 0.f;
 #pragma unroll
-            for (int i = 0; i < RS_PER; ++i) mine += (g + 16 * i < nparts) ? rs_part[i] : 0.f;
-            part_s[g][r] = mine;
+            for (int i = 0; i < RS_PER; ++i) mine += (g + rs_groups * i < nparts) ? rs_part[i] : 0.f;
+            part_s[g * rs_rows + r] = mine;
             __syncthreads();
-            if (threadIdx.x < 16) {
-                float sq = part_s[0][threadIdx.x];
-#pragma unroll
-                for (int q = 1; q < 16; ++q) sq += part_s[q][threadIdx.x];
+            if ((int)threadIdx.x < rs_rows) {
+                float sq = part_s[threadIdx.x];
+                for (int q = 1; q < rs_groups; ++q) sq += part_s[q * rs_rows + threadIdx.x];
                 inv_s[threadIdx.x] = 1.0f / sqrtf(sq / (float)K + eps);
             }
             __syncthreads();
@@ -1085,7 +1086,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                 const float* us = &uband[(16 * (wave & 1) + rr) * ES + ecol];
                 float v[8];
                 float f = 1.0f;
-                if constexpr (ROWSCALE) f = row_parts ? row_inv[row & 15] : 1.0f;      // (row_parts: M <= 16, so row < 16 here)
+                if constexpr (ROWSCALE) f = row_parts ? row_inv[row & 31] : 1.0f;      // (row_parts: M <= 32, so row < 32 here)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = swiglu_bf16(gs[e] * f, us[e] * f);
                 const size_t o_idx = (size_t)row * NO + col;
@@ -1122,8 +1123,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const bf16_t* __rest
                 for (int r = 0; r < 16; ++r) {
                     float gv = acc[i][j][r], uv = acc[i][j + 1][r];
                     if constexpr (ROWSCALE) {
-                        if (row_parts) {                 // (M <= 16: only the tile's first 16 rows are written)
-                            const float f = row_inv[(wm + 32 * i + 8 * (r >> 2) + crow + (r & 3)) & 15];
+                        if (row_parts) {                 // (M <= 32: only the tile's first 32 rows are written)
+                            const float f = row_inv[(wm + 32 * i + 8 * (r >> 2) + crow + (r & 3)) & 31];
                             gv *= f;
                             uv *= f;
                         }
@@ -1181,7 +1182,7 @@ template <int BM, int BN, int BK, int NSTAGE, bool SWIGLU, typename TO, int WLM 
 static int launch_dma(const bf16_t* x, const bf16_t* w, const float* bias, TO* out, int M, int N, int K,
                       int accumulate, hipStream_t stream, int nsplit = 1, const float* row_parts = nullptr,
                       int nparts = 0, float eps = 0.f) {
-    if (row_parts && !(SWIGLU && BM == 64 && M <= 16 && nparts > 0)) return LI_ERR_SIZE;
+    if (row_parts && !(SWIGLU && BM == 64 && M <= 32 && nparts > 0)) return LI_ERR_SIZE;
     const long mtiles = (M + BM - 1) / BM, ntiles = (N + BN - 1) / BN;
     if (nsplit < 1 || nsplit > 65535 || nsplit > K / BK) return LI_ERR_SIZE;
     const long blocks = TileOrder::blocks(mtiles, ntiles, nsplit);
@@ -1316,14 +1317,15 @@ struct SkinnyArgs {
     bf16_t* kc;
     bf16_t* vc;
     int nh, nkv, dh, page_size, num_pages;
-    // An RMS norm between two products of up to 16 rows, without a pass of its own.  The product
+    // An RMS norm between two products of up to 32 rows, without a pass of its own.  The product
     // BEFORE it (float out with accumulate: the residual sum) also writes xg[m, n] = bf16(gamma[n] *
-    // out[m, n]) and, per block, the sums of squares of its columns of out to sq_parts[block * 16 + m].
+    // out[m, n]) and, per block, the sums of squares of its columns of out to sq_parts[block * R + m],
+    // R = 16 up to 16 rows and 32 above.
     const float* gamma;
     bf16_t* xg;
     float* sq_parts;
     // The product AFTER it takes such an xg as its x and scales row m's sums by
-    // 1 / sqrt(sum_p row_parts[p * 16 + m] / K + eps): the factor of a row does not depend on k.
+    // 1 / sqrt(sum_p row_parts[p * R + m] / K + eps): the factor of a row does not depend on k.
     const float* row_parts;
     int nparts;
     float eps;
@@ -1335,9 +1337,13 @@ struct SkinnyArgs {
 
 template <int MT, int NT, int WAVES, bool SWIGLU, typename TO, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs a) {
-    static_assert(!ROPE || (MT == 1 && !SWIGLU), "the rotary epilogue takes one tile of rows");
+    static_assert(!ROPE || (MT <= 2 && !SWIGLU), "the rotary epilogue takes one or two tiles of rows");
+    static_assert(MT <= WAVES, "wave mt writes the results of row tile mt");
     __shared__ floatx4 red[WAVES][MT * NT][64];
-    __shared__ float part_sums[WAVES * 4][16];
+    __shared__ float part_sums[WAVES * 64];          // [group of threads][row]: the rows' sums of squares, a share a group
+    // rows that the shares of the sums of squares are kept for, a block and a step: 16 up to 16 rows, else 32
+    // (the products on both sides of a norm see the same M)
+    constexpr int RP = MT <= 1 ? 16 : 32;
     const int M = a.M, N = a.N, K = a.K;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // (the same for a wave's lanes: its branches are scalar)
     const int g = lane >> 4, r16 = lane & 15;
@@ -1383,12 +1389,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
     // weights, the rotation's cosines and sines, the page slot) is asked for now, by the wave
     // that will write the results: the answers arrive with the first chunk, and the epilogue
     // waits for no memory.  Never conditional per lane: a place past the end reads the last one.
-    constexpr bool PRE = MT == 1 && !SWIGLU;
+    constexpr bool PRE = MT <= 2 && !SWIGLU;        // (wave mt writes row tile mt: thread t of the epilogue is lane t % 64 of wave t / 64)
     float pre_bias[NT][4], pre_res[NT][4], pre_gamma[NT][4], pre_cos[NT][4], pre_sin[NT][4];
     int pre_slot = 0;
     if constexpr (PRE) {
-        if (wave == 0) {
-            const int m = (lane & 15) < M ? (lane & 15) : M - 1;
+        if (wave < MT) {
+            const int m = 16 * wave + (lane & 15) < M ? 16 * wave + (lane & 15) : M - 1;
             if constexpr (ROPE) {
                 const bool second = (lane >> 4) >= 2;
                 pre_slot = a.slot_map[m];
@@ -1488,26 +1494,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
         // those of the first chunk, only as many rounds as there are parts, and never conditional
         // within a round (a part past the end reads the last one).  They are added up behind the
         // loads of the second chunk: the wait for them is the wait the first multiplication has anyway.
-        constexpr int G = WAVES * 4, PER = SK_MAX_PARTS / G;
+        constexpr int G = WAVES * 64 / RP, PER = SK_MAX_PARTS / G;
         float part[PER];
         if (a.row_parts) {
-            const int m = threadIdx.x & 15, q = threadIdx.x >> 4;
+            const int m = threadIdx.x % RP, q = threadIdx.x / RP;
 #pragma unroll
             for (int i = 0; i < PER; ++i) {
                 part[i] = 0.f;
                 if (i * G < a.nparts) {
                     const int p = q + i * G;
-                    part[i] = a.row_parts[(size_t)(p < a.nparts ? p : a.nparts - 1) * 16 + m];
+                    part[i] = a.row_parts[(size_t)(p < a.nparts ? p : a.nparts - 1) * RP + m];
                 }
             }
         }
         if (wave + WAVES < nfull) load_chunk(wave + WAVES, wbuf[1], xbuf[1], std::false_type{});
         if (a.row_parts) {
-            const int m = threadIdx.x & 15, q = threadIdx.x >> 4;
+            const int m = threadIdx.x % RP, q = threadIdx.x / RP;
             float mine = 0.f;
 #pragma unroll
             for (int i = 0; i < PER; ++i) mine += (q + i * G < a.nparts) ? part[i] : 0.f;
-            part_sums[q][m] = mine;
+            part_sums[q * RP + m] = mine;
         }
         // (the first turn is written out: its loads of the second chunk stand above, before the parts are added up)
         if (wave < nfull) multiply(wbuf[0], xbuf[0]);
@@ -1563,9 +1569,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
             }
         }
         if (AHEAD && a.row_parts) {
-            float sq = part_sums[0][m & 15];
+            float sq = part_sums[m % RP];
 #pragma unroll
-            for (int q = 1; q < WAVES * 4; ++q) sq += part_sums[q][m & 15];
+            for (int q = 1; q < WAVES * 64 / RP; ++q) sq += part_sums[q * RP + m % RP];
             const float inv = 1.0f / sqrtf(sq / (float)K + a.eps);
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) { s[nt][0] *= inv; s[nt][1] *= inv; s[nt][2] *= inv; s[nt][3] *= inv; }
@@ -1573,7 +1579,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
         if constexpr (ROPE) {
             const int dh = a.dh;
             const bool second = (l >> 4) >= 2;                       // this lane holds the pairs' second members
-            const int slot = pre_slot;                               // (MT is 1: thread t is lane l of wave 0, which asked for these)
+            const int slot = pre_slot;                               // (thread t is lane l of wave mt, which asked for these)
             const int page = slot / a.page_size, in_page = slot - page * a.page_size;
             const bool page_ok = page >= 0 && page < a.num_pages;
 #pragma unroll
@@ -1611,7 +1617,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                 }
             }
         } else {
-            if constexpr (sizeof(TO) == 4 && MT == 1) {
+            if constexpr (sizeof(TO) == 4 && MT <= 2) {
                 if (a.xg) {                          // the sum goes out three ways (see SkinnyArgs)
                     float sq = 0.f;
 #pragma unroll
@@ -1630,7 +1636,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(SkinnyArgs
                     // the four lanes of a row (l, l ^ 16, l ^ 32, l ^ 48: all of them are here, or none)
                     sq += __shfl_xor(sq, 16, 64);
                     sq += __shfl_xor(sq, 32, 64);
-                    if ((l >> 4) == 0) a.sq_parts[(size_t)blockIdx.x * 16 + m] = sq;
+                    if ((l >> 4) == 0) a.sq_parts[(size_t)blockIdx.x * RP + m] = sq;
                     continue;
                 }
             }
@@ -1728,8 +1734,9 @@ extern "C" int li_linear_skinny(const void* x, const void* w, const float* bias,
 }
 
 // The product before an RMS norm that is fused into its neighbours (see SkinnyArgs): out += x w^T + bias
-// in float32, xg = bf16(gamma * out), sq_parts[block * 16 + m] = the block's share of row m's sum of
-// squares.  Up to 16 rows.  li_residual_norm_parts(N) is the number of blocks, i.e. of parts.
+// in float32, xg = bf16(gamma * out), sq_parts[block * R + m] = the block's share of row m's sum of
+// squares (R = 16 up to 16 rows, 32 above).  Up to 32 rows.  li_residual_norm_parts(N) is the number of
+// blocks, i.e. of parts.
 extern "C" int li_residual_norm_parts(int N) {
     int per = 32;                                      // as launch_skinny tiles the columns of few rows
     if (N < 8192) { per = balanced_per_block(N, 16); per = per ? per : 16; }
@@ -1738,7 +1745,7 @@ extern "C" int li_residual_norm_parts(int N) {
 
 extern "C" int li_linear_residual_norm(const void* x, const void* w, const float* bias, float* out, int M, int N,
                                        int K, const float* gamma, void* xg, float* sq_parts, hipStream_t stream) {
-    if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K % 8) || !gamma || !xg || !sq_parts) return LI_ERR_SIZE;
+    if (M <= 0 || M > 32 || N <= 0 || K <= 0 || (K % 8) || !gamma || !xg || !sq_parts) return LI_ERR_SIZE;
     if (li_residual_norm_parts(N) > SK_MAX_PARTS) return LI_ERR_SIZE;
     SkinnyArgs a{(const bf16_t*)x, (const bf16_t*)w, bias, out, M, N, K, 1,
                  nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, gamma, (bf16_t*)xg, sq_parts, nullptr, 0, 0.f};
@@ -1763,9 +1770,22 @@ extern "C" int li_linear_residual_norm(const void* x, const void* w, const float
 // of 16 requests at the 7B sizes 4.28 against 4.43 ms, at the 1.5B sizes 2.22 against 1.94 ms).
 #define FEW_ROWS_FUSED 12
 #define FEW_ROWS_LARGE_BYTES (100l << 20)
+// 17 to 32 rows (two tiles of rows a block, the fused epilogues as with one): every block reads all of x, 32
+// rows of it now, so the few-row kernel wins only against small matrices, and of those with long rows only
+// against the smallest.  Alone, tiles with their adding-up kernel against the few-row kernel at 24 rows: the
+// 7B's q/k/v (33 MB) 12.4 / 8.7 us and o 12.3 / 8.5; the 1.5B's q/k/v 11.6 / 6.4, o 11.8 / 6.6, gate/up (55 MB)
+// 16.8 / 15.7, down (27 MB, rows of 8,960) 14.2 / 12.9; the 3B's down (45 MB, rows of 11,008) 17.6 / 19.0; the
+// 14B's q/k/v (73 MB) 19.7 / 19.5 and o (52 MB, rows of 5,120) 16.9 / 17.6.
+#define FEW_ROWS_TWO_TILES 32
+#define FEW_ROWS_TWO_TILES_BYTES (56l << 20)
+#define FEW_ROWS_TWO_TILES_LONG_K 4096
+#define FEW_ROWS_TWO_TILES_LONG_K_BYTES (32l << 20)
 #define SWIGLU_TILES_BYTES (160l << 20)      // (see li_linear_swiglu)
 extern "C" int li_few_rows_preferred(int M, long N, long K) {
-    return M <= FEW_ROWS_FUSED || (M <= 16 && N * K * 2 < FEW_ROWS_LARGE_BYTES);
+    if (M <= FEW_ROWS_FUSED || (M <= 16 && N * K * 2 < FEW_ROWS_LARGE_BYTES)) return 1;
+    if (M > FEW_ROWS_TWO_TILES || K % 8) return 0;
+    const long bytes = N * K * 2;
+    return bytes <= FEW_ROWS_TWO_TILES_BYTES && (K <= FEW_ROWS_TWO_TILES_LONG_K || bytes <= FEW_ROWS_TWO_TILES_LONG_K_BYTES);
 }
 
 static bool mid_rows_take(int M, int N, int K) {
@@ -2047,7 +2067,7 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
                                 const float* row_parts, int nparts, float eps, hipStream_t stream) {
     if (M <= 0 || I <= 0 || K <= 0 || I > 0x3fffffff) return LI_ERR_SIZE;
     const int N = 2 * I;
-    if (row_parts && (M > 16 || (K % 8) || nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f)) return LI_ERR_SIZE;
+    if (row_parts && (M > 32 || (K % 8) || nparts <= 0 || nparts > SK_MAX_PARTS || eps < 0.f)) return LI_ERR_SIZE;
     // Up to 64 rows the product waits for w.  From 17 rows on (more than the few-row kernel's fused form takes),
     // and from 13 on where the matrix is large (li_few_rows_preferred: the 7B's at 16 rows 51.8 against 59.6 us),
     // it goes to tiles of 64 rows if the matrix has tiles enough to fill the chip: the width with the least
@@ -2122,7 +2142,7 @@ extern "C" int li_linear_swiglu(const void* x, const void* w, void* out, int M, 
 #undef LI_DMA
 }
 
-// The packed q/k/v projection of up to 16 rows with the half-split rotary encoding of query and key
+// The packed q/k/v projection of up to 32 rows with the half-split rotary encoding of query and key
 // heads and the write of keys and values into their page slots as its epilogue (see ROPE above).
 // w [(nh + 2 nkv) dh, K] bfloat16, bias float32 or null, out [M, (nh + 2 nkv) dh] bfloat16 (rotated
 // q, rotated k, v), cos/sin float32 [M, dh / 2], slot_map int32 [M], kc/vc the cache layer.
@@ -2131,7 +2151,7 @@ extern "C" int li_linear_rope_store(const void* x, const void* w, const float* b
                                     const float* cos, const float* sin, const int* slot_map, void* kc, void* vc,
                                     int nh, int nkv, int dh, int page_size, int num_pages,
                                     const float* row_parts, int nparts, float eps, hipStream_t stream) {
-    if (M <= 0 || M > 16 || K <= 0 || K % 8 || nh <= 0 || nkv <= 0 || dh <= 0 || dh % 16 || page_size <= 0 ||
+    if (M <= 0 || M > 32 || K <= 0 || K % 8 || nh <= 0 || nkv <= 0 || dh <= 0 || dh % 16 || page_size <= 0 ||
         num_pages <= 0 || (long)(nh + 2 * nkv) * dh > 0x7fffffffL)
         return LI_ERR_SIZE;
     const int N = (nh + 2 * nkv) * dh;
@@ -2142,7 +2162,12 @@ extern "C" int li_linear_rope_store(const void* x, const void* w, const float* b
     const int pairs = N / 2;
     a.cols = balanced_per_block(pairs, 8);
     const int per = a.cols ? a.cols : 8, blocks = (pairs + per - 1) / per;
-    if (per > 8) gemm_bf16_skinny_kernel<1, 2, 8, false, bf16_t, true><<<blocks, 8 * 64, 0, stream>>>(a);
-    else gemm_bf16_skinny_kernel<1, 1, 8, false, bf16_t, true><<<blocks, 8 * 64, 0, stream>>>(a);
+    if (M <= 16) {
+        if (per > 8) gemm_bf16_skinny_kernel<1, 2, 8, false, bf16_t, true><<<blocks, 8 * 64, 0, stream>>>(a);
+        else gemm_bf16_skinny_kernel<1, 1, 8, false, bf16_t, true><<<blocks, 8 * 64, 0, stream>>>(a);
+    } else {                                            // (two tiles of rows: four waves, as for the plain product)
+        if (per > 8) gemm_bf16_skinny_kernel<2, 2, 4, false, bf16_t, true><<<blocks, 4 * 64, 0, stream>>>(a);
+        else gemm_bf16_skinny_kernel<2, 1, 4, false, bf16_t, true><<<blocks, 4 * 64, 0, stream>>>(a);
+    }
     return li_launch_status();
 }

@@ -403,11 +403,11 @@ def swiglu_takes(m: int, k: int, w_dtype: torch.dtype) -> bool:
 # bfloat16 and each block's share of the rows' sums of squares (`linear_residual_norm`); the product
 # after it multiplies those rows and scales each row's result by the norm's factor (`row_scale` of
 # `linear_swiglu` and `linear_rope_store`).
-RESIDUAL_NORM_MAX_ROWS = 16
+RESIDUAL_NORM_MAX_ROWS = 32
 RESIDUAL_NORM_MAX_PARTS = 512
-# The few-row kernels with their fused epilogues take up to 16 rows; at 13 to 16 rows the 64-row tiles with
-# K in parts (and the kernels that add the parts up doing the norm, the rotation and the page write) are
-# faster where the matrix is large.  Parts ask `few_rows_preferred` beside the `*_takes` of the few-row
+# The few-row kernels with their fused epilogues take up to 32 rows (two tiles of 16 a block); from 13 rows on
+# the 64-row tiles with K in parts (and the kernels that add the parts up doing the norm, the rotation and the
+# page write) are faster where the matrix is large, from 17 on also where it is of middling size.  Parts ask `few_rows_preferred` beside the `*_takes` of the few-row
 # kernels; the kernel library holds the rule (its own entry points decide by it too).
 
 
@@ -423,7 +423,7 @@ def few_rows_preferred(m: int, n: int, k: int) -> bool:
 
 class RowScale:
     """What the product after a fused RMS norm needs beside its rows: the shares of the rows' sums
-    of squares [nparts * 16] float32 and the norm's eps."""
+    of squares [nparts * R] float32 (R = 16 for up to 16 rows, 32 above) and the norm's eps."""
     def __init__(self, sq_parts: torch.Tensor, nparts: int, eps: float):
         self.sq_parts, self.nparts, self.eps = sq_parts, int(nparts), float(eps)
 
@@ -444,10 +444,15 @@ def residual_norm_takes(m: int, n: int, k: int, w_dtype: torch.dtype) -> bool:
             and residual_norm_parts(n) <= RESIDUAL_NORM_MAX_PARTS)
 
 
+def row_scale_rows(m: int) -> int:
+    """Places a block's shares of the rows' sums of squares take: 16 for up to 16 rows, 32 above."""
+    return 16 if m <= 16 else 32
+
+
 def linear_residual_norm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                          gamma: torch.Tensor, xg: torch.Tensor, sq_parts: torch.Tensor) -> int:
-    """out += x w^T + bias (float32); xg = bfloat16(gamma * out); sq_parts[p * 16 + m] = block p's
-    share of sum_n out[m, n]^2.  Returns the number of blocks p."""
+    """out += x w^T + bias (float32); xg = bfloat16(gamma * out); sq_parts[p * R + m] = block p's
+    share of sum_n out[m, n]^2 (R = `row_scale_rows(m)`).  Returns the number of blocks p."""
     _gpu(x, w, bias, out, gamma, xg, sq_parts)
     m, k = x.shape
     n = w.shape[0]
@@ -460,8 +465,8 @@ def linear_residual_norm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.
          "linear_residual_norm: bias must be float32 [N]")
     _chk(gamma.dtype is torch.float32 and gamma.shape == (n,) and gamma.is_contiguous(), "linear_residual_norm: gamma must be float32 [N]")
     parts = residual_norm_parts(n)
-    _chk(sq_parts.dtype is torch.float32 and sq_parts.is_contiguous() and sq_parts.numel() >= parts * 16,
-         "linear_residual_norm: sq_parts must be float32 with 16 places a block")
+    _chk(sq_parts.dtype is torch.float32 and sq_parts.is_contiguous() and sq_parts.numel() >= parts * row_scale_rows(m),
+         "linear_residual_norm: sq_parts must be float32 with 16 places a block (32 above 16 rows)")
     _run("gemm", "li_linear_residual_norm", x.data_ptr(), w.data_ptr(), 0 if bias is None else bias.data_ptr(),
          out.data_ptr(), m, n, k, gamma.data_ptr(), xg.data_ptr(), sq_parts.data_ptr())
     return parts
@@ -508,7 +513,8 @@ def _check_row_scale(what: str, m: int, row_scale: Optional[RowScale]):
     _chk(0 < m <= RESIDUAL_NORM_MAX_ROWS, f"{what}: a row scale goes with up to {RESIDUAL_NORM_MAX_ROWS} rows")
     _chk(0 < row_scale.nparts <= RESIDUAL_NORM_MAX_PARTS and row_scale.eps >= 0, f"{what}: row scale out of range")
     _chk(row_scale.sq_parts.dtype is torch.float32 and row_scale.sq_parts.is_contiguous()
-         and row_scale.sq_parts.numel() >= row_scale.nparts * 16, f"{what}: the row scale's parts must be float32 [nparts * 16]")
+         and row_scale.sq_parts.numel() >= row_scale.nparts * row_scale_rows(m),
+         f"{what}: the row scale's parts must be float32 [nparts * {row_scale_rows(m)}]")
     return row_scale.sq_parts.data_ptr(), row_scale.nparts, row_scale.eps
 
 
@@ -535,7 +541,7 @@ def linear_swiglu(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, row_scale
          *_check_row_scale("linear_swiglu", m, row_scale))
 
 
-ROPE_STORE_MAX_ROWS = 16
+ROPE_STORE_MAX_ROWS = 32
 
 
 def rope_store_takes(m: int, k: int, w_dtype: torch.dtype, dh: int, rotary_dim: int) -> bool:

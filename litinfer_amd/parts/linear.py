@@ -37,7 +37,7 @@ class Linear:
     def add_with_scaling(self, x: torch.Tensor, out: torch.Tensor, scaling, rows: torch.Tensor, ws):
         """out += x W^T + b; rows = scaling.weight * out.  Returns what the product
         behind the norm needs for the rows' factors."""
-        parts = ws.buffer("linear.sq_parts", (ops.RESIDUAL_NORM_MAX_PARTS * 16,), torch.float32)
+        parts = ws.buffer("linear.sq_parts", (ops.RESIDUAL_NORM_MAX_PARTS * ops.RESIDUAL_NORM_MAX_ROWS,), torch.float32)
         n = ops.linear_residual_norm(x, self.weight, self.bias, out, scaling.weight, rows, parts)
         return ops.RowScale(parts, n, scaling.eps)
 

@@ -148,7 +148,7 @@ def plain_cache():
 
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", list(CASES))
-@pytest.mark.parametrize("n_live", [8, 12, 13, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("n_live", [8, 12, 13, 16, 17, 24, 32, 33, 64])
 def test_decode_batches_match_the_plain_implementation(tiny_models, plain_cache, name, dt, n_live):
     cfg, page, seed = CASES[name]
     d = tiny_models[(name, dt)]
@@ -219,7 +219,7 @@ def model_7b(tmp_path_factory):
     return helpers.make_model(tmp_path_factory.mktemp("db7b"), SHAPE_7B, 21, torch.bfloat16)
 
 
-@pytest.mark.parametrize("n_live", [8, 13, 64])
+@pytest.mark.parametrize("n_live", [8, 13, 24, 64])
 def test_decode_batches_at_the_7b_layer_sizes(model_7b, n_live):
     """The sizes the benchmark times (two layers of them, a small vocabulary), in bfloat16."""
     toks, prompts = many_requests(SHAPE_7B["vocab_size"], n_live, 900 + n_live, long_every=16, longest=260)

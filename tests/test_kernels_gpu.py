@@ -294,6 +294,13 @@ def test_float32_few_row_product_with_swiglu_epilogue(ops, m, inter, k):
     (5, 200, 136, 301, 0.1),         # a ragged last block of 16 columns; an eps that counts
     (9, 264, 72, 8210, 1e-5),        # many outputs, ragged; fewer chunks of K than waves
     (4, 1096, 40, 9000, 1e-6),
+    (17, 3584, 512, 1024, 1e-6),     # two tiles of rows a block: the same three ways out, 32 places a block for the shares
+    (32, 1536, 8960, 8960, 1e-6),    # the 1.5B's sizes at 32 rows: few-row kernels on both sides
+    (24, 3584, 512, 18944, 1e-6),    # the 7B's gate/up at 24 rows: tiles of 64 x 192 scale 24 rows
+    (29, 5120, 128, 20480, 1e-5),    # gates and ups in two waves
+    (19, 8200, 64, 48, 1e-5),
+    (32, 200, 136, 301, 0.1),
+    (21, 264, 72, 8210, 1e-5),
 ])
 def test_rms_norm_shared_between_the_products_on_its_two_sides(ops, m, n, kprev, inter, eps):
     """x += h Wo^T leaves gamma * x and the shares of the rows' sums of squares; the gate/up product
@@ -308,13 +315,14 @@ def test_rms_norm_shared_between_the_products_on_its_two_sides(ops, m, n, kprev,
     assert ops.residual_norm_takes(m, n, kprev, wo.dtype)
     out = base.to(DEV)
     xg = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
-    parts = torch.full((ops.RESIDUAL_NORM_MAX_PARTS * 16,), float("nan"), device=DEV)
+    places = ops.row_scale_rows(m)                       # 16 up to 16 rows, 32 above
+    parts = torch.full((ops.RESIDUAL_NORM_MAX_PARTS * places,), float("nan"), device=DEV)
     nparts = ops.linear_residual_norm(h.to(DEV), wo.to(DEV), bias.to(DEV), out, gamma.to(DEV), xg, parts)
     assert nparts == ops.residual_norm_parts(n) <= ops.RESIDUAL_NORM_MAX_PARTS
     for i in range(m):
         assert rel(out[i], x[i]) < 1e-5, i
         assert rel(xg[i], gamma.double().numpy() * x[i]) < 2.0 ** -8, i
-    sq = parts[:nparts * 16].view(nparts, 16)[:, :m].double().sum(dim=0).cpu().numpy()
+    sq = parts[:nparts * places].view(nparts, places)[:, :m].double().sum(dim=0).cpu().numpy()
     assert np.allclose(sq, (x * x).sum(axis=1), rtol=1e-5)
     # the same sum as the product alone leaves it
     alone = base.to(DEV)
@@ -366,8 +374,8 @@ def test_rms_norm_shared_between_the_products_on_its_two_sides(ops, m, n, kprev,
         assert torch.equal(kc[sl // page, :, sl % page].cpu(), qv[i, nh:nh + nkv])
         assert torch.equal(vc[sl // page, :, sl % page].cpu(), qv[i, nh + nkv:])
     with pytest.raises(ValueError):                      # more rows than the kernels scale
-        ops.linear_swiglu(torch.zeros(17, n, dtype=torch.bfloat16, device=DEV), w.to(DEV),
-                          torch.empty(17, inter, dtype=torch.bfloat16, device=DEV), row_scale=scale)
+        ops.linear_swiglu(torch.zeros(33, n, dtype=torch.bfloat16, device=DEV), w.to(DEV),
+                          torch.empty(33, inter, dtype=torch.bfloat16, device=DEV), row_scale=scale)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -388,11 +396,14 @@ def test_the_rule_for_few_rows_is_the_same_in_the_library_and_in_the_host_stand_
     # parts ask the kernel library which kernels few rows should take; the stand-in that the host-side tests
     # run the parts with answers the same
     import torch_ops
-    for m in (1, 8, 12, 13, 16, 17, 64, 65):
-        for n, k in ((1536, 1536), (3584, 18944), (18944, 3584), (4608, 3584), (5120, 27648), (10240, 8192), (14000, 3745)):
+    for m in (1, 8, 12, 13, 16, 17, 24, 32, 33, 64, 65):
+        for n, k in ((1536, 1536), (3584, 18944), (18944, 3584), (4608, 3584), (5120, 27648), (10240, 8192), (14000, 3745),
+                     (17920, 1536), (1536, 8960), (2048, 11008), (5120, 5120), (7168, 5120), (22016, 2048), (300, 100)):
             assert ops.few_rows_preferred(m, n, k) == torch_ops.few_rows_preferred(m, n, k), (m, n, k)
     assert ops.few_rows_preferred(12, 3584, 18944) and not ops.few_rows_preferred(13, 3584, 18944)
-    assert ops.few_rows_preferred(16, 3584, 3584) and not ops.few_rows_preferred(17, 3584, 3584)
+    assert ops.few_rows_preferred(16, 3584, 3584) and ops.few_rows_preferred(32, 3584, 3584) and not ops.few_rows_preferred(33, 3584, 3584)
+    assert not ops.few_rows_preferred(17, 3584, 18944) and not ops.few_rows_preferred(17, 5120, 5120)
+    assert ops.few_rows_preferred(32, 1536, 8960) and not ops.few_rows_preferred(17, 2048, 11008)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -805,10 +816,16 @@ def test_projection_cut_along_k_with_rotary_encoding_and_page_write_in_the_addin
     (5, 35, 1, 80, 72, True),           # 1480 rotation pairs: 6 a block, blocks that straddle heads, a ragged last one
     (16, 40, 8, 128, 64, False),        # 3584 pairs: 14 a block, two tiles
     (2, 70, 1, 128, 40, True),          # more pairs than two tiles a compute unit hold: whole tiles again
+    (17, 28, 4, 128, 3584, True),       # two tiles of rows a block
+    (32, 12, 2, 128, 1536, True),
+    (25, 5, 5, 48, 120, False),
+    (31, 35, 1, 80, 72, True),
+    (20, 70, 1, 128, 40, False),
 ])
 def test_projection_with_rotary_encoding_and_page_write_as_its_epilogue(ops, t, nh, nkv, dh, k, bias):
     g = torch.Generator().manual_seed(16)
     n, page, pages = (nh + 2 * nkv) * dh, 8, 9
+    assert t <= page * pages
     x = (torch.randn(t, k, generator=g) * 2).to(torch.bfloat16)
     w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(torch.bfloat16)
     b = torch.randn(n, generator=g) if bias else None

@@ -144,11 +144,13 @@ def residual_norm_parts(n):
 
 
 def few_rows_preferred(m, n, k):
-    return m <= 12 or (m <= 16 and n * k * 2 < (100 << 20))
+    if m <= 12 or (m <= 16 and n * k * 2 < (100 << 20)):
+        return True
+    return m <= 32 and k % 8 == 0 and n * k * 2 <= (56 << 20) and (k <= 4096 or n * k * 2 <= (32 << 20))
 
 
 def residual_norm_takes(m, n, k, w_dtype):
-    return w_dtype is torch.bfloat16 and 0 < m <= 16 and k % 8 == 0 and residual_norm_parts(n) <= RESIDUAL_NORM_MAX_PARTS
+    return w_dtype is torch.bfloat16 and 0 < m <= 32 and k % 8 == 0 and residual_norm_parts(n) <= RESIDUAL_NORM_MAX_PARTS
 
 
 def linear_residual_norm(x, w, bias, out, gamma, xg, sq_parts):
@@ -156,8 +158,9 @@ def linear_residual_norm(x, w, bias, out, gamma, xg, sq_parts):
     xg.copy_((gamma * out).to(xg.dtype))
     per = 32 if out.shape[1] >= 8192 else 16
     parts = residual_norm_parts(out.shape[1])
-    for p in range(parts):                               # one share a block of columns, 16 places each
-        sq_parts[p * 16:p * 16 + out.shape[0]] = (out[:, p * per:(p + 1) * per] ** 2).sum(dim=1)
+    r = 16 if out.shape[0] <= 16 else 32
+    for p in range(parts):                               # one share a block of columns, 16 places each (32 above 16 rows)
+        sq_parts[p * r:p * r + out.shape[0]] = (out[:, p * per:(p + 1) * per] ** 2).sum(dim=1)
     return parts
 
 
@@ -166,7 +169,8 @@ def linear_then_norm(x, w, bias, out, gamma, eps, xn, ws):
 
 
 def _row_factors(row_scale, m, k):
-    sq = row_scale.sq_parts[:row_scale.nparts * 16].view(row_scale.nparts, 16)[:, :m].sum(dim=0)
+    r = 16 if m <= 16 else 32
+    sq = row_scale.sq_parts[:row_scale.nparts * r].view(row_scale.nparts, r)[:, :m].sum(dim=0)
     return (1.0 / torch.sqrt(sq / k + row_scale.eps))[:, None]
 
 
@@ -180,7 +184,7 @@ def linear_swiglu(x, w, out, row_scale=None):
 
 
 def rope_store_takes(m, k, w_dtype, dh, rotary_dim):
-    return w_dtype is torch.bfloat16 and 0 < m <= 16 and k % 8 == 0 and dh % 16 == 0 and rotary_dim == dh
+    return w_dtype is torch.bfloat16 and 0 < m <= 32 and k % 8 == 0 and dh % 16 == 0 and rotary_dim == dh
 
 
 def linear_rope_store_parts(*args, **kwargs):
