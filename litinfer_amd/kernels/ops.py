@@ -640,6 +640,12 @@ def _simd_count(device: torch.device) -> int:
 DECODE_QUAD = 4              # runs of a token's keys that one block of the matrix-core decode kernel takes, one a wave
 # measurements only: single-wave blocks and a merge kernel behind them, as before the blocks joined their runs
 _decode_single_waves = False
+# Share of the SIMDs that a step's waves must fill for the blocks of four waves (below).  Most batch sizes give a
+# number of runs whose waves fill the SIMDs nearly, not wholly (17 requests x 2 kv heads x 28 runs = 952 of
+# 1,024); asked for all of them, those took single-wave blocks and the merge kernel: 17 / 24 / 28 requests of
+# 4,096 keys at the 1.5B head layout 23.5 / 29.4 / 31.5 us a layer against 21.8 / 26.9 / 29.9 with the blocks of
+# four (7B layout, 28 requests: 53.6 against 50.0); from a half on the short contexts lose (17.0 against 16.0 us).
+_DECODE_FILLS = 0.7
 
 
 def decode_splits(pairs: int, keys: int, simds: int = _DEC_WAVES, quad: int = DECODE_QUAD) -> int:
@@ -769,7 +775,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k: torch.Tensor, v: to
             quad = DECODE_QUAD
             planned = decode_splits(n_single * nkv, keys, simds, quad)
             nsplit = _ragged_splits(planned, meta, window)
-            fills = n_single * nkv * nsplit >= simds
+            fills = n_single * nkv * nsplit >= _DECODE_FILLS * simds
             if (_decode_single_waves or nsplit > planned
                     or not (nsplit == DECODE_QUAD or (fills and (nsplit <= 32 or keys >= 8192)))):
                 quad = 1
