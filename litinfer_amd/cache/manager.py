@@ -310,6 +310,11 @@ class CacheManager:
         if self._lib.li_book_commit(self._book, self._handle(rid), int(n_new)) < 0:
             raise PagePoolError(self._error())
 
+    @property
+    def has_state(self) -> bool:
+        """Whether any mixer keeps per-request state of fixed size in this cache."""
+        return bool(self._entry_state)
+
     def rewind(self, rid, n: int) -> None:
         """Forget the last `n` tokens of `rid`: their positions will be computed and written
         again.  The pages stay with the request.  Refused (ValueError) where a windowed group has

@@ -58,7 +58,8 @@ class Engine:
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  max_seqs: int = 64, page_order_seed: Optional[int] = None,
                  config: Any = None, use_graphs: bool = True, graph_after: int = 4,
-                 keep_stored_precision: bool = False, max_graphs: int = 64, step_tokens: int = 2048):
+                 keep_stored_precision: bool = False, max_graphs: int = 64, step_tokens: int = 2048,
+                 pad_rows_to: int = 4):
         """keep_stored_precision: with dtype bfloat16, leave matrices that the checkpoint stores in
         32-bit or half precision in 32-bit (their products then run in the 32-bit kernels) instead of
         rounding them once to bfloat16 when they are bound."""
@@ -97,6 +98,8 @@ class Engine:
         # `max_graphs` recorded ones are kept
         self._graphs: "OrderedDict[Any, Any]" = OrderedDict()
         self.max_graphs = max(1, int(max_graphs))
+        # recorded steps of more than `pad_rows_to` requests take whole multiples of it (see `step`); 1: as they come
+        self.pad_rows_to = max(1, int(pad_rows_to))
         self._graph_generation = (-1, -1)
         self.graph_replays = 0
         self.graphs_recorded = 0
@@ -270,6 +273,24 @@ class Engine:
             raise
         decode_only = int(counts.max()) == 1
         key = self._graph_key(entries, handles) if decode_only else None
+        rows = None
+        if key is not None:
+            # A recorded step serves one number of requests.  Where requests come and go that number
+            # changes every few steps, and most steps would run eagerly or be recorded anew; so a batch
+            # is filled up to the next multiple of `pad_rows_to` with copies of its LAST entry: the
+            # copies read the same token, position, pages and table row, write the same key and value
+            # to the same place, and their logits are dropped.  Not where a mixer keeps state of fixed
+            # size (a copy would step the state a second time).
+            n = len(entries)
+            fill = -n % self.pad_rows_to if (n > self.pad_rows_to and not self.cache.has_state) else 0
+            if fill:
+                rows = sum(len(e.want) for e in entries)
+                last = entries[-1]
+                entries = list(entries) + [StepEntry(last.rid, last.tokens, [0], take=last.take)] * fill
+                step_handles = np.concatenate([handles, np.full(fill, handles[-1], dtype=handles.dtype)])
+                key = (n + fill, key[1] + fill, key[2])
+            else:
+                step_handles = handles
         if profiler.enabled:
             profiler.phase = "decode" if decode_only else "prefill"
         if self._trace:
@@ -281,7 +302,9 @@ class Engine:
             if key is None:
                 logits = self.model.forward(self._build_context(entries, handles=handles), cache)
             else:
-                logits = self._forward_graphed(key, self._build_context(entries, pad_blocks=key[2], handles=handles))
+                logits = self._forward_graphed(key, self._build_context(entries, pad_blocks=key[2], handles=step_handles))
+                if rows is not None:
+                    logits = logits[:rows] if rows else None
         except BaseException:
             for rid in admitted:
                 cache.release(rid)

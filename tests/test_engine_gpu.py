@@ -107,6 +107,52 @@ def test_recorded_decode_steps_equal_eager_ones_on_every_replay(models, dt):
     assert schedules.rel_err(outs[0][at].cpu().numpy()[0], ref["r5"][pos]) < TOL[dt]
 
 
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "E"])
+def test_recorded_steps_filled_up_with_copies_of_the_last_entry(models, name, dt):
+    """A recorded decode step of more than four requests is filled up to a multiple of four with copies of its
+    last entry, so that one recording serves several numbers of requests.  5 to 11 requests that come and go:
+    the logits of every request and step are the plain implementation's, requests that are never last and the
+    one that is copied alike, nothing is counted twice in the cache, and few shapes are recorded."""
+    from litinfer_amd.engine import StepEntry
+    cfg, page, _ = CASES[name]
+    d, _, _ = models[(name, dt)]
+    lengths = [40, 33, 47, 38, 52, 36, 44, 41, 35, 49, 43]
+    reqs = helpers.random_requests(cfg["vocab_size"], lengths, 123)
+    ref = helpers.plain_logits(d, reqs)
+    from litinfer_amd.engine import Engine
+    eng = Engine.from_dir(d, dtype=dt, device="cuda:0", page_size=page, max_tokens=16 * 64, max_seqs=12, graph_after=2)
+    assert eng.pad_rows_to == 4
+    names = list(reqs)
+    at = {}
+    for r in names[:5]:                                     # five start with 20 tokens each
+        eng.step([StepEntry(r, reqs[r][:20], [])])
+        at[r] = 20
+    worst, steps = 0.0, 0
+    waiting = names[5:]
+    while at:
+        if waiting and steps % 3 == 2:                      # another request joins, its prompt in one portion
+            r = waiting.pop(0)
+            eng.step([StepEntry(r, reqs[r][:20], [])])
+            at[r] = 20
+        live = [r for r in names if r in at]
+        out = eng.step([StepEntry(r, [reqs[r][at[r]]], [0]) for r in live])
+        assert out.shape[0] == len(live)                    # the copies' rows are not handed out
+        got = out.cpu().numpy()
+        for i, r in enumerate(live):
+            worst = max(worst, schedules.rel_err(got[i], ref[r][at[r]]))
+            at[r] += 1
+            assert eng.cache.cached_len(r) == at[r]
+            if at[r] == len(reqs[r]):
+                eng.finish(r)
+                del at[r]
+        steps += 1
+    eng.cache.check_invariants()
+    print(f"[observed] {name} {dt}: {worst:.3e}; {eng.graphs_recorded} recordings, {eng.graph_replays} replays in {steps} steps")
+    assert worst < TOL[dt]
+    assert eng.graph_replays > steps // 2 and eng.graphs_recorded <= 8
+
+
 @pytest.mark.parametrize("dt,name", [("bfloat16", "D"), ("bfloat16", "E"), ("float32", "B")])
 def test_a_long_prompt_in_portions_then_decoding(tmp_path, dt, name):
     """Thousands of positions: many tiles of queries, block tables of hundreds of pages, many
