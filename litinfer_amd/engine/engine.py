@@ -57,7 +57,7 @@ class Engine:
     def __init__(self, spec: ModelSpec, *, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: Optional[int] = None, max_tokens: Optional[int] = None,
                  max_seqs: int = 64, page_order_seed: Optional[int] = None,
-                 config: Any = None, use_graphs: bool = True, graph_after: int = 4,
+                 config: Any = None, use_graphs: bool = True, graph_after: int = 2,
                  keep_stored_precision: bool = False, max_graphs: int = 64, step_tokens: int = 2048,
                  pad_rows_to: int = 4):
         """keep_stored_precision: with dtype bfloat16, leave matrices that the checkpoint stores in
@@ -89,9 +89,11 @@ class Engine:
         # shape, and replayed: a step is some hundred small launches otherwise
         self.use_graphs = bool(use_graphs) and self.rt.device.type == "cuda" and not profiler.enabled
         # A decode step of a shape (requests, wanted rows, table widths) is recorded at its graph_after-th
-        # occurrence and replayed from then on; before that it runs eagerly.  Recording costs about as much
-        # as a few steps and drains the queue of work once: where requests come and go and a shape lasts
-        # a few steps, recording every shape at its second step costs more than replays give back.
+        # occurrence and replayed from then on; before that it runs eagerly (the first occurrence sizes the
+        # buffers).  The recording runs in the eager pass's place, on a stream of its own and without a
+        # device-wide wait (`_record`), so that a recorded step costs what an eager one costs: where requests
+        # come and go a shape lasts a few steps only, and a recording that cost several steps' time (as one
+        # made with `torch.cuda.graph` after the eager pass did) ate what the replays gave back.
         self.graph_after = max(2, int(graph_after))
         self._trace = trace_enabled()
         # shape -> ("seen", times) | ("graph", graph, its output), least recently used first; at most
@@ -100,6 +102,7 @@ class Engine:
         self.max_graphs = max(1, int(max_graphs))
         # recorded steps of more than `pad_rows_to` requests take whole multiples of it (see `step`); 1: as they come
         self.pad_rows_to = max(1, int(pad_rows_to))
+        self._record_stream = None
         self._graph_generation = (-1, -1)
         self.graph_replays = 0
         self.graphs_recorded = 0
@@ -332,6 +335,26 @@ class Engine:
         widths = tuple(max(16, 1 << (max(need, 1) - 1).bit_length()) for need in self.cache.max_table_len(handles))
         return (len(entries), sum(len(e.want) for e in entries), widths)
 
+    def _record(self, ctx: StepContext):
+        """The model's forward pass for `ctx` as a graph (nothing runs).  Recorded on a stream of its own,
+        as a capture must be, that waits for the step's stream and is waited for by it; without the
+        device-wide wait and the emptying of the allocator's cache that `torch.cuda.graph` begins with:
+        where requests come and go a shape is recorded every few steps, the device should not run dry
+        for it, and memory handed back to the driver is asked for again a step later."""
+        if self._record_stream is None:
+            self._record_stream = torch.cuda.Stream(self.rt.device)
+        here = torch.cuda.current_stream(self.rt.device)
+        self._record_stream.wait_stream(here)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(self._record_stream):
+            graph.capture_begin()
+            try:
+                out = self.model.forward(ctx, self.cache)
+            finally:
+                graph.capture_end()
+        here.wait_stream(self._record_stream)
+        return graph, out
+
     def _buffers_at(self):
         """Changes whenever a buffer that a recorded step may address has moved."""
         return (self.ws.generation, self._uploader.generation)
@@ -354,31 +377,33 @@ class Engine:
             state[1].replay()
             self.graph_replays += 1
             return state[2]
-        # the first steps of a shape run eagerly (the first sizes the buffers), the graph_after-th is recorded
-        logits = self.model.forward(ctx, self.cache)
-        if self._graph_generation != self._buffers_at():
-            # this pass itself made a buffer grow (a larger batch than any before): what was
-            # recorded for OTHER shapes addresses the old one
-            self._drop_graphs()
-            self._graph_generation = self._buffers_at()
+        # the first steps of a shape run eagerly (the first sizes the buffers); at its graph_after-th the
+        # step is recorded and the recording run in the eager pass's place
         seen = 1 if state is None else state[1] + 1
         graphs[key] = ("seen", seen)
         graphs.move_to_end(key)
+        logits = None
         if seen >= self.graph_after:
             made = self.ws.allocations
-            torch.cuda.synchronize(self.rt.device)
-            ctx.forget_shared()                   # what the eager pass prepared must be prepared in the graph too
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                out = self.model.forward(ctx, self.cache)
+            graph, out = self._record(ctx)
             if self._graph_generation != self._buffers_at() or self.ws.allocations != made:
                 # recording itself allocated (the buffer would live in the graph's own pool) or
                 # moved a buffer: do not keep it, and nothing recorded before it either
                 self._drop_graphs()
                 self._graph_generation = self._buffers_at()
+                ctx.forget_shared()               # (what the recording prepared has not run)
             else:
                 graphs[key] = ("graph", graph, out)
                 self.graphs_recorded += 1
+                graph.replay()
+                logits = out
+        if logits is None:
+            logits = self.model.forward(ctx, self.cache)
+            if self._graph_generation != self._buffers_at():
+                # this pass itself made a buffer grow (a larger batch than any before): what was
+                # recorded for OTHER shapes addresses the old one
+                self._drop_graphs()
+                self._graph_generation = self._buffers_at()
         # the least recently used shapes go: a long-lived engine sees hundreds of them, and every
         # recorded one holds its graph and its output buffer
         recorded = sum(1 for s in graphs.values() if s[0] == "graph")
